@@ -1,0 +1,150 @@
+"""Pins the oracle's extension formats (int8 per-channel, per-token int8
+activations, uint4 group-wise asymmetric, fp8 e4m3fn).  The reference
+implements none of these, so there are no reference vectors: each function is
+pinned against a library routine (numpy integer matmul, numpy float16,
+torch.float8_e4m3fn, numpy.round) or a brute-force numpy re-derivation written
+independently of the C code.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+
+def test_w8a8_int32_accumulators_vs_numpy():
+    rng = np.random.default_rng(0)
+    for M, N, K in [(1, 256, 256), (9, 8, 64), (5, 33, 4096)]:
+        xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        want = xq.astype(np.int32) @ w.astype(np.int32).T
+        assert np.array_equal(O.w8a8_acc_i32(xq, w), want)
+    # the extreme: every product 127*127 at K = 4096 stays inside int32
+    xq = np.full((1, 4096), 127, np.int8)
+    w = np.full((2, 4096), -127, np.int8)
+    assert (O.w8a8_acc_i32(xq, w) == -4096 * 127 * 127).all()
+
+
+def test_quantize_rows_i8_vs_numpy():
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((17, 64)).astype(np.float32)
+    x[3] = 0.0                      # absmax 0 -> scale 1, codes 0
+    x[4, :] = np.float32(0.5) * np.arange(64, dtype=np.float32) - 16   # ties at scale 1?  see below
+    x[4, 0] = -127.0                # absmax 127 -> scale exactly 1 -> halves are exact ties
+    q, s = O.quantize_rows_i8(x)
+    amax = np.abs(x).max(axis=1)
+    s_want = (amax / np.float32(127)).astype(np.float32)
+    s_want[s_want == 0] = 1
+    assert np.array_equal(s.view(np.uint32), s_want.view(np.uint32))
+    q_want = np.clip(np.round(x / s_want[:, None]), -127, 127).astype(np.int8)  # np.round: ties to even
+    assert np.array_equal(q, q_want)
+    assert not q[3].any() and s[3] == 1.0
+    assert q[4, 1] == -16 and q[4, 2] == -15  # -15.5 -> -16 (even), -15.0
+    assert (np.abs(q.astype(np.int32)) <= 127).all() and (np.abs(q).max(axis=1)[amax > 0] == 127).all()
+
+
+def test_w8_forward_fp32_and_fp64():
+    rng = np.random.default_rng(2)
+    M, N, K = 3, 40, 512
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    b = (rng.standard_normal(N) * 0.02).astype(np.float32)
+    exact = (x.astype(np.float64) @ w.astype(np.float64).T) * s.astype(np.float64) + b.astype(np.float64)
+    y64 = O.w8_forward_f64(w, s, x, b)
+    assert np.abs(y64 - exact).max() <= 1e-12 * np.abs(exact).max()
+    y = O.w8_forward_f32(w, s, x, b)
+    assert np.abs(y - exact).max() / np.sqrt((exact ** 2).mean()) < 1e-5
+    yr = O.w8_forward_f32(w, s, x, b, relu=True)
+    assert np.array_equal(yr, np.where(y > 0, y, np.float32(0)))
+    assert np.array_equal(O.w8_forward_f64(w, s, x, b, relu=True), np.where(y64 > 0, y64, 0.0))
+    # small integers: fp32 arithmetic is exact, so the result equals the integer closed form
+    xi = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    yi = O.w8_forward_f32(w, np.ones(N, np.float32), xi)
+    assert np.array_equal(yi, (xi.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32))
+
+
+def test_w8a8_epilogue_closed_form():
+    rng = np.random.default_rng(3)
+    M, N = 6, 10
+    acc = rng.integers(-2 ** 20, 2 ** 20, (M, N), dtype=np.int32)
+    sx = rng.uniform(1e-3, 1e-1, M).astype(np.float32)
+    sw = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    want = acc.astype(np.float32) * (sx[:, None] * sw[None, :]) + b[None, :]
+    assert np.array_equal(O.w8a8_epilogue(acc, sx, sw, b), want)
+    assert np.array_equal(O.w8a8_epilogue(acc, sx, sw, b, relu=True), np.where(want > 0, want, np.float32(0)))
+    assert np.array_equal(O.w8a8_epilogue(acc, sx, sw), acc.astype(np.float32) * (sx[:, None] * sw[None, :]))
+
+
+@pytest.mark.parametrize("K,group", [(960, 128), (2560, 128), (128, 32), (64, 128)])
+def test_w4g_dequantize_vs_bruteforce(K, group):
+    rng = np.random.default_rng(K + group)
+    N = 5
+    G = -(-K // group)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    z = rng.integers(0, 16, (N, G), dtype=np.uint8)
+    s = rng.uniform(1e-3, 1e-1, (N, G)).astype(np.float16)
+    codes = (q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8)
+    zp = np.zeros((N, (G + 1) // 2), np.uint8)
+    for g in range(G):
+        zp[:, g // 2] |= (z[:, g] << (4 * (g & 1))).astype(np.uint8)
+    got = O.w4g_dequantize(codes, s.view(np.uint16), zp, N, K, group)
+    want = np.empty((N, K), np.float32)
+    for n in range(N):
+        for k in range(K):
+            g = k // group
+            want[n, k] = (np.float32(q[n, k]) - np.float32(z[n, g])) * np.float32(s[n, g])
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    if K == 960:
+        assert G == 8  # ragged: the 8th group is 64 wide
+
+
+def test_e4m3_decode_all_codes_vs_torch():
+    codes = torch.arange(256, dtype=torch.uint8)
+    want = codes.view(torch.float8_e4m3fn).float().numpy()
+    got = O.e4m3_decode_table()
+    nan = np.isnan(want)
+    assert nan.sum() == 2 and np.array_equal(np.isnan(got), nan)  # 0x7F and 0xFF only: no infinities
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert got[0x7E] == 448.0 and got[0xFE] == -448.0 and got[0x01] == 2.0 ** -9
+
+
+def test_e4m3_encode_vs_torch_in_range_and_saturation():
+    rng = np.random.default_rng(4)
+    tbl = O.e4m3_decode_table()
+    fin = np.sort(tbl[:0x7F])
+    mids = ((fin[:-1].astype(np.float64) + fin[1:].astype(np.float64)) / 2).astype(np.float32)  # exact ties
+    x = np.concatenate([
+        np.clip(rng.standard_normal(40000).astype(np.float32), -448, 448),
+        (rng.standard_normal(20000) * 100).clip(-448, 448).astype(np.float32),
+        (rng.standard_normal(20000) * 1e-2).astype(np.float32),
+        fin, -fin, mids, -mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)),
+        np.array([0.0, -0.0, 448.0, -448.0, 2.0 ** -10, 2.0 ** -10 * 1.001, 2.0 ** -9, 1e-9], np.float32),
+    ])
+    x = x[np.abs(x) <= 448]
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = O.e4m3_encode(x)
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:10]
+    # saturating above the largest finite (BASELINE: "clipped to the e4m3 range")
+    big = np.array([449.0, 464.0, 480.0, 1e6, np.inf, -500.0, -np.inf], np.float32)
+    assert np.array_equal(O.e4m3_encode(big), np.array([0x7E, 0x7E, 0x7E, 0x7E, 0x7E, 0xFE, 0xFE], np.uint8))
+    assert (O.e4m3_encode(np.array([np.nan], np.float32))[0] & 0x7F) == 0x7F
+    # encode ∘ decode is the identity on every non-NaN code (−0 keeps its sign)
+    ok = ~np.isnan(tbl)
+    assert np.array_equal(O.e4m3_encode(tbl[ok]), np.arange(256, dtype=np.uint8)[ok])
+
+
+def test_fp8_forward_vs_numpy():
+    rng = np.random.default_rng(5)
+    M, N, K = 4, 9, 256
+    a = O.e4m3_encode(np.clip(rng.standard_normal((M, K)), -448, 448).astype(np.float32))
+    b = O.e4m3_encode(np.clip(rng.standard_normal((N, K)), -448, 448).astype(np.float32))
+    sa, sb = np.float32(0.37), np.float32(1.9)
+    fa = torch.from_numpy(a).view(torch.float8_e4m3fn).double().numpy()
+    fb = torch.from_numpy(b).view(torch.float8_e4m3fn).double().numpy()
+    want = (fa @ fb.T) * np.float64(sa * sb)
+    y64, ybf = O.fp8_forward_f64(a, b, sa, sb)
+    assert np.abs(y64 - want).max() <= 1e-12 * np.abs(want).max()
+    want_bf = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(ybf, want_bf)
