@@ -1,0 +1,186 @@
+/* noeira_qlinear.h — C ABI of libnoeira_qlinear.so, the MI355X (gfx950)
+ * implementation of noeira's quantized-linear inference path.
+ *
+ * The reference has no C ABI for this operator: its boundary is the Mojo
+ * `Module` surface implemented by `QLinear[IN, OUT]`
+ * (noeira/nn/quant/qlinear.mojo:208-524).  This header is what a Mojo host
+ * binds through the reference's own FFI idiom
+ *     var lib = OwnedDLHandle(path); var f = lib.get_function[c_int]("sym")
+ * (benchmarks/_test_cuda_ffi.mojo:61-80, noeira/io/serial/native.mojo:44-109).
+ * That idiom fixes the rules followed here: every function has a fixed arity
+ * (no variadics: noeira/io/serial/native.mojo:6-14), takes only integers,
+ * floats and raw addresses, and returns an int32 status (0 = NQ_OK).  Each
+ * entry point cites the reference method it stands in for.
+ *
+ * Conventions
+ *   - W is [OUT, IN] row-major (torch's orientation, qlinear.mojo:3), x is
+ *     [M, IN] row-major, y is [M, OUT] row-major, dense strides.
+ *   - Host pointers are named *_host; every other data pointer is a device
+ *     address valid on the current HIP device.
+ *   - `stream` is a hipStream_t passed as an address (NULL = the default
+ *     stream).  Compute entry points only enqueue: they never synchronise and,
+ *     after the first call at a given M, never allocate (the capture rule of
+ *     qlinear.mojo:60-68 gated by tests/nn/quant/test_qlinear_gpu.mojo:55-130).
+ *   - A layer handle is used by one host thread at a time; different handles
+ *     may be used from different threads/streams.  Identical inputs give
+ *     bit-identical outputs on every call (test_qlinear_gpu.mojo:96,128).
+ *   - On failure a function returns a non-zero status and leaves a sentence
+ *     for nq_last_error(); the wording follows the reference's `raise Error`
+ *     messages so a wrapper can re-raise them verbatim.
+ *   - This table is append-only; nq_abi_version() guards it.
+ */
+#ifndef NOEIRA_QLINEAR_H
+#define NOEIRA_QLINEAR_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NQ_ABI_VERSION 1
+
+/* status codes */
+#define NQ_OK 0
+#define NQ_ERR_INVALID 1     /* bad argument / shape / dtype combination */
+#define NQ_ERR_NOT_LOADED 2  /* forward before set_weight / set_blocks */
+#define NQ_ERR_NO_BLOCKS 3   /* logical blocks were dropped (keep_only_repacked) */
+#define NQ_ERR_SIZE 4        /* wrong byte count / scratch too small */
+#define NQ_ERR_HIP 5         /* a HIP runtime call failed */
+#define NQ_ERR_UNSUPPORTED 6
+
+/* weight formats */
+#define NQ_FMT_Q4_0 0        /* the reference's format: groups of 32 along IN,
+                                18-byte blocks [fp16 d][16 B nibbles], value
+                                (q-8)*d  (noeira/nn/quant/q4_0.mojo:1-8) */
+#define NQ_FMT_W8_CHANNEL 1  /* int8 [OUT, IN] + fp32 scale per output channel */
+#define NQ_FMT_W4_GROUP 2    /* uint4, 2 per byte (low nibble = even k), fp16
+                                scale and uint4 zero-point per group along IN */
+#define NQ_FMT_FP8_E4M3 3    /* OCP e4m3fn [OUT, IN] + one fp32 scale */
+
+/* element types of x, y, bias */
+#define NQ_DT_F32 0
+#define NQ_DT_BF16 1
+#define NQ_DT_I8 2        /* x only: int8 codes with a per-row fp32 scale */
+#define NQ_DT_FP8_E4M3 3  /* x only: e4m3fn codes with one fp32 scale */
+#define NQ_DT_I32 4       /* y only: raw int32 accumulators (W8 x I8) */
+
+/* epilogues (LinearAct's, noeira/nn/primitives/linear_act.mojo:81-115) */
+#define NQ_EPI_NONE 0
+#define NQ_EPI_RELU 1     /* z > 0 ? z : 0  (ops/relu_op.mojo:29-31) */
+
+typedef struct nq_layer* nq_handle;
+
+/* ---- library ----------------------------------------------------------- */
+
+/* NQ_ABI_VERSION of the loaded library ("APPEND ONLY" tables are an ABI in
+ * the reference: noeira/io/serial/native.mojo LAYOUT_N). */
+int32_t nq_abi_version(void);
+
+/* Copies the calling thread's last error sentence (NUL-terminated, truncated
+ * to n) and returns its full length.  Stands in for the Mojo `Error` a
+ * QLinear method raises (qlinear.mojo:276-281,334-338,358-369). */
+int64_t nq_last_error(char* buf, int64_t n);
+
+/* ---- layer lifecycle ---------------------------------------------------- */
+
+/* `QLinear[IN, OUT].make` (qlinear.mojo:253-260): an empty layer.  `group` is
+ * 32 for NQ_FMT_Q4_0 (IN % 32 == 0 is required, qlinear.mojo:243-245), the
+ * group width for NQ_FMT_W4_GROUP, ignored otherwise.  flags = 0. */
+int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t out_features,
+                  int32_t group, int32_t flags);
+
+/* Frees the layer's device and host storage. */
+int32_t nq_destroy(nq_handle h);
+
+/* `QLinear.set_blocks` (qlinear.mojo:271-320): load Q4_0 blocks
+ * [OUT, IN/32*18] from the host.  nbytes must equal OUT*(IN/32)*18, otherwise
+ * NQ_ERR_SIZE "... bytes, expected ...".  The bytes are copied (host copy kept
+ * for nq_get_blocks), uploaded, and re-laid-out on the device once; the call
+ * returns after the upload has completed. */
+int32_t nq_set_blocks(nq_handle h, const uint8_t* blocks_host, int64_t nbytes, void* stream);
+
+/* `QLinear.set_weight` (qlinear.mojo:264-269): round-to-nearest quantisation
+ * of an fp32 [OUT, IN] weight on the Q4_0 grid (q4_0.mojo:98-154), run on the
+ * device, then loaded as by nq_set_blocks.  n_values must be OUT*IN. */
+int32_t nq_set_weight_f32(nq_handle h, const float* w_host, int64_t n_values, void* stream);
+
+/* NQ_FMT_W8_CHANNEL: int8 weight [OUT, IN] and fp32 scales [OUT]. */
+int32_t nq_set_weight_i8(nq_handle h, const int8_t* w_host, const float* scales_host, void* stream);
+
+/* NQ_FMT_W4_GROUP: codes [OUT, IN/2], fp16 scale bits [OUT, G], packed uint4
+ * zero-points [OUT, ceil(G/2)] (low nibble = even group), G = ceil(IN/group). */
+int32_t nq_set_weight_w4g(nq_handle h, const uint8_t* codes_host, const uint16_t* scales_f16_host,
+                          const uint8_t* zps_host, void* stream);
+
+/* NQ_FMT_FP8_E4M3: e4m3fn codes [OUT, IN] and the per-tensor scale. */
+int32_t nq_set_weight_fp8(nq_handle h, const uint8_t* w_host, float scale, void* stream);
+
+/* Bytes of the logical weight (`QLinear.BYTES`, qlinear.mojo:216-217, for
+ * Q4_0; the codes' byte count for the other formats). */
+int64_t nq_blocks_bytes(nq_handle h);
+
+/* `QLinear.blocks()` (qlinear.mojo:322-324): the Q4_0 blocks back, byte for
+ * byte.  NQ_ERR_NOT_LOADED / NQ_ERR_NO_BLOCKS as `_need_blocks` (:358-369). */
+int32_t nq_get_blocks(nq_handle h, uint8_t* out_host, int64_t nbytes);
+
+/* `QLinear.keep_only_repacked` (qlinear.mojo:342-356): drop the host copy of
+ * the logical blocks; only the device layout the forward reads is kept. */
+int32_t nq_keep_only_repacked(nq_handle h);
+
+/* ---- compute ------------------------------------------------------------ */
+
+/* `QLinear.forward` (qlinear.mojo:407-477) generalised to the formats above
+ * and to `LinearAct`'s bias/activation epilogue:
+ *     y[M, OUT] = epi( x[M, IN] @ deq(W)^T  (+ bias[OUT]) )
+ * x_dtype: F32 or BF16 for Q4_0 / W8_CHANNEL / W4_GROUP; I8 for W8_CHANNEL
+ * (x_scale = fp32 [M], one per row); FP8_E4M3 for FP8_E4M3 weights
+ * (x_scale = fp32 [1]).  x_scale is NULL otherwise.
+ * y_dtype: F32 or BF16; I32 with x_dtype I8 returns the raw accumulators
+ * (no scale, bias or epilogue).  bias may be NULL; bias_dtype F32 or BF16.
+ * The dequantised weight is never materialised. */
+int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
+                   int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype,
+                   int32_t epilogue, void* stream);
+
+/* The device twin of `dequantize_q4_0` (`dequant_q4_0_kernel`,
+ * q4_0.mojo:242-266; `QLinear.dequantized`, qlinear.mojo:326-328): deq(W)
+ * [OUT, IN] fp32 into out_dev (n_values >= OUT*IN else NQ_ERR_SIZE, the
+ * `share_scratch` rule of qlinear.mojo:330-340).  Any format. */
+int32_t nq_dequantize(nq_handle h, float* out_dev, int64_t n_values, void* stream);
+
+/* `QLinear.vjp` (qlinear.mojo:479-518): gx[M, IN] = gy[M, OUT] @ deq(W),
+ * fp32 in and out, overwriting gx.  Q4_0 only. */
+int32_t nq_grad_input(nq_handle h, const float* gy, float* gx, int32_t M, void* stream);
+
+/* Per-row (token) absmax int8 quantisation of activations [M, K]:
+ *     s[m] = absmax(x[m,:]) / 127 (1 where 0);  q = clip(rhe(x / s), -127, 127)
+ * divide and ties-to-even, as the RTN grid insists (q4_0.mojo:30-32).
+ * x_dtype F32 or BF16. */
+int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M,
+                            int32_t K, void* stream);
+
+/* `_cast_pad_kernel` (qlinear.mojo:152-172): fp32 [rows, cols] -> bf16
+ * [rows, cols_pad] with a zero tail. */
+int32_t nq_cast_pad_bf16(const float* src, uint16_t* dst, int32_t rows, int32_t cols,
+                         int32_t cols_pad, void* stream);
+
+/* `_slice_cast_kernel` (qlinear.mojo:175-192): bf16 [rows, cols_pad] -> fp32
+ * [rows, cols]. */
+int32_t nq_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int32_t cols,
+                          int32_t cols_pad, void* stream);
+
+/* Three W8_CHANNEL layers run as one launch for batched-env actor inference
+ * (SAC/PPO actor MLP; `LinearAct` chain): per token
+ *     h1 = relu(L1(q8(x))), h2 = relu(L2(q8(h1))), y = L3(q8(h2)) (+ relu if
+ *     final_epilogue), q8 = nq_quantize_rows_i8's rule, int32 accumulation.
+ * x fp32 [M, IN1], y fp32 [M, OUT3]; b1..b3 fp32 or NULL.  The layers'
+ * shapes must chain (OUT1 == IN2, OUT2 == IN3), IN <= 256, OUT <= 256. */
+int32_t nq_mlp3_w8a8_forward(nq_handle l1, nq_handle l2, nq_handle l3, const float* x, float* y,
+                             int32_t M, const float* b1, const float* b2, const float* b3,
+                             int32_t final_epilogue, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NOEIRA_QLINEAR_H */

@@ -1,0 +1,127 @@
+"""dlopen of libnoeira_qlinear.so and its C prototypes.
+
+Resolution order mirrors the reference's native-shim loaders
+(noeira/io/serial/native.mojo:57-71): ``$NOEIRA_QLINEAR_LIB`` -> the package
+directory -> the bare name.  A missing library is an error, never a fallback:
+there is no CPU path behind this package.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libnoeira_qlinear.so"
+
+# status codes / enums of include/noeira_qlinear.h
+NQ_OK, NQ_ERR_INVALID, NQ_ERR_NOT_LOADED, NQ_ERR_NO_BLOCKS, NQ_ERR_SIZE, NQ_ERR_HIP, NQ_ERR_UNSUPPORTED = range(7)
+FMT_Q4_0, FMT_W8_CHANNEL, FMT_W4_GROUP, FMT_FP8_E4M3 = range(4)
+DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
+EPI_NONE, EPI_RELU = 0, 1
+ABI_VERSION = 1
+
+EXPORTS = [
+    "nq_abi_version", "nq_last_error", "nq_create", "nq_destroy", "nq_set_blocks", "nq_set_weight_f32",
+    "nq_set_weight_i8", "nq_set_weight_w4g", "nq_set_weight_fp8", "nq_blocks_bytes", "nq_get_blocks",
+    "nq_keep_only_repacked", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
+    "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward",
+]
+
+
+class NQError(RuntimeError):
+    """A non-zero status from the library, carrying its sentence (the Mojo
+    wrapper raises ``Error(msg)`` from the same text)."""
+
+    def __init__(self, code: int, msg: str):
+        super().__init__(msg)
+        self.code = code
+
+
+def candidates():
+    out = []
+    override = os.environ.get("NOEIRA_QLINEAR_LIB", "")
+    if override:
+        out.append(override)
+    out.append(os.path.join(_HERE, LIB_NAME))
+    out.append(LIB_NAME)
+    return out
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    last = None
+    for path in candidates():
+        if os.sep in path and not os.path.exists(path):
+            continue
+        try:
+            L = C.CDLL(path)
+            break
+        except OSError as e:  # keep looking, report all at the end
+            last = e
+    else:
+        raise OSError(
+            "libnoeira_qlinear.so not found. Tried:\n  - " + "\n  - ".join(candidates())
+            + "\nBuild it with `python -m noeira_amd.build`, or set NOEIRA_QLINEAR_LIB=/path/to/"
+            + LIB_NAME + (f"\n(last loader error: {last})" if last else ""))
+    i32, i64, p, f32 = C.c_int32, C.c_int64, C.c_void_p, C.c_float
+    L.nq_abi_version.restype = i32
+    L.nq_abi_version.argtypes = []
+    L.nq_last_error.restype = i64
+    L.nq_last_error.argtypes = [C.c_char_p, i64]
+    L.nq_create.restype = i32
+    L.nq_create.argtypes = [C.POINTER(p), i32, i32, i32, i32, i32]
+    L.nq_destroy.restype = i32
+    L.nq_destroy.argtypes = [p]
+    L.nq_set_blocks.restype = i32
+    L.nq_set_blocks.argtypes = [p, p, i64, p]
+    L.nq_set_weight_f32.restype = i32
+    L.nq_set_weight_f32.argtypes = [p, p, i64, p]
+    L.nq_set_weight_i8.restype = i32
+    L.nq_set_weight_i8.argtypes = [p, p, p, p]
+    L.nq_set_weight_w4g.restype = i32
+    L.nq_set_weight_w4g.argtypes = [p, p, p, p, p]
+    L.nq_set_weight_fp8.restype = i32
+    L.nq_set_weight_fp8.argtypes = [p, p, f32, p]
+    L.nq_blocks_bytes.restype = i64
+    L.nq_blocks_bytes.argtypes = [p]
+    L.nq_get_blocks.restype = i32
+    L.nq_get_blocks.argtypes = [p, p, i64]
+    L.nq_keep_only_repacked.restype = i32
+    L.nq_keep_only_repacked.argtypes = [p]
+    L.nq_forward.restype = i32
+    L.nq_forward.argtypes = [p, p, i32, p, p, i32, i32, p, i32, i32, p]
+    L.nq_dequantize.restype = i32
+    L.nq_dequantize.argtypes = [p, p, i64, p]
+    L.nq_grad_input.restype = i32
+    L.nq_grad_input.argtypes = [p, p, p, i32, p]
+    L.nq_quantize_rows_i8.restype = i32
+    L.nq_quantize_rows_i8.argtypes = [p, i32, p, p, i32, i32, p]
+    L.nq_cast_pad_bf16.restype = i32
+    L.nq_cast_pad_bf16.argtypes = [p, p, i32, i32, i32, p]
+    L.nq_slice_cast_f32.restype = i32
+    L.nq_slice_cast_f32.argtypes = [p, p, i32, i32, i32, p]
+    L.nq_mlp3_w8a8_forward.restype = i32
+    L.nq_mlp3_w8a8_forward.argtypes = [p, p, p, p, p, i32, p, p, p, i32, p]
+    got = L.nq_abi_version()
+    if got != ABI_VERSION:
+        raise OSError(f"{LIB_NAME}: ABI version {got}, this package binds version {ABI_VERSION}")
+    _lib = L
+    return L
+
+
+def last_error() -> str:
+    L = lib()
+    n = L.nq_last_error(None, 0)
+    buf = C.create_string_buffer(int(n) + 1)
+    L.nq_last_error(buf, n + 1)
+    return buf.value.decode("utf-8", "replace")
+
+
+def check(rc: int):
+    if rc != NQ_OK:
+        raise NQError(rc, last_error())

@@ -1,0 +1,434 @@
+// The C ABI of libnoeira_qlinear.so (include/noeira_qlinear.h): argument
+// checking, the layer's storage, and dispatch to the kernels.  No C++
+// exception crosses the boundary and nothing here aborts; every failure is a
+// status code plus a sentence for nq_last_error().
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "nq_common.h"
+
+namespace nq {
+
+static thread_local std::string g_last_error;
+
+int32_t fail(int32_t code, const std::string& msg) {
+    g_last_error = msg;
+    return code;
+}
+
+int32_t fail_hip(hipError_t e, const char* what) {
+    g_last_error = std::string("HIP error ") + hipGetErrorName(e) + " (" + hipGetErrorString(e) + ") in " + what;
+    return NQ_ERR_HIP;
+}
+
+namespace {
+
+const char* fmt_name(int f) {
+    switch (f) {
+        case NQ_FMT_Q4_0: return "Q4_0";
+        case NQ_FMT_W8_CHANNEL: return "W8_CHANNEL";
+        case NQ_FMT_W4_GROUP: return "W4_GROUP";
+        case NQ_FMT_FP8_E4M3: return "FP8_E4M3";
+    }
+    return "?";
+}
+
+std::string shape_tag(const nq_layer* L) {
+    return "QLinear[" + std::to_string(L->in) + ", " + std::to_string(L->out) + "]";
+}
+
+int64_t logical_bytes(const nq_layer* L) {
+    switch (L->format) {
+        case NQ_FMT_Q4_0: return (int64_t)L->out * (L->in / Q4_GROUP) * Q4_BLOCK;
+        case NQ_FMT_W4_GROUP: return (int64_t)L->out * (L->in / 2);
+        default: return (int64_t)L->out * L->in;
+    }
+}
+
+void free_device(nq_layer* L) {
+    if (L->d_codes) (void)hipFree(L->d_codes);
+    if (L->d_scales) (void)hipFree(L->d_scales);
+    if (L->d_zps) (void)hipFree(L->d_zps);
+    L->d_codes = nullptr, L->d_scales = nullptr, L->d_zps = nullptr;
+}
+
+int32_t check_handle(nq_handle h, const char* what) {
+    if (!h) return fail(NQ_ERR_INVALID, std::string(what) + ": null layer handle");
+    return NQ_OK;
+}
+
+// the `_need_blocks` rule of noeira/nn/quant/qlinear.mojo:358-369
+int32_t need_loaded(const nq_layer* L, const char* what) {
+    if (!L->loaded)
+        return fail(NQ_ERR_NOT_LOADED,
+                    std::string("QLinear.") + what + ": no weights (set_weight or set_blocks first)");
+    return NQ_OK;
+}
+
+int32_t need_blocks(const nq_layer* L, const char* what) {
+    int32_t rc = need_loaded(L, what);
+    if (rc) return rc;
+    if (!L->has_host_blocks)
+        return fail(NQ_ERR_NO_BLOCKS, std::string("QLinear.") + what +
+                                          ": no blocks are kept (keep_only_repacked); only the forward is left");
+    return NQ_OK;
+}
+
+int32_t bind_device(nq_layer* L) {
+    int dev = 0;
+    NQ_HIP(hipGetDevice(&dev));
+    if (L->device >= 0 && L->device != dev && L->loaded)
+        return fail(NQ_ERR_INVALID, "layer was loaded on device " + std::to_string(L->device) +
+                                        " but the current device is " + std::to_string(dev));
+    L->device = dev;
+    return NQ_OK;
+}
+
+// upload the split Q4_0 layout from raw blocks that already sit on the device
+int32_t adopt_q4_0_blocks(nq_layer* L, const uint8_t* raw_dev, hipStream_t s) {
+    const int64_t nblocks = (int64_t)L->out * (L->in / Q4_GROUP);
+    free_device(L);
+    NQ_HIP(hipMalloc((void**)&L->d_codes, (size_t)nblocks * 16 + 16));
+    NQ_HIP(hipMalloc(&L->d_scales, (size_t)nblocks * 2 + 16));
+    int32_t rc = launch_q4_0_repack(raw_dev, L->d_codes, reinterpret_cast<uint16_t*>(L->d_scales), nblocks, s);
+    if (rc) return rc;
+    L->row_bytes = (int64_t)(L->in / Q4_GROUP) * 16;
+    return NQ_OK;
+}
+
+}  // namespace
+}  // namespace nq
+
+using namespace nq;
+
+extern "C" {
+
+int32_t nq_abi_version(void) { return NQ_ABI_VERSION; }
+
+int64_t nq_last_error(char* buf, int64_t n) {
+    const std::string& e = g_last_error;
+    if (buf && n > 0) {
+        size_t k = std::min((size_t)(n - 1), e.size());
+        std::memcpy(buf, e.data(), k);
+        buf[k] = 0;
+    }
+    return (int64_t)e.size();
+}
+
+int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t out_features, int32_t group,
+                  int32_t flags) {
+    if (!out) return fail(NQ_ERR_INVALID, "nq_create: null output handle");
+    *out = nullptr;
+    if (format < NQ_FMT_Q4_0 || format > NQ_FMT_FP8_E4M3)
+        return fail(NQ_ERR_INVALID, "nq_create: unknown format " + std::to_string(format));
+    if (in_features <= 0 || out_features <= 0)
+        return fail(NQ_ERR_INVALID, "nq_create: IN and OUT must be positive");
+    if (flags != 0) return fail(NQ_ERR_INVALID, "nq_create: flags must be 0");
+    if (format == NQ_FMT_Q4_0) {
+        // qlinear.mojo:243-245
+        if (in_features % Q4_GROUP != 0)
+            return fail(NQ_ERR_INVALID, "QLinear: IN must be a multiple of 32 (one Q4_0 group)");
+        if (group != 0 && group != Q4_GROUP)
+            return fail(NQ_ERR_INVALID, "nq_create: Q4_0 groups are 32 wide");
+        group = Q4_GROUP;
+    } else if (format == NQ_FMT_W4_GROUP) {
+        if (group <= 0 || group % 32 != 0)
+            return fail(NQ_ERR_INVALID, "nq_create: W4_GROUP needs a group width that is a multiple of 32");
+        if (in_features % 32 != 0)
+            return fail(NQ_ERR_INVALID, "nq_create: W4_GROUP needs IN to be a multiple of 32");
+    } else {
+        if (in_features % 16 != 0)
+            return fail(NQ_ERR_INVALID, std::string("nq_create: ") + fmt_name(format) +
+                                            " needs IN to be a multiple of 16");
+        group = 0;
+    }
+    nq_layer* L = new (std::nothrow) nq_layer();
+    if (!L) return fail(NQ_ERR_INVALID, "nq_create: out of host memory");
+    L->format = format, L->in = in_features, L->out = out_features, L->group = group;
+    L->groups = group ? (in_features + group - 1) / group : 0;
+    *out = L;
+    return NQ_OK;
+}
+
+int32_t nq_destroy(nq_handle h) {
+    if (!h) return NQ_OK;
+    free_device(h);
+    delete h;
+    return NQ_OK;
+}
+
+int32_t nq_set_blocks(nq_handle h, const uint8_t* blocks_host, int64_t nbytes, void* stream) {
+    int32_t rc = check_handle(h, "nq_set_blocks");
+    if (rc) return rc;
+    if (h->format != NQ_FMT_Q4_0)
+        return fail(NQ_ERR_INVALID, "nq_set_blocks: the layer's format is not Q4_0");
+    const int64_t want = logical_bytes(h);
+    if (nbytes != want)  // qlinear.mojo:276-281
+        return fail(NQ_ERR_SIZE, shape_tag(h) + ".set_blocks: " + std::to_string(nbytes) + " bytes, expected " +
+                                     std::to_string(want));
+    if (!blocks_host) return fail(NQ_ERR_INVALID, "nq_set_blocks: null blocks");
+    hipStream_t s = (hipStream_t)stream;
+    h->loaded = false;
+    if ((rc = bind_device(h))) return rc;
+    h->host_blocks.assign(blocks_host, blocks_host + nbytes);
+    h->has_host_blocks = true;
+    uint8_t* raw = nullptr;
+    NQ_HIP(hipMalloc((void**)&raw, (size_t)nbytes + 16));
+    hipError_t e = hipMemcpyAsync(raw, h->host_blocks.data(), (size_t)nbytes, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) {
+        rc = adopt_q4_0_blocks(h, raw, s);
+        if (rc == NQ_OK) e = hipStreamSynchronize(s);
+    }
+    (void)hipFree(raw);
+    if (e != hipSuccess) return fail_hip(e, "nq_set_blocks upload");
+    if (rc) return rc;
+    h->loaded = true;
+    return NQ_OK;
+}
+
+int32_t nq_set_weight_f32(nq_handle h, const float* w_host, int64_t n_values, void* stream) {
+    int32_t rc = check_handle(h, "nq_set_weight_f32");
+    if (rc) return rc;
+    if (h->format != NQ_FMT_Q4_0)
+        return fail(NQ_ERR_INVALID, "nq_set_weight_f32: the layer's format is not Q4_0");
+    const int64_t want = (int64_t)h->in * h->out;
+    if (n_values != want)  // q4_0.mojo:139-143
+        return fail(NQ_ERR_SIZE, "quantize_rtn_q4_0: " + std::to_string(n_values) + " values for a [" +
+                                     std::to_string(h->out) + ", " + std::to_string(h->in) + "] weight");
+    if (!w_host) return fail(NQ_ERR_INVALID, "nq_set_weight_f32: null weight");
+    hipStream_t s = (hipStream_t)stream;
+    h->loaded = false;
+    if ((rc = bind_device(h))) return rc;
+    const int64_t nbytes = logical_bytes(h);
+    float* wd = nullptr;
+    uint8_t* raw = nullptr;
+    NQ_HIP(hipMalloc((void**)&wd, (size_t)want * 4));
+    hipError_t e = hipMalloc((void**)&raw, (size_t)nbytes + 16);
+    if (e != hipSuccess) {
+        (void)hipFree(wd);
+        return fail_hip(e, "nq_set_weight_f32 alloc");
+    }
+    h->host_blocks.resize((size_t)nbytes);
+    e = hipMemcpyAsync(wd, w_host, (size_t)want * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) rc = launch_q4_0_rtn(wd, raw, h->out, h->in, s);
+    if (e == hipSuccess && rc == NQ_OK)
+        e = hipMemcpyAsync(h->host_blocks.data(), raw, (size_t)nbytes, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess && rc == NQ_OK) rc = adopt_q4_0_blocks(h, raw, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
+    (void)hipFree(wd);
+    (void)hipFree(raw);
+    if (e != hipSuccess) return fail_hip(e, "nq_set_weight_f32");
+    if (rc) return rc;
+    h->has_host_blocks = true;
+    h->loaded = true;
+    return NQ_OK;
+}
+
+int32_t nq_set_weight_i8(nq_handle h, const int8_t* w_host, const float* scales_host, void* stream) {
+    int32_t rc = check_handle(h, "nq_set_weight_i8");
+    if (rc) return rc;
+    if (h->format != NQ_FMT_W8_CHANNEL)
+        return fail(NQ_ERR_INVALID, "nq_set_weight_i8: the layer's format is not W8_CHANNEL");
+    if (!w_host || !scales_host) return fail(NQ_ERR_INVALID, "nq_set_weight_i8: null weight or scales");
+    hipStream_t s = (hipStream_t)stream;
+    h->loaded = false;
+    if ((rc = bind_device(h))) return rc;
+    free_device(h);
+    const size_t n = (size_t)h->in * h->out;
+    NQ_HIP(hipMalloc((void**)&h->d_codes, n + 16));
+    NQ_HIP(hipMalloc(&h->d_scales, (size_t)h->out * 4 + 16));
+    h->host_blocks.assign(reinterpret_cast<const uint8_t*>(w_host), reinterpret_cast<const uint8_t*>(w_host) + n);
+    h->has_host_blocks = true;
+    NQ_HIP(hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s));
+    NQ_HIP(hipMemcpyAsync(h->d_scales, scales_host, (size_t)h->out * 4, hipMemcpyHostToDevice, s));
+    NQ_HIP(hipStreamSynchronize(s));
+    h->row_bytes = h->in;
+    h->loaded = true;
+    return NQ_OK;
+}
+
+int32_t nq_set_weight_w4g(nq_handle h, const uint8_t* codes_host, const uint16_t* scales_f16_host,
+                          const uint8_t* zps_host, void* stream) {
+    int32_t rc = check_handle(h, "nq_set_weight_w4g");
+    if (rc) return rc;
+    if (h->format != NQ_FMT_W4_GROUP)
+        return fail(NQ_ERR_INVALID, "nq_set_weight_w4g: the layer's format is not W4_GROUP");
+    if (!codes_host || !scales_f16_host || !zps_host)
+        return fail(NQ_ERR_INVALID, "nq_set_weight_w4g: null codes, scales or zero-points");
+    hipStream_t s = (hipStream_t)stream;
+    h->loaded = false;
+    if ((rc = bind_device(h))) return rc;
+    free_device(h);
+    const size_t n = (size_t)h->out * (h->in / 2);
+    const size_t ng = (size_t)h->out * h->groups;
+    const size_t nz = (size_t)h->out * ((h->groups + 1) / 2);
+    uint8_t* zp_packed = nullptr;
+    NQ_HIP(hipMalloc((void**)&h->d_codes, n + 16));
+    NQ_HIP(hipMalloc(&h->d_scales, ng * 2 + 16));
+    NQ_HIP(hipMalloc((void**)&h->d_zps, ng + 16));
+    NQ_HIP(hipMalloc((void**)&zp_packed, nz + 16));
+    h->host_blocks.assign(codes_host, codes_host + n);
+    h->has_host_blocks = true;
+    hipError_t e = hipMemcpyAsync(h->d_codes, codes_host, n, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(h->d_scales, scales_f16_host, ng * 2, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(zp_packed, zps_host, nz, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) rc = launch_w4g_unpack_zps(zp_packed, h->d_zps, h->out, h->groups, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
+    (void)hipFree(zp_packed);
+    if (e != hipSuccess) return fail_hip(e, "nq_set_weight_w4g upload");
+    if (rc) return rc;
+    h->row_bytes = h->in / 2;
+    h->loaded = true;
+    return NQ_OK;
+}
+
+int32_t nq_set_weight_fp8(nq_handle h, const uint8_t* w_host, float scale, void* stream) {
+    int32_t rc = check_handle(h, "nq_set_weight_fp8");
+    if (rc) return rc;
+    if (h->format != NQ_FMT_FP8_E4M3)
+        return fail(NQ_ERR_INVALID, "nq_set_weight_fp8: the layer's format is not FP8_E4M3");
+    if (!w_host) return fail(NQ_ERR_INVALID, "nq_set_weight_fp8: null weight");
+    hipStream_t s = (hipStream_t)stream;
+    h->loaded = false;
+    if ((rc = bind_device(h))) return rc;
+    free_device(h);
+    const size_t n = (size_t)h->in * h->out;
+    NQ_HIP(hipMalloc((void**)&h->d_codes, n + 16));
+    h->host_blocks.assign(w_host, w_host + n);
+    h->has_host_blocks = true;
+    NQ_HIP(hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s));
+    NQ_HIP(hipStreamSynchronize(s));
+    h->scale = scale;
+    h->row_bytes = h->in;
+    h->loaded = true;
+    return NQ_OK;
+}
+
+int64_t nq_blocks_bytes(nq_handle h) {
+    if (!h) return 0;
+    return logical_bytes(h);
+}
+
+int32_t nq_get_blocks(nq_handle h, uint8_t* out_host, int64_t nbytes) {
+    int32_t rc = check_handle(h, "nq_get_blocks");
+    if (rc) return rc;
+    if ((rc = need_blocks(h, "blocks"))) return rc;
+    if (nbytes != (int64_t)h->host_blocks.size())
+        return fail(NQ_ERR_SIZE, shape_tag(h) + ".blocks: a buffer of " + std::to_string(nbytes) +
+                                     " bytes, expected " + std::to_string(h->host_blocks.size()));
+    if (!out_host) return fail(NQ_ERR_INVALID, "nq_get_blocks: null buffer");
+    std::memcpy(out_host, h->host_blocks.data(), (size_t)nbytes);
+    return NQ_OK;
+}
+
+int32_t nq_keep_only_repacked(nq_handle h) {
+    int32_t rc = check_handle(h, "nq_keep_only_repacked");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "keep_only_repacked"))) return rc;
+    std::vector<uint8_t>().swap(h->host_blocks);
+    h->has_host_blocks = false;
+    return NQ_OK;
+}
+
+int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y, int32_t y_dtype,
+                   int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue, void* stream) {
+    int32_t rc = check_handle(h, "nq_forward");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!x || !y) return fail(NQ_ERR_INVALID, "nq_forward: null x or y");
+    if (((uintptr_t)x & 15) || ((uintptr_t)y & 3))
+        return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
+    if (epilogue != NQ_EPI_NONE && epilogue != NQ_EPI_RELU)
+        return fail(NQ_ERR_INVALID, "nq_forward: unknown epilogue " + std::to_string(epilogue));
+    if (bias && bias_dtype != NQ_DT_F32 && bias_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "nq_forward: bias must be fp32 or bf16");
+    ForwardArgs a{h, x, x_dtype, x_scale, y, y_dtype, M, bias, bias_dtype, epilogue, (hipStream_t)stream};
+    if (x_dtype == NQ_DT_I8) {
+        if (h->format != NQ_FMT_W8_CHANNEL)
+            return fail(NQ_ERR_INVALID, "nq_forward: int8 activations need a W8_CHANNEL layer");
+        if (y_dtype == NQ_DT_I32) {
+            if (bias || epilogue != NQ_EPI_NONE)
+                return fail(NQ_ERR_INVALID, "nq_forward: raw int32 accumulators take no bias or epilogue");
+        } else {
+            if (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16)
+                return fail(NQ_ERR_INVALID, "nq_forward: y must be fp32, bf16 or int32");
+            if (!x_scale) return fail(NQ_ERR_INVALID, "nq_forward: int8 activations need per-row scales");
+        }
+        return launch_gemv_i8(a);
+    }
+    if (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "nq_forward: y must be fp32 or bf16");
+    if (x_dtype == NQ_DT_FP8_E4M3) {
+        if (h->format != NQ_FMT_FP8_E4M3)
+            return fail(NQ_ERR_INVALID, "nq_forward: fp8 activations need an FP8_E4M3 layer");
+        if (!x_scale) return fail(NQ_ERR_INVALID, "nq_forward: fp8 activations need a scale");
+    } else if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16) {
+        return fail(NQ_ERR_INVALID, "nq_forward: unknown x dtype " + std::to_string(x_dtype));
+    }
+    return launch_gemv(a);
+}
+
+int32_t nq_dequantize(nq_handle h, float* out_dev, int64_t n_values, void* stream) {
+    int32_t rc = check_handle(h, "nq_dequantize");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "dequantized"))) return rc;
+    if (n_values < (int64_t)h->in * h->out)  // qlinear.mojo:334-338
+        return fail(NQ_ERR_SIZE, "QLinear.share_scratch: " + std::to_string(n_values) + " values for a [" +
+                                     std::to_string(h->out) + ", " + std::to_string(h->in) + "] weight");
+    if (!out_dev || ((uintptr_t)out_dev & 15))
+        return fail(NQ_ERR_INVALID, "nq_dequantize: the output must be a 16-byte aligned device buffer");
+    return launch_dequantize(h, out_dev, (hipStream_t)stream);
+}
+
+int32_t nq_grad_input(nq_handle h, const float* gy, float* gx, int32_t M, void* stream) {
+    int32_t rc = check_handle(h, "nq_grad_input");
+    if (rc) return rc;
+    if ((rc = need_blocks(h, "vjp"))) return rc;
+    if (h->format != NQ_FMT_Q4_0) return fail(NQ_ERR_UNSUPPORTED, "nq_grad_input: Q4_0 layers only");
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_grad_input: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!gy || !gx) return fail(NQ_ERR_INVALID, "nq_grad_input: null gy or gx");
+    return launch_grad_input_q4_0(h, gy, gx, M, (hipStream_t)stream);
+}
+
+int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M, int32_t K,
+                            void* stream) {
+    if (M < 0 || K <= 0 || K % 4 != 0)
+        return fail(NQ_ERR_INVALID, "nq_quantize_rows_i8: M >= 0 and K a positive multiple of 4 are required");
+    if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "nq_quantize_rows_i8: x must be fp32 or bf16");
+    if (M == 0) return NQ_OK;
+    if (!x || !q || !scales) return fail(NQ_ERR_INVALID, "nq_quantize_rows_i8: null pointer");
+    if (((uintptr_t)x & 15) || ((uintptr_t)q & 3))
+        return fail(NQ_ERR_INVALID, "nq_quantize_rows_i8: x must be 16-byte and q 4-byte aligned");
+    return launch_quantize_rows_i8(x, x_dtype, q, scales, M, K, (hipStream_t)stream);
+}
+
+int32_t nq_cast_pad_bf16(const float* src, uint16_t* dst, int32_t rows, int32_t cols, int32_t cols_pad,
+                         void* stream) {
+    if (rows < 0 || cols < 0 || cols_pad < cols)
+        return fail(NQ_ERR_INVALID, "nq_cast_pad_bf16: need rows >= 0 and cols_pad >= cols >= 0");
+    if (rows && cols_pad && (!src || !dst)) return fail(NQ_ERR_INVALID, "nq_cast_pad_bf16: null pointer");
+    return launch_cast_pad_bf16(src, dst, rows, cols, cols_pad, (hipStream_t)stream);
+}
+
+int32_t nq_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int32_t cols, int32_t cols_pad,
+                          void* stream) {
+    if (rows < 0 || cols < 0 || cols_pad < cols)
+        return fail(NQ_ERR_INVALID, "nq_slice_cast_f32: need rows >= 0 and cols_pad >= cols >= 0");
+    if (rows && cols && (!src || !dst)) return fail(NQ_ERR_INVALID, "nq_slice_cast_f32: null pointer");
+    return launch_slice_cast_f32(src, dst, rows, cols, cols_pad, (hipStream_t)stream);
+}
+
+int32_t nq_mlp3_w8a8_forward(nq_handle l1, nq_handle l2, nq_handle l3, const float* x, float* y, int32_t M,
+                             const float* b1, const float* b2, const float* b3, int32_t final_epilogue,
+                             void* stream) {
+    (void)l1, (void)l2, (void)l3, (void)x, (void)y, (void)M, (void)b1, (void)b2, (void)b3;
+    (void)final_epilogue, (void)stream;
+    return fail(NQ_ERR_UNSUPPORTED, "nq_mlp3_w8a8_forward: not built yet");
+}
+
+}  // extern "C"

@@ -1,0 +1,93 @@
+// Internal declarations shared by the translation units of libnoeira_qlinear.so.
+// Nothing here crosses the C ABI (include/noeira_qlinear.h does).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "../../include/noeira_qlinear.h"
+
+namespace nq {
+
+constexpr int Q4_GROUP = 32;  // weights per Q4_0 group (noeira/nn/quant/q4_0.mojo:49)
+constexpr int Q4_BLOCK = 18;  // bytes per Q4_0 block   (noeira/nn/quant/q4_0.mojo:51)
+constexpr int CHUNK = 16;     // bytes one lane loads per weight fetch (128-bit)
+
+// Sets the calling thread's error sentence and returns `code`.
+int32_t fail(int32_t code, const std::string& msg);
+int32_t fail_hip(hipError_t e, const char* what);
+
+#define NQ_HIP(expr)                                        \
+    do {                                                    \
+        hipError_t _e = (expr);                             \
+        if (_e != hipSuccess) return nq::fail_hip(_e, #expr); \
+    } while (0)
+
+}  // namespace nq
+
+// One quantized linear layer.  Device layouts (all row-major over OUT):
+//   Q4_0        codes  [OUT][G][16 B]   the nibble bytes of each block, so that
+//                                        every group is one aligned 128-bit load
+//               scales [OUT][G] fp16    the block scales, split off the blocks
+//   W8_CHANNEL  codes  [OUT][IN] int8,  scales [OUT] fp32
+//   W4_GROUP    codes  [OUT][IN/2]      (low nibble = even k)
+//               scales [OUT][G] fp16,   zps [OUT][G] uint8 (unpacked)
+//   FP8_E4M3    codes  [OUT][IN],       scale = one fp32
+struct nq_layer {
+    int32_t format = 0;
+    int32_t in = 0;
+    int32_t out = 0;
+    int32_t group = 0;
+    int32_t groups = 0;        // G = ceil(IN / group) for the grouped formats
+    bool loaded = false;
+    bool has_host_blocks = false;
+    std::vector<uint8_t> host_blocks;  // logical bytes as handed to set_* (Q4_0: the blocks)
+    int device = -1;
+    uint8_t* d_codes = nullptr;
+    void* d_scales = nullptr;
+    uint8_t* d_zps = nullptr;
+    float scale = 1.0f;
+    int64_t row_bytes = 0;     // bytes of one row of d_codes
+};
+
+namespace nq {
+
+struct ForwardArgs {
+    const nq_layer* L;
+    const void* x;
+    int32_t x_dtype;
+    const float* x_scale;
+    void* y;
+    int32_t y_dtype;
+    int32_t M;
+    const void* bias;
+    int32_t bias_dtype;
+    int32_t epilogue;
+    hipStream_t stream;
+};
+
+// nq_q4_0.hip
+int32_t launch_q4_0_repack(const uint8_t* raw_dev, uint8_t* codes, uint16_t* scales, int64_t nblocks,
+                           hipStream_t s);
+int32_t launch_q4_0_rtn(const float* w_dev, uint8_t* blocks_dev, int64_t n, int64_t k, hipStream_t s);
+int32_t launch_dequantize(const nq_layer* L, float* out, hipStream_t s);
+int32_t launch_grad_input_q4_0(const nq_layer* L, const float* gy, float* gx, int32_t M, hipStream_t s);
+int32_t launch_w4g_unpack_zps(const uint8_t* packed, uint8_t* out, int64_t rows, int64_t groups,
+                              hipStream_t s);
+
+// nq_gemv.hip: dequant-GEMV for small M (also the any-M fallback)
+int32_t launch_gemv(const ForwardArgs& a);
+int32_t launch_gemv_i8(const ForwardArgs& a);
+
+// nq_quant.hip
+int32_t launch_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M,
+                                int32_t K, hipStream_t s);
+int32_t launch_cast_pad_bf16(const float* src, uint16_t* dst, int32_t rows, int32_t cols,
+                             int32_t cols_pad, hipStream_t s);
+int32_t launch_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int32_t cols,
+                              int32_t cols_pad, hipStream_t s);
+
+}  // namespace nq

@@ -1,0 +1,319 @@
+"""Host-side mirror of the reference's quantized linear operator over the C ABI.
+
+``QLinear`` keeps the public surface of ``QLinear[IN, OUT]``
+(noeira/nn/quant/qlinear.mojo:208-524): ``make``, ``set_weight``,
+``set_blocks``, ``blocks``, ``dequantized``, ``share_scratch``,
+``keep_only_repacked``, ``forward``, ``vjp``, ``release_buffers`` with the
+same argument meaning and the same error sentences, so the gates read like the
+reference's (tests/nn/quant/test_qlinear_gpu.mojo).  ``W8Linear``,
+``W4GroupLinear`` and ``FP8Linear`` are the int8 / group-wise uint4 / fp8
+layers BASELINE names, in the shape of ``Linear`` / ``LinearAct`` (a bias and an
+optional ReLU, noeira/nn/primitives/linear_act.mojo:81-115) but holding the
+weight as [OUT, IN] like ``QLinear`` does.
+
+torch is used only for device memory and streams; every computation is a call
+into libnoeira_qlinear.so.  There is no CPU path: ``target="cpu"`` raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import numpy as np
+import torch
+
+from . import _lib as L
+
+Q4_GROUP = 32
+Q4_BLOCK = 18
+
+_TORCH_DT = {torch.float32: L.DT_F32, torch.bfloat16: L.DT_BF16}
+
+
+def _stream_ptr() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need_gpu(target: str):
+    if target != "gpu":
+        raise L.NQError(L.NQ_ERR_UNSUPPORTED,
+                        "noeira_amd has no CPU path: target must be \"gpu\" (got \"" + str(target) + "\")")
+    if not torch.cuda.is_available():
+        raise L.NQError(L.NQ_ERR_HIP, "noeira_amd: no HIP device is visible")
+
+
+def _dev_ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _check_x(x: torch.Tensor, IN: int, what: str):
+    if not x.is_cuda or not x.is_contiguous():
+        raise L.NQError(L.NQ_ERR_INVALID, what + ": x must be a contiguous device tensor")
+    if x.numel() % IN != 0:
+        raise L.NQError(L.NQ_ERR_INVALID, f"{what}: x has {x.numel()} values, not a multiple of IN = {IN}")
+    return x.numel() // IN
+
+
+class _Layer:
+    """Owns one nq_handle."""
+
+    FORMAT = -1
+
+    def __init__(self, IN: int, OUT: int, group: int = 0):
+        self.IN, self.OUT, self.group = int(IN), int(OUT), int(group)
+        h = C.c_void_p()
+        L.check(L.lib().nq_create(C.byref(h), self.FORMAT, self.IN, self.OUT, self.group, 0))
+        self._h = h
+        self._loaded = False
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h is not None and h.value:
+            try:
+                L.lib().nq_destroy(h)
+            except Exception:
+                pass
+            self._h = None
+
+    # shared by every format ------------------------------------------------
+    def _forward(self, x: torch.Tensor, x_dtype: int, x_scale: Optional[torch.Tensor], out: Optional[torch.Tensor],
+                 out_dtype: torch.dtype, bias: Optional[torch.Tensor], epilogue: str, what: str) -> torch.Tensor:
+        M = _check_x(x, self.IN, what)
+        if out is None or out.numel() < M * self.OUT or out.dtype != out_dtype:
+            out = torch.empty((M, self.OUT), dtype=out_dtype, device=x.device)
+        y_dt = {torch.float32: L.DT_F32, torch.bfloat16: L.DT_BF16, torch.int32: L.DT_I32}[out_dtype]
+        b_dt = L.DT_F32
+        if bias is not None:
+            if bias.dtype not in _TORCH_DT or bias.numel() != self.OUT or not bias.is_cuda:
+                raise L.NQError(L.NQ_ERR_INVALID, what + ": bias must be a device fp32/bf16 tensor of OUT values")
+            b_dt = _TORCH_DT[bias.dtype]
+        epi = {"none": L.EPI_NONE, "relu": L.EPI_RELU}[epilogue]
+        L.check(L.lib().nq_forward(self._h, _dev_ptr(x), x_dtype, _dev_ptr(x_scale), _dev_ptr(out), y_dt, M,
+                                   _dev_ptr(bias), b_dt, epi, _stream_ptr()))
+        return out
+
+    def dequantized_dev(self, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """deq(W) [OUT, IN] fp32 on the device (`dequant_q4_0_kernel`, q4_0.mojo:242-266)."""
+        if out is None:
+            out = torch.empty((self.OUT, self.IN), dtype=torch.float32, device="cuda")
+        L.check(L.lib().nq_dequantize(self._h, _dev_ptr(out), out.numel(), _stream_ptr()))
+        return out
+
+
+class QLinear(_Layer):
+    """A frozen Q4_0 linear: y[T, OUT] = x[T, IN] @ deq(W)^T, W [OUT, IN]
+    (qlinear.mojo:1-11).  fp32 activations at its boundary, no bias, no Param."""
+
+    FORMAT = L.FMT_Q4_0
+    ARITY = 1
+
+    def __init__(self, IN: int, OUT: int):
+        if IN % Q4_GROUP != 0:  # the comptime assert of qlinear.mojo:243-245
+            raise L.NQError(L.NQ_ERR_INVALID, "QLinear: IN must be a multiple of 32 (one Q4_0 group)")
+        super().__init__(IN, OUT, Q4_GROUP)
+        self.W_SIZE = IN * OUT
+        self.ROW_BYTES = (IN // Q4_GROUP) * Q4_BLOCK
+        self.BYTES = OUT * self.ROW_BYTES
+        self.deq: Optional[torch.Tensor] = None  # shared dequantize scratch (share_scratch)
+
+    @staticmethod
+    def display_label() -> str:
+        return "QLinear"
+
+    @classmethod
+    def make(cls, IN: int, OUT: int, target: str = "gpu", ctx=None) -> "QLinear":
+        """An empty layer: weights come from set_weight or set_blocks, never
+        from an initializer (qlinear.mojo:253-260)."""
+        _need_gpu(target)
+        return cls(IN, OUT)
+
+    # ── weights ────────────────────────────────────────────────────────────
+    def set_weight(self, w, target: str = "gpu", ctx=None):
+        """Quantize an fp32 [OUT, IN] weight by RTN on the Q4_0 grid and load it
+        (qlinear.mojo:264-269)."""
+        _need_gpu(target)
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        L.check(L.lib().nq_set_weight_f32(self._h, w.ctypes.data_as(C.c_void_p), w.size, _stream_ptr()))
+        self._loaded = True
+
+    def set_blocks(self, blocks, target: str = "gpu", ctx=None):
+        """Load Q4_0 blocks [OUT, IN/32*18] (qlinear.mojo:271-320)."""
+        _need_gpu(target)
+        b = np.ascontiguousarray(blocks, dtype=np.uint8)
+        L.check(L.lib().nq_set_blocks(self._h, b.ctypes.data_as(C.c_void_p), b.size, _stream_ptr()))
+        self._loaded = True
+
+    def blocks(self) -> np.ndarray:
+        """A copy of the Q4_0 blocks (for a file) (qlinear.mojo:322-324)."""
+        out = np.empty(self.BYTES, np.uint8)
+        L.check(L.lib().nq_get_blocks(self._h, out.ctypes.data_as(C.c_void_p), out.size))
+        return out
+
+    def dequantized(self) -> np.ndarray:
+        """deq(W) [OUT, IN] fp32 on the host (for gates) (qlinear.mojo:326-328)."""
+        self.blocks()  # the `_need_blocks` rule: raises once the blocks were dropped
+        return self.dequantized_dev().cpu().numpy()
+
+    def share_scratch(self, buf: torch.Tensor, n: int):
+        """Use `buf` (n fp32 values, at least OUT*IN) as the dequantize scratch
+        (qlinear.mojo:330-340).  This build's forward never materialises
+        deq(W); the buffer is what `dequantized_dev` without an argument
+        writes."""
+        if n < self.W_SIZE:
+            raise L.NQError(L.NQ_ERR_SIZE,
+                            f"QLinear.share_scratch: {n} values for a [{self.OUT}, {self.IN}] weight")
+        self.deq = buf
+
+    def keep_only_repacked(self):
+        """Drop the logical blocks, keep the device layout the forward reads
+        (qlinear.mojo:342-356).  blocks(), dequantized() and vjp raise after."""
+        L.check(L.lib().nq_keep_only_repacked(self._h))
+
+    # ── Module ─────────────────────────────────────────────────────────────
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, target: str = "gpu",
+                ctx=None) -> torch.Tensor:
+        """y[B, OUT] = x[B, IN] @ deq(W)^T (qlinear.mojo:407-477).  x fp32 (the
+        reference's boundary) or bf16; y fp32."""
+        _need_gpu(target)
+        if x.dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "QLinear.forward: x must be fp32 or bf16")
+        return self._forward(x, _TORCH_DT[x.dtype], None, out, torch.float32, None, "none", "QLinear.forward")
+
+    def vjp(self, forward_input: torch.Tensor, grad_output: torch.Tensor,
+            grad_input: Optional[torch.Tensor] = None, target: str = "gpu", ctx=None) -> torch.Tensor:
+        """grad_input = grad_output @ deq(W), overwriting it (qlinear.mojo:479-518)."""
+        _need_gpu(target)
+        M = _check_x(grad_output, self.OUT, "QLinear.vjp")
+        if grad_output.dtype != torch.float32:
+            raise L.NQError(L.NQ_ERR_INVALID, "QLinear.vjp: grad_output must be fp32")
+        if grad_input is None or grad_input.numel() < M * self.IN:
+            grad_input = torch.empty((M, self.IN), dtype=torch.float32, device=grad_output.device)
+        L.check(L.lib().nq_grad_input(self._h, _dev_ptr(grad_output), _dev_ptr(grad_input), M, _stream_ptr()))
+        return grad_input
+
+    def release_buffers(self):
+        """The reference drops its bf16 activation staging here
+        (qlinear.mojo:520-524); this build has none to drop."""
+
+
+class W8Linear(_Layer):
+    """int8 weight [OUT, IN] with one fp32 scale per output channel.
+    Activations fp32/bf16 (W8A32 / W8A16) or int8 with per-token scales (W8A8)."""
+
+    FORMAT = L.FMT_W8_CHANNEL
+
+    def set_weight(self, w_i8, scales):
+        w = np.ascontiguousarray(w_i8, dtype=np.int8)
+        s = np.ascontiguousarray(scales, dtype=np.float32)
+        if w.size != self.IN * self.OUT or s.size != self.OUT:
+            raise L.NQError(L.NQ_ERR_SIZE, f"W8Linear.set_weight: expected [{self.OUT}, {self.IN}] codes and "
+                                           f"{self.OUT} scales")
+        L.check(L.lib().nq_set_weight_i8(self._h, w.ctypes.data_as(C.c_void_p), s.ctypes.data_as(C.c_void_p),
+                                         _stream_ptr()))
+        self._loaded = True
+
+    def forward(self, x, bias=None, epilogue="none", out=None, out_dtype=torch.float32):
+        if x.dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "W8Linear.forward: x must be fp32 or bf16")
+        return self._forward(x, _TORCH_DT[x.dtype], None, out, out_dtype, bias, epilogue, "W8Linear.forward")
+
+    def forward_a8(self, xq, x_scales, bias=None, epilogue="none", out=None, out_dtype=torch.float32):
+        """int8 activations [M, IN] with per-token scales [M]: int32
+        accumulation, then epi(acc * sx * sw + bias).  out_dtype=torch.int32
+        returns the raw accumulators."""
+        if xq.dtype != torch.int8:
+            raise L.NQError(L.NQ_ERR_INVALID, "W8Linear.forward_a8: xq must be int8")
+        return self._forward(xq, L.DT_I8, x_scales, out, out_dtype, bias, epilogue, "W8Linear.forward_a8")
+
+
+class W4GroupLinear(_Layer):
+    """Asymmetric uint4, group-wise along IN: codes [OUT, IN/2] (low nibble =
+    even k), fp16 scales [OUT, G], packed uint4 zero-points [OUT, ceil(G/2)]."""
+
+    FORMAT = L.FMT_W4_GROUP
+
+    def __init__(self, IN, OUT, group=128):
+        super().__init__(IN, OUT, group)
+        self.G = -(-IN // group)
+
+    def set_weight(self, codes, scales_f16, zps):
+        c = np.ascontiguousarray(codes, dtype=np.uint8)
+        s = np.ascontiguousarray(scales_f16)
+        if s.dtype == np.float16:
+            s = s.view(np.uint16)
+        s = np.ascontiguousarray(s, dtype=np.uint16)
+        z = np.ascontiguousarray(zps, dtype=np.uint8)
+        if c.size != self.OUT * self.IN // 2 or s.size != self.OUT * self.G or z.size != self.OUT * ((self.G + 1) // 2):
+            raise L.NQError(L.NQ_ERR_SIZE, "W4GroupLinear.set_weight: inconsistent sizes")
+        L.check(L.lib().nq_set_weight_w4g(self._h, c.ctypes.data_as(C.c_void_p), s.ctypes.data_as(C.c_void_p),
+                                          z.ctypes.data_as(C.c_void_p), _stream_ptr()))
+        self._loaded = True
+
+    def forward(self, x, bias=None, epilogue="none", out=None, out_dtype=torch.float32):
+        if x.dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "W4GroupLinear.forward: x must be fp32 or bf16")
+        return self._forward(x, _TORCH_DT[x.dtype], None, out, out_dtype, bias, epilogue, "W4GroupLinear.forward")
+
+
+class FP8Linear(_Layer):
+    """OCP e4m3fn weight [OUT, IN] with one fp32 scale; activations e4m3fn with
+    one fp32 scale (or fp32/bf16); fp32 accumulation; bf16 or fp32 output."""
+
+    FORMAT = L.FMT_FP8_E4M3
+
+    def set_weight(self, w_codes, scale: float):
+        w = np.ascontiguousarray(w_codes, dtype=np.uint8)
+        if w.size != self.IN * self.OUT:
+            raise L.NQError(L.NQ_ERR_SIZE, f"FP8Linear.set_weight: expected [{self.OUT}, {self.IN}] codes")
+        L.check(L.lib().nq_set_weight_fp8(self._h, w.ctypes.data_as(C.c_void_p), C.c_float(scale), _stream_ptr()))
+        self._loaded = True
+
+    def forward(self, x_codes, x_scale, bias=None, epilogue="none", out=None, out_dtype=torch.bfloat16):
+        """x_codes: uint8 (or torch.float8_e4m3fn) [M, IN]; x_scale: device fp32 [1]."""
+        if x_codes.dtype == torch.float8_e4m3fn:
+            x_codes = x_codes.view(torch.uint8)
+        if x_codes.dtype != torch.uint8:
+            raise L.NQError(L.NQ_ERR_INVALID, "FP8Linear.forward: x must be e4m3fn codes")
+        return self._forward(x_codes, L.DT_FP8_E4M3, x_scale, out, out_dtype, bias, epilogue, "FP8Linear.forward")
+
+
+def quantize_rows_i8(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None):
+    """Per-token absmax int8 quantisation on the device: (q int8 [M, K], s fp32 [M])."""
+    if x.dtype not in _TORCH_DT or x.dim() != 2 or not x.is_contiguous():
+        raise L.NQError(L.NQ_ERR_INVALID, "quantize_rows_i8: x must be a contiguous fp32/bf16 [M, K] device tensor")
+    M, K = x.shape
+    if q is None:
+        q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    if scales is None:
+        scales = torch.empty((M,), dtype=torch.float32, device=x.device)
+    L.check(L.lib().nq_quantize_rows_i8(_dev_ptr(x), _TORCH_DT[x.dtype], _dev_ptr(q), _dev_ptr(scales), M, K,
+                                        _stream_ptr()))
+    return q, scales
+
+
+def cast_pad_bf16(x: torch.Tensor, cols_pad: int) -> torch.Tensor:
+    """fp32 [rows, cols] -> bf16 [rows, cols_pad], zero tail (qlinear.mojo:152-172)."""
+    rows, cols = x.shape
+    out = torch.empty((rows, cols_pad), dtype=torch.bfloat16, device=x.device)
+    L.check(L.lib().nq_cast_pad_bf16(_dev_ptr(x), _dev_ptr(out), rows, cols, cols_pad, _stream_ptr()))
+    return out
+
+
+def slice_cast_f32(xb: torch.Tensor, cols: int) -> torch.Tensor:
+    """bf16 [rows, cols_pad] -> fp32 [rows, cols] (qlinear.mojo:175-192)."""
+    rows, cols_pad = xb.shape
+    out = torch.empty((rows, cols), dtype=torch.float32, device=xb.device)
+    L.check(L.lib().nq_slice_cast_f32(_dev_ptr(xb), _dev_ptr(out), rows, cols, cols_pad, _stream_ptr()))
+    return out
+
+
+def mlp3_w8a8_forward(l1: W8Linear, l2: W8Linear, l3: W8Linear, x: torch.Tensor, b1=None, b2=None, b3=None,
+                      final_relu: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The three-layer W8A8 actor MLP as one launch (per-token int8 requantisation
+    between layers, int32 accumulation, fused ReLU)."""
+    M = _check_x(x, l1.IN, "mlp3_w8a8_forward")
+    if out is None:
+        out = torch.empty((M, l3.OUT), dtype=torch.float32, device=x.device)
+    L.check(L.lib().nq_mlp3_w8a8_forward(l1._h, l2._h, l3._h, _dev_ptr(x), _dev_ptr(out), M, _dev_ptr(b1),
+                                         _dev_ptr(b2), _dev_ptr(b3), int(final_relu), _stream_ptr()))
+    return out

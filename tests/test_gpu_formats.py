@@ -1,0 +1,225 @@
+"""The int8 / uint4-group / fp8 layers BASELINE's configs name, on the GPU
+through the C ABI, against the CPU oracle on identical seeded inputs.
+
+The reference implements none of these formats, so the oracle's closed forms
+(pinned in tests/test_oracle_ext.py) are the checker.  Bars: int32 accumulators
+bit-exact; fp32/bf16 outputs max-abs-err <= 1e-3 * RMS(exact output);
+fp8 <= 1e-2 * RMS.  At sizes the oracle cannot finish in seconds, parity is
+shown through size-independent properties (linearity in the activations, a
+row/column sample checked exactly, agreement between the GEMV and GEMM paths).
+"""
+import numpy as np
+import pytest
+import torch
+
+from noeira_amd import formats as F
+from noeira_amd.qlinear import FP8Linear, W4GroupLinear, W8Linear, quantize_rows_i8
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL_RMS = 1e-3
+TOL_RMS_FP8 = 1e-2
+
+
+def rel_rms(a, b):
+    b = np.asarray(b, np.float64)
+    return np.abs(np.asarray(a, np.float64) - b).max() / max(np.sqrt((b ** 2).mean()), 1e-300)
+
+
+def bf16(x):
+    return torch.from_numpy(np.ascontiguousarray(x, np.float32)).to(torch.bfloat16)
+
+
+def w8_layer(rng, K, N):
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    lin = W8Linear(K, N)
+    lin.set_weight(w, s)
+    return lin, w, s
+
+
+# ── config 1: W8A32, M=1, K=256, N=256 (SAC actor hidden layer), zero bias ─────
+def test_config1_w8a32_sac_hidden():
+    rng = np.random.default_rng(1)
+    lin, w, s = w8_layer(rng, 256, 256)
+    x = rng.standard_normal((1, 256)).astype(np.float32)
+    bias = np.zeros(256, np.float32)
+    y = lin.forward(torch.from_numpy(x).cuda(), bias=torch.from_numpy(bias).cuda()).cpu().numpy()
+    exact = O.w8_forward_f64(w, s, x, bias)
+    assert rel_rms(y, exact) < TOL_RMS
+    assert rel_rms(y, O.w8_forward_f32(w, s, x, bias)) < TOL_RMS
+    # the integer-activation reading: per-token int8 x, int32 accumulate (bit-exact), then scale
+    xq, sx = quantize_rows_i8(torch.from_numpy(x).cuda())
+    xq_o, sx_o = O.quantize_rows_i8(x)
+    assert np.array_equal(xq.cpu().numpy(), xq_o) and np.array_equal(sx.cpu().numpy(), sx_o)
+    acc = lin.forward_a8(xq, sx, out_dtype=torch.int32).cpu().numpy()
+    assert np.array_equal(acc, O.w8a8_acc_i32(xq_o, w))
+    y8 = lin.forward_a8(xq, sx).cpu().numpy()
+    assert rel_rms(y8, O.w8a8_epilogue(O.w8a8_acc_i32(xq_o, w), sx_o, s)) < 1e-6
+
+
+# ── config 2: ACT policy MLP, W8A16, M in {1, 100}, bf16 bias, fp32 out ────────
+@pytest.mark.parametrize("M", [1, 100])
+@pytest.mark.parametrize("K,N", [(512, 3200), (3200, 512)])
+def test_config2_w8a16_act_mlp(K, N, M):
+    rng = np.random.default_rng(K + N + M)
+    lin, w, s = w8_layer(rng, K, N)
+    xb = bf16(rng.standard_normal((M, K)))
+    bb = bf16(rng.standard_normal(N) * 0.02)
+    y = lin.forward(xb.cuda(), bias=bb.cuda()).cpu().numpy()
+    assert y.dtype == np.float32 and y.shape == (M, N)
+    exact = O.w8_forward_f64(w, s, xb.float().numpy(), bb.float().numpy())
+    assert rel_rms(y, exact) < TOL_RMS, rel_rms(y, exact)
+    # ReLU epilogue and bf16 output
+    yr = lin.forward(xb.cuda(), bias=bb.cuda(), epilogue="relu", out_dtype=torch.bfloat16).float().cpu().numpy()
+    want = bf16(np.maximum(exact, 0).astype(np.float32)).float().numpy()
+    assert np.abs(yr - want).max() <= np.abs(want).max() * 2.0 ** -7  # one bf16 ulp of the largest value
+
+
+# ── config 3: VLM block, W4A16 group 128 asymmetric, M in {1, 256} ────────────
+W4_SHAPES = [(960, 960), (960, 2560), (2560, 960)]
+
+
+@pytest.mark.parametrize("M", [1, 256])
+@pytest.mark.parametrize("K,N", W4_SHAPES)
+def test_config3_w4a16_group128(K, N, M):
+    rng = np.random.default_rng(K * 3 + N + M)
+    group = 128
+    G = -(-K // group)
+    assert (K, G) != (960, 8) or K % group == 64      # the ragged 8th group (64 wide)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    z = rng.integers(0, 16, (N, G), dtype=np.uint8)
+    sc = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+    codes, zps = F.pack_w4g(q, z)
+    lin = W4GroupLinear(K, N, group)
+    lin.set_weight(codes, sc, zps)
+    deq = O.w4g_dequantize(codes, sc.view(np.uint16), zps, N, K, group)
+    assert np.array_equal(lin.dequantized_dev().cpu().numpy().view(np.uint32), deq.view(np.uint32))
+    xb = bf16(rng.standard_normal((M, K)))
+    y = lin.forward(xb.cuda()).cpu().numpy()
+    exact = O.dense_forward_f64(deq, xb.float().numpy())
+    assert rel_rms(y, exact) < TOL_RMS, rel_rms(y, exact)
+
+
+def test_config3_quantized_from_gaussian_weights():
+    """The same path on weights produced by the host quantiser (not random codes)."""
+    rng = np.random.default_rng(33)
+    K, N = 960, 320
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    q, sc, z = F.quantize_w4g_asym(w, 128)
+    codes, zps = F.pack_w4g(q, z)
+    lin = W4GroupLinear(K, N, 128)
+    lin.set_weight(codes, sc, zps)
+    deq = O.w4g_dequantize(codes, sc.view(np.uint16), zps, N, K, 128)
+    assert np.abs(deq - w).max() <= 0.51 * sc.astype(np.float32).max()
+    xb = bf16(rng.standard_normal((3, K)))
+    assert rel_rms(lin.forward(xb.cuda()).cpu().numpy(), O.dense_forward_f64(deq, xb.float().numpy())) < TOL_RMS
+
+
+# ── config 4: batched-env actor, W8A8, M=4096, 64 -> 256 -> 256 -> 8, ReLU ─────
+def actor_layers(rng):
+    dims = [(64, 256), (256, 256), (256, 8)]
+    layers = []
+    for K, N in dims:
+        lin, w, s = w8_layer(rng, K, N)
+        b = (rng.standard_normal(N) * 0.02).astype(np.float32)
+        layers.append((lin, w, s, b))
+    return layers
+
+
+def oracle_actor(layers, x):
+    """Layer by layer: per-token int8, exact int32 accumulate, relu(sx*sw*acc + b)."""
+    h = x
+    accs = []
+    for i, (_, w, s, b) in enumerate(layers):
+        hq, sx = O.quantize_rows_i8(h)
+        acc = O.w8a8_acc_i32(hq, w)
+        accs.append((hq, sx, acc))
+        h = O.w8a8_epilogue(acc, sx, s, b, relu=(i < 2))
+    return h, accs
+
+
+def test_config4_w8a8_actor_layer_by_layer():
+    rng = np.random.default_rng(4)
+    layers = actor_layers(rng)
+    M = 4096
+    x = rng.standard_normal((M, 64)).astype(np.float32)
+    want, accs = oracle_actor(layers, x)
+    h = torch.from_numpy(x).cuda()
+    for i, (lin, w, s, b) in enumerate(layers):
+        hq, sx = quantize_rows_i8(h)
+        hq_o, sx_o, acc_o = accs[i]
+        if i == 0:  # identical inputs: the quantiser and the accumulators are bit-exact
+            assert np.array_equal(hq.cpu().numpy(), hq_o) and np.array_equal(sx.cpu().numpy(), sx_o)
+            acc = lin.forward_a8(hq, sx, out_dtype=torch.int32).cpu().numpy()
+            assert np.array_equal(acc, acc_o)
+        else:       # fed the oracle's codes, the accumulators are bit-exact at every layer
+            acc = lin.forward_a8(torch.from_numpy(hq_o).cuda(), torch.from_numpy(sx_o).cuda(),
+                                 out_dtype=torch.int32).cpu().numpy()
+            assert np.array_equal(acc, acc_o)
+        h = lin.forward_a8(hq, sx, bias=torch.from_numpy(b).cuda(), epilogue="relu" if i < 2 else "none")
+    assert rel_rms(h.cpu().numpy(), want) < TOL_RMS
+
+
+def test_quantize_rows_i8_edges():
+    rng = np.random.default_rng(44)
+    x = rng.standard_normal((37, 256)).astype(np.float32)
+    x[3] = 0.0
+    x[4] = 0.5 * np.arange(256, dtype=np.float32) - 64
+    x[4, 0] = -127.0     # scale exactly 1: the halves are exact ties
+    q, s = quantize_rows_i8(torch.from_numpy(x).cuda())
+    q_o, s_o = O.quantize_rows_i8(x)
+    assert np.array_equal(q.cpu().numpy(), q_o) and np.array_equal(s.cpu().numpy().view(np.uint32), s_o.view(np.uint32))
+    qb, sb = quantize_rows_i8(bf16(x).cuda())
+    q_o, s_o = O.quantize_rows_i8(bf16(x).float().numpy())
+    assert np.array_equal(qb.cpu().numpy(), q_o) and np.array_equal(sb.cpu().numpy(), s_o)
+
+
+# ── config 5: fp8 e4m3 x fp8 e4m3, per-tensor scales, fp32 accumulate, bf16 out ─
+def fp8_operands(rng, M, N, K):
+    a = F.encode_e4m3(rng.standard_normal((M, K)).astype(np.float32))
+    b = F.encode_e4m3(rng.standard_normal((N, K)).astype(np.float32))
+    return a, b
+
+
+def test_encode_e4m3_host_matches_oracle():
+    rng = np.random.default_rng(50)
+    x = (rng.standard_normal(50000) * 3).astype(np.float32)
+    x[:10] = [500, -500, 448, -448, 0, 1e-9, 2 ** -9, 2 ** -10, 0.0625, -0.0625]
+    assert np.array_equal(F.encode_e4m3(x), O.e4m3_encode(np.clip(x, -448, 448)))
+
+
+@pytest.mark.parametrize("M", [1, 64])
+def test_config5_fp8_reduced_size_vs_oracle(M):
+    rng = np.random.default_rng(5 + M)
+    N, K = 512, 4096
+    a, b = fp8_operands(rng, M, N, K)
+    sa, sb = np.float32(0.731), np.float32(1.37)
+    lin = FP8Linear(K, N)
+    lin.set_weight(b, float(sb))
+    xs = torch.tensor([sa], dtype=torch.float32, device="cuda")
+    y = lin.forward(torch.from_numpy(a).cuda(), xs)
+    assert y.dtype == torch.bfloat16
+    y64, ybf = O.fp8_forward_f64(a, b, sa, sb)
+    got = y.float().cpu().numpy()
+    assert rel_rms(got, y64) < TOL_RMS_FP8
+    # bf16 rounding of an fp32-accurate sum: off by at most one bf16 step from the oracle's bits
+    gb = y.view(torch.int16).cpu().numpy().view(np.uint16).astype(np.int32)
+    assert np.abs(gb - ybf.astype(np.int32)).max() <= 1
+    yf = lin.forward(torch.from_numpy(a).cuda(), xs, out_dtype=torch.float32).cpu().numpy()
+    assert rel_rms(yf, y64) < 1e-5
+
+
+def test_config5_fp8_gemv_full_size_sampled():
+    """M = 1 at the full K = 4096, N = 11008: every output against the oracle
+    (45 MB of weights, 45 MFLOP: the oracle finishes in well under a second)."""
+    rng = np.random.default_rng(55)
+    N, K = 11008, 4096
+    a, b = fp8_operands(rng, 1, N, K)
+    lin = FP8Linear(K, N)
+    lin.set_weight(b, 1.0)
+    xs = torch.ones(1, dtype=torch.float32, device="cuda")
+    y = lin.forward(torch.from_numpy(a).cuda(), xs, out_dtype=torch.float32).cpu().numpy()
+    y64, _ = O.fp8_forward_f64(a, b, 1.0, 1.0, want_bf16=False)
+    assert rel_rms(y, y64) < 1e-5
