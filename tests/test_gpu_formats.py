@@ -202,13 +202,16 @@ def test_config5_fp8_reduced_size_vs_oracle(M):
     y = lin.forward(torch.from_numpy(a).cuda(), xs)
     assert y.dtype == torch.bfloat16
     y64, ybf = O.fp8_forward_f64(a, b, sa, sb)
-    got = y.float().cpu().numpy()
-    assert rel_rms(got, y64) < TOL_RMS_FP8
-    # bf16 rounding of an fp32-accurate sum: off by at most one bf16 step from the oracle's bits
-    gb = y.view(torch.int16).cpu().numpy().view(np.uint16).astype(np.int32)
-    assert np.abs(gb - ybf.astype(np.int32)).max() <= 1
+    # The bar (1e-2 of RMS) is applied to the fp32 accumulator-times-scale value.  bf16 itself
+    # carries up to 2^-8 relative rounding, i.e. up to 1.5e-2 of RMS on a 4-sigma output, so the
+    # bf16 output is held to a tighter, exact statement instead: it is the round-to-nearest-even
+    # bf16 of that fp32 value, and within one bf16 step of the oracle's bits.
     yf = lin.forward(torch.from_numpy(a).cuda(), xs, out_dtype=torch.float32).cpu().numpy()
+    assert rel_rms(yf, y64) < TOL_RMS_FP8
     assert rel_rms(yf, y64) < 1e-5
+    gb = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(gb, O.bf16_bits(yf))
+    assert np.abs(gb.astype(np.int32) - ybf.astype(np.int32)).max() <= 1
 
 
 def test_config5_fp8_gemv_full_size_sampled():
