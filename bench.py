@@ -1,0 +1,395 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--no-sweep]
+
+Prints ONE JSON line.  The headline workload is BASELINE.json's configs[1] at
+M = 1: the ACT-style policy MLP's two W8A16 linears (512 -> 3200 and
+3200 -> 512, bf16 activations, int8 weights with per-channel fp32 scales, bf16
+bias, fp32 output).  A step is one pass over both linears.  Weights, inputs
+and outputs are resident in HBM before the timed region.  Because a 1.6 MB
+weight sits in the 256 MB Infinity Cache, the step rotates through enough
+distinct copies of the two layers (>= 512 MB) that every call streams from
+HBM ("cold"); the warm figure (one copy, the reference's own protocol,
+benchmarks/quant/bench_qlinear_smolvla.mojo:37-38,89-137) is reported beside
+it.  `value` is algorithmic GB/s: every operand counted once (weights, scales,
+bias, x, y), no scratch, no padding.
+
+`results` carries every other BASELINE config measured with the reference's
+protocol (warm-up, 7 samples of N calls between two synchronisations, median
+sample / N), each with its own roofline fraction; `roofline` is the headline
+workload's kernel; `roofline_mfma` is the large-M fp8 GEMM (config 5).
+
+`cpu_baseline` times the CPU oracle's restatement of the reference's CPU
+forward (a fresh dequantize to an fp32 scratch, then the serial triple loop;
+noeira/nn/quant/qlinear.mojo:416-426, noeira/nn/core/cpu_gemm.mojo:88-98) on
+one host core, on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TOPS = {"fp8": 5000.0, "int8": 5000.0, "bf16": 2500.0}
+SAMPLES, COLD_BYTES = 7, 512 << 20
+
+
+def ensure_built():
+    from noeira_amd import _lib
+
+    try:
+        _lib.lib()
+    except OSError:
+        from noeira_amd import build as nq_build
+
+        nq_build.build()
+        _lib.lib()
+
+
+def bf16_t(x):
+    import numpy as np
+    import torch
+
+    return torch.from_numpy(np.ascontiguousarray(x, np.float32)).to(torch.bfloat16)
+
+
+class Timer:
+    """HIP events on torch's current stream (the stream every launch goes to)."""
+
+    def __init__(self):
+        import torch
+
+        self.t = torch
+        self.a = torch.cuda.Event(enable_timing=True)
+        self.b = torch.cuda.Event(enable_timing=True)
+
+    def run(self, fn, n):
+        self.t.cuda.synchronize()
+        self.a.record()
+        for i in range(n):
+            fn(i)
+        self.b.record()
+        self.t.cuda.synchronize()
+        return self.a.elapsed_time(self.b) * 1e-3  # seconds
+
+
+def median_per_call(fn, calls):
+    """The reference's protocol: warm once, SAMPLES samples of `calls` calls."""
+    tm = Timer()
+    fn(0)
+    ts = [tm.run(fn, calls) / calls for _ in range(SAMPLES)]
+    return statistics.median(ts)
+
+
+# ── workloads ───────────────────────────────────────────────────────────────
+def make_act_w8a16(M, copies, seed=2):
+    """configs[1]: two W8A16 linears, K=512->N=3200 and K=3200->N=512."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import W8Linear
+
+    rng = np.random.default_rng(seed)
+    dims = [(512, 3200), (3200, 512)]
+    sets = []
+    for _ in range(copies):
+        pair = []
+        for K, N in dims:
+            lin = W8Linear(K, N)
+            lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8),
+                           rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+            pair.append(lin)
+        sets.append(pair)
+    xs = [bf16_t(rng.standard_normal((M, K))).cuda() for K, _ in dims]
+    bs = [bf16_t(rng.standard_normal(N) * 0.02).cuda() for _, N in dims]
+    ys = [torch.empty((M, N), dtype=torch.float32, device="cuda") for _, N in dims]
+    nbytes = sum(N * K + 4 * N + 2 * N + 2 * K * M + 4 * N * M for K, N in dims)
+    ops = sum(2 * M * N * K for K, N in dims)
+
+    def step(i):
+        pair = sets[i % copies]
+        pair[0].forward(xs[0], bias=bs[0], out=ys[0])
+        pair[1].forward(xs[1], bias=bs[1], out=ys[1])
+
+    return dict(step=step, bytes=nbytes, ops=ops, launches=2, keep=(sets, xs, bs, ys))
+
+
+def make_q4_0(IN, OUT, M, copies, seed=3):
+    """The reference's own layer: Q4_0 group 32, fp32 activations, fp32 out."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import QLinear
+
+    rng = np.random.default_rng(seed)
+    nb = OUT * (IN // 32) * 18
+    layers = []
+    for _ in range(copies):
+        blocks = rng.integers(0, 256, nb, dtype=np.uint8)
+        sc = rng.uniform(1e-3, 2e-3, OUT * (IN // 32)).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        blocks.reshape(-1, 18)[:, 0:2] = sc
+        ql = QLinear.make(IN, OUT, "gpu")
+        ql.set_blocks(blocks)
+        layers.append(ql)
+    x = torch.from_numpy(rng.standard_normal((M, IN)).astype(np.float32)).cuda()
+    y = torch.empty((M, OUT), dtype=torch.float32, device="cuda")
+
+    def step(i):
+        layers[i % copies].forward(x, out=y)
+
+    return dict(step=step, bytes=nb + 4 * IN * M + 4 * OUT * M, ops=2 * M * IN * OUT, launches=1,
+                keep=(layers, x, y))
+
+
+def make_w4g(K, N, M, copies, seed=4):
+    """configs[2]: asymmetric uint4, group 128, fp16 scales, bf16 activations."""
+    import numpy as np
+    import torch
+
+    from noeira_amd import formats as F
+    from noeira_amd.qlinear import W4GroupLinear
+
+    rng = np.random.default_rng(seed)
+    G = -(-K // 128)
+    layers = []
+    for _ in range(copies):
+        codes = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+        sc = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+        zps = F.pack_u4_pairs(rng.integers(0, 16, (N, G), dtype=np.uint8))
+        lin = W4GroupLinear(K, N, 128)
+        lin.set_weight(codes, sc, zps)
+        layers.append(lin)
+    x = bf16_t(rng.standard_normal((M, K))).cuda()
+    y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+
+    def step(i):
+        layers[i % copies].forward(x, out=y)
+
+    nbytes = N * K // 2 + 2 * N * G + N * ((G + 1) // 2) + 2 * K * M + 4 * N * M
+    return dict(step=step, bytes=nbytes, ops=2 * M * N * K, launches=1, keep=(layers, x, y))
+
+
+def make_w8a32(seed=1):
+    """configs[0]: W8A32, M=1, K=N=256."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import W8Linear
+
+    rng = np.random.default_rng(seed)
+    lin = W8Linear(256, 256)
+    lin.set_weight(rng.integers(-127, 128, (256, 256), dtype=np.int8), rng.uniform(1e-3, 1e-2, 256).astype(np.float32))
+    x = torch.from_numpy(rng.standard_normal((1, 256)).astype(np.float32)).cuda()
+    b = torch.zeros(256, dtype=torch.float32, device="cuda")
+    y = torch.empty((1, 256), dtype=torch.float32, device="cuda")
+    return dict(step=lambda i: lin.forward(x, bias=b, out=y), bytes=68608, ops=2 * 256 * 256, launches=1,
+                keep=(lin, x, b, y))
+
+
+def make_actor_w8a8(M=4096, seed=5):
+    """configs[3]: 64 -> 256 -> 256 -> 8, per-token int8 activations, ReLU."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import W8Linear, quantize_rows_i8
+
+    rng = np.random.default_rng(seed)
+    dims = [(64, 256), (256, 256), (256, 8)]
+    lins, biases = [], []
+    for K, N in dims:
+        lin = W8Linear(K, N)
+        lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        lins.append(lin)
+        biases.append(torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda())
+    x = torch.from_numpy(rng.standard_normal((M, 64)).astype(np.float32)).cuda()
+    qs = [torch.empty((M, K), dtype=torch.int8, device="cuda") for K, _ in dims]
+    ss = [torch.empty((M,), dtype=torch.float32, device="cuda") for _ in dims]
+    hs = [torch.empty((M, N), dtype=torch.float32, device="cuda") for _, N in dims]
+
+    def step(i):
+        h = x
+        for j, lin in enumerate(lins):
+            quantize_rows_i8(h, qs[j], ss[j])
+            h = lin.forward_a8(qs[j], ss[j], bias=biases[j], epilogue="relu" if j < 2 else "none", out=hs[j])
+
+    ops = sum(2 * M * K * N for K, N in dims)
+    nbytes = sum(K * N + 4 * N for K, N in dims) + 4 * M * 64 + 4 * M * 8
+    return dict(step=step, bytes=nbytes, ops=ops, launches=6, keep=(lins, biases, x, qs, ss, hs))
+
+
+def make_fp8(M, N, K=4096, copies=1, seed=6):
+    """configs[4]: e4m3 x e4m3, per-tensor scales, fp32 accumulate, bf16 out."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import FP8Linear
+
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    layers = []
+    for _ in range(copies):
+        w = torch.randn((N, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        lin = FP8Linear(K, N)
+        lin.set_weight(w, 1.0 / 16)
+        layers.append(lin)
+    a = torch.randn((M, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).cuda()
+    sa = torch.tensor([1.0 / 16], dtype=torch.float32, device="cuda")
+    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def step(i):
+        layers[i % copies].forward(a, sa, out=y)
+
+    return dict(step=step, bytes=N * K + M * K + 2 * M * N + 8, ops=2 * M * N * K, launches=1, keep=(layers, a, sa, y))
+
+
+def report(name, wl, seconds, bound, peak_key=None):
+    gbps = wl["bytes"] / seconds / 1e9
+    tops = wl["ops"] / seconds / 1e12
+    r = {"workload": name, "us_per_call": round(seconds * 1e6, 3), "GBps": round(gbps, 2), "TOPS": round(tops, 4),
+         "bound": bound}
+    if bound == "hbm":
+        r["frac_of_roofline"] = round(gbps / HBM_PEAK_GBPS, 4)
+    else:
+        r["frac_of_roofline"] = round(tops / MFMA_PEAK_TOPS[peak_key], 4)
+    return r
+
+
+def sweep(skip_large=False):
+    """Every BASELINE config, the reference's timing protocol."""
+    import torch
+
+    out = []
+
+    def run(name, maker, bound, peak_key=None, calls=50, **kw):
+        wl = maker(**kw)
+        copies = kw.get("copies", 1)
+        t = median_per_call(wl["step"], max(calls, copies))
+        out.append(report(name, wl, t, bound, peak_key))
+        del wl
+        torch.cuda.empty_cache()
+
+    run("cfg0 W8A32 256->256 M=1 (warm)", make_w8a32, "hbm")
+    run("cfg1 W8A16 ACT MLP M=100 (warm)", make_act_w8a16, "hbm", M=100, copies=1)
+    for (K, N) in [(960, 960), (960, 2560), (2560, 960)]:
+        c = max(1, COLD_BYTES // (N * K // 2))
+        run(f"cfg2 W4A16 g128 {K}->{N} M=1 (cold)", make_w4g, "hbm", K=K, N=N, M=1, copies=c, calls=c)
+        run(f"cfg2 W4A16 g128 {K}->{N} M=256 (warm)", make_w4g, "mfma", "bf16", K=K, N=N, M=256, copies=1, calls=20)
+    for (IN, OUT) in [(960, 960), (960, 320), (960, 2560), (2560, 960)]:
+        c = max(1, COLD_BYTES // (OUT * IN * 9 // 16))
+        run(f"ref Q4_0 g32 {IN}->{OUT} M=1 fp32 (cold)", make_q4_0, "hbm", IN=IN, OUT=OUT, M=1, copies=c, calls=c)
+        run(f"ref Q4_0 g32 {IN}->{OUT} M=135 fp32 (warm)", make_q4_0, "mfma", "bf16", IN=IN, OUT=OUT, M=135,
+            copies=1, calls=20)
+    run("cfg3 W8A8 actor 64->256->256->8 M=4096 (6 launches)", make_actor_w8a8, "mfma", "int8", calls=20)
+    for N in (4096, 11008):
+        c = max(1, COLD_BYTES // (N * 4096))
+        run(f"cfg4 fp8 GEMV K=4096 N={N} M=1 (cold)", make_fp8, "hbm", M=1, N=N, copies=c, calls=max(c, 20))
+        if not skip_large:
+            run(f"cfg4 fp8 GEMM M=8192 K=4096 N={N}", make_fp8, "mfma", "fp8", M=8192, N=N, copies=1, calls=3)
+    return out
+
+
+def cpu_baseline(budget_s=12.0):
+    """The oracle's restatement of the reference's CPU forward, one core, on the
+    headline workload's two linears (M = 1) for about `budget_s` seconds."""
+    import numpy as np
+
+    from oracle import oracle as O
+
+    rng = np.random.default_rng(2)
+    dims = [(512, 3200), (3200, 512)]
+    ws = [(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32)) for K, N in dims]
+    xs = [bf16_t(rng.standard_normal((1, K))).float().numpy() for K, _ in dims]
+    bs = [bf16_t(rng.standard_normal(N) * 0.02).float().numpy() for _, N in dims]
+    nbytes = sum(N * K + 4 * N + 2 * N + 2 * K + 4 * N for K, N in dims)
+    O.w8_qlinear_forward_cpu(ws[0][0], ws[0][1], xs[0], bs[0])
+    n, t0 = 0, time.perf_counter()
+    while True:
+        for (w, s), x, b in zip(ws, xs, bs):
+            O.w8_qlinear_forward_cpu(w, s, x, b)
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s and n >= 3:
+            break
+    return {"value": round(nbytes * n / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "ms_per_step": round(dt / n * 1e3, 3),
+            "sample": f"{n} steps of the headline workload (both W8 linears at M=1): a fresh dequantize to an "
+                      f"fp32 [OUT, IN] scratch then the serial triple loop, single thread, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--only", default="", help="time only the headline loop (for rocprofv3 runs)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {a.gpus} is not supported "
+              "(one layer's forward needs no second device).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    ensure_built()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    per_pair = 2 * 512 * 3200
+    copies = -(-COLD_BYTES // per_pair)
+    wl = make_act_w8a16(1, copies)
+    tm = Timer()
+    for i in range(a.warmup):
+        wl["step"](i)
+    sec = tm.run(wl["step"], a.steps)
+    ms_per_step = sec / a.steps * 1e3
+    value = wl["bytes"] / (sec / a.steps) / 1e9
+    launch_s = sec / (a.steps * wl["launches"])
+    achieved = (wl["bytes"] / wl["launches"]) / launch_s / 1e9
+
+    warm = make_act_w8a16(1, 1)
+    warm_s = median_per_call(warm["step"], 200)
+
+    line = {
+        "metric": "qlinear GB/s at M=1 and TOPS at M=4096, as % of MI355X roofline",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 weights x bf16 activations, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1], ACT-style policy MLP W8A16 at M=1: linears 512->3200 and "
+                               "3200->512, int8 weights + per-channel fp32 scales, bf16 x, bf16 bias, fp32 y; "
+                               f"cold: rotating over {copies} distinct weight copies ({copies * per_pair >> 20} MiB)",
+                   "algorithmic_bytes_per_step": wl["bytes"], "launches_per_step": wl["launches"]},
+        "pct_of_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 3),
+        "warm": {"GBps": round(warm["bytes"] / warm_s / 1e9, 2), "us_per_step": round(warm_s * 1e6, 3),
+                 "note": "one weight copy, resident in L2 / Infinity Cache (the reference's protocol)"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 5), "traffic": None,
+                     "kernel": "nq::gemv_kernel<W8_CHANNEL, MT=1>", "avg_launch_us": round(launch_s * 1e6, 3)},
+    }
+    if a.only:
+        print(json.dumps(line))
+        return
+    if not a.no_sweep:
+        line["results"] = sweep()
+        mf = [r for r in line["results"] if "fp8 GEMM" in r["workload"]]
+        if mf:
+            best = max(mf, key=lambda r: r["TOPS"])
+            line["roofline_mfma"] = {"bound": "mfma", "achieved": best["TOPS"], "peak": MFMA_PEAK_TOPS["fp8"],
+                                     "unit": "TFLOP/s", "frac": round(best["TOPS"] / MFMA_PEAK_TOPS["fp8"], 5),
+                                     "workload": best["workload"]}
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

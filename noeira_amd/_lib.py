@@ -54,6 +54,11 @@ def lib() -> C.CDLL:
     global _lib
     if _lib is not None:
         return _lib
+    # torch first: the device pointers and streams this package hands to the library come from
+    # torch, so both must run on the one HIP runtime torch ships (same SONAME; the first one
+    # loaded into the process wins).
+    import torch  # noqa: F401
+
     last = None
     for path in candidates():
         if os.sep in path and not os.path.exists(path):

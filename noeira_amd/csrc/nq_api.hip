@@ -357,6 +357,7 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
                 return fail(NQ_ERR_INVALID, "nq_forward: y must be fp32, bf16 or int32");
             if (!x_scale) return fail(NQ_ERR_INVALID, "nq_forward: int8 activations need per-row scales");
         }
+        if (gemm8_applicable(a)) return launch_gemm8(a);
         return launch_gemv_i8(a);
     }
     if (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16)
@@ -368,6 +369,7 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
     } else if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16) {
         return fail(NQ_ERR_INVALID, "nq_forward: unknown x dtype " + std::to_string(x_dtype));
     }
+    if (gemm8_applicable(a)) return launch_gemm8(a);
     return launch_gemv(a);
 }
 

@@ -82,6 +82,10 @@ int32_t launch_w4g_unpack_zps(const uint8_t* packed, uint8_t* out, int64_t rows,
 int32_t launch_gemv(const ForwardArgs& a);
 int32_t launch_gemv_i8(const ForwardArgs& a);
 
+// nq_gemm8.hip: LDS-tiled fp8 / int8 MFMA GEMM for large M
+bool gemm8_applicable(const ForwardArgs& a);
+int32_t launch_gemm8(const ForwardArgs& a);
+
 // nq_quant.hip
 int32_t launch_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M,
                                 int32_t K, hipStream_t s);

@@ -1,0 +1,290 @@
+// Large-M GEMM over 8-bit operands on the CDNA4 matrix cores:
+//     fp8 e4m3 x fp8 e4m3 -> fp32   (v_mfma_f32_32x32x64_f8f6f4)
+//     int8     x int8     -> int32  (v_mfma_i32_32x32x32_i8)
+//   y[M, N] = epi( (x[M, K] . w[N, K]^T) * scale + bias[N] )
+// Both operands are K-contiguous, which is the layout the MFMA wants: a lane
+// supplies 32 consecutive bytes of one row.
+//
+// Tiling.  One workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 tile of y;
+// each wavefront owns 128 x 128 of it as 4 x 4 MFMA tiles of 32 x 32, i.e. 256
+// fp32/int32 accumulators per lane (the AGPR half of the unified register
+// file), one workgroup per CU.  A wavefront tile this large is what keeps the
+// kernel MFMA-bound: per 64-byte k-step a wavefront issues 16 MFMAs (1024
+// cycles) for 16 KiB of LDS reads, half the LDS bandwidth; at 64 x 64 the LDS
+// would be the limit.
+//
+// K loop.  Stages of BK = 128 bytes: x tile 256 x 128 B and w tile 256 x 128 B
+// (64 KiB), double-buffered in LDS (128 of the CU's 160 KiB).  While a stage is
+// being multiplied, the next stage's 16 128-bit global loads per lane are in
+// flight into registers; they are written to the other LDS buffer after the
+// MFMAs, so there is one barrier per stage.
+//
+// LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
+// permuted by slot ^= (row >> 1) & 7.  Rows r and r + 1 then sit 128 B apart in
+// different bank halves and rows two apart in different slots, so both the
+// 128-bit fragment reads (32 rows x 2 slots per wavefront instruction) and the
+// staging writes are conflict free.
+//
+// Workgroup order.  Hardware deals consecutive workgroup ids round-robin to
+// the 8 XCDs, each with its own L2.  Ids are first regrouped so that each XCD
+// gets one contiguous run of tiles, and runs walk the tile grid in bands of 8
+// row tiles, so the ~32 tiles resident on an XCD share 8 x-tiles and 4 w-tiles
+// in that XCD's L2 instead of 32 + 32.
+#include <type_traits>
+
+#include "nq_common.h"
+
+namespace nq {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+constexpr int BM = 256, BN = 256, BK = 128;
+constexpr int STAGE_BYTES = (BM + BN) * BK;  // 64 KiB
+
+struct Gemm8Params {
+    const uint8_t* a;  // x [M][K]
+    const uint8_t* b;  // w [N][K]
+    void* y;
+    const void* bias;
+    const float* row_scale;  // int8: per-row activation scales [M]; fp8: [1]
+    const float* col_scale;  // int8: per-channel weight scales [N]
+    float tscale;            // fp8: the weight's per-tensor scale
+    int32_t M, N, K;
+    int32_t tiles_m, tiles_n;
+    int32_t y_dtype, bias_dtype, epilogue;
+};
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float v) {
+    uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
+__device__ __forceinline__ int lds_off(int row, int slot) {
+    return row * BK + ((slot ^ ((row >> 1) & 7)) << 4);
+}
+
+template <bool FP8>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm8_kernel(const Gemm8Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // ---- XCD-aware tile assignment
+    const int nb = gridDim.x;
+    const int bid = blockIdx.x;
+    const int per = nb / 8, rem = nb % 8;
+    const int xcd = bid % 8, local = bid / 8;
+    const int lid = xcd * per + min(xcd, rem) + local;
+    constexpr int GM = 8;
+    const int band = lid / (GM * p.tiles_n);
+    const int first_m = band * GM;
+    const int band_rows = min(GM, p.tiles_m - first_m);
+    const int in_band = lid - band * GM * p.tiles_n;
+    const int tm = first_m + in_band % band_rows;
+    const int tn = in_band / band_rows;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // ---- global -> register staging: 8 pieces of x and 8 of w per lane per stage
+    const uint8_t* ga[8];
+    const uint8_t* gb[8];
+    int so[8];  // LDS offset of piece i (same for the x and the w tile)
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int piece = tid + 256 * i;
+        const int row = piece >> 3, slot = piece & 7;
+        ga[i] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.K + slot * 16;
+        gb[i] = p.b + (int64_t)min(n0 + row, p.N - 1) * p.K + slot * 16;
+        so[i] = lds_off(row, slot);
+    }
+    u32x4 ra[8], rb[8];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            ra[i] = *reinterpret_cast<const u32x4*>(ga[i] + k0);
+            rb[i] = *reinterpret_cast<const u32x4*>(gb[i] + k0);
+        }
+    };
+    auto stash = [&](int buf) {
+        uint8_t* base = lds + buf * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            *reinterpret_cast<u32x4*>(base + so[i]) = ra[i];
+            *reinterpret_cast<u32x4*>(base + BM * BK + so[i]) = rb[i];
+        }
+    };
+
+    typedef typename std::conditional<FP8, f32x16, i32x16>::type acc_t;
+    acc_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // Fragment addressing.  fp8: a 64-byte k-step, this lane supplies bytes [32 h, 32 h + 32) of
+    // its row (h = lane / 32), i.e. slots 4 s + 2 h and 4 s + 2 h + 1.  int8: a 32-byte k-step,
+    // bytes [16 h, 16 h + 16), slot 2 s + h.  Tile bases are multiples of 32 rows, so the swizzle
+    // term depends on the row within the tile only.
+    const int frow = lane & 31;
+    const int fh = lane >> 5;
+    const int fsw = (frow >> 1) & 7;
+
+    const int KT = p.K / BK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; kt++) {
+        if (kt + 1 < KT) fetch((kt + 1) * BK);
+        const uint8_t* sa = lds + (kt & 1) * STAGE_BYTES + (wm * 128 + frow) * BK;
+        const uint8_t* sb = lds + (kt & 1) * STAGE_BYTES + BM * BK + (wn * 128 + frow) * BK;
+        if constexpr (FP8) {
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                const int o0 = ((4 * s + 2 * fh) ^ fsw) << 4, o1 = ((4 * s + 2 * fh + 1) ^ fsw) << 4;
+                i32x8 af[4], bf[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const i32x4 lo = *reinterpret_cast<const i32x4*>(sa + i * 32 * BK + o0);
+                    const i32x4 hi = *reinterpret_cast<const i32x4*>(sa + i * 32 * BK + o1);
+                    af[i] = (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    const i32x4 lo2 = *reinterpret_cast<const i32x4*>(sb + i * 32 * BK + o0);
+                    const i32x4 hi2 = *reinterpret_cast<const i32x4*>(sb + i * 32 * BK + o1);
+                    bf[i] = (i32x8){lo2[0], lo2[1], lo2[2], lo2[3], hi2[0], hi2[1], hi2[2], hi2[3]};
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], 0, 0, 0,
+                                                                                     0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                const int o0 = ((2 * s + fh) ^ fsw) << 4;
+                i32x4 af[4], bf[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    af[i] = *reinterpret_cast<const i32x4*>(sa + i * 32 * BK + o0);
+                    bf[i] = *reinterpret_cast<const i32x4*>(sb + i * 32 * BK + o0);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        if (kt + 1 < KT) stash((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds column n = l % 32 and rows 8*(r/4) + 4*(l/32) + r%4 of each tile.
+    // The output type is resolved once, outside the unrolled loops.
+    const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;
+    auto emit = [&](auto kind) {
+        constexpr int KIND = decltype(kind)::value;  // 0: fp32, 1: bf16, 2: raw int32
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int mb = m0 + wm * 128 + i * 32 + 4 * (lane >> 5);
+            float rs[16];
+            if constexpr (!FP8 && KIND != 2) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) rs[r] = p.row_scale[min(mb + 8 * (r >> 2) + (r & 3), p.M - 1)];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int n = n0 + wn * 128 + j * 32 + (lane & 31);
+                if (n >= p.N) continue;
+                float cscale = 1.0f, bias = 0.0f;
+                if constexpr (!FP8 && KIND != 2) cscale = p.col_scale[n];
+                if (p.bias)
+                    bias = (p.bias_dtype == NQ_DT_F32)
+                               ? reinterpret_cast<const float*>(p.bias)[n]
+                               : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = mb + 8 * (r >> 2) + (r & 3);
+                    if (m >= p.M) continue;
+                    const int64_t o = (int64_t)m * p.N + n;
+                    if constexpr (KIND == 2) {
+                        reinterpret_cast<int32_t*>(p.y)[o] = (int32_t)acc[i][j][r];
+                    } else {
+                        float z;
+                        if constexpr (FP8)
+                            z = acc[i][j][r] * fp8_scale;
+                        else
+                            z = (float)acc[i][j][r] * (rs[r] * cscale);
+                        z += bias;
+                        if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                        if constexpr (KIND == 0)
+                            reinterpret_cast<float*>(p.y)[o] = z;
+                        else
+                            reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16(z);
+                    }
+                }
+            }
+        }
+    };
+    if (p.y_dtype == NQ_DT_F32)
+        emit(std::integral_constant<int, 0>{});
+    else if (p.y_dtype == NQ_DT_BF16)
+        emit(std::integral_constant<int, 1>{});
+    else if constexpr (!FP8)
+        emit(std::integral_constant<int, 2>{});
+}
+
+}  // namespace
+
+bool gemm8_applicable(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    const bool fp8 = (a.x_dtype == NQ_DT_FP8_E4M3 && L->format == NQ_FMT_FP8_E4M3);
+    const bool i8 = (a.x_dtype == NQ_DT_I8 && L->format == NQ_FMT_W8_CHANNEL);
+    return (fp8 || i8) && (L->in % BK == 0) && a.M >= 64;
+}
+
+int32_t launch_gemm8(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    Gemm8Params p{};
+    p.a = reinterpret_cast<const uint8_t*>(a.x);
+    p.b = L->d_codes;
+    p.y = a.y, p.bias = a.bias;
+    p.row_scale = a.x_scale;
+    p.col_scale = reinterpret_cast<const float*>(L->d_scales);
+    p.tscale = L->scale;
+    p.M = a.M, p.N = L->out, p.K = L->in;
+    p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + BN - 1) / BN;
+    p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    const dim3 grid(p.tiles_m * p.tiles_n);
+    const size_t lds = 2 * STAGE_BYTES;
+    static bool attr_set[2] = {false, false};
+    if (a.x_dtype == NQ_DT_FP8_E4M3) {
+        if (!attr_set[0]) {
+            NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            attr_set[0] = true;
+        }
+        hipLaunchKernelGGL(gemm8_kernel<true>, grid, dim3(256), lds, a.stream, p);
+    } else {
+        if (!attr_set[1]) {
+            NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            attr_set[1] = true;
+        }
+        hipLaunchKernelGGL(gemm8_kernel<false>, grid, dim3(256), lds, a.stream, p);
+    }
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+}  // namespace nq

@@ -543,3 +543,21 @@ void nqo_f16_bits_array(const float* x, int64_t n, uint16_t* out) {
 void nqo_f16_value_array(const uint16_t* h, int64_t n, float* out) {
     for (int64_t i = 0; i < n; i++) out[i] = nqo_f16_value(h[i]);
 }
+
+/* The reference's CPU forward (qlinear.mojo:416-426: a FRESH dequantize to an
+ * fp32 [OUT, IN] scratch, then the serial gemm_cpu) restated for an int8
+ * per-channel weight: deq[n,k] = float(w[n,k]) * s[n], y = x @ deq^T (+ bias).
+ * Used as the single-core CPU baseline of the W8 workloads. */
+int nqo_w8_qlinear_forward_cpu(const int8_t* w, const float* s, int64_t N, int64_t K, const float* x,
+                               int64_t M, const float* bias, float* y) {
+    float* deq = (float*)malloc(sizeof(float) * (size_t)(N * K));
+    if (!deq) return NQO_ENOMEM;
+    for (int64_t n = 0; n < N; n++)
+        for (int64_t k = 0; k < K; k++) deq[n * K + k] = (float)w[n * K + k] * s[n];
+    nqo_gemm_cpu(0, 1, M, N, K, 1.0f, x, K, deq, K, 0.0f, y, N);
+    if (bias)
+        for (int64_t m = 0; m < M; m++)
+            for (int64_t n = 0; n < N; n++) y[m * N + n] += bias[n];
+    free(deq);
+    return NQO_OK;
+}

@@ -100,6 +100,8 @@ def lib() -> C.CDLL:
         L.nqo_fp8_forward_f64.argtypes = [p, p, i64, i64, i64, f32, f32, p, p]
         L.nqo_e4m3_dequantize.restype = None
         L.nqo_e4m3_dequantize.argtypes = [p, i64, p]
+        L.nqo_w8_qlinear_forward_cpu.restype = C.c_int
+        L.nqo_w8_qlinear_forward_cpu.argtypes = [p, p, i64, i64, p, i64, p, p]
         for name in ("nqo_e4m3_encode_array", "nqo_f16_bits_array", "nqo_f16_value_array"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [p, i64, p]
@@ -306,6 +308,21 @@ def w8_forward_f64(w, s, x, bias=None, relu=False):
     b = _c(bias, np.float32) if bias is not None else None
     y = np.empty((M, N), np.float64)
     lib().nqo_w8_forward_f64(_ptr(w), _ptr(s), N, K, _ptr(x), M, _ptr(b), int(relu), _ptr(y))
+    return y
+
+
+def w8_qlinear_forward_cpu(w, s, x, bias=None, out=None):
+    """Dequantize-to-scratch then serial GEMM, as QLinear.forward["cpu"] does."""
+    w = _c(w, np.int8)
+    s = _c(s, np.float32)
+    x = _c(x, np.float32)
+    N, K = w.shape
+    M = x.size // K
+    b = _c(bias, np.float32) if bias is not None else None
+    y = out if out is not None else np.empty((M, N), np.float32)
+    rc = lib().nqo_w8_qlinear_forward_cpu(_ptr(w), _ptr(s), N, K, _ptr(x), M, _ptr(b), _ptr(y))
+    if rc:
+        raise MemoryError("w8_qlinear_forward_cpu")
     return y
 
 
