@@ -274,6 +274,7 @@ int32_t nq_set_weight_w4g(nq_handle h, const uint8_t* codes_host, const uint16_t
     if (e == hipSuccess) e = hipMemcpyAsync(h->d_scales, scales_f16_host, ng * 2, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = hipMemcpyAsync(zp_packed, zps_host, nz, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) rc = launch_w4g_unpack_zps(zp_packed, h->d_zps, h->out, h->groups, s);
+    if (e == hipSuccess && rc == NQ_OK) rc = launch_w4g_repack(h->d_codes, (int64_t)h->out * (h->in / 32), s);
     if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
     (void)hipFree(zp_packed);
     if (e != hipSuccess) return fail_hip(e, "nq_set_weight_w4g upload");
@@ -370,6 +371,7 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
         return fail(NQ_ERR_INVALID, "nq_forward: unknown x dtype " + std::to_string(x_dtype));
     }
     if (gemm8_applicable(a)) return launch_gemm8(a);
+    if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
     return launch_gemv(a);
 }
 

@@ -78,6 +78,12 @@ int32_t launch_grad_input_q4_0(const nq_layer* L, const float* gy, float* gx, in
 int32_t launch_w4g_unpack_zps(const uint8_t* packed, uint8_t* out, int64_t rows, int64_t groups,
                               hipStream_t s);
 
+int32_t launch_w4g_repack(uint8_t* codes, int64_t nchunks, hipStream_t s);
+
+// nq_gemm_a16.hip: medium-M dequant GEMM on the bf16 matrix cores
+bool gemm_a16_applicable(const ForwardArgs& a);
+int32_t launch_gemm_a16(const ForwardArgs& a);
+
 // nq_gemv.hip: dequant-GEMV for small M (also the any-M fallback)
 int32_t launch_gemv(const ForwardArgs& a);
 int32_t launch_gemv_i8(const ForwardArgs& a);

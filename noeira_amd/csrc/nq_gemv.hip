@@ -181,10 +181,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
                 float4 xa[MT], xb[MT];
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
-                    if (FMT == NQ_FMT_Q4_0) {          // word jw: elements 4jw.. (low), 16+4jw.. (high)
-                        xa[m] = xs[(m * QPC + jw) * p.psq + c];
-                        xb[m] = xs[(m * QPC + jw + 4) * p.psq + c];
-                    } else if (FMT == NQ_FMT_W4_GROUP) {  // word jw: elements 8jw .. 8jw+7
+                    if (FOUR_BIT) {                    // word jw: elements 8jw .. 8jw+7
                         xa[m] = xs[(m * QPC + 2 * jw) * p.psq + c];
                         xb[m] = xs[(m * QPC + 2 * jw + 1) * p.psq + c];
                     } else {                           // word jw: elements 4jw .. 4jw+3
@@ -194,23 +191,16 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
 #pragma unroll
                 for (int r = 0; r < RPL; r++) {
                     const uint32_t word = wv[r][jw];
-                    if (FMT == NQ_FMT_Q4_0) {
+                    if (FOUR_BIT) {
+                        // device nibble order (nq_nib.h): low nibbles of the four bytes are elements
+                        // 0, 4, 1, 5; high nibbles are elements 2, 6, 3, 7
                         const uint32_t lo = word & 0x0F0F0F0Fu, hi = (word >> 4) & 0x0F0F0F0Fu;
-                        const float l0 = ub0(lo), l1 = ub1(lo), l2 = ub2(lo), l3 = ub3(lo);
-                        const float h0 = ub0(hi), h1 = ub1(hi), h2 = ub2(hi), h3 = ub3(hi);
+                        const float e0 = ub0(lo), e4 = ub1(lo), e1 = ub2(lo), e5 = ub3(lo);
+                        const float e2 = ub0(hi), e6 = ub1(hi), e3 = ub2(hi), e7 = ub3(hi);
 #pragma unroll
                         for (int m = 0; m < MT; m++) {
-                            dot[r][m] = dot4(xa[m], l0, l1, l2, l3, dot[r][m]);
-                            dot[r][m] = dot4(xb[m], h0, h1, h2, h3, dot[r][m]);
-                        }
-                    } else if (FMT == NQ_FMT_W4_GROUP) {
-                        const uint32_t lo = word & 0x0F0F0F0Fu, hi = (word >> 4) & 0x0F0F0F0Fu;
-                        const float l0 = ub0(lo), l1 = ub1(lo), l2 = ub2(lo), l3 = ub3(lo);
-                        const float h0 = ub0(hi), h1 = ub1(hi), h2 = ub2(hi), h3 = ub3(hi);
-#pragma unroll
-                        for (int m = 0; m < MT; m++) {
-                            dot[r][m] = dot4(xa[m], l0, h0, l1, h1, dot[r][m]);
-                            dot[r][m] = dot4(xb[m], l2, h2, l3, h3, dot[r][m]);
+                            dot[r][m] = dot4(xa[m], e0, e1, e2, e3, dot[r][m]);
+                            dot[r][m] = dot4(xb[m], e4, e5, e6, e7, dot[r][m]);
                         }
                     } else if (FMT == NQ_FMT_W8_CHANNEL) {
                         const uint32_t t = word ^ 0x80808080u;  // int8 + 128 as unsigned bytes

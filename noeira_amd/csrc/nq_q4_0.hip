@@ -3,14 +3,17 @@
 #include <hip/hip_fp16.h>
 
 #include "nq_common.h"
+#include "nq_nib.h"
 
 namespace nq {
 
 // ---------------------------------------------------------------------------
-// Q4_0 blocks [nblocks][18] -> nibble bytes [nblocks][16] + fp16 scale bits.
+// Q4_0 blocks [nblocks][18] -> device chunks [nblocks][16] + fp16 scale bits.
 // The 18-byte block is only 2-byte aligned; splitting the scale off makes each
-// group one aligned 128-bit load for the forward kernels.  Bytes are moved,
-// never reinterpreted, so NaN/inf/subnormal scales survive unchanged.
+// group one aligned 128-bit load for the forward kernels, and the nibbles are
+// re-ordered from the block's split-half order (byte j = element j | element
+// j+16 << 4) to the device order of nq_nib.h.  Scale bytes are moved, never
+// reinterpreted, so NaN/inf/subnormal scales survive unchanged.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void q4_0_repack_kernel(const uint8_t* __restrict__ raw,
                                                           uint8_t* __restrict__ codes,
@@ -23,11 +26,15 @@ __global__ __launch_bounds__(256) void q4_0_repack_kernel(const uint8_t* __restr
 #pragma unroll
     for (int i = 0; i < 9; i++) h[i] = src[i];
     scales[b] = h[0];
+    uint8_t e[Q4_GROUP];
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const uint8_t byte = (uint8_t)(h[1 + (j >> 1)] >> (8 * (j & 1)));
+        e[j] = byte & 0xF;
+        e[j + 16] = byte >> 4;
+    }
     uint4 v;
-    v.x = (uint32_t)h[1] | ((uint32_t)h[2] << 16);
-    v.y = (uint32_t)h[3] | ((uint32_t)h[4] << 16);
-    v.z = (uint32_t)h[5] | ((uint32_t)h[6] << 16);
-    v.w = (uint32_t)h[7] | ((uint32_t)h[8] << 16);
+    v.x = nib_pack8(e), v.y = nib_pack8(e + 8), v.z = nib_pack8(e + 16), v.w = nib_pack8(e + 24);
     reinterpret_cast<uint4*>(codes)[b] = v;
 }
 
@@ -129,6 +136,30 @@ int32_t launch_w4g_unpack_zps(const uint8_t* packed, uint8_t* out, int64_t rows,
     return NQ_OK;
 }
 
+// W4_GROUP codes, in place: logical bytes (byte i = element 2i | element 2i+1 << 4) -> device order
+__global__ __launch_bounds__(256) void w4g_repack_kernel(uint8_t* __restrict__ codes, int64_t nchunks) {
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= nchunks) return;
+    uint4 v = reinterpret_cast<uint4*>(codes)[c];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint8_t e[32];
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const uint8_t byte = (uint8_t)(w[j >> 2] >> (8 * (j & 3)));
+        e[2 * j] = byte & 0xF;
+        e[2 * j + 1] = byte >> 4;
+    }
+    v.x = nib_pack8(e), v.y = nib_pack8(e + 8), v.z = nib_pack8(e + 16), v.w = nib_pack8(e + 24);
+    reinterpret_cast<uint4*>(codes)[c] = v;
+}
+
+int32_t launch_w4g_repack(uint8_t* codes, int64_t nchunks, hipStream_t s) {
+    if (nchunks == 0) return NQ_OK;
+    hipLaunchKernelGGL(w4g_repack_kernel, dim3((unsigned)((nchunks + 255) / 256)), dim3(256), 0, s, codes, nchunks);
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
 // ---------------------------------------------------------------------------
 // deq(W) [OUT, IN] fp32.  The device twin of dequantize_q4_0
 // (`dequant_q4_0_kernel`, q4_0.mojo:242-266), one thread per 128-bit chunk of
@@ -158,24 +189,21 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restri
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     float* dst = out + r * (int64_t)K + (int64_t)c * EPC;
     float o[EPC];
-    if (FMT == NQ_FMT_Q4_0) {
-        float d = __half2float(__ushort_as_half(reinterpret_cast<const uint16_t*>(scales)[i]));
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xFFu;
-            o[j] = ((float)(int)(byte & 0xF) - 8.0f) * d;
-            o[j + 16] = ((float)(int)(byte >> 4) - 8.0f) * d;
+    if (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP) {
+        float d, z;
+        if (FMT == NQ_FMT_Q4_0) {
+            d = __half2float(__ushort_as_half(reinterpret_cast<const uint16_t*>(scales)[i]));
+            z = 8.0f;
+        } else {
+            const int g = (c * EPC) / group;
+            d = __half2float(__ushort_as_half(reinterpret_cast<const uint16_t*>(scales)[r * groups + g]));
+            z = (float)zps[r * groups + g];
         }
-    } else if (FMT == NQ_FMT_W4_GROUP) {
-        int g = (c * EPC) / group;
-        float d = __half2float(__ushort_as_half(reinterpret_cast<const uint16_t*>(scales)[r * groups + g]));
-        float z = (float)zps[r * groups + g];
+        float q[EPC];
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xFFu;
-            o[2 * j] = ((float)(int)(byte & 0xF) - z) * d;
-            o[2 * j + 1] = ((float)(int)(byte >> 4) - z) * d;
-        }
+        for (int t = 0; t < 4; t++) nib_unpack8(w[t], q + 8 * t);
+#pragma unroll
+        for (int j = 0; j < EPC; j++) o[j] = (q[j] - z) * d;
     } else if (FMT == NQ_FMT_W8_CHANNEL) {
         float s = reinterpret_cast<const float*>(scales)[r];
 #pragma unroll
@@ -249,16 +277,14 @@ __global__ __launch_bounds__(256) void grad_input_q4_0_kernel(const uint8_t* __r
             float gv[GI_MT];
 #pragma unroll
             for (int m = 0; m < GI_MT; m++) gv[m] = (m0 + m < M) ? gy[(int64_t)(m0 + m) * N + o] : 0.0f;
+            float q[Q4_GROUP];
 #pragma unroll
-            for (int j = 0; j < 16; j++) {
-                uint32_t byte = (w[j >> 2] >> (8 * (j & 3))) & 0xFFu;
-                float lo = ((float)(int)(byte & 0xF) - 8.0f) * d;
-                float hi = ((float)(int)(byte >> 4) - 8.0f) * d;
+            for (int t = 0; t < 4; t++) nib_unpack8(w[t], q + 8 * t);
 #pragma unroll
-                for (int m = 0; m < GI_MT; m++) {
-                    acc[m][j] = fmaf(gv[m], lo, acc[m][j]);
-                    acc[m][j + 16] = fmaf(gv[m], hi, acc[m][j + 16]);
-                }
+            for (int j = 0; j < Q4_GROUP; j++) {
+                const float wv = (q[j] - 8.0f) * d;
+#pragma unroll
+                for (int m = 0; m < GI_MT; m++) acc[m][j] = fmaf(gv[m], wv, acc[m][j]);
             }
         }
     }
