@@ -430,9 +430,30 @@ int32_t nq_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int32_t
 int32_t nq_mlp3_w8a8_forward(nq_handle l1, nq_handle l2, nq_handle l3, const float* x, float* y, int32_t M,
                              const float* b1, const float* b2, const float* b3, int32_t final_epilogue,
                              void* stream) {
-    (void)l1, (void)l2, (void)l3, (void)x, (void)y, (void)M, (void)b1, (void)b2, (void)b3;
-    (void)final_epilogue, (void)stream;
-    return fail(NQ_ERR_UNSUPPORTED, "nq_mlp3_w8a8_forward: not built yet");
+    nq_handle ls[3] = {l1, l2, l3};
+    for (int i = 0; i < 3; i++) {
+        int32_t rc = check_handle(ls[i], "nq_mlp3_w8a8_forward");
+        if (rc) return rc;
+        if ((rc = need_loaded(ls[i], "forward"))) return rc;
+        if (ls[i]->format != NQ_FMT_W8_CHANNEL)
+            return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: every layer must be W8_CHANNEL");
+        if (ls[i]->in > 256 || ls[i]->out > 256)
+            return fail(NQ_ERR_UNSUPPORTED, "nq_mlp3_w8a8_forward: layer " + std::to_string(i + 1) + " is [" +
+                                                std::to_string(ls[i]->in) + " -> " + std::to_string(ls[i]->out) +
+                                                "]; the fused kernel holds at most 256 features per token");
+    }
+    if (l1->out != l2->in || l2->out != l3->in)
+        return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: the layers do not chain (" + std::to_string(l1->in) + " -> " +
+                                        std::to_string(l1->out) + ", " + std::to_string(l2->in) + " -> " +
+                                        std::to_string(l2->out) + ", " + std::to_string(l3->in) + " -> " +
+                                        std::to_string(l3->out) + ")");
+    if (final_epilogue != NQ_EPI_NONE && final_epilogue != NQ_EPI_RELU)
+        return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: unknown epilogue " + std::to_string(final_epilogue));
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!x || !y) return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: null x or y");
+    if ((uintptr_t)x & 15) return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: x must be 16-byte aligned");
+    return launch_mlp3_w8a8(l1, l2, l3, x, y, M, b1, b2, b3, final_epilogue, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -92,6 +92,11 @@ int32_t launch_gemv_i8(const ForwardArgs& a);
 bool gemm8_applicable(const ForwardArgs& a);
 int32_t launch_gemm8(const ForwardArgs& a);
 
+// nq_mlp.hip: three W8A8 layers in one launch
+int32_t launch_mlp3_w8a8(const nq_layer* l1, const nq_layer* l2, const nq_layer* l3, const float* x, float* y,
+                         int32_t M, const float* b1, const float* b2, const float* b3, int32_t final_relu,
+                         hipStream_t s);
+
 // nq_quant.hip
 int32_t launch_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M,
                                 int32_t K, hipStream_t s);

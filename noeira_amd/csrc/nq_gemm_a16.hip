@@ -31,6 +31,8 @@
 // the B operand of four MFMAs.
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
+
 #include "nq_common.h"
 
 namespace nq {
@@ -119,12 +121,14 @@ __device__ __forceinline__ void load_a(const void* x, int64_t elem_off, bool val
 }
 
 template <int FMT, bool XF32, int MW, int NW>
-__global__ __launch_bounds__(256) void gemm_a16_kernel(const A16Params p) {
+__global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
     constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL);
     constexpr int NT = XF32 ? 3 : 1;
     constexpr int KSTEP = FOUR_BIT ? 128 : 64;  // k covered by one 16-byte weight load per lane x 4 lanes
     constexpr int NMF = FOUR_BIT ? 4 : 2;       // MFMAs (32 k each) per k-step
-    __shared__ float red[3][MW * NW * 4 * 64];
+    constexpr int RED = MW * NW * 4 * 64;       // floats one wavefront contributes to the reduction
+    extern __shared__ float red[];              // [KW - 1][RED]
+    const int KW = blockDim.x >> 6;             // wavefronts splitting K
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kb = lane >> 4;
@@ -155,13 +159,16 @@ __global__ __launch_bounds__(256) void gemm_a16_kernel(const A16Params p) {
     const u32x4* wq = reinterpret_cast<const u32x4*>(p.codes);
 
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
-    for (int ks = wave; ks < nsteps; ks += 4) {
-        // ---- weights: one 128-bit load per lane per n-tile
-        u32x4 wv[NW];
+    auto load_w = [&](int ks, u32x4 (&dst)[NW]) {
         const int c = ks * 4 + kb;  // the 16-byte chunk this lane loads
-        const bool cvalid = c < p.nch;
+        const bool cvalid = ks < nsteps && c < p.nch;
 #pragma unroll
-        for (int j = 0; j < NW; j++) wv[j] = cvalid ? wq[wrow[j] + c] : (u32x4){0, 0, 0, 0};
+        for (int j = 0; j < NW; j++) dst[j] = cvalid ? wq[wrow[j] + c] : (u32x4){0, 0, 0, 0};
+    };
+    u32x4 wv[NW], wnext[NW];
+    load_w(wave, wv);
+    for (int ks = wave; ks < nsteps; ks += KW) {
+        load_w(ks + KW, wnext);  // in flight while this k-step is multiplied
 
         if constexpr (FOUR_BIT) {
             // per-chunk scale and zero point for chunks 4ks .. 4ks+3 of row n (lane's own column)
@@ -253,6 +260,8 @@ __global__ __launch_bounds__(256) void gemm_a16_kernel(const A16Params p) {
                 }
             }
         }
+#pragma unroll
+        for (int j = 0; j < NW; j++) wv[j] = wnext[j];
     }
 
     if constexpr (!FOUR_BIT) {
@@ -271,7 +280,7 @@ __global__ __launch_bounds__(256) void gemm_a16_kernel(const A16Params p) {
 #pragma unroll
             for (int j = 0; j < NW; j++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) red[wave - 1][((i * NW + j) * 4 + r) * 64 + lane] = acc[i][j][r];
+                for (int r = 0; r < 4; r++) red[(wave - 1) * RED + ((i * NW + j) * 4 + r) * 64 + lane] = acc[i][j][r];
     }
     __syncthreads();
     if (wave != 0) return;
@@ -293,9 +302,7 @@ __global__ __launch_bounds__(256) void gemm_a16_kernel(const A16Params p) {
                 if (m >= p.M) continue;
                 const int ri = ((i * NW + j) * 4 + r) * 64 + lane;
                 float z = acc[i][j][r];
-                z += red[0][ri];
-                z += red[1][ri];
-                z += red[2][ri];
+                for (int w = 0; w < KW - 1; w++) z += red[w * RED + ri];
                 if (FMT == NQ_FMT_W8_CHANNEL) z *= rs;
                 z += b;
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
@@ -309,28 +316,34 @@ __global__ __launch_bounds__(256) void gemm_a16_kernel(const A16Params p) {
 }
 
 template <int FMT, bool XF32, int MW>
-int32_t launch_nw(const A16Params& p, int nw, dim3 grid, hipStream_t s) {
+int32_t launch_nw(const A16Params& p, int nw, int kw, dim3 grid, hipStream_t s) {
+    const size_t lds = (size_t)(kw - 1) * MW * nw * 4 * 64 * sizeof(float);
     if (nw == 1)
-        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW, 1>), grid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW, 1>), grid, dim3(64 * kw), lds, s, p);
     else
-        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW, 2>), grid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW, 2>), grid, dim3(64 * kw), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
 
 template <int FMT, bool XF32>
-int32_t launch_mw(const A16Params& p, int mw, int nw, dim3 grid, hipStream_t s) {
+int32_t launch_mw(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
     switch (mw) {
-        case 1: return launch_nw<FMT, XF32, 1>(p, nw, grid, s);
-        case 2: return launch_nw<FMT, XF32, 2>(p, nw, grid, s);
-        case 3: return launch_nw<FMT, XF32, 3>(p, nw, grid, s);
-        default: return launch_nw<FMT, XF32, 4>(p, nw, grid, s);
+        case 1: return launch_nw<FMT, XF32, 1>(p, nw, kw, grid, s);
+        case 2: return launch_nw<FMT, XF32, 2>(p, nw, kw, grid, s);
+        case 3: return launch_nw<FMT, XF32, 3>(p, nw, kw, grid, s);
+        default: return launch_nw<FMT, XF32, 4>(p, nw, kw, grid, s);
     }
 }
 
 template <int FMT>
-int32_t launch_x(const A16Params& p, bool xf32, int mw, int nw, dim3 grid, hipStream_t s) {
-    return xf32 ? launch_mw<FMT, true>(p, mw, nw, grid, s) : launch_mw<FMT, false>(p, mw, nw, grid, s);
+int32_t launch_x(const A16Params& p, bool xf32, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
+    return xf32 ? launch_mw<FMT, true>(p, mw, nw, kw, grid, s) : launch_mw<FMT, false>(p, mw, nw, kw, grid, s);
+}
+
+int env_int(const char* name, int dflt) {
+    const char* v = std::getenv(name);
+    return v ? std::atoi(v) : dflt;
 }
 
 }  // namespace
@@ -366,13 +379,27 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
             if (tiles < best_tiles) best_tiles = tiles, mw = c;
         }
     }
-    const int nw = (L->out >= 1024) ? 2 : 1;
+    int nw = (L->out >= 1024) ? 2 : 1;
+    if (mw * nw > 6) nw = 1;  // 4 x 2 MFMA tiles per wavefront would spill under the 256-register budget
+    // wavefronts along K: as many as it takes to leave each one at most two k-steps (the call is
+    // latency-bound: a k-step is one dependent round trip to memory), within the LDS the
+    // fixed-order reduction needs
+    const int kstep = four_bit ? 128 : 64;
+    const int nsteps = (L->in + kstep - 1) / kstep;
+    int kw = 4;
+    while (kw < 8 && (nsteps + kw - 1) / kw > 2) kw *= 2;
+    while ((size_t)(kw - 1) * mw * nw * 1024 > 60 * 1024) {
+        if (nw > 1) nw = 1;
+        else if (mw > 1) mw--;
+        else kw /= 2;
+    }
+    kw = env_int("NQ_A16_KW", kw);
     dim3 grid((L->out + 16 * nw - 1) / (16 * nw), (a.M + 16 * mw - 1) / (16 * mw));
     const bool xf32 = a.x_dtype == NQ_DT_F32;
     switch (L->format) {
-        case NQ_FMT_Q4_0: return launch_x<NQ_FMT_Q4_0>(p, xf32, mw, nw, grid, a.stream);
-        case NQ_FMT_W4_GROUP: return launch_x<NQ_FMT_W4_GROUP>(p, xf32, mw, nw, grid, a.stream);
-        case NQ_FMT_W8_CHANNEL: return launch_x<NQ_FMT_W8_CHANNEL>(p, xf32, mw, nw, grid, a.stream);
+        case NQ_FMT_Q4_0: return launch_x<NQ_FMT_Q4_0>(p, xf32, mw, nw, kw, grid, a.stream);
+        case NQ_FMT_W4_GROUP: return launch_x<NQ_FMT_W4_GROUP>(p, xf32, mw, nw, kw, grid, a.stream);
+        case NQ_FMT_W8_CHANNEL: return launch_x<NQ_FMT_W8_CHANNEL>(p, xf32, mw, nw, kw, grid, a.stream);
     }
     return fail(NQ_ERR_INVALID, "nq_forward: unknown format");
 }

@@ -284,3 +284,44 @@ def test_int8_gemm_bit_exact(M, K, N):
     yb = lin.forward_a8(xd, sd, bias=torch.from_numpy(bias).cuda(), out_dtype=torch.bfloat16)
     want_b = O.w8a8_epilogue(acc_o, sx, s, bias)
     assert np.abs(yb.float().cpu().numpy() - want_b).max() <= np.abs(want_b).max() * 2.0 ** -8
+
+
+def test_config4_w8a8_actor_fused_single_launch():
+    """The same MLP as one launch (nq_mlp3_w8a8_forward) against the layer-by-layer oracle."""
+    from noeira_amd.qlinear import mlp3_w8a8_forward
+    rng = np.random.default_rng(4)
+    layers = actor_layers(rng)
+    for M in (4096, 1, 37):
+        x = rng.standard_normal((M, 64)).astype(np.float32)
+        want, _ = oracle_actor(layers, x)
+        bs = [torch.from_numpy(l[3]).cuda() for l in layers]
+        y = torch.full((M, 8), float("nan"), device="cuda")
+        mlp3_w8a8_forward(layers[0][0], layers[1][0], layers[2][0], torch.from_numpy(x).cuda(), bs[0], bs[1], bs[2],
+                          out=y)
+        got = y.cpu().numpy()
+        assert not np.isnan(got).any()
+        assert rel_rms(got, want) < TOL_RMS, rel_rms(got, want)
+        # no requantisation flips at all on this seed: the fused path equals the unfused oracle to fp32 rounding
+        assert rel_rms(got, want) < 1e-5
+
+
+def test_mlp3_other_shapes_and_errors():
+    from noeira_amd import _lib as L
+    from noeira_amd.qlinear import mlp3_w8a8_forward
+    rng = np.random.default_rng(41)
+    dims = [(48, 112), (112, 64), (64, 24)]      # K not a multiple of 64, N not a multiple of 64
+    layers = []
+    for K, N in dims:
+        lin, w, s = w8_layer(rng, K, N)
+        layers.append((lin, w, s, (rng.standard_normal(N) * 0.02).astype(np.float32)))
+    x = rng.standard_normal((50, 48)).astype(np.float32)
+    h = x
+    for i, (_, w, s, b) in enumerate(layers):
+        hq, sx = O.quantize_rows_i8(h)
+        h = O.w8a8_epilogue(O.w8a8_acc_i32(hq, w), sx, s, b, relu=True)
+    bs = [torch.from_numpy(l[3]).cuda() for l in layers]
+    y = mlp3_w8a8_forward(layers[0][0], layers[1][0], layers[2][0], torch.from_numpy(x).cuda(), bs[0], bs[1], bs[2],
+                          final_relu=True).cpu().numpy()
+    assert rel_rms(y, h) < TOL_RMS
+    with pytest.raises(L.NQError, match="do not chain"):
+        mlp3_w8a8_forward(layers[0][0], layers[2][0], layers[1][0], torch.from_numpy(x).cuda())
