@@ -372,6 +372,7 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
     }
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
+    if (gemv_m1_applicable(a)) return launch_gemv_m1(a);
     return launch_gemv(a);
 }
 

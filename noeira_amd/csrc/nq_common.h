@@ -88,6 +88,10 @@ int32_t launch_gemm_a16(const ForwardArgs& a);
 int32_t launch_gemv(const ForwardArgs& a);
 int32_t launch_gemv_i8(const ForwardArgs& a);
 
+// nq_gemv_m1.hip: register-resident GEMV for a single activation row
+bool gemv_m1_applicable(const ForwardArgs& a);
+int32_t launch_gemv_m1(const ForwardArgs& a);
+
 // nq_gemm8.hip: LDS-tiled fp8 / int8 MFMA GEMM for large M
 bool gemm8_applicable(const ForwardArgs& a);
 int32_t launch_gemm8(const ForwardArgs& a);

@@ -158,6 +158,18 @@ __global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
     }
     const u32x4* wq = reinterpret_cast<const u32x4*>(p.codes);
 
+    // the epilogue's operands are requested up front: nothing is loaded after the reduction
+    float ep_scale[NW], ep_bias[NW];
+#pragma unroll
+    for (int j = 0; j < NW; j++) {
+        ep_scale[j] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[nrow[j]] : 1.0f;
+        ep_bias[j] = 0.0f;
+        if (p.bias)
+            ep_bias[j] = (p.bias_dtype == NQ_DT_F32)
+                             ? reinterpret_cast<const float*>(p.bias)[nrow[j]]
+                             : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[nrow[j]] << 16);
+    }
+
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
     auto load_w = [&](int ks, u32x4 (&dst)[NW]) {
         const int c = ks * 4 + kb;  // the 16-byte chunk this lane loads
@@ -288,12 +300,7 @@ __global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
     for (int j = 0; j < NW; j++) {
         const int n = n_base + 16 * j + ln;
         if (n >= p.N) continue;
-        float rs = 1.0f, b = 0.0f;
-        if (FMT == NQ_FMT_W8_CHANNEL) rs = reinterpret_cast<const float*>(p.scales)[n];
-        if (p.bias)
-            b = (p.bias_dtype == NQ_DT_F32)
-                    ? reinterpret_cast<const float*>(p.bias)[n]
-                    : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+        const float rs = ep_scale[j], b = ep_bias[j];
 #pragma unroll
         for (int i = 0; i < MW; i++)
 #pragma unroll

@@ -140,6 +140,18 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
 #pragma unroll
         for (int r = 0; r < RPL; r++) rows[r] = min(row0 + r, (int64_t)p.N - 1);
 
+        // the epilogue's operands are requested before the K loop, not after the reduction
+        float ep_scale[RPL], ep_bias[RPL];
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            ep_scale[r] = 1.0f, ep_bias[r] = 0.0f;
+            if (FMT == NQ_FMT_W8_CHANNEL) ep_scale[r] = reinterpret_cast<const float*>(p.scales)[rows[r]];
+            if (FMT == NQ_FMT_FP8_E4M3) ep_scale[r] = p.tscale * (p.x_scale ? p.x_scale[0] : 1.0f);
+            if (p.bias)
+                ep_bias[r] = (p.bias_dtype == NQ_DT_F32)
+                                 ? reinterpret_cast<const float*>(p.bias)[rows[r]]
+                                 : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[rows[r]]);
+        }
         float acc[RPL][MT];
 #pragma unroll
         for (int r = 0; r < RPL; r++)
@@ -244,15 +256,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(const GemvParams p) {
             for (int r = 0; r < RPL; r++) {
                 const int64_t n = row0 + r;
                 if (n >= p.N) continue;
-                float rs = 1.0f;
-                if (FMT == NQ_FMT_W8_CHANNEL) rs = reinterpret_cast<const float*>(p.scales)[n];
-                if (FMT == NQ_FMT_FP8_E4M3) rs = p.tscale * (p.x_scale ? p.x_scale[0] : 1.0f);
-                float b = 0.0f;
-                if (p.bias) {
-                    b = (p.bias_dtype == NQ_DT_F32)
-                            ? reinterpret_cast<const float*>(p.bias)[n]
-                            : bf16_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]);
-                }
+                const float rs = ep_scale[r], b = ep_bias[r];
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     if (m0 + m >= p.M) continue;

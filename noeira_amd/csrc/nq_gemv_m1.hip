@@ -1,0 +1,440 @@
+// Dequant-GEMV for one activation row (M = 1): y[N] = epi(deq(W) x + bias).
+//
+// The regime is HBM- or latency-bound: the only large operand is the packed
+// weight, read exactly once with 128-bit non-temporal loads.  x is small and
+// shared by every row, so each lane keeps the slice of x it needs IN REGISTERS
+// for the whole kernel: `lpr` lanes (a power of two) share a row, lane j owns
+// the 16-byte chunks j, j + lpr, ... (CPL of them), and the x values under
+// those chunks are loaded once, up front, together with the first weights -
+// one round trip to memory, no LDS, no barrier.  A lane group then walks its
+// rows RPL at a time (RPL x CPL independent loads in flight per lane).
+//
+//   8-bit weights (int8, fp8):  x held as fp32, one v_cvt per code + one FMA.
+//   4-bit weights, bf16 x:      x held as packed bf16 pairs; a word of eight
+//       codes becomes four bf16 pairs (16 + q) with a shift and an and-or each
+//       (device nibble order, nq_nib.h) and goes through v_dot2_f32_bf16:
+//       1.5 VALU ops per weight instead of 2.25.
+//   4-bit weights, fp32 x:      x held as fp32, v_cvt + FMA (exact fp32
+//       products, the reference's 1e-5 band).
+// Offsets and zero points leave the inner loop through xsum, the sum of x
+// under a chunk: sum x (q - z) = sum x q - z xsum.
+//
+// The cross-lane sum is a fixed butterfly, so a repeated call returns the same
+// bits (tests/nn/quant/test_qlinear_gpu.mojo:96,128).
+#include <hip/hip_fp16.h>
+
+#include <cstdlib>
+
+#include "nq_common.h"
+
+namespace nq {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+struct M1Params {
+    const uint8_t* codes;
+    const void* scales;
+    const uint8_t* zps;
+    const void* x;
+    const float* x_scale;
+    void* y;
+    const void* bias;
+    int32_t N, K;
+    int32_t group, groups;
+    float tscale;
+    int32_t nch;   // 16-byte chunks per row
+    int32_t lpr;   // lanes per row (a power of two)
+    int32_t lpr_log2;
+    int32_t rpw;   // rows per lane group (a multiple of RPL)
+    int32_t x_dtype, y_dtype, bias_dtype, epilogue;
+};
+
+__device__ __forceinline__ float bf16lo(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t pair) { return __uint_as_float(pair & 0xFFFF0000u); }
+
+__device__ __forceinline__ uint16_t to_bf16(float v) {
+    uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
+// Sum over a group of `lpr` consecutive lanes (a power of two); every lane of the group ends with
+// the total.  Butterfly in a fixed order: quad swaps, half-row and row mirrors (DPP), then the
+// 16- and 32-lane swaps (v_permlane16_swap / v_permlane32_swap).  No LDS traffic.
+__device__ __forceinline__ float group_sum(float v, int lpr) {
+    int t;
+    if (lpr > 1) {
+        t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+        v += __int_as_float(t);
+    }
+    if (lpr > 2) {
+        t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+        v += __int_as_float(t);
+    }
+    if (lpr > 4) {
+        t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false);  // row_half_mirror
+        v += __int_as_float(t);
+    }
+    if (lpr > 8) {
+        t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false);  // row_mirror
+        v += __int_as_float(t);
+    }
+    if (lpr > 16) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+    if (lpr > 32) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+    return v;
+}
+
+template <int FMT, bool DOT2, int CPL, int RPL>
+__global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
+    constexpr bool FOUR_BIT = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP);
+    constexpr int EPC = FOUR_BIT ? 32 : 16;
+    constexpr int XR = DOT2 ? EPC / 2 : EPC;  // registers of x per chunk
+    static_assert(!DOT2 || FOUR_BIT, "the bf16 dot path is for 4-bit weights");
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lpr = p.lpr;
+    const int rg = lane >> p.lpr_log2, lj = lane & (lpr - 1);
+
+    const u32x4* wq = reinterpret_cast<const u32x4*>(p.codes);
+    const int64_t group_id = (((int64_t)blockIdx.x * 4 + wave) << (6 - p.lpr_log2)) + rg;
+    const int64_t row_begin = group_id * p.rpw;
+    bool cval[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; i++) cval[i] = (lj + i * lpr) < p.nch;
+
+    // One batch = RPL rows x CPL chunks of codes (+ their scales) for this lane.  The first batch is
+    // requested before x so that both arrive in one round trip; afterwards batch b+1 is in flight
+    // while batch b is multiplied.
+    auto fetch = [&](int64_t row0, u32x4 (&wv)[RPL][CPL], float (&cs)[RPL][CPL], float (&cz)[RPL][CPL],
+                     float (&rs)[RPL], float (&rbias)[RPL]) {
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            const int64_t row = min(row0 + r, (int64_t)p.N - 1);
+            // the epilogue's operands travel with the codes, so nothing is loaded after the reduction
+            rs[r] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[row] : 1.0f;
+            rbias[r] = 0.0f;
+            if (p.bias)
+                rbias[r] = (p.bias_dtype == NQ_DT_F32)
+                               ? reinterpret_cast<const float*>(p.bias)[row]
+                               : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[row] << 16);
+#pragma unroll
+            for (int i = 0; i < CPL; i++) {
+                const int c = lj + i * lpr;
+                const bool ok = cval[i] && row0 < p.N;
+                wv[r][i] = ok ? __builtin_nontemporal_load(&wq[row * p.nch + c]) : (u32x4){0, 0, 0, 0};
+                cs[r][i] = 0.0f, cz[r][i] = 0.0f;
+                if constexpr (FOUR_BIT) {
+                    if (ok) {
+                        if (FMT == NQ_FMT_Q4_0) {
+                            cs[r][i] = __half2float(
+                                __ushort_as_half(reinterpret_cast<const uint16_t*>(p.scales)[row * p.nch + c]));
+                            cz[r][i] = 8.0f;
+                        } else {
+                            const int g = (c * EPC) / p.group;
+                            cs[r][i] = __half2float(
+                                __ushort_as_half(reinterpret_cast<const uint16_t*>(p.scales)[row * p.groups + g]));
+                            cz[r][i] = (float)p.zps[row * p.groups + g];
+                        }
+                    }
+                }
+            }
+        }
+    };
+    u32x4 wv[RPL][CPL], wn[RPL][CPL];
+    float cs[RPL][CPL], cz[RPL][CPL], csn[RPL][CPL], czn[RPL][CPL];
+    float rs[RPL], rbias[RPL], rsn[RPL], rbiasn[RPL];
+    const float tscale = (FMT == NQ_FMT_FP8_E4M3) ? p.tscale * (p.x_scale ? p.x_scale[0] : 1.0f) : 1.0f;
+    fetch(row_begin, wv, cs, cz, rs, rbias);
+
+    // ---- this lane's slice of x, loaded once
+    uint32_t xr[CPL][XR];  // fp32 bits, or bf16 pairs when DOT2
+    float xsum[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; i++) {
+        const int c = lj + i * lpr;
+        const int64_t k0 = (int64_t)c * EPC;
+        float s = 0.0f;
+        if constexpr (DOT2) {
+#pragma unroll
+            for (int v = 0; v < EPC / 8; v++) {
+                u32x4 t = {0, 0, 0, 0};
+                if (cval[i]) t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    xr[i][4 * v + e] = t[e];
+                    s += bf16lo(t[e]) + bf16hi(t[e]);
+                }
+            }
+        } else {
+            float f[EPC];
+            if (!cval[i]) {
+#pragma unroll
+                for (int e = 0; e < EPC; e++) f[e] = 0.0f;
+            } else if (p.x_dtype == NQ_DT_F32) {
+#pragma unroll
+                for (int v = 0; v < EPC / 4; v++) {
+                    const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.x) + k0 + 4 * v);
+                    f[4 * v] = t.x, f[4 * v + 1] = t.y, f[4 * v + 2] = t.z, f[4 * v + 3] = t.w;
+                }
+            } else if (p.x_dtype == NQ_DT_BF16) {
+#pragma unroll
+                for (int v = 0; v < EPC / 8; v++) {
+                    const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) f[8 * v + 2 * e] = bf16lo(t[e]), f[8 * v + 2 * e + 1] = bf16hi(t[e]);
+                }
+            } else {  // fp8 e4m3
+#pragma unroll
+                for (int v = 0; v < EPC / 16; v++) {
+                    const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(p.x) + k0 + 16 * v);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)t[e], false);
+                        const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)t[e], true);
+                        f[16 * v + 4 * e] = a[0], f[16 * v + 4 * e + 1] = a[1];
+                        f[16 * v + 4 * e + 2] = b[0], f[16 * v + 4 * e + 3] = b[1];
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < EPC; e++) {
+                xr[i][e] = __float_as_uint(f[e]);
+                s += f[e];
+            }
+        }
+        xsum[i] = s;
+    }
+
+#define XF(i, e) __uint_as_float(xr[(i)][(e)])
+    for (int rb = 0; rb < p.rpw; rb += RPL) {
+        const int64_t row0 = row_begin + rb;
+        if (row0 >= p.N) break;
+        if (rb + RPL < p.rpw) fetch(row0 + RPL, wn, csn, czn, rsn, rbiasn);
+
+        float acc[RPL];
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            acc[r] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < CPL; i++) {
+                float dot = 0.0f;
+                if constexpr (FOUR_BIT) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const uint32_t w = wv[r][i][t];
+                        if constexpr (DOT2) {
+                            // pair s of the word = elements 2s, 2s+1 -> bf16 (16 + q, 16 + q')
+                            const uint32_t w0 = ((w << 3) & 0x00780078u) | 0x41804180u;
+                            const uint32_t w1 = ((w >> 1) & 0x00780078u) | 0x41804180u;
+                            const uint32_t w2 = ((w >> 5) & 0x00780078u) | 0x41804180u;
+                            const uint32_t w3 = ((w >> 9) & 0x00780078u) | 0x41804180u;
+                            dot = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, xr[i][4 * t]),
+                                                                  __builtin_bit_cast(bf16x2, w0), dot, false);
+                            dot = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, xr[i][4 * t + 1]),
+                                                                  __builtin_bit_cast(bf16x2, w1), dot, false);
+                            dot = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, xr[i][4 * t + 2]),
+                                                                  __builtin_bit_cast(bf16x2, w2), dot, false);
+                            dot = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, xr[i][4 * t + 3]),
+                                                                  __builtin_bit_cast(bf16x2, w3), dot, false);
+                        } else {
+                            // low nibbles of the four bytes: elements 0, 4, 1, 5; high nibbles: 2, 6, 3, 7
+                            const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+                            dot = fmaf(XF(i, 8 * t + 0), (float)(lo & 0xFFu), dot);
+                            dot = fmaf(XF(i, 8 * t + 4), (float)((lo >> 8) & 0xFFu), dot);
+                            dot = fmaf(XF(i, 8 * t + 1), (float)((lo >> 16) & 0xFFu), dot);
+                            dot = fmaf(XF(i, 8 * t + 5), (float)(lo >> 24), dot);
+                            dot = fmaf(XF(i, 8 * t + 2), (float)(hi & 0xFFu), dot);
+                            dot = fmaf(XF(i, 8 * t + 6), (float)((hi >> 8) & 0xFFu), dot);
+                            dot = fmaf(XF(i, 8 * t + 3), (float)((hi >> 16) & 0xFFu), dot);
+                            dot = fmaf(XF(i, 8 * t + 7), (float)(hi >> 24), dot);
+                        }
+                    }
+                    const float zoff = DOT2 ? cz[r][i] + 16.0f : cz[r][i];
+                    acc[r] = fmaf(cs[r][i], fmaf(-zoff, xsum[i], dot), acc[r]);
+                } else if constexpr (FMT == NQ_FMT_W8_CHANNEL) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const uint32_t u = wv[r][i][t] ^ 0x80808080u;  // int8 + 128 as unsigned bytes
+                        dot = fmaf(XF(i, 4 * t + 0), (float)(u & 0xFFu), dot);
+                        dot = fmaf(XF(i, 4 * t + 1), (float)((u >> 8) & 0xFFu), dot);
+                        dot = fmaf(XF(i, 4 * t + 2), (float)((u >> 16) & 0xFFu), dot);
+                        dot = fmaf(XF(i, 4 * t + 3), (float)(u >> 24), dot);
+                    }
+                    acc[r] += fmaf(-128.0f, xsum[i], dot);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv[r][i][t], false);
+                        const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)wv[r][i][t], true);
+                        dot = fmaf(XF(i, 4 * t + 0), a[0], dot);
+                        dot = fmaf(XF(i, 4 * t + 1), a[1], dot);
+                        dot = fmaf(XF(i, 4 * t + 2), b[0], dot);
+                        dot = fmaf(XF(i, 4 * t + 3), b[1], dot);
+                    }
+                    acc[r] += dot;
+                }
+            }
+        }
+
+#pragma unroll
+        for (int r = 0; r < RPL; r++) acc[r] = group_sum(acc[r], lpr);
+
+        if (lj == 0) {
+#pragma unroll
+            for (int r = 0; r < RPL; r++) {
+                const int64_t n = row0 + r;
+                if (n >= p.N) continue;
+                float z = acc[r];
+                if (FMT == NQ_FMT_W8_CHANNEL) z *= rs[r];
+                if (FMT == NQ_FMT_FP8_E4M3) z *= tscale;
+                z += rbias[r];
+                if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(p.y)[n] = z;
+                else
+                    reinterpret_cast<uint16_t*>(p.y)[n] = to_bf16(z);
+            }
+        }
+        if (rb + RPL < p.rpw) {
+#pragma unroll
+            for (int r = 0; r < RPL; r++)
+#pragma unroll
+                for (int i = 0; i < CPL; i++) wv[r][i] = wn[r][i], cs[r][i] = csn[r][i], cz[r][i] = czn[r][i];
+#pragma unroll
+            for (int r = 0; r < RPL; r++) rs[r] = rsn[r], rbias[r] = rbiasn[r];
+        }
+    }
+}
+
+#undef XF
+
+int env_int(const char* name, int dflt) {
+    const char* v = std::getenv(name);
+    return v ? std::atoi(v) : dflt;
+}
+
+// Only the combinations the host picks are instantiated: at most 8 loads in flight per lane
+// (RPL x CPL), and at most 96 registers of x (CPL <= 3 when a chunk of x takes 32 registers).
+template <int FMT, bool DOT2, int CPL>
+int32_t launch_rpl(const M1Params& p, int rpl, dim3 grid, hipStream_t s) {
+    if constexpr (CPL <= 2) {
+        if (rpl >= 4) {
+            hipLaunchKernelGGL((gemv_m1_kernel<FMT, DOT2, CPL, 4>), grid, dim3(256), 0, s, p);
+            NQ_HIP(hipGetLastError());
+            return NQ_OK;
+        }
+    }
+    if constexpr (CPL <= 4) {
+        if (rpl >= 2) {
+            hipLaunchKernelGGL((gemv_m1_kernel<FMT, DOT2, CPL, 2>), grid, dim3(256), 0, s, p);
+            NQ_HIP(hipGetLastError());
+            return NQ_OK;
+        }
+    }
+    hipLaunchKernelGGL((gemv_m1_kernel<FMT, DOT2, CPL, 1>), grid, dim3(256), 0, s, p);
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+template <int FMT, bool DOT2>
+int32_t launch_cpl(const M1Params& p, int cpl, int rpl, dim3 grid, hipStream_t s) {
+    constexpr bool WIDE_X = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP) && !DOT2;
+    switch (cpl) {
+        case 1: return launch_rpl<FMT, DOT2, 1>(p, rpl, grid, s);
+        case 2: return launch_rpl<FMT, DOT2, 2>(p, rpl, grid, s);
+        case 3: return launch_rpl<FMT, DOT2, 3>(p, rpl, grid, s);
+    }
+    if constexpr (!WIDE_X) {
+        switch (cpl) {
+            case 4: return launch_rpl<FMT, DOT2, 4>(p, rpl, grid, s);
+            case 5: return launch_rpl<FMT, DOT2, 5>(p, rpl, grid, s);
+            case 6: return launch_rpl<FMT, DOT2, 6>(p, rpl, grid, s);
+        }
+    }
+    return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no single-row GEMV variant for this IN");
+}
+
+// (lanes per row, chunks per lane) covering nch chunks with the fewest idle slots
+bool pick_split(int nch, int cpl_max, int* lpr_out, int* cpl_out) {
+    int best = -1;
+    for (int lpr = 64; lpr >= 1; lpr >>= 1) {
+        const int cpl = (nch + lpr - 1) / lpr;
+        if (cpl > cpl_max) break;
+        const int slots = lpr * cpl;
+        if (best < 0 || slots < best) best = slots, *lpr_out = lpr, *cpl_out = cpl;
+    }
+    return best >= 0;
+}
+
+}  // namespace
+
+bool gemv_m1_applicable(const ForwardArgs& a) {
+    if (a.M != 1) return false;
+    const nq_layer* L = a.L;
+    if (a.x_dtype == NQ_DT_I8) return false;
+    const bool four_bit = (L->format == NQ_FMT_Q4_0 || L->format == NQ_FMT_W4_GROUP);
+    const bool dot2 = four_bit && a.x_dtype == NQ_DT_BF16;
+    const int nch = L->in / (four_bit ? 32 : 16);
+    int lpr, cpl;
+    // x registers per chunk: 16 (8-bit, or 4-bit through the bf16 dot) or 32 (4-bit with fp32 x)
+    return pick_split(nch, (four_bit && !dot2) ? 3 : 6, &lpr, &cpl);
+}
+
+int32_t launch_gemv_m1(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    const bool four_bit = (L->format == NQ_FMT_Q4_0 || L->format == NQ_FMT_W4_GROUP);
+    const bool dot2 = four_bit && a.x_dtype == NQ_DT_BF16;
+    M1Params p{};
+    p.codes = L->d_codes, p.scales = L->d_scales, p.zps = L->d_zps;
+    p.x = a.x, p.x_scale = a.x_scale, p.y = a.y, p.bias = a.bias;
+    p.N = L->out, p.K = L->in, p.group = L->group, p.groups = L->groups, p.tscale = L->scale;
+    p.nch = L->in / (four_bit ? 32 : 16);
+    p.x_dtype = a.x_dtype, p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    int lpr = 64, cpl = 1;
+    pick_split(p.nch, (four_bit && !dot2) ? 3 : 6, &lpr, &cpl);
+    // Small matrices are latency-bound: one row per lane group, as many wavefronts as possible.
+    // Large ones are bandwidth-bound: keep about eight 128-bit loads outstanding per lane and give
+    // each lane group a second batch, so the next rows are in flight while a batch is multiplied.
+    const int64_t wbytes = (int64_t)L->out * p.nch * 16;
+    int rpl = 1, mult = 1;
+    if (wbytes >= (4 << 20)) {
+        rpl = cpl <= 2 ? 4 : (cpl <= 4 ? 2 : 1);
+        const int64_t waves = (((int64_t)L->out + rpl - 1) / rpl * lpr + 63) / 64;
+        if (waves >= 4096) mult = 2;
+    }
+    lpr = env_int("NQ_M1_LPR", lpr);
+    rpl = env_int("NQ_M1_RPL", rpl);
+    mult = env_int("NQ_M1_MULT", mult);
+    cpl = (p.nch + lpr - 1) / lpr;
+    rpl = cpl <= 2 ? (rpl >= 4 ? 4 : (rpl >= 2 ? 2 : 1)) : (cpl <= 4 ? (rpl >= 2 ? 2 : 1) : 1);
+    p.lpr = lpr;
+    p.lpr_log2 = 0;
+    while ((1 << p.lpr_log2) < lpr) p.lpr_log2++;
+    p.rpw = rpl * mult;
+    const int64_t groups = ((int64_t)L->out + p.rpw - 1) / p.rpw;
+    const int64_t groups_per_block = 4 * (64 / lpr);
+    dim3 grid((unsigned)((groups + groups_per_block - 1) / groups_per_block));
+    switch (L->format) {
+        case NQ_FMT_Q4_0:
+            return dot2 ? launch_cpl<NQ_FMT_Q4_0, true>(p, cpl, rpl, grid, a.stream)
+                        : launch_cpl<NQ_FMT_Q4_0, false>(p, cpl, rpl, grid, a.stream);
+        case NQ_FMT_W4_GROUP:
+            return dot2 ? launch_cpl<NQ_FMT_W4_GROUP, true>(p, cpl, rpl, grid, a.stream)
+                        : launch_cpl<NQ_FMT_W4_GROUP, false>(p, cpl, rpl, grid, a.stream);
+        case NQ_FMT_W8_CHANNEL: return launch_cpl<NQ_FMT_W8_CHANNEL, false>(p, cpl, rpl, grid, a.stream);
+        case NQ_FMT_FP8_E4M3: return launch_cpl<NQ_FMT_FP8_E4M3, false>(p, cpl, rpl, grid, a.stream);
+    }
+    return fail(NQ_ERR_INVALID, "nq_forward: unknown format");
+}
+
+}  // namespace nq
