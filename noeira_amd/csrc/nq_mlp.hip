@@ -4,22 +4,24 @@
 // noeira/deep_agents/sac/config.mojo:58-67).  At M = 4096 the three GEMMs are
 // 0.69 GOP, a fraction of a microsecond of matrix-core time, so the cost of the
 // unfused chain is its six launches and the activations it writes and re-reads.
-// Here one wavefront carries 16 tokens through all three layers without ever
-// leaving registers.
+// Here one workgroup of four wavefronts carries 16 tokens through all three
+// layers; activations never leave the CU (registers, plus 4 KB of LDS to hand a
+// layer's int8 codes to the next one).
 //
 // Orientation.  The MFMA (v_mfma_i32_16x16x64_i8) is issued "transposed":
 // the weight tile is the A operand (16 output channels x 64 k) and the tokens
 // are the B operand (64 k x 16 tokens), so in the result a lane holds one token
 // (column = lane % 16) and four consecutive output channels per tile (rows
-// 4 * (lane / 16) + r).  That makes the per-token work lane-local:
-//   - the absmax of a token's activations is a max over the lane's own values
-//     and the three other lanes of its column (two shuffles);
-//   - four consecutive int8 codes pack into one dword;
-//   - the next layer's B operand (16 consecutive k per lane) is those dwords
-//     gathered from the four lanes of the column: a 4 x 4 dword transpose done
-//     with v_permlane32_swap / v_permlane16_swap, no LDS.
+// 4 * (lane / 16) + r).  That makes the per-token work lane-local: the absmax
+// of a token's activations is a max over the lane's own values, the three
+// other lanes of its column (two shuffles) and the other wavefronts (16 floats
+// through LDS); four consecutive int8 codes pack into one dword, stored to
+// LDS row `token`; the next layer's B operand is one 128-bit LDS read.
+// The output channels of a layer are split over the four wavefronts (each owns
+// a quarter of the 16-channel tiles), because the call is bound by the serial
+// instruction stream of a wavefront, not by the matrix cores.
 // Weights stay in L2 (84 KB for the actor); each wavefront reads its fragments
-// with 128-bit loads.
+// with 128-bit loads, four tiles at a time.
 //
 // Arithmetic is the unfused path's: per-token scale s = absmax / 127 (1 where
 // 0), q = clip(rint(v / s), -127, 127) with a true division, exact int32
@@ -62,85 +64,107 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
            (((uint32_t)d & 0xFFu) << 24);
 }
 
-// One layer for this wavefront's 16 tokens.  `bop[s]` is the B operand of k-step s (16 int8 of
-// the lane's token), `sx` the token's activation scale.  Returns z[j][r] = the layer's fp32
-// output for channel 16 j + 4 kb + r of the lane's token (zero for channels >= N).
-__device__ __forceinline__ void layer_forward(const MlpLayer& L, const i32x4 (&bop)[MAXS], float sx, bool relu,
-                                              int ln, int kb, float (&z)[MAXT][4]) {
-    const int tiles = (L.N + 15) >> 4;
-    const int steps = (L.K + 63) >> 6;
+constexpr int TPW = MAXT / 4;      // tiles per wavefront
+constexpr int HROW = 256 + 16;     // LDS row stride of the int8 hand-over buffer (bytes)
+
+// This wavefront's share of one layer: tiles 4 w .. 4 w + 3 for the 16 tokens of the workgroup.
+// `bop[s]` is the B operand of k-step s (16 int8 of the lane's token), `sx` the token's scale.
+// z[u][r] = fp32 output for channel 16 (4 w + u) + 4 kb + r of the lane's token (0 beyond N).
+// All of the wavefront's loads (4 x STEPS weight fragments, channel scales, biases) are requested
+// together, clamped rather than branched around, then masked at use.
+template <int STEPS>
+__device__ __forceinline__ void layer_steps(const MlpLayer& L, const i32x4 (&bop)[MAXS], float sx, bool relu, int wave,
+                                            int ln, int kb, float (&z)[TPW][4]) {
+    i32x4 a[TPW][STEPS];
+    float swv[TPW][4], bsv[TPW][4];
 #pragma unroll
-    for (int j = 0; j < MAXT; j++) {
-        if (j >= tiles) {
+    for (int u = 0; u < TPW; u++) {
+        const int j = TPW * wave + u;
+        const int n_a = min(16 * j + ln, L.N - 1);  // the weight row this lane supplies to the A operand
 #pragma unroll
-            for (int r = 0; r < 4; r++) z[j][r] = 0.0f;
-            continue;
+        for (int s = 0; s < STEPS; s++) {
+            const int k0 = min(64 * s + 16 * kb, L.K - 16);
+            a[u][s] = *reinterpret_cast<const i32x4*>(L.w + (int64_t)n_a * L.K + k0);
         }
-        i32x4 acc = {0, 0, 0, 0};
-        const int n_a = 16 * j + ln;  // the weight row this lane supplies to the A operand
 #pragma unroll
-        for (int s = 0; s < MAXS; s++) {
-            if (s >= steps) break;
-            const int k0 = 64 * s + 16 * kb;
-            i32x4 a = {0, 0, 0, 0};
-            if (n_a < L.N && k0 < L.K) a = *reinterpret_cast<const i32x4*>(L.w + (int64_t)n_a * L.K + k0);
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bop[s], acc, 0, 0, 0);
+        for (int r = 0; r < 4; r++) {
+            const int n = min(16 * j + 4 * kb + r, L.N - 1);
+            swv[u][r] = L.sw[n];
+            bsv[u][r] = L.bias ? L.bias[n] : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < TPW; u++) {
+        const int j = TPW * wave + u;
+        i32x4 acc = {0, 0, 0, 0};
+        const bool row_ok = (16 * j + ln) < L.N;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const bool ok = row_ok && (64 * s + 16 * kb) < L.K;
+            const i32x4 av = ok ? a[u][s] : (i32x4){0, 0, 0, 0};
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bop[s], acc, 0, 0, 0);
         }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int n = 16 * j + 4 * kb + r;
-            float v = 0.0f;
-            if (n < L.N) {
-                v = (float)acc[r] * (sx * L.sw[n]);
-                if (L.bias) v += L.bias[n];
-                if (relu) v = v > 0.0f ? v : 0.0f;
-            }
-            z[j][r] = v;
+            float v = (float)acc[r] * (sx * swv[u][r]) + bsv[u][r];
+            if (relu) v = v > 0.0f ? v : 0.0f;
+            z[u][r] = (n < L.N) ? v : 0.0f;
         }
     }
 }
 
-// Per-token int8 requantisation of z (channels 0 .. N-1) into the next layer's B operands.
-__device__ __forceinline__ void requantize(const float (&z)[MAXT][4], int N, i32x4 (&bop)[MAXS], float& sx) {
-    const int tiles = (N + 15) >> 4;
+__device__ __forceinline__ void layer_forward(const MlpLayer& L, const i32x4 (&bop)[MAXS], float sx, bool relu,
+                                              int wave, int ln, int kb, float (&z)[TPW][4]) {
+    const int steps = (L.K + 63) >> 6;
+    if (steps == 1)
+        layer_steps<1>(L, bop, sx, relu, wave, ln, kb, z);
+    else if (steps == 2)
+        layer_steps<2>(L, bop, sx, relu, wave, ln, kb, z);
+    else if (steps == 3)
+        layer_steps<3>(L, bop, sx, relu, wave, ln, kb, z);
+    else
+        layer_steps<4>(L, bop, sx, relu, wave, ln, kb, z);
+}
+
+// Per-token int8 requantisation of a layer's output (channels 0 .. N-1, spread over the four
+// wavefronts) into the next layer's B operands, through LDS.
+__device__ __forceinline__ void requantize(const float (&z)[TPW][4], uint8_t* hq, float* amax_part, int wave, int ln,
+                                           int kb, i32x4 (&bop)[MAXS], float& sx) {
     float amax = 0.0f;
 #pragma unroll
-    for (int j = 0; j < MAXT; j++) {
-        if (j >= tiles) break;
+    for (int u = 0; u < TPW; u++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) amax = fmaxf(amax, fabsf(z[j][r]));
-    }
+        for (int r = 0; r < 4; r++) amax = fmaxf(amax, fabsf(z[u][r]));  // channels beyond N hold 0
     amax = fmaxf(amax, __shfl_xor(amax, 16));
     amax = fmaxf(amax, __shfl_xor(amax, 32));
+    if (kb == 0) amax_part[wave * 16 + ln] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(amax_part[ln], amax_part[16 + ln]), fmaxf(amax_part[32 + ln], amax_part[48 + ln]));
     float s = amax / 127.0f;
     if (s == 0.0f) s = 1.0f;
     sx = s;
-    // tile j of this lane = channels 16 j + 4 kb .. + 3: one dword.  k-step t needs, in lane kb',
-    // the dwords of tile 4 t + kb' from the four lanes of the column, in lane order.
 #pragma unroll
-    for (int t = 0; t < MAXS; t++) {
-        uint32_t d[4];
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int j = 4 * t + u;
-            d[u] = (j < tiles) ? pack4(q8(z[j][0], s), q8(z[j][1], s), q8(z[j][2], s), q8(z[j][3], s)) : 0u;
-        }
-        auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-        auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-        d[0] = s02[0], d[2] = s02[1], d[1] = s13[0], d[3] = s13[1];
-        auto t01 = __builtin_amdgcn_permlane16_swap(d[0], d[1], false, false);
-        auto t23 = __builtin_amdgcn_permlane16_swap(d[2], d[3], false, false);
-        bop[t] = (i32x4){(int)t01[0], (int)t01[1], (int)t23[0], (int)t23[1]};
+    for (int u = 0; u < TPW; u++) {
+        const int j = TPW * wave + u;
+        const uint32_t d = pack4(q8(z[u][0], s), q8(z[u][1], s), q8(z[u][2], s), q8(z[u][3], s));
+        *reinterpret_cast<uint32_t*>(hq + ln * HROW + 16 * j + 4 * kb) = d;
     }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < MAXS; t++) bop[t] = *reinterpret_cast<const i32x4*>(hq + ln * HROW + 64 * t + 16 * kb);
 }
 
-__global__ __launch_bounds__(64) void mlp3_w8a8_kernel(const MlpParams p) {
-    const int lane = threadIdx.x;
+__global__ __launch_bounds__(256) void mlp3_w8a8_kernel(const MlpParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t hq[2][16 * HROW];
+    __shared__ float amax_part[2][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kb = lane >> 4;
     const int m = blockIdx.x * 16 + ln;          // this lane's token
     const int mc = min(m, p.M - 1);
 
     // ---- layer 1 input: fp32 x, 16 consecutive k per lane per k-step, quantised in registers
+    // (every wavefront does this for the same 16 tokens: cheaper than a hand-over)
     const int K0 = p.l[0].K;
     const int steps0 = (K0 + 63) >> 6;
     float xv[MAXS][16];
@@ -172,23 +196,25 @@ __global__ __launch_bounds__(64) void mlp3_w8a8_kernel(const MlpParams p) {
                                    q8(xv[s][4 * q + 3], sx));
     }
 
-    float z[MAXT][4];
-    layer_forward(p.l[0], bop, sx, true, ln, kb, z);
-    requantize(z, p.l[0].N, bop, sx);
-    layer_forward(p.l[1], bop, sx, true, ln, kb, z);
-    requantize(z, p.l[1].N, bop, sx);
-    layer_forward(p.l[2], bop, sx, p.final_relu != 0, ln, kb, z);
+    // zero the hand-over rows once: channels a layer does not produce must read as 0
+    for (int i = threadIdx.x; i < 2 * 16 * HROW / 4; i += 256) reinterpret_cast<uint32_t*>(&hq[0][0])[i] = 0u;
+    __syncthreads();
+
+    float z[TPW][4];
+    layer_forward(p.l[0], bop, sx, true, wave, ln, kb, z);
+    requantize(z, hq[0], amax_part[0], wave, ln, kb, bop, sx);
+    layer_forward(p.l[1], bop, sx, true, wave, ln, kb, z);
+    requantize(z, hq[1], amax_part[1], wave, ln, kb, bop, sx);
+    layer_forward(p.l[2], bop, sx, p.final_relu != 0, wave, ln, kb, z);
 
     if (m >= p.M) return;
     const int N2 = p.l[2].N;
-    const int tiles2 = (N2 + 15) >> 4;
 #pragma unroll
-    for (int j = 0; j < MAXT; j++) {
-        if (j >= tiles2) break;
+    for (int u = 0; u < TPW; u++) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int n = 16 * j + 4 * kb + r;
-            if (n < N2) p.y[(int64_t)m * N2 + n] = z[j][r];
+            const int n = 16 * (TPW * wave + u) + 4 * kb + r;
+            if (n < N2) p.y[(int64_t)m * N2 + n] = z[u][r];
         }
     }
 }
@@ -208,7 +234,7 @@ int32_t launch_mlp3_w8a8(const nq_layer* l1, const nq_layer* l2, const nq_layer*
         p.l[i].N = ls[i]->out, p.l[i].K = ls[i]->in;
     }
     p.x = x, p.y = y, p.M = M, p.final_relu = final_relu;
-    hipLaunchKernelGGL(mlp3_w8a8_kernel, dim3((M + 15) / 16), dim3(64), 0, s, p);
+    hipLaunchKernelGGL(mlp3_w8a8_kernel, dim3((M + 15) / 16), dim3(256), 0, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
