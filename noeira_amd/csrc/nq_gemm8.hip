@@ -25,6 +25,12 @@
 // 128-bit fragment reads (32 rows x 2 slots per wavefront instruction) and the
 // staging writes are conflict free.
 //
+// Epilogue.  The MFMA takes the weight tile as its first operand, so a lane
+// ends up with one token and runs of four consecutive channels; results are
+// staged per wavefront through LDS and leave as 128-bit stores covering whole
+// 256/512-byte row segments of y (2-byte scattered stores cost 37 % of the
+// kernel before).
+//
 // Workgroup order.  Hardware deals consecutive workgroup ids round-robin to
 // the 8 XCDs, each with its own L2.  Ids are first regrouped so that each XCD
 // gets one contiguous run of tiles, and runs walk the tile grid in bands of 8
@@ -43,6 +49,8 @@ typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(16))) int i32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 
 constexpr int BM = 256, BN = 256, BK = 128;
 constexpr int STAGE_BYTES = (BM + BN) * BK;  // 64 KiB
@@ -165,7 +173,7 @@ void gemm8_kernel(const Gemm8Params p) {
                 for (int i = 0; i < 4; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], 0, 0, 0,
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0, 0,
                                                                                      0, 0, 0);
             }
         } else {
@@ -182,58 +190,127 @@ void gemm8_kernel(const Gemm8Params p) {
                 for (int i = 0; i < 4; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
             }
         }
         if (kt + 1 < KT) stash((kt + 1) & 1);
         __syncthreads();
     }
 
-    // ---- epilogue: lane holds column n = l % 32 and rows 8*(r/4) + 4*(l/32) + r%4 of each tile.
-    // The output type is resolved once, outside the unrolled loops.
+    // ---- epilogue.  The MFMA was issued with the weight tile as its first operand, so in
+    // acc[i][j] a lane holds ONE token m = 32 i + lane % 32 (MFMA column) and, for g = 0..3, the
+    // four consecutive channels n = 32 j + 8 g + 4 (lane / 32) + 0..3 (MFMA rows, registers 4g..4g+3).
+    // Per-token work is lane-local and four outputs of a row of y are adjacent.  Each wavefront
+    // stages its results through its own LDS region (free now: the loop ended on a barrier) as
+    // [token][channel] rows, and writes them out as 128-bit stores, 256 B (bf16) or 512 B (fp32 /
+    // int32) contiguous per row of y.
     const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;
+    const int wm0 = m0 + wm * 128, wn0 = n0 + wn * 128;
+    const int lm = lane & 31, lh = lane >> 5;
+    const bool full_tile = (m0 + BM <= p.M) && (n0 + BN <= p.N) && (p.N % 8 == 0);
+
+    // channel scale and bias for the lane's channels of tile j, group g (needs n < N: clamped)
+    auto chan = [&](int j, int g, float (&cs)[4], float (&cb)[4], bool need_scale) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int n = min(wn0 + 32 * j + 8 * g + 4 * lh + r, p.N - 1);
+            cs[r] = need_scale ? p.col_scale[n] : 1.0f;
+            cb[r] = 0.0f;
+            if (p.bias)
+                cb[r] = (p.bias_dtype == NQ_DT_F32)
+                            ? reinterpret_cast<const float*>(p.bias)[n]
+                            : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+        }
+    };
+
     auto emit = [&](auto kind) {
         constexpr int KIND = decltype(kind)::value;  // 0: fp32, 1: bf16, 2: raw int32
+        constexpr int ES = (KIND == 1) ? 2 : 4;      // bytes per output element
+        constexpr int IP = (KIND == 1) ? 2 : 1;      // token tiles (of 32) staged per pass
+        constexpr int ROWB = 128 * ES + 16;          // staged row: 128 channels + pad (bank spread)
+        uint8_t* stage = lds + wave * (32 * IP * ROWB);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int mb = m0 + wm * 128 + i * 32 + 4 * (lane >> 5);
-            float rs[16];
-            if constexpr (!FP8 && KIND != 2) {
+        for (int ip = 0; ip < 4; ip += IP) {
+            // ---- registers -> LDS (this wavefront's region only).  Channel scales and biases are
+            // fetched per channel tile j; the compiler barrier keeps it from hoisting all 16 (j, g)
+            // sets above the loop, which would spill.
+            float rscale[IP];
 #pragma unroll
-                for (int r = 0; r < 16; r++) rs[r] = p.row_scale[min(mb + 8 * (r >> 2) + (r & 3), p.M - 1)];
+            for (int ii = 0; ii < IP; ii++) {
+                rscale[ii] = 1.0f;
+                if constexpr (!FP8 && KIND != 2) rscale[ii] = p.row_scale[min(wm0 + 32 * (ip + ii) + lm, p.M - 1)];
             }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int n = n0 + wn * 128 + j * 32 + (lane & 31);
-                if (n >= p.N) continue;
-                float cscale = 1.0f, bias = 0.0f;
-                if constexpr (!FP8 && KIND != 2) cscale = p.col_scale[n];
-                if (p.bias)
-                    bias = (p.bias_dtype == NQ_DT_F32)
-                               ? reinterpret_cast<const float*>(p.bias)[n]
-                               : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+                float cs[4][4], cb[4][4];
+                if constexpr (KIND != 2) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int m = mb + 8 * (r >> 2) + (r & 3);
-                    if (m >= p.M) continue;
-                    const int64_t o = (int64_t)m * p.N + n;
-                    if constexpr (KIND == 2) {
-                        reinterpret_cast<int32_t*>(p.y)[o] = (int32_t)acc[i][j][r];
-                    } else {
-                        float z;
-                        if constexpr (FP8)
-                            z = acc[i][j][r] * fp8_scale;
-                        else
-                            z = (float)acc[i][j][r] * (rs[r] * cscale);
-                        z += bias;
-                        if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
-                        if constexpr (KIND == 0)
-                            reinterpret_cast<float*>(p.y)[o] = z;
-                        else
-                            reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16(z);
+                    for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8);
+                }
+#pragma unroll
+                for (int ii = 0; ii < IP; ii++) {
+                    const int i = ip + ii;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        uint8_t* dst = stage + (32 * ii + lm) * ROWB + (32 * j + 8 * g + 4 * lh) * ES;
+                        if constexpr (KIND == 2) {
+                            *reinterpret_cast<i32x4*>(dst) = (i32x4){(int)acc[i][j][4 * g], (int)acc[i][j][4 * g + 1],
+                                                                      (int)acc[i][j][4 * g + 2], (int)acc[i][j][4 * g + 3]};
+                        } else {
+                            float z[4];
+#pragma unroll
+                            for (int r = 0; r < 4; r++) {
+                                if constexpr (FP8)
+                                    z[r] = acc[i][j][4 * g + r] * fp8_scale + cb[g][r];
+                                else
+                                    z[r] = (float)acc[i][j][4 * g + r] * (rscale[ii] * cs[g][r]) + cb[g][r];
+                                if (p.epilogue == NQ_EPI_RELU) z[r] = z[r] > 0.0f ? z[r] : 0.0f;
+                            }
+                            if constexpr (KIND == 0) {
+                                *reinterpret_cast<float4*>(dst) = make_float4(z[0], z[1], z[2], z[3]);
+                            } else {
+                                // v_cvt_pk_bf16_f32: round to nearest even in hardware
+                                const bf16x4 pk = __builtin_convertvector((f32x4){z[0], z[1], z[2], z[3]}, bf16x4);
+                                *reinterpret_cast<bf16x4*>(dst) = pk;
+                            }
+                        }
+                    }
+                }
+                asm volatile("" ::: "memory");
+            }
+            // the region is this wavefront's own and DS operations of a wavefront execute in order:
+            // no block barrier, only a fence against compiler reordering
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // ---- LDS -> global: 16 bytes per lane, rows of y contiguous
+            constexpr int LPRW = 128 * ES / 16;          // lanes per staged row (16 or 32)
+            constexpr int RPI = 64 / LPRW;               // rows per wavefront instruction
+#pragma unroll
+            for (int t = 0; t < 32 * IP / RPI; t++) {
+                const int row = t * RPI + lane / LPRW, c16 = lane % LPRW;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * ROWB + c16 * 16);
+                const int m = wm0 + 32 * ip + row;
+                const int n = wn0 + c16 * (16 / ES);
+                if (full_tile) {
+                    *reinterpret_cast<i32x4*>(reinterpret_cast<uint8_t*>(p.y) + ((int64_t)m * p.N + n) * ES) = v;
+                } else if (m < p.M) {
+                    // ragged edge: element by element
+#pragma unroll
+                    for (int e = 0; e < 16 / ES; e++) {
+                        if (n + e >= p.N) break;
+                        if constexpr (ES == 2) {
+                            const uint32_t wv = (uint32_t)v[e >> 1];
+                            reinterpret_cast<uint16_t*>(p.y)[(int64_t)m * p.N + n + e] = (uint16_t)(wv >> (16 * (e & 1)));
+                        } else {
+                            reinterpret_cast<int32_t*>(p.y)[(int64_t)m * p.N + n + e] = v[e];
+                        }
                     }
                 }
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     };
     if (p.y_dtype == NQ_DT_F32)
