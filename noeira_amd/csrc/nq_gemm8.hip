@@ -15,9 +15,9 @@
 //
 // K loop.  Stages of BK = 128 bytes: x tile 256 x 128 B and w tile 256 x 128 B
 // (64 KiB), double-buffered in LDS (128 of the CU's 160 KiB).  While a stage is
-// being multiplied, the next stage's 16 128-bit global loads per lane are in
-// flight into registers; they are written to the other LDS buffer after the
-// MFMAs, so there is one barrier per stage.
+// being multiplied, the next stage streams from global memory straight into the
+// other LDS buffer (global_load_lds_dwordx4, 16 per lane per stage): no
+// registers, no ds_write, one wait + one barrier per stage.
 //
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= (row >> 1) & 7.  Rows r and r + 1 then sit 128 B apart in
@@ -101,34 +101,30 @@ void gemm8_kernel(const Gemm8Params p) {
     const int tn = in_band / band_rows;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // ---- global -> register staging: 8 pieces of x and 8 of w per lane per stage
-    const uint8_t* ga[8];
-    const uint8_t* gb[8];
-    int so[8];  // LDS offset of piece i (same for the x and the w tile)
+    // ---- global -> LDS, direct (global_load_lds_dwordx4): no register round trip.  One
+    // instruction fills 1 KiB of LDS, lane l at byte 16 l, i.e. 8 rows of 128 B; wavefront w owns
+    // rows [64 w, 64 w + 64) of both tiles.  The slot swizzle is applied on the global side: the
+    // lane that lands in physical slot l % 8 of its row fetches logical slot (l % 8) ^ swz(row).
+    typedef __attribute__((address_space(1))) const void gptr_t;
+    typedef __attribute__((address_space(3))) void lptr_t;
+    const uint8_t* da[8];
+    const uint8_t* db[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int piece = tid + 256 * i;
-        const int row = piece >> 3, slot = piece & 7;
-        ga[i] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.K + slot * 16;
-        gb[i] = p.b + (int64_t)min(n0 + row, p.N - 1) * p.K + slot * 16;
-        so[i] = lds_off(row, slot);
+    for (int t = 0; t < 8; t++) {
+        const int row = wave * 64 + t * 8 + (lane >> 3);
+        const int slot = (lane & 7) ^ ((row >> 1) & 7);
+        da[t] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.K + slot * 16;
+        db[t] = p.b + (int64_t)min(n0 + row, p.N - 1) * p.K + slot * 16;
     }
-    u32x4 ra[8], rb[8];
-    auto fetch = [&](int k0) {
+    auto dma = [&](int k0, int buf) {
+        uint8_t* base = lds + buf * STAGE_BYTES + wave * 64 * BK;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            ra[i] = *reinterpret_cast<const u32x4*>(ga[i] + k0);
-            rb[i] = *reinterpret_cast<const u32x4*>(gb[i] + k0);
+        for (int t = 0; t < 8; t++) {
+            __builtin_amdgcn_global_load_lds((gptr_t*)(da[t] + k0), (lptr_t*)(base + t * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t*)(db[t] + k0), (lptr_t*)(base + BM * BK + t * 1024), 16, 0, 0);
         }
     };
-    auto stash = [&](int buf) {
-        uint8_t* base = lds + buf * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            *reinterpret_cast<u32x4*>(base + so[i]) = ra[i];
-            *reinterpret_cast<u32x4*>(base + BM * BK + so[i]) = rb[i];
-        }
-    };
+    const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;  // requested now, used in the epilogue
 
     typedef typename std::conditional<FP8, f32x16, i32x16>::type acc_t;
     acc_t acc[4][4];
@@ -148,11 +144,13 @@ void gemm8_kernel(const Gemm8Params p) {
     const int fsw = (frow >> 1) & 7;
 
     const int KT = p.K / BK;
-    fetch(0);
-    stash(0);
+    dma(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     for (int kt = 0; kt < KT; kt++) {
-        if (kt + 1 < KT) fetch((kt + 1) * BK);
+        // stage kt+1 streams into the other buffer while stage kt is multiplied; the barrier at
+        // the end of the previous iteration guarantees nobody still reads that buffer
+        if (kt + 1 < KT) dma((kt + 1) * BK, (kt + 1) & 1);
         const uint8_t* sa = lds + (kt & 1) * STAGE_BYTES + (wm * 128 + frow) * BK;
         const uint8_t* sb = lds + (kt & 1) * STAGE_BYTES + BM * BK + (wn * 128 + frow) * BK;
         if constexpr (FP8) {
@@ -193,7 +191,7 @@ void gemm8_kernel(const Gemm8Params p) {
                         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
             }
         }
-        if (kt + 1 < KT) stash((kt + 1) & 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
@@ -204,7 +202,6 @@ void gemm8_kernel(const Gemm8Params p) {
     // stages its results through its own LDS region (free now: the loop ended on a barrier) as
     // [token][channel] rows, and writes them out as 128-bit stores, 256 B (bf16) or 512 B (fp32 /
     // int32) contiguous per row of y.
-    const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;
     const int wm0 = m0 + wm * 128, wn0 = n0 + wn * 128;
     const int lm = lane & 31, lh = lane >> 5;
     const bool full_tile = (m0 + BM <= p.M) && (n0 + BN <= p.N) && (p.N % 8 == 0);
