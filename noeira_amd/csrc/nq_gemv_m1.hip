@@ -94,7 +94,7 @@ __device__ __forceinline__ float group_sum(float v, int lpr) {
     return v;
 }
 
-template <int FMT, bool DOT2, int CPL, int RPL>
+template <int FMT, int XDT, bool DOT2, int CPL, int RPL>
 __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     constexpr bool FOUR_BIT = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP);
     constexpr int EPC = FOUR_BIT ? 32 : 16;
@@ -129,23 +129,21 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
                                : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[row] << 16);
 #pragma unroll
             for (int i = 0; i < CPL; i++) {
-                const int c = lj + i * lpr;
-                const bool ok = cval[i] && row0 < p.N;
-                wv[r][i] = ok ? __builtin_nontemporal_load(&wq[row * p.nch + c]) : (u32x4){0, 0, 0, 0};
+                // Unconditional loads from clamped addresses: a lane whose chunk index runs past the
+                // row re-reads the last chunk, and its contribution vanishes because its x is zero.
+                // (A predicated load would become a branch around the load and serialise the batch.)
+                const int c = min(lj + i * lpr, p.nch - 1);
+                wv[r][i] = __builtin_nontemporal_load(&wq[row * p.nch + c]);
                 cs[r][i] = 0.0f, cz[r][i] = 0.0f;
-                if constexpr (FOUR_BIT) {
-                    if (ok) {
-                        if (FMT == NQ_FMT_Q4_0) {
-                            cs[r][i] = __half2float(
-                                __ushort_as_half(reinterpret_cast<const uint16_t*>(p.scales)[row * p.nch + c]));
-                            cz[r][i] = 8.0f;
-                        } else {
-                            const int g = (c * EPC) / p.group;
-                            cs[r][i] = __half2float(
-                                __ushort_as_half(reinterpret_cast<const uint16_t*>(p.scales)[row * p.groups + g]));
-                            cz[r][i] = (float)p.zps[row * p.groups + g];
-                        }
-                    }
+                if constexpr (FMT == NQ_FMT_Q4_0) {
+                    cs[r][i] = __half2float(
+                        __ushort_as_half(reinterpret_cast<const uint16_t*>(p.scales)[row * p.nch + c]));
+                    cz[r][i] = 8.0f;
+                } else if constexpr (FMT == NQ_FMT_W4_GROUP) {
+                    const int g = (c * EPC) / p.group;
+                    cs[r][i] = __half2float(
+                        __ushort_as_half(reinterpret_cast<const uint16_t*>(p.scales)[row * p.groups + g]));
+                    cz[r][i] = (float)p.zps[row * p.groups + g];
                 }
             }
         }
@@ -161,32 +159,28 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     float xsum[CPL];
 #pragma unroll
     for (int i = 0; i < CPL; i++) {
-        const int c = lj + i * lpr;
-        const int64_t k0 = (int64_t)c * EPC;
+        // clamped, unconditional loads; a chunk past the end of the row gets x = 0 afterwards
+        const int64_t k0 = (int64_t)min(lj + i * lpr, p.nch - 1) * EPC;
         float s = 0.0f;
         if constexpr (DOT2) {
 #pragma unroll
             for (int v = 0; v < EPC / 8; v++) {
-                u32x4 t = {0, 0, 0, 0};
-                if (cval[i]) t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
+                const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    xr[i][4 * v + e] = t[e];
-                    s += bf16lo(t[e]) + bf16hi(t[e]);
+                    xr[i][4 * v + e] = cval[i] ? t[e] : 0u;
+                    s += bf16lo(xr[i][4 * v + e]) + bf16hi(xr[i][4 * v + e]);
                 }
             }
         } else {
             float f[EPC];
-            if (!cval[i]) {
-#pragma unroll
-                for (int e = 0; e < EPC; e++) f[e] = 0.0f;
-            } else if (p.x_dtype == NQ_DT_F32) {
+            if constexpr (XDT == NQ_DT_F32) {
 #pragma unroll
                 for (int v = 0; v < EPC / 4; v++) {
                     const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.x) + k0 + 4 * v);
                     f[4 * v] = t.x, f[4 * v + 1] = t.y, f[4 * v + 2] = t.z, f[4 * v + 3] = t.w;
                 }
-            } else if (p.x_dtype == NQ_DT_BF16) {
+            } else if constexpr (XDT == NQ_DT_BF16) {
 #pragma unroll
                 for (int v = 0; v < EPC / 8; v++) {
                     const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
@@ -208,8 +202,9 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
             }
 #pragma unroll
             for (int e = 0; e < EPC; e++) {
-                xr[i][e] = __float_as_uint(f[e]);
-                s += f[e];
+                const float fv = cval[i] ? f[e] : 0.0f;
+                xr[i][e] = __float_as_uint(fv);
+                s += fv;
             }
         }
         xsum[i] = s;
@@ -325,40 +320,40 @@ int env_int(const char* name, int dflt) {
 
 // Only the combinations the host picks are instantiated: at most 8 loads in flight per lane
 // (RPL x CPL), and at most 96 registers of x (CPL <= 3 when a chunk of x takes 32 registers).
-template <int FMT, bool DOT2, int CPL>
+template <int FMT, int XDT, bool DOT2, int CPL>
 int32_t launch_rpl(const M1Params& p, int rpl, dim3 grid, hipStream_t s) {
     if constexpr (CPL <= 2) {
         if (rpl >= 4) {
-            hipLaunchKernelGGL((gemv_m1_kernel<FMT, DOT2, CPL, 4>), grid, dim3(256), 0, s, p);
+            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 4>), grid, dim3(256), 0, s, p);
             NQ_HIP(hipGetLastError());
             return NQ_OK;
         }
     }
     if constexpr (CPL <= 4) {
         if (rpl >= 2) {
-            hipLaunchKernelGGL((gemv_m1_kernel<FMT, DOT2, CPL, 2>), grid, dim3(256), 0, s, p);
+            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 2>), grid, dim3(256), 0, s, p);
             NQ_HIP(hipGetLastError());
             return NQ_OK;
         }
     }
-    hipLaunchKernelGGL((gemv_m1_kernel<FMT, DOT2, CPL, 1>), grid, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 1>), grid, dim3(256), 0, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
 
-template <int FMT, bool DOT2>
+template <int FMT, int XDT, bool DOT2>
 int32_t launch_cpl(const M1Params& p, int cpl, int rpl, dim3 grid, hipStream_t s) {
     constexpr bool WIDE_X = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP) && !DOT2;
     switch (cpl) {
-        case 1: return launch_rpl<FMT, DOT2, 1>(p, rpl, grid, s);
-        case 2: return launch_rpl<FMT, DOT2, 2>(p, rpl, grid, s);
-        case 3: return launch_rpl<FMT, DOT2, 3>(p, rpl, grid, s);
+        case 1: return launch_rpl<FMT, XDT, DOT2, 1>(p, rpl, grid, s);
+        case 2: return launch_rpl<FMT, XDT, DOT2, 2>(p, rpl, grid, s);
+        case 3: return launch_rpl<FMT, XDT, DOT2, 3>(p, rpl, grid, s);
     }
     if constexpr (!WIDE_X) {
         switch (cpl) {
-            case 4: return launch_rpl<FMT, DOT2, 4>(p, rpl, grid, s);
-            case 5: return launch_rpl<FMT, DOT2, 5>(p, rpl, grid, s);
-            case 6: return launch_rpl<FMT, DOT2, 6>(p, rpl, grid, s);
+            case 4: return launch_rpl<FMT, XDT, DOT2, 4>(p, rpl, grid, s);
+            case 5: return launch_rpl<FMT, XDT, DOT2, 5>(p, rpl, grid, s);
+            case 6: return launch_rpl<FMT, XDT, DOT2, 6>(p, rpl, grid, s);
         }
     }
     return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no single-row GEMV variant for this IN");
@@ -402,16 +397,16 @@ int32_t launch_gemv_m1(const ForwardArgs& a) {
     p.x_dtype = a.x_dtype, p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     int lpr = 64, cpl = 1;
     pick_split(p.nch, (four_bit && !dot2) ? 3 : 6, &lpr, &cpl);
-    // Small matrices are latency-bound: one row per lane group, as many wavefronts as possible.
-    // Large ones are bandwidth-bound: keep about eight 128-bit loads outstanding per lane and give
-    // each lane group a second batch, so the next rows are in flight while a batch is multiplied.
-    const int64_t wbytes = (int64_t)L->out * p.nch * 16;
-    int rpl = 1, mult = 1;
-    if (wbytes >= (4 << 20)) {
-        rpl = cpl <= 2 ? 4 : (cpl <= 4 ? 2 : 1);
-        const int64_t waves = (((int64_t)L->out + rpl - 1) / rpl * lpr + 63) / 64;
-        if (waves >= 4096) mult = 2;
+    // a small matrix wants wavefronts more than it wants busy lanes: widen the lane group until the
+    // launch has ~1k wavefronts (idle lanes cost nothing, a short dependency chain is the point)
+    while (lpr < 64 && (int64_t)L->out * lpr / 64 < 1024) {
+        lpr *= 2;
+        cpl = (p.nch + lpr - 1) / lpr;
     }
+    // One row per lane group and one batch per wavefront: the most wavefronts, the shortest
+    // dependency chain.  Measured best from 68 KB to 45 MB of weights (memory-level parallelism
+    // comes from occupancy, not from rows per lane).
+    int rpl = 1, mult = 1;
     lpr = env_int("NQ_M1_LPR", lpr);
     rpl = env_int("NQ_M1_RPL", rpl);
     mult = env_int("NQ_M1_MULT", mult);
@@ -424,15 +419,22 @@ int32_t launch_gemv_m1(const ForwardArgs& a) {
     const int64_t groups = ((int64_t)L->out + p.rpw - 1) / p.rpw;
     const int64_t groups_per_block = 4 * (64 / lpr);
     dim3 grid((unsigned)((groups + groups_per_block - 1) / groups_per_block));
+    const int xd = a.x_dtype;
     switch (L->format) {
         case NQ_FMT_Q4_0:
-            return dot2 ? launch_cpl<NQ_FMT_Q4_0, true>(p, cpl, rpl, grid, a.stream)
-                        : launch_cpl<NQ_FMT_Q4_0, false>(p, cpl, rpl, grid, a.stream);
+            if (dot2) return launch_cpl<NQ_FMT_Q4_0, NQ_DT_BF16, true>(p, cpl, rpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_Q4_0, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
         case NQ_FMT_W4_GROUP:
-            return dot2 ? launch_cpl<NQ_FMT_W4_GROUP, true>(p, cpl, rpl, grid, a.stream)
-                        : launch_cpl<NQ_FMT_W4_GROUP, false>(p, cpl, rpl, grid, a.stream);
-        case NQ_FMT_W8_CHANNEL: return launch_cpl<NQ_FMT_W8_CHANNEL, false>(p, cpl, rpl, grid, a.stream);
-        case NQ_FMT_FP8_E4M3: return launch_cpl<NQ_FMT_FP8_E4M3, false>(p, cpl, rpl, grid, a.stream);
+            if (dot2) return launch_cpl<NQ_FMT_W4_GROUP, NQ_DT_BF16, true>(p, cpl, rpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_W4_GROUP, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
+        case NQ_FMT_W8_CHANNEL:
+            if (xd == NQ_DT_BF16) return launch_cpl<NQ_FMT_W8_CHANNEL, NQ_DT_BF16, false>(p, cpl, rpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_W8_CHANNEL, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
+        case NQ_FMT_FP8_E4M3:
+            if (xd == NQ_DT_FP8_E4M3)
+                return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_FP8_E4M3, false>(p, cpl, rpl, grid, a.stream);
+            if (xd == NQ_DT_BF16) return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_BF16, false>(p, cpl, rpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
     }
     return fail(NQ_ERR_INVALID, "nq_forward: unknown format");
 }
