@@ -52,7 +52,9 @@ struct A16Params {
     void* y;
     const void* bias;
     int32_t M, N, K;
-    int32_t group, groups;
+    int32_t groups;
+    float inv_cpg;    // W4_GROUP: 1 / (16-byte chunks per group)
+    int32_t s_pairs;  // Q4_0: scale rows are 4-byte (1) or 8-byte (2) aligned, else 0
     int32_t nch;      // 16-byte chunks per weight row
     int32_t y_dtype, bias_dtype, epilogue;
 };
@@ -64,6 +66,20 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
 }
 
 __device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// loads at a uniform base plus a 32-bit byte offset (one address register per lane)
+__device__ __forceinline__ u32x4 ld16(const void* base, uint32_t off) {
+    return *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(base) + off);
+}
+__device__ __forceinline__ uint32_t ld4(const void* base, uint32_t off) {
+    return *reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(base) + off);
+}
+__device__ __forceinline__ uint32_t ld2(const void* base, uint32_t off) {
+    return *reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(base) + off);
+}
+__device__ __forceinline__ uint32_t ld1(const void* base, uint32_t off) {
+    return *reinterpret_cast<const uint8_t*>(reinterpret_cast<const char*>(base) + off);
+}
 
 // eight 4-bit codes of one word (pair s = elements 2s, 2s+1 in nibbles s and s+4) -> bf16 16+q
 __device__ __forceinline__ u32x4 nib_word_to_bf16(uint32_t w) {
@@ -81,54 +97,59 @@ __device__ __forceinline__ void i8_word_to_bf16(uint32_t w, uint32_t& p0, uint32
     const float f0 = (float)(t & 0xFFu), f1 = (float)((t >> 8) & 0xFFu);
     const float f2 = (float)((t >> 16) & 0xFFu), f3 = (float)(t >> 24);
     // values <= 255 have at most 8 significant bits: the high half of the fp32 is the exact bf16
-    p0 = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xFFFF0000u);
-    p1 = (__float_as_uint(f2) >> 16) | (__float_as_uint(f3) & 0xFFFF0000u);
+    p0 = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+    p1 = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
 }
 
-// A-operand terms for 8 consecutive activations.  NT = 1 (bf16 input) or 3 (fp32 split).
+// A-operand terms of 8 consecutive activations held raw in registers: one term for bf16
+// input, three for fp32 (hi + mid + lo = the fp32 value exactly: each split truncates, so
+// each residual is exact in fp32 and the third has at most 8 significant bits).  A term pair
+// is the two high halves, gathered with one byte permute.
 template <bool XF32>
-__device__ __forceinline__ void load_a(const void* x, int64_t elem_off, bool valid, u32x4 (&t)[XF32 ? 3 : 1]) {
+__device__ __forceinline__ void make_terms(const u32x4 (&raw)[XF32 ? 2 : 1], u32x4 (&t)[XF32 ? 3 : 1]) {
     if constexpr (!XF32) {
-        t[0] = valid ? *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(x) + elem_off)
-                     : (u32x4){0, 0, 0, 0};
+        t[0] = raw[0];
     } else {
-        float v[8];
-        if (valid) {
-            const float4 a = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(x) + elem_off)[0];
-            const float4 b = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(x) + elem_off)[1];
-            v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = 0.0f;
-        }
-        uint32_t h[8], m[8], l[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            // truncating splits: each residual is exact in fp32, the third term is exact in bf16
-            const uint32_t hb = __float_as_uint(v[i]) & 0xFFFF0000u;
-            const float r1 = v[i] - __uint_as_float(hb);
-            const uint32_t mb = __float_as_uint(r1) & 0xFFFF0000u;
-            const float r2 = r1 - __uint_as_float(mb);
-            h[i] = hb, m[i] = mb, l[i] = __float_as_uint(r2) & 0xFFFF0000u;
-        }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            t[0][i] = (h[2 * i] >> 16) | h[2 * i + 1];
-            t[1][i] = (m[2 * i] >> 16) | m[2 * i + 1];
-            t[2][i] = (l[2 * i] >> 16) | l[2 * i + 1];
+            const uint32_t a = raw[i >> 1][(2 * i) & 3], b = raw[i >> 1][(2 * i + 1) & 3];
+            const float ra = __uint_as_float(a) - __uint_as_float(a & 0xFFFF0000u);
+            const float rb = __uint_as_float(b) - __uint_as_float(b & 0xFFFF0000u);
+            const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+            const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+            t[0][i] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+            t[1][i] = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+            t[2][i] = __builtin_amdgcn_perm(__float_as_uint(sb), __float_as_uint(sa), 0x07060302u);
         }
     }
 }
 
-template <int FMT, bool XF32, int MW, int NW>
-__global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
+// One workgroup computes a [16 MW] x [16 NW] output tile; its KW wavefronts split K by
+// k-steps (wave w takes k-steps w, w + KW, ...).  Calls of this size are bound by how many
+// instructions one wavefront executes back to back and by how many cache lines its loads
+// touch, not by the matrix cores or by bytes, which shapes the kernel:
+//   - a wavefront's activations are the large operand (2 or 4 bytes an element against half
+//     a byte or one byte of weight), so the tile is wide in N: every activation fragment,
+//     and for fp32 input its three-term split, is formed once for NW weight tiles;
+//   - all loads are issued one k-step ahead from clamped addresses (a fragment register is
+//     refilled as soon as it has been read), so a wavefront waits for memory once;
+//   - scale records come in as few loads as their alignment allows, since every load costs
+//     one cache-line look-up per weight row whatever its width;
+//   - the zero-point term enters the MFMA as its C operand, and where a whole k-step lies in
+//     one group (WHOLE) the scale is applied once per k-step instead of once per chunk.
+template <int FMT, bool XF32, int MW, int NW, int KW, bool WHOLE>
+__global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL);
-    constexpr int NT = XF32 ? 3 : 1;
+    constexpr int NT = XF32 ? 3 : 1;            // bf16 terms per activation
+    constexpr int NL = XF32 ? 2 : 1;            // 16-byte loads per activation fragment
+    constexpr int ES = XF32 ? 4 : 2;            // bytes per activation
     constexpr int KSTEP = FOUR_BIT ? 128 : 64;  // k covered by one 16-byte weight load per lane x 4 lanes
     constexpr int NMF = FOUR_BIT ? 4 : 2;       // MFMAs (32 k each) per k-step
-    constexpr int RED = MW * NW * 4 * 64;       // floats one wavefront contributes to the reduction
-    extern __shared__ float red[];              // [KW - 1][RED]
-    const int KW = blockDim.x >> 6;             // wavefronts splitting K
+    constexpr int NS = WHOLE ? 1 : 4;           // scale records per k-step and weight row
+    constexpr int TA = MW * NW * 4;             // accumulator registers per lane
+    constexpr int RED = TA * 64;                // floats one wavefront contributes to the reduction
+    constexpr int EPW = (TA + KW - 1) / KW;     // accumulators one wavefront finishes
+    extern __shared__ float red[];              // [KW][RED]
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kb = lane >> 4;
@@ -146,120 +167,224 @@ __global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
         for (int j = 0; j < NW; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
     }
 
-    int64_t xrow[MW];
+    // byte offsets of this lane's rows (the host has checked that every operand is < 4 GiB)
+    uint32_t xoff[MW], woff[NW], soff[NW];
 #pragma unroll
-    for (int i = 0; i < MW; i++) xrow[i] = (int64_t)min(m_base + 16 * i + ln, p.M - 1) * p.K;
-    int64_t wrow[NW];
-    int nrow[NW];
+    for (int i = 0; i < MW; i++) xoff[i] = (uint32_t)min(m_base + 16 * i + ln, p.M - 1) * (uint32_t)p.K * ES;
 #pragma unroll
     for (int j = 0; j < NW; j++) {
-        nrow[j] = min(n_base + 16 * j + ln, p.N - 1);
-        wrow[j] = (int64_t)nrow[j] * p.nch;
+        const uint32_t n = (uint32_t)min(n_base + 16 * j + ln, p.N - 1);
+        woff[j] = n * (uint32_t)p.nch * 16u;
+        soff[j] = n * (uint32_t)(FMT == NQ_FMT_Q4_0 ? p.nch : p.groups);  // in elements
     }
-    const u32x4* wq = reinterpret_cast<const u32x4*>(p.codes);
 
-    // the epilogue's operands are requested up front: nothing is loaded after the reduction
-    float ep_scale[NW], ep_bias[NW];
+    // the accumulators this wavefront finishes after the reduction are idx = wave + t KW; their
+    // per-channel operands are requested now so that nothing is loaded after the reduction
+    float ep_scale[EPW], ep_bias[EPW];
 #pragma unroll
-    for (int j = 0; j < NW; j++) {
-        ep_scale[j] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[nrow[j]] : 1.0f;
-        ep_bias[j] = 0.0f;
+    for (int t = 0; t < EPW; t++) {
+        const int idx = min(wave + t * KW, TA - 1);
+        const int n = min(n_base + 16 * ((idx >> 2) % NW) + ln, p.N - 1);
+        ep_scale[t] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[n] : 1.0f;
+        ep_bias[t] = 0.0f;
         if (p.bias)
-            ep_bias[j] = (p.bias_dtype == NQ_DT_F32)
-                             ? reinterpret_cast<const float*>(p.bias)[nrow[j]]
-                             : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[nrow[j]] << 16);
+            ep_bias[t] = (p.bias_dtype == NQ_DT_F32)
+                             ? reinterpret_cast<const float*>(p.bias)[n]
+                             : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
     }
 
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
-    auto load_w = [&](int ks, u32x4 (&dst)[NW]) {
-        const int c = ks * 4 + kb;  // the 16-byte chunk this lane loads
-        const bool cvalid = ks < nsteps && c < p.nch;
-#pragma unroll
-        for (int j = 0; j < NW; j++) dst[j] = cvalid ? wq[wrow[j] + c] : (u32x4){0, 0, 0, 0};
-    };
-    u32x4 wv[NW], wnext[NW];
-    load_w(wave, wv);
-    for (int ks = wave; ks < nsteps; ks += KW) {
-        load_w(ks + KW, wnext);  // in flight while this k-step is multiplied
 
-        if constexpr (FOUR_BIT) {
-            // per-chunk scale and zero point for chunks 4ks .. 4ks+3 of row n (lane's own column)
-            float cs[NW][4], cz[NW][4];
+    // ---- loaders: unconditional, from clamped addresses; what lies past K is multiplied by a
+    // zero scale (4-bit formats) or replaced by zero activations (W8)
+    auto load_w = [&](int ks, u32x4 (&dst)[NW]) {
+        const uint32_t c = (uint32_t)min(ks * 4 + kb, p.nch - 1) * 16u;  // the 16-byte chunk this lane loads
 #pragma unroll
-            for (int j = 0; j < NW; j++)
+        for (int j = 0; j < NW; j++) dst[j] = ld16(p.codes, woff[j] + c);
+    };
+    // scale records of a k-step: fp16 scale | zero point << 16
+    auto load_s = [&](int ks, uint32_t (&dst)[NW][NS]) {
+        if constexpr (FMT == NQ_FMT_Q4_0) {
+            if (p.s_pairs) {  // rows are 4- or 8-byte aligned (the last load may run 4 bytes past a row)
+                const uint32_t c0 = (uint32_t)min(ks, nsteps - 1) * 8u;
+#pragma unroll
+                for (int j = 0; j < NW; j++) {
+                    uint32_t v0, v1;
+                    if (p.s_pairs == 2) {
+                        const u32x2 v = *reinterpret_cast<const u32x2*>(reinterpret_cast<const char*>(p.scales) +
+                                                                        (soff[j] * 2u + c0));
+                        v0 = v[0], v1 = v[1];
+                    } else {
+                        v0 = ld4(p.scales, soff[j] * 2u + c0), v1 = ld4(p.scales, soff[j] * 2u + c0 + 4u);
+                    }
+                    dst[j][0] = v0 & 0xFFFFu, dst[j][1] = v0 >> 16, dst[j][2] = v1 & 0xFFFFu, dst[j][3] = v1 >> 16;
+                }
+            } else {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const int cc = ks * 4 + q;
-                    if (cc < p.nch) {
-                        if (FMT == NQ_FMT_Q4_0) {
-                            cs[j][q] = __half2float(__ushort_as_half(
-                                reinterpret_cast<const uint16_t*>(p.scales)[(int64_t)nrow[j] * p.nch + cc]));
-                            cz[j][q] = 24.0f;  // 16 (conversion offset) + 8 (Q4_0's implicit zero point)
-                        } else {
-                            const int g = (cc * 32) / p.group;
-                            cs[j][q] = __half2float(__ushort_as_half(
-                                reinterpret_cast<const uint16_t*>(p.scales)[(int64_t)nrow[j] * p.groups + g]));
-                            cz[j][q] = 16.0f + (float)p.zps[(int64_t)nrow[j] * p.groups + g];
-                        }
-                    } else {
-                        cs[j][q] = 0.0f, cz[j][q] = 0.0f;
-                    }
+                    const uint32_t cc = (uint32_t)min(ks * 4 + q, p.nch - 1);
+#pragma unroll
+                    for (int j = 0; j < NW; j++) dst[j][q] = ld2(p.scales, (soff[j] + cc) * 2u);
                 }
+            }
+        } else if constexpr (FMT == NQ_FMT_W4_GROUP) {
+#pragma unroll
+            for (int q = 0; q < NS; q++) {
+                const int cc = min(ks * 4 + q, p.nch - 1);
+                const uint32_t g = (uint32_t)(((float)cc + 0.5f) * p.inv_cpg);  // cc / chunks per group
+#pragma unroll
+                for (int j = 0; j < NW; j++)
+                    dst[j][q] = ld2(p.scales, (soff[j] + g) * 2u) | (ld1(p.zps, soff[j] + g) << 16);
+            }
+        }
+    };
+    auto k_of = [&](int ks, int q) { return FOUR_BIT ? ks * 128 + q * 32 + kb * 8 : ks * 64 + kb * 16 + q * 8; };
+    auto load_x = [&](int ks, int q, int i, u32x4 (&dst)[NL]) {
+        int k0 = k_of(ks, q);
+        if (k0 >= p.K) k0 = 0;
+        const uint32_t o = xoff[i] + (uint32_t)k0 * ES;
+        dst[0] = ld16(p.x, o);
+        if constexpr (XF32) dst[1] = ld16(p.x, o + 16u);
+    };
+    auto scale_of = [&](uint32_t rec, bool valid) {
+        return valid ? __half2float(__ushort_as_half((uint16_t)(rec & 0xFFFFu))) : 0.0f;
+    };
+    auto zero_of = [&](uint32_t rec) {  // 16 (the conversion offset) + the zero point
+        return (FMT == NQ_FMT_Q4_0) ? 24.0f : 16.0f + (float)(rec >> 16);
+    };
+
+    u32x4 wv[NW];
+    uint32_t sv[NW][NS];
+    u32x4 xr[MW][NMF][NL];
+    load_w(wave, wv);
+#pragma unroll
+    for (int q = 0; q < NMF; q++)
+#pragma unroll
+        for (int i = 0; i < MW; i++) load_x(wave, q, i, xr[i][q]);
+    load_s(wave, sv);
+
+    for (int ks = wave; ks < nsteps; ks += KW) {
+        const int kn = ks + KW;  // the k-step the registers are refilled for
+        u32x4 wc[NW];
+        uint32_t sc[NW][NS];
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            wc[j] = wv[j];
+#pragma unroll
+            for (int q = 0; q < NS; q++) sc[j][q] = sv[j][q];
+        }
+        load_w(kn, wv);
+        load_s(kn, sv);
+
+        if constexpr (FOUR_BIT) {
             // ---- transpose words among the four lanes (kb = 0..3) that share a row
 #pragma unroll
             for (int j = 0; j < NW; j++) {
-                auto s02 = __builtin_amdgcn_permlane32_swap(wv[j][0], wv[j][2], false, false);
-                auto s13 = __builtin_amdgcn_permlane32_swap(wv[j][1], wv[j][3], false, false);
-                wv[j][0] = s02[0], wv[j][2] = s02[1], wv[j][1] = s13[0], wv[j][3] = s13[1];
-                auto t01 = __builtin_amdgcn_permlane16_swap(wv[j][0], wv[j][1], false, false);
-                auto t23 = __builtin_amdgcn_permlane16_swap(wv[j][2], wv[j][3], false, false);
-                wv[j][0] = t01[0], wv[j][1] = t01[1], wv[j][2] = t23[0], wv[j][3] = t23[1];
+                auto s02 = __builtin_amdgcn_permlane32_swap(wc[j][0], wc[j][2], false, false);
+                auto s13 = __builtin_amdgcn_permlane32_swap(wc[j][1], wc[j][3], false, false);
+                wc[j][0] = s02[0], wc[j][2] = s02[1], wc[j][1] = s13[0], wc[j][3] = s13[1];
+                auto t01 = __builtin_amdgcn_permlane16_swap(wc[j][0], wc[j][1], false, false);
+                auto t23 = __builtin_amdgcn_permlane16_swap(wc[j][2], wc[j][3], false, false);
+                wc[j][0] = t01[0], wc[j][1] = t01[1], wc[j][2] = t23[0], wc[j][3] = t23[1];
             }
-#pragma unroll
-            for (int q = 0; q < NMF; q++) {
-                const int k0 = ks * KSTEP + q * 32 + kb * 8;
-                const bool kvalid = k0 < p.K;
-                u32x4 bop[NW];
-#pragma unroll
-                for (int j = 0; j < NW; j++) bop[j] = nib_word_to_bf16(wv[j][q]);
+            if constexpr (WHOLE) {
+                // one group for the whole k-step: sum the four chunks in the MFMA accumulator
+                f32x4 xs[MW], pp[MW][NW];
 #pragma unroll
                 for (int i = 0; i < MW; i++) {
-                    u32x4 at[NT];
-                    load_a<XF32>(p.x, xrow[i] + k0, kvalid, at);
-                    f32x4 xs = {0, 0, 0, 0};
+                    xs[i] = (f32x4){0, 0, 0, 0};
 #pragma unroll
-                    for (int t = 0; t < NT; t++)
-                        xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xs, 0, 0, 0);
+                    for (int j = 0; j < NW; j++) pp[i][j] = (f32x4){0, 0, 0, 0};
+                }
 #pragma unroll
-                    for (int j = 0; j < NW; j++) {
-                        f32x4 pp = {0, 0, 0, 0};
+                for (int q = 0; q < NMF; q++) {
+                    const bool kvalid = k_of(ks, q) < p.K;  // the last group may be cut short by K
+                    u32x4 bop[NW];
 #pragma unroll
-                        for (int t = 0; t < NT; t++)
-                            pp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]), pp, 0, 0,
-                                                                          0);
+                    for (int j = 0; j < NW; j++) bop[j] = nib_word_to_bf16(wc[j][q]);
+#pragma unroll
+                    for (int i = 0; i < MW; i++) {
+                        u32x4 raw[NL], at[NT];
+#pragma unroll
+                        for (int t = 0; t < NL; t++) raw[t] = kvalid ? xr[i][q][t] : (u32x4){0, 0, 0, 0};
+                        load_x(kn, q, i, xr[i][q]);  // refill
+                        make_terms<XF32>(raw, at);
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            xs[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xs[i],
+                                                                             0, 0, 0);
+#pragma unroll
+                            for (int j = 0; j < NW; j++)
+                                pp[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]),
+                                                                                   pp[i][j], 0, 0, 0);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < NW; j++) {
+                    const float cs = scale_of(sc[j][0], true), cz = zero_of(sc[j][0]);
+#pragma unroll
+                    for (int i = 0; i < MW; i++)
 #pragma unroll
                         for (int r = 0; r < 4; r++)
-                            acc[i][j][r] = fmaf(cs[j][q], fmaf(-cz[j][q], xs[r], pp[r]), acc[i][j][r]);
+                            acc[i][j][r] = fmaf(cs, fmaf(-cz, xs[i][r], pp[i][j][r]), acc[i][j][r]);
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < NMF; q++) {
+                    const bool cvalid = ks * 4 + q < p.nch;
+                    u32x4 bop[NW];
+#pragma unroll
+                    for (int j = 0; j < NW; j++) bop[j] = nib_word_to_bf16(wc[j][q]);
+#pragma unroll
+                    for (int i = 0; i < MW; i++) {
+                        u32x4 raw[NL], at[NT];
+#pragma unroll
+                        for (int t = 0; t < NL; t++) raw[t] = xr[i][q][t];
+                        load_x(kn, q, i, xr[i][q]);  // refill
+                        make_terms<XF32>(raw, at);
+                        f32x4 xs = {0, 0, 0, 0};
+#pragma unroll
+                        for (int t = 0; t < NT; t++)
+                            xs = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xs, 0, 0,
+                                                                          0);
+#pragma unroll
+                        for (int j = 0; j < NW; j++) {
+                            // the zero-point term -(16 + z) sum_k x_k is the MFMA's C operand
+                            const float cz = zero_of(sc[j][q]);
+                            f32x4 pp;
+#pragma unroll
+                            for (int r = 0; r < 4; r++) pp[r] = -cz * xs[r];
+#pragma unroll
+                            for (int t = 0; t < NT; t++)
+                                pp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]), pp,
+                                                                              0, 0, 0);
+                            const float cs = scale_of(sc[j][q], cvalid);
+#pragma unroll
+                            for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf(cs, pp[r], acc[i][j][r]);
+                        }
                     }
                 }
             }
         } else {
 #pragma unroll
             for (int q = 0; q < NMF; q++) {
-                const int k0 = ks * KSTEP + kb * 16 + q * 8;
-                const bool kvalid = k0 < p.K;
+                const bool kvalid = k_of(ks, q) < p.K;
                 u32x4 bop[NW];
 #pragma unroll
                 for (int j = 0; j < NW; j++) {
                     uint32_t b0, b1, b2, b3;
-                    i8_word_to_bf16(wv[j][2 * q], b0, b1);
-                    i8_word_to_bf16(wv[j][2 * q + 1], b2, b3);
+                    i8_word_to_bf16(wc[j][2 * q], b0, b1);
+                    i8_word_to_bf16(wc[j][2 * q + 1], b2, b3);
                     bop[j] = (u32x4){b0, b1, b2, b3};
                 }
 #pragma unroll
                 for (int i = 0; i < MW; i++) {
-                    u32x4 at[NT];
-                    load_a<XF32>(p.x, xrow[i] + k0, kvalid, at);
+                    u32x4 raw[NL], at[NT];
+#pragma unroll
+                    for (int t = 0; t < NL; t++) raw[t] = kvalid ? xr[i][q][t] : (u32x4){0, 0, 0, 0};
+                    load_x(kn, q, i, xr[i][q]);
+                    make_terms<XF32>(raw, at);
 #pragma unroll
                     for (int t = 0; t < NT; t++) {
                         xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xacc[i], 0,
@@ -272,8 +397,6 @@ __global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
                 }
             }
         }
-#pragma unroll
-        for (int j = 0; j < NW; j++) wv[j] = wnext[j];
     }
 
     if constexpr (!FOUR_BIT) {
@@ -285,67 +408,61 @@ __global__ __launch_bounds__(512) void gemm_a16_kernel(const A16Params p) {
                 for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf(-128.0f, xacc[i][r], acc[i][j][r]);
     }
 
-    // ---- combine the four K-slices in wave order (fixed, so results repeat bit for bit)
-    if (wave > 0) {
+    // ---- combine the K-slices: every wavefront posts its partial tile, then wavefront w sums
+    // accumulators w, w + KW, ... over the slices in wave order (fixed, so results repeat bit
+    // for bit) and stores them
 #pragma unroll
-        for (int i = 0; i < MW; i++)
+    for (int i = 0; i < MW; i++)
 #pragma unroll
-            for (int j = 0; j < NW; j++)
+        for (int j = 0; j < NW; j++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) red[(wave - 1) * RED + ((i * NW + j) * 4 + r) * 64 + lane] = acc[i][j][r];
-    }
+            for (int r = 0; r < 4; r++) red[wave * RED + ((i * NW + j) * 4 + r) * 64 + lane] = acc[i][j][r];
     __syncthreads();
-    if (wave != 0) return;
 #pragma unroll
-    for (int j = 0; j < NW; j++) {
+    for (int t = 0; t < EPW; t++) {
+        const int idx = wave + t * KW;
+        if (TA % KW != 0 && idx >= TA) break;
+        float part[KW];
+#pragma unroll
+        for (int w = 0; w < KW; w++) part[w] = red[w * RED + idx * 64 + lane];
+        float z = part[0];
+#pragma unroll
+        for (int w = 1; w < KW; w++) z += part[w];
+        const int r = idx & 3, j = (idx >> 2) % NW, i = (idx >> 2) / NW;
         const int n = n_base + 16 * j + ln;
-        if (n >= p.N) continue;
-        const float rs = ep_scale[j], b = ep_bias[j];
-#pragma unroll
-        for (int i = 0; i < MW; i++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int m = m_base + 16 * i + 4 * kb + r;  // D layout: row 4*(lane/16) + r, column lane%16
-                if (m >= p.M) continue;
-                const int ri = ((i * NW + j) * 4 + r) * 64 + lane;
-                float z = acc[i][j][r];
-                for (int w = 0; w < KW - 1; w++) z += red[w * RED + ri];
-                if (FMT == NQ_FMT_W8_CHANNEL) z *= rs;
-                z += b;
-                if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
-                const int64_t o = (int64_t)m * p.N + n;
-                if (p.y_dtype == NQ_DT_F32)
-                    reinterpret_cast<float*>(p.y)[o] = z;
-                else
-                    reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(z);
-            }
+        const int m = m_base + 16 * i + 4 * kb + r;  // D layout: row 4*(lane/16) + r, column lane%16
+        if (FMT == NQ_FMT_W8_CHANNEL) z *= ep_scale[t];
+        z += ep_bias[t];
+        if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+        if (n < p.N && m < p.M) {
+            const int64_t o = (int64_t)m * p.N + n;
+            if (p.y_dtype == NQ_DT_F32)
+                reinterpret_cast<float*>(p.y)[o] = z;
+            else
+                reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(z);
+        }
     }
 }
 
-template <int FMT, bool XF32, int MW>
-int32_t launch_nw(const A16Params& p, int nw, int kw, dim3 grid, hipStream_t s) {
-    const size_t lds = (size_t)(kw - 1) * MW * nw * 4 * 64 * sizeof(float);
-    if (nw == 1)
-        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW, 1>), grid, dim3(64 * kw), lds, s, p);
-    else
-        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW, 2>), grid, dim3(64 * kw), lds, s, p);
-    NQ_HIP(hipGetLastError());
-    return NQ_OK;
-}
-
-template <int FMT, bool XF32>
-int32_t launch_mw(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
-    switch (mw) {
-        case 1: return launch_nw<FMT, XF32, 1>(p, nw, kw, grid, s);
-        case 2: return launch_nw<FMT, XF32, 2>(p, nw, kw, grid, s);
-        case 3: return launch_nw<FMT, XF32, 3>(p, nw, kw, grid, s);
-        default: return launch_nw<FMT, XF32, 4>(p, nw, kw, grid, s);
+template <int FMT, bool XF32, bool WHOLE>
+int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
+    const size_t lds = (size_t)kw * mw * nw * 4 * 64 * sizeof(float);
+    const dim3 block(64 * kw);
+#define NQ_A16_CASE(MW_, NW_, KW_)                                                                         \
+    if (mw == MW_ && nw == NW_ && kw == KW_) {                                                             \
+        hipLaunchKernelGGL((gemm_a16_kernel<FMT, XF32, MW_, NW_, KW_, WHOLE>), grid, block, lds, s, p);    \
+        NQ_HIP(hipGetLastError());                                                                         \
+        return NQ_OK;                                                                                      \
     }
-}
-
-template <int FMT>
-int32_t launch_x(const A16Params& p, bool xf32, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
-    return xf32 ? launch_mw<FMT, true>(p, mw, nw, kw, grid, s) : launch_mw<FMT, false>(p, mw, nw, kw, grid, s);
+#define NQ_A16_TILE(MW_, NW_) NQ_A16_CASE(MW_, NW_, 4) NQ_A16_CASE(MW_, NW_, 8)
+    NQ_A16_TILE(1, 1)
+    NQ_A16_TILE(1, 2)
+    NQ_A16_TILE(1, 4)
+    NQ_A16_TILE(2, 2)
+    if constexpr (!XF32) { NQ_A16_TILE(2, 4) }
+#undef NQ_A16_TILE
+#undef NQ_A16_CASE
+    return fail(NQ_ERR_INVALID, "nq_forward: no medium-M kernel of that tile shape");
 }
 
 int env_int(const char* name, int dflt) {
@@ -361,52 +478,61 @@ bool gemm_a16_applicable(const ForwardArgs& a) {
     if (L->format == NQ_FMT_FP8_E4M3) return false;
     if (L->format != NQ_FMT_W8_CHANNEL && L->in % 32 != 0) return false;
     if (L->format == NQ_FMT_W8_CHANNEL && L->in % 16 != 0) return false;
+    // the kernel addresses each operand with 32-bit byte offsets
+    const int64_t lim = (int64_t)1 << 32;
+    if ((int64_t)a.M * L->in * 4 >= lim || (int64_t)L->out * L->in >= lim) return false;
     return a.M >= 5;
 }
 
 int32_t launch_gemm_a16(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     const bool four_bit = L->format != NQ_FMT_W8_CHANNEL;
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
     A16Params p{};
     p.codes = L->d_codes, p.scales = L->d_scales, p.zps = L->d_zps;
     p.x = a.x, p.y = a.y, p.bias = a.bias;
     p.M = a.M, p.N = L->out, p.K = L->in;
-    p.group = L->group, p.groups = L->groups;
+    p.groups = L->groups;
+    p.inv_cpg = L->group ? 32.0f / (float)L->group : 1.0f;
+    p.s_pairs = L->format != NQ_FMT_Q4_0 ? 0 : (L->in / 32) % 4 == 0 ? 2 : (L->in / 32) % 2 == 0 ? 1 : 0;
     p.nch = L->in / (four_bit ? 32 : 16);
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
-    // M tile: the smallest multiple of 16 rows (<= 64) that wastes the least padding
-    int mw = 4;
-    if (a.M <= 16) mw = 1;
-    else if (a.M <= 32) mw = 2;
-    else if (a.M <= 48) mw = 3;
-    else {
-        int best_tiles = 1 << 30;
-        for (int c = 4; c >= 2; c--) {
-            const int tiles = (a.M + 16 * c - 1) / (16 * c) * c;  // 16-row MFMA tiles computed
-            if (tiles < best_tiles) best_tiles = tiles, mw = c;
-        }
+    // Tile shape: as wide in N as still leaves enough workgroups to occupy the chip (the
+    // activations are the operand that is re-read per N tile), two M tiles per wavefront only
+    // when that costs no extra padded rows
+    // (measured at M = 100..256: the 2 x 4 tile only pays once there is work for several
+    // rounds of workgroups, and below ~128 workgroups a narrower tile wins)
+    static const int shapes[5][2] = {{2, 4}, {2, 2}, {1, 4}, {1, 2}, {1, 1}};
+    int mw = 1, nw = 1;
+    const int mt = (a.M + 15) / 16;
+    for (int c = 0; c < 5; c++) {
+        mw = shapes[c][0], nw = shapes[c][1];
+        if (mw == 2 && (mt & 1) && mt < 16) continue;
+        if (mw * nw == 8 && xf32) continue;  // would not fit the register budget
+        const int64_t wgs = (int64_t)((mt + mw - 1) / mw) * ((L->out + 16 * nw - 1) / (16 * nw));
+        if (wgs >= (mw * nw == 8 ? 2048 : 128)) break;
     }
-    int nw = (L->out >= 1024) ? 2 : 1;
-    if (mw * nw > 6) nw = 1;  // 4 x 2 MFMA tiles per wavefront would spill under the 256-register budget
-    // wavefronts along K: as many as it takes to leave each one at most two k-steps (the call is
-    // latency-bound: a k-step is one dependent round trip to memory), within the LDS the
-    // fixed-order reduction needs
+    mw = env_int("NQ_A16_MW", mw), nw = env_int("NQ_A16_NW", nw);
+    // K split: 8 wavefronts when there are more than 4 k-steps
     const int kstep = four_bit ? 128 : 64;
     const int nsteps = (L->in + kstep - 1) / kstep;
-    int kw = 4;
-    while (kw < 8 && (nsteps + kw - 1) / kw > 2) kw *= 2;
-    while ((size_t)(kw - 1) * mw * nw * 1024 > 60 * 1024) {
-        if (nw > 1) nw = 1;
-        else if (mw > 1) mw--;
-        else kw /= 2;
-    }
+    int kw = nsteps > 4 ? 8 : 4;
     kw = env_int("NQ_A16_KW", kw);
     dim3 grid((L->out + 16 * nw - 1) / (16 * nw), (a.M + 16 * mw - 1) / (16 * mw));
-    const bool xf32 = a.x_dtype == NQ_DT_F32;
     switch (L->format) {
-        case NQ_FMT_Q4_0: return launch_x<NQ_FMT_Q4_0>(p, xf32, mw, nw, kw, grid, a.stream);
-        case NQ_FMT_W4_GROUP: return launch_x<NQ_FMT_W4_GROUP>(p, xf32, mw, nw, kw, grid, a.stream);
-        case NQ_FMT_W8_CHANNEL: return launch_x<NQ_FMT_W8_CHANNEL>(p, xf32, mw, nw, kw, grid, a.stream);
+        case NQ_FMT_Q4_0:
+            return xf32 ? launch_tile<NQ_FMT_Q4_0, true, false>(p, mw, nw, kw, grid, a.stream)
+                        : launch_tile<NQ_FMT_Q4_0, false, false>(p, mw, nw, kw, grid, a.stream);
+        case NQ_FMT_W4_GROUP:
+            // a k-step (128 k) lies in one group when the group width is a multiple of 128
+            if (L->group % 128 == 0)
+                return xf32 ? launch_tile<NQ_FMT_W4_GROUP, true, true>(p, mw, nw, kw, grid, a.stream)
+                            : launch_tile<NQ_FMT_W4_GROUP, false, true>(p, mw, nw, kw, grid, a.stream);
+            return xf32 ? launch_tile<NQ_FMT_W4_GROUP, true, false>(p, mw, nw, kw, grid, a.stream)
+                        : launch_tile<NQ_FMT_W4_GROUP, false, false>(p, mw, nw, kw, grid, a.stream);
+        case NQ_FMT_W8_CHANNEL:
+            return xf32 ? launch_tile<NQ_FMT_W8_CHANNEL, true, false>(p, mw, nw, kw, grid, a.stream)
+                        : launch_tile<NQ_FMT_W8_CHANNEL, false, false>(p, mw, nw, kw, grid, a.stream);
     }
     return fail(NQ_ERR_INVALID, "nq_forward: unknown format");
 }
