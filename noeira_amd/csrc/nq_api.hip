@@ -370,6 +370,7 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
     } else if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16) {
         return fail(NQ_ERR_INVALID, "nq_forward: unknown x dtype " + std::to_string(x_dtype));
     }
+    if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
     if (gemv_m1_applicable(a)) return launch_gemv_m1(a);

@@ -92,6 +92,10 @@ int32_t launch_gemv_i8(const ForwardArgs& a);
 bool gemv_m1_applicable(const ForwardArgs& a);
 int32_t launch_gemv_m1(const ForwardArgs& a);
 
+// nq_gemv_fp8.hip: fp8 x fp8 GEMV for 1..16 activation rows on the matrix cores
+bool gemv_fp8_applicable(const ForwardArgs& a);
+int32_t launch_gemv_fp8(const ForwardArgs& a);
+
 // nq_gemm8.hip: LDS-tiled fp8 / int8 MFMA GEMM for large M
 bool gemm8_applicable(const ForwardArgs& a);
 int32_t launch_gemm8(const ForwardArgs& a);

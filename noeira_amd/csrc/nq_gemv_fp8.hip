@@ -1,0 +1,294 @@
+// fp8 x fp8 GEMV for 1..16 activation rows on the matrix cores:
+//     y[M, N] = epi( (x[M, K] @ W[N, K]^T) * s_w * s_x + bias ),  x and W in e4m3.
+//
+// The call is bound by the weight stream (K = 4096, N = 11008 is 45 MB), and what a
+// streaming kernel can lose is issue slots: converting an fp8 code and multiplying it on the
+// vector ALU costs about two instructions per weight per wavefront, which at one row per
+// wavefront is more instruction issue than the loads leave room for.  One
+// v_mfma_f32_16x16x128_f8f6f4 multiplies a 16-row x 128-k slab of weights (2 KB) by up to 16
+// activation rows in a single instruction, so the kernel is loads plus a handful of MFMAs:
+//   - a workgroup owns 16 weight rows; its KW wavefronts split K, SPW steps of 128 k each;
+//   - lane (n = lane % 16, kb = lane / 16) loads the 32 bytes of row n under k-block kb of a
+//     step (two 128-bit loads, 128 contiguous bytes per row across the four lanes) - this is
+//     exactly its share of the MFMA's B operand, so nothing is shuffled or converted;
+//   - the activations are the A operand: row m = lane % 16 (clamped to M - 1), same k-block;
+//     they are 16 x K bytes at most and stay in L1/L2;
+//   - all of a wavefront's loads are issued before its first MFMA (SPW x 32 bytes per lane,
+//     up to 16 KB per wavefront in flight);
+//   - the KW partial 16 x 16 tiles are summed through LDS in wave order (fixed, so a repeated
+//     call returns the same bits) and thread (m, n) applies scale, bias and epilogue.
+//
+// A single activation row (M = 1) takes a second kernel whose loads are fully coalesced: one
+// wavefront owns ONE weight row and reads it as 1 KB contiguous per load instruction (lane l
+// takes the 16-byte chunks l, l + 64, ...).  The MFMA is then used "diagonally": the 16 B
+// columns are 16 different 128-byte segments of that row and the 16 A rows are the matching
+// segments of x (lane l of A holds x at the very offsets lane l of B holds W), so
+// D[c][c] = <x segment c, W segment c> and the row's dot product is the trace of D.  15/16 of
+// the MFMA is wasted, which costs nothing here: the instruction replaces ~250 VALU
+// instructions per KB-row and the kernel issues little besides its loads.
+#include "nq_common.h"
+
+#include <cstdlib>
+
+namespace nq {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+struct Fp8GemvParams {
+    const uint8_t* w;
+    const uint8_t* x;
+    const float* x_scale;
+    void* y;
+    const void* bias;
+    int32_t M, N, K;
+    int32_t nsteps;  // K / 128
+    float tscale;
+    int32_t y_dtype, bias_dtype, epilogue;
+};
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
+    uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
+template <int SPW, int KW>
+__global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p) {
+    __shared__ float red[KW][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ln = lane & 15, kb = lane >> 4;
+    const int n_base = blockIdx.x * 16;
+
+    const int64_t wrow = (int64_t)min(n_base + ln, p.N - 1) * p.K;
+    const int64_t xrow = (int64_t)min(ln, p.M - 1) * p.K;
+
+    f32x4 acc = {0, 0, 0, 0};
+    for (int s0 = wave * SPW; s0 < p.nsteps; s0 += KW * SPW) {
+        u32x4 wv[SPW][2], xv[SPW][2];
+        // unconditional loads from clamped step indices; a step past K is multiplied by zero
+#pragma unroll
+        for (int s = 0; s < SPW; s++) {
+            const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128 + kb * 32;
+            const u32x4* src = reinterpret_cast<const u32x4*>(p.w + wrow + k0);
+            wv[s][0] = __builtin_nontemporal_load(src);
+            wv[s][1] = __builtin_nontemporal_load(src + 1);
+        }
+#pragma unroll
+        for (int s = 0; s < SPW; s++) {
+            const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128 + kb * 32;
+            const u32x4* src = reinterpret_cast<const u32x4*>(p.x + xrow + k0);
+            const bool valid = s0 + s < p.nsteps;
+            const u32x4 t0 = src[0], t1 = src[1];
+            xv[s][0] = valid ? t0 : (u32x4){0, 0, 0, 0};
+            xv[s][1] = valid ? t1 : (u32x4){0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int s = 0; s < SPW; s++) {
+            const i32x8 a = {(int)xv[s][0][0], (int)xv[s][0][1], (int)xv[s][0][2], (int)xv[s][0][3],
+                             (int)xv[s][1][0], (int)xv[s][1][1], (int)xv[s][1][2], (int)xv[s][1][3]};
+            const i32x8 b = {(int)wv[s][0][0], (int)wv[s][0][1], (int)wv[s][0][2], (int)wv[s][0][3],
+                             (int)wv[s][1][0], (int)wv[s][1][1], (int)wv[s][1][2], (int)wv[s][1][3]};
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+        }
+    }
+
+    // D layout: lane holds column n = lane % 16, rows m = 4 (lane / 16) + r
+#pragma unroll
+    for (int r = 0; r < 4; r++) red[wave][(4 * kb + r) * 16 + ln] = acc[r];
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < 256) {
+        const int m = t >> 4, n = n_base + (t & 15);
+        if (m < p.M && n < p.N) {
+            float z = red[0][t];
+#pragma unroll
+            for (int w = 1; w < KW; w++) z += red[w][t];
+            z *= p.tscale * p.x_scale[0];
+            if (p.bias)
+                z += (p.bias_dtype == NQ_DT_F32)
+                         ? reinterpret_cast<const float*>(p.bias)[n]
+                         : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+            const int64_t o = (int64_t)m * p.N + n;
+            if (p.y_dtype == NQ_DT_F32)
+                reinterpret_cast<float*>(p.y)[o] = z;
+            else
+                reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(z);
+        }
+    }
+}
+
+
+int env_int(const char* name, int dflt) {
+    const char* v = std::getenv(name);
+    return v ? std::atoi(v) : dflt;
+}
+
+// ---- M = 1: one wavefront per weight row, coalesced loads, trace of the MFMA tile
+template <int CPL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvParams p) {
+    __shared__ u32x4 xs[CPL * 64];  // the activation row, shared by the workgroup's rows
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row = (int64_t)blockIdx.x * WAVES + wave;
+    const int nch = p.K >> 4;  // 16-byte chunks per row
+    const u32x4* wr = reinterpret_cast<const u32x4*>(p.w + min(row, (int64_t)p.N - 1) * p.K);
+    const u32x4* xr = reinterpret_cast<const u32x4*>(p.x);
+
+    // x goes first so that waiting for it leaves the weight loads in flight; every load is
+    // unconditional from a clamped chunk index, and a chunk past K meets x = 0
+    constexpr int XPT = (CPL * 64 + 64 * WAVES - 1) / (64 * WAVES);  // chunks of x per thread
+    u32x4 xg[XPT];
+#pragma unroll
+    for (int i = 0; i < XPT; i++) xg[i] = xr[min((int)threadIdx.x + i * 64 * WAVES, nch - 1)];
+    u32x4 wv[CPL], xv[CPL];
+#pragma unroll
+    for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wr + min(j * 64 + lane, nch - 1));
+#pragma unroll
+    for (int i = 0; i < XPT; i++) {
+        const int c = (int)threadIdx.x + i * 64 * WAVES;
+        if (c < CPL * 64) xs[c] = (c < nch) ? xg[i] : (u32x4){0, 0, 0, 0};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < CPL; j++) xv[j] = xs[j * 64 + lane];
+    // the epilogue's operands travel with the codes
+    const float scale = p.tscale * p.x_scale[0];
+    float bias = 0.0f;
+    if (p.bias) {
+        const int64_t n = min(row, (int64_t)p.N - 1);
+        bias = (p.bias_dtype == NQ_DT_F32)
+                   ? reinterpret_cast<const float*>(p.bias)[n]
+                   : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+    }
+
+    f32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < CPL; j += 2) {
+        const u32x4 x1 = (j + 1 < CPL) ? xv[j + 1] : (u32x4){0, 0, 0, 0};
+        const u32x4 w1 = (j + 1 < CPL) ? wv[j + 1] : (u32x4){0, 0, 0, 0};
+        const i32x8 a = {(int)xv[j][0], (int)xv[j][1], (int)xv[j][2], (int)xv[j][3],
+                         (int)x1[0],    (int)x1[1],    (int)x1[2],    (int)x1[3]};
+        const i32x8 b = {(int)wv[j][0], (int)wv[j][1], (int)wv[j][2], (int)wv[j][3],
+                         (int)w1[0],    (int)w1[1],    (int)w1[2],    (int)w1[3]};
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+    }
+    // lane holds D[4 (lane / 16) + r][lane % 16]: its diagonal entry, if any, is r = c % 4 where
+    // c = lane % 16 and c / 4 == lane / 16
+    const int c = lane & 15, r = c & 3;
+    float v = r == 0 ? acc[0] : r == 1 ? acc[1] : r == 2 ? acc[2] : acc[3];
+    v = ((c >> 2) == (lane >> 4)) ? v : 0.0f;
+    // fixed butterfly over the 64 lanes (so a repeated call returns the same bits)
+    int t;
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false);
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false);
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false);
+    v += __int_as_float(t);
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false);
+    v += __int_as_float(t);
+    {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+    {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+    }
+    if (lane == 0 && row < p.N) {
+        float z = v * scale + bias;
+        if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+        if (p.y_dtype == NQ_DT_F32)
+            reinterpret_cast<float*>(p.y)[row] = z;
+        else
+            reinterpret_cast<uint16_t*>(p.y)[row] = f32_to_bf16_rne(z);
+    }
+}
+
+template <int CPL>
+int32_t launch_row(const Fp8GemvParams& p, int waves, hipStream_t s) {
+    if (waves == 4)
+        hipLaunchKernelGGL((gemv_fp8_row_kernel<CPL, 4>), dim3((unsigned)((p.N + 3) / 4)), dim3(256), 0, s, p);
+    else if (waves == 8)
+        hipLaunchKernelGGL((gemv_fp8_row_kernel<CPL, 8>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
+    else
+        hipLaunchKernelGGL((gemv_fp8_row_kernel<CPL, 16>), dim3((unsigned)((p.N + 15) / 16)), dim3(1024), 0, s, p);
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+
+template <int SPW>
+int32_t launch_kw(const Fp8GemvParams& p, int kw, dim3 grid, hipStream_t s) {
+    if (kw == 4)
+        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 4>), grid, dim3(256), 0, s, p);
+    else if (kw == 8)
+        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 8>), grid, dim3(512), 0, s, p);
+    else if constexpr (SPW <= 4)
+        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 16>), grid, dim3(1024), 0, s, p);
+    else
+        return fail(NQ_ERR_INVALID, "nq_forward: no fp8 GEMV of that shape");
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+}  // namespace
+
+// a row of 768..8192 codes takes the one-row kernel (M = 1, K a multiple of 16); otherwise the
+// 16-row tile kernel needs whole MFMA steps (K a multiple of 128)
+static bool row_kernel_fits(const ForwardArgs& a) {
+    return a.M == 1 && a.L->in % 16 == 0 && a.L->in >= 768 && a.L->in <= 8192;
+}
+
+bool gemv_fp8_applicable(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (L->format != NQ_FMT_FP8_E4M3 || a.x_dtype != NQ_DT_FP8_E4M3 || a.x_scale == nullptr) return false;
+    return row_kernel_fits(a) || (a.M >= 1 && a.M <= 16 && L->in % 128 == 0);
+}
+
+int32_t launch_gemv_fp8(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    Fp8GemvParams p{};
+    p.w = L->d_codes, p.x = reinterpret_cast<const uint8_t*>(a.x), p.x_scale = a.x_scale;
+    p.y = a.y, p.bias = a.bias;
+    p.M = a.M, p.N = L->out, p.K = L->in, p.nsteps = L->in / 128;
+    p.tscale = L->scale;
+    p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    // one row: a wavefront per weight row once a row fills most of its 64 lanes (K >= 768)
+    const int cpl = (L->in / 16 + 63) / 64;
+    if (row_kernel_fits(a) && (L->in % 128 != 0 || env_int("NQ_FP8V_ROW", 1))) {
+        const int waves = env_int("NQ_FP8V_WAVES", 8);
+        switch (cpl) {
+            case 1: return launch_row<1>(p, waves, a.stream);
+            case 2: return launch_row<2>(p, waves, a.stream);
+            case 3: return launch_row<3>(p, waves, a.stream);
+            case 4: return launch_row<4>(p, waves, a.stream);
+            case 5: return launch_row<5>(p, waves, a.stream);
+            case 6: return launch_row<6>(p, waves, a.stream);
+            case 7: return launch_row<7>(p, waves, a.stream);
+            default: return launch_row<8>(p, waves, a.stream);
+        }
+    }
+    // K split: up to 8 steps (16 KB) per wavefront, and enough wavefronts per workgroup that a
+    // small N still fills the chip
+    int kw = 4, spw = 8;
+    const int64_t wgs = ((int64_t)L->out + 15) / 16;
+    if (wgs < 512) kw = 8;
+    if (wgs < 128) kw = 16;
+    while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
+    if (kw == 16 && spw > 4) spw = 4;
+    kw = env_int("NQ_FP8V_KW", kw), spw = env_int("NQ_FP8V_SPW", spw);
+    const dim3 grid((unsigned)wgs);
+    switch (spw) {
+        case 1: return launch_kw<1>(p, kw, grid, a.stream);
+        case 2: return launch_kw<2>(p, kw, grid, a.stream);
+        case 4: return launch_kw<4>(p, kw, grid, a.stream);
+        default: return launch_kw<8>(p, kw, grid, a.stream);
+    }
+}
+
+}  // namespace nq

@@ -190,10 +190,10 @@ def test_encode_e4m3_host_matches_oracle():
     assert np.array_equal(F.encode_e4m3(x), O.e4m3_encode(np.clip(x, -448, 448)))
 
 
-@pytest.mark.parametrize("M", [1, 64])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 64])
 def test_config5_fp8_reduced_size_vs_oracle(M):
     rng = np.random.default_rng(5 + M)
-    N, K = 512, 4096
+    N, K = (504 if M in (7, 17) else 512), 4096  # 504 = 31.5 row tiles of 16
     a, b = fp8_operands(rng, M, N, K)
     sa, sb = np.float32(0.731), np.float32(1.37)
     lin = FP8Linear(K, N)
@@ -210,7 +210,7 @@ def test_config5_fp8_reduced_size_vs_oracle(M):
     assert rel_rms(yf, y64) < TOL_RMS_FP8
     # far inside the bar: the matrix cores add fp8 products in fp32 (their internal alignment
     # costs a little against a serial fp32 chain: ~6e-5 of RMS at K = 4096)
-    assert rel_rms(yf, y64) < (1e-5 if M == 1 else 3e-4)
+    assert rel_rms(yf, y64) < 3e-4
     gb = y.view(torch.int16).cpu().numpy().view(np.uint16)
     assert np.array_equal(gb, O.bf16_bits(yf))
     # and so it sits within bf16's own half-step (2^-9 relative) of the exact value, plus the
@@ -230,7 +230,30 @@ def test_config5_fp8_gemv_full_size_sampled():
     xs = torch.ones(1, dtype=torch.float32, device="cuda")
     y = lin.forward(torch.from_numpy(a).cuda(), xs, out_dtype=torch.float32).cpu().numpy()
     y64, _ = O.fp8_forward_f64(a, b, 1.0, 1.0, want_bf16=False)
-    assert rel_rms(y, y64) < 1e-5
+    assert rel_rms(y, y64) < 3e-4  # MFMA fp32 accumulation; the bar is 1e-2
+    # repeated calls return the same bits (fixed-order K split)
+    y2 = lin.forward(torch.from_numpy(a).cuda(), xs, out_dtype=torch.float32).cpu().numpy()
+    assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 128, 16), (3, 384, 40), (16, 2560, 100), (2, 8192, 33),
+                                   (1, 784, 37), (1, 1024, 5), (1, 2576, 130), (1, 8192, 19), (1, 8208, 9)])
+def test_fp8_small_m_bias_relu_and_shapes(M, K, N):
+    """fp8 x fp8 at 1..16 rows: ragged N, K from one MFMA step to several rounds of the K split,
+    fp32 bias and ReLU fused; checked against the float64 oracle."""
+    rng = np.random.default_rng(1000 + M + K)
+    a, b = fp8_operands(rng, M, N, K)
+    sa, sb = np.float32(0.5), np.float32(0.25)
+    bias = rng.standard_normal(N).astype(np.float32)
+    lin = FP8Linear(K, N)
+    lin.set_weight(b, float(sb))
+    xs = torch.tensor([sa], dtype=torch.float32, device="cuda")
+    y = lin.forward(torch.from_numpy(a).cuda(), xs, bias=torch.from_numpy(bias).cuda(), epilogue="relu",
+                    out_dtype=torch.float32).cpu().numpy()
+    y64, _ = O.fp8_forward_f64(a, b, sa, sb, want_bf16=False)
+    ref = np.maximum(y64 + bias.astype(np.float64), 0.0)
+    rms = np.sqrt(((y64 + bias) ** 2).mean())
+    assert np.abs(y - ref).max() <= 3e-4 * rms
 
 
 @pytest.mark.parametrize("N", [4096, 11008])
@@ -260,7 +283,7 @@ def test_config5_fp8_gemm_full_size_sampled(N):
     assert rel_rms(got, y64) < TOL_RMS_FP8
     assert rel_rms(got, y64) < 3e-4
     gemv = lin.forward(ad[int(rows[5])].reshape(1, K).contiguous(), xs, out_dtype=torch.float32).cpu().numpy()
-    assert rel_rms(gemv, y64[5:6]) < 1e-5
+    assert rel_rms(gemv, y64[5:6]) < 3e-4
 
 
 @pytest.mark.parametrize("M,K,N", [(4096, 256, 256), (300, 384, 520), (64, 128, 8), (1000, 1024, 264)])
