@@ -143,56 +143,92 @@ void gemm8_kernel(const Gemm8Params p) {
     const int fh = lane >> 5;
     const int fsw = (frow >> 1) & 7;
 
+    // ---- main loop, software-pipelined by hand.  A wavefront has its SIMD to itself (the
+    // 128 x 128 accumulator leaves room for one), so nothing hides an LDS round trip unless
+    // the program order does: every fragment is read one MFMA group (4 MFMAs, ~256 cycles)
+    // before the group that consumes it, the next sub-step's weight fragments are spread over
+    // the four groups of the current one, and the one barrier of a K step sits before its LAST
+    // group, followed at once by the first reads of the next stage, so that barrier skew and
+    // read latency are both covered by matrix-core work already queued.
+    // __builtin_amdgcn_sched_barrier(0) pins that order against the instruction scheduler.
+    constexpr int NS = FP8 ? 2 : 4;  // sub-steps (one MFMA k-extent each) per K step
+    typedef typename std::conditional<FP8, i32x8, i32x4>::type frag_t;
+    auto read_frag = [&](const uint8_t* base, int sub, int t) -> frag_t {
+        if constexpr (FP8) {
+            const int o0 = ((4 * sub + 2 * fh) ^ fsw) << 4, o1 = ((4 * sub + 2 * fh + 1) ^ fsw) << 4;
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(base + t * 32 * BK + o0);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(base + t * 32 * BK + o1);
+            return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        } else {
+            const int o0 = ((2 * sub + fh) ^ fsw) << 4;
+            return *reinterpret_cast<const i32x4*>(base + t * 32 * BK + o0);
+        }
+    };
+    auto stage_a = [&](int kt) { return lds + (kt & 1) * STAGE_BYTES + (wm * 128 + frow) * BK; };
+    auto stage_b = [&](int kt) { return lds + (kt & 1) * STAGE_BYTES + BM * BK + (wn * 128 + frow) * BK; };
+
     const int KT = p.K / BK;
     dma(0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    // Fragment registers are two named sets used in turn (groups alternate between af[0] and
+    // af[1], sub-steps between bf[0] and bf[1]); a K step has an even number of both, so the
+    // sets line up again at the loop's back edge and nothing is copied.
+    frag_t af[2], bf[2][4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) bf[0][j] = read_frag(stage_b(0), 0, j);
+    af[0] = read_frag(stage_a(0), 0, 0);
     for (int kt = 0; kt < KT; kt++) {
-        // stage kt+1 streams into the other buffer while stage kt is multiplied; the barrier at
-        // the end of the previous iteration guarantees nobody still reads that buffer
+        // stage kt+1 streams into the other buffer while stage kt is multiplied; the barrier
+        // inside the previous iteration guarantees nobody still reads that buffer
         if (kt + 1 < KT) dma((kt + 1) * BK, (kt + 1) & 1);
-        const uint8_t* sa = lds + (kt & 1) * STAGE_BYTES + (wm * 128 + frow) * BK;
-        const uint8_t* sb = lds + (kt & 1) * STAGE_BYTES + BM * BK + (wn * 128 + frow) * BK;
-        if constexpr (FP8) {
+        const uint8_t* sa = stage_a(kt);
+        const uint8_t* sb = stage_b(kt);
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                const int o0 = ((4 * s + 2 * fh) ^ fsw) << 4, o1 = ((4 * s + 2 * fh + 1) ^ fsw) << 4;
-                i32x8 af[4], bf[4];
+        for (int sub = 0; sub < NS; sub++) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const i32x4 lo = *reinterpret_cast<const i32x4*>(sa + i * 32 * BK + o0);
-                    const i32x4 hi = *reinterpret_cast<const i32x4*>(sa + i * 32 * BK + o1);
-                    af[i] = (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    const i32x4 lo2 = *reinterpret_cast<const i32x4*>(sb + i * 32 * BK + o0);
-                    const i32x4 hi2 = *reinterpret_cast<const i32x4*>(sb + i * 32 * BK + o1);
-                    bf[i] = (i32x8){lo2[0], lo2[1], lo2[2], lo2[3], hi2[0], hi2[1], hi2[2], hi2[3]};
+            for (int i = 0; i < 4; i++) {
+                const int g = sub * 4 + i;  // group index within the K step
+                const bool last = (sub == NS - 1 && i == 3);
+                frag_t& acur = af[g & 1];
+                frag_t& anext = af[(g + 1) & 1];
+                frag_t(&bcur)[4] = bf[sub & 1];
+                frag_t(&bnext)[4] = bf[(sub + 1) & 1];
+                if (last) {
+                    // every read of stage kt has been issued and waited for; once all wavefronts
+                    // are here stage kt+1 is complete and stage kt's buffer may be overwritten
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
                 }
+                __builtin_amdgcn_sched_barrier(0);
+                // the first MFMA of the group goes ahead of the prefetch so that the reads are
+                // issued while the matrix core is busy and have the rest of the group to land
+                if constexpr (FP8)
+                    acc[i][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bcur[0], acur, acc[i][0], 0, 0, 0, 0,
+                                                                                 0, 0);
+                else
+                    acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bcur[0], acur, acc[i][0], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (!last) {
+                    anext = (i < 3) ? read_frag(sa, sub, i + 1) : read_frag(sa, sub + 1, 0);
+                    if (sub + 1 < NS) bnext[i] = read_frag(sb, sub + 1, i);
+                } else if (kt + 1 < KT) {
+                    anext = read_frag(stage_a(kt + 1), 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                    for (int j = 0; j < 4; j++) bnext[j] = read_frag(stage_b(kt + 1), 0, j);
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, 0, 0,
+                for (int j = 1; j < 4; j++) {
+                    if constexpr (FP8)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bcur[j], acur, acc[i][j], 0, 0, 0,
                                                                                      0, 0, 0);
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                const int o0 = ((2 * s + fh) ^ fsw) << 4;
-                i32x4 af[4], bf[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    af[i] = *reinterpret_cast<const i32x4*>(sa + i * 32 * BK + o0);
-                    bf[i] = *reinterpret_cast<const i32x4*>(sb + i * 32 * BK + o0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bcur[j], acur, acc[i][j], 0, 0, 0);
                 }
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
     }
 
     // ---- epilogue.  The MFMA was issued with the weight tile as its first operand, so in
@@ -244,34 +280,55 @@ void gemm8_kernel(const Gemm8Params p) {
 #pragma unroll
                     for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8);
                 }
+                if constexpr (KIND == 2) {
 #pragma unroll
-                for (int ii = 0; ii < IP; ii++) {
-                    const int i = ip + ii;
+                    for (int ii = 0; ii < IP; ii++) {
+                        const int i = ip + ii;
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        uint8_t* dst = stage + (32 * ii + lm) * ROWB + (32 * j + 8 * g + 4 * lh) * ES;
-                        if constexpr (KIND == 2) {
+                        for (int g = 0; g < 4; g++) {
+                            uint8_t* dst = stage + (32 * ii + lm) * ROWB + (32 * j + 8 * g + 4 * lh) * ES;
                             *reinterpret_cast<i32x4*>(dst) = (i32x4){(int)acc[i][j][4 * g], (int)acc[i][j][4 * g + 1],
                                                                       (int)acc[i][j][4 * g + 2], (int)acc[i][j][4 * g + 3]};
-                        } else {
-                            float z[4];
+                        }
+                    }
+                } else {
+                    float z[IP][4][4];
+#pragma unroll
+                    for (int ii = 0; ii < IP; ii++)
+#pragma unroll
+                        for (int g = 0; g < 4; g++)
 #pragma unroll
                             for (int r = 0; r < 4; r++) {
                                 if constexpr (FP8)
-                                    z[r] = acc[i][j][4 * g + r] * fp8_scale + cb[g][r];
+                                    z[ii][g][r] = acc[ip + ii][j][4 * g + r] * fp8_scale + cb[g][r];
                                 else
-                                    z[r] = (float)acc[i][j][4 * g + r] * (rscale[ii] * cs[g][r]) + cb[g][r];
-                                if (p.epilogue == NQ_EPI_RELU) z[r] = z[r] > 0.0f ? z[r] : 0.0f;
+                                    z[ii][g][r] = (float)acc[ip + ii][j][4 * g + r] * (rscale[ii] * cs[g][r]) + cb[g][r];
                             }
+                    if (p.epilogue == NQ_EPI_RELU) {
+                        // a real (uniform) branch: one v_max per value when asked for, nothing otherwise
+                        asm volatile("" ::: "memory");
+#pragma unroll
+                        for (int ii = 0; ii < IP; ii++)
+#pragma unroll
+                            for (int g = 0; g < 4; g++)
+#pragma unroll
+                                for (int r = 0; r < 4; r++) z[ii][g][r] = z[ii][g][r] > 0.0f ? z[ii][g][r] : 0.0f;
+                    }
+#pragma unroll
+                    for (int ii = 0; ii < IP; ii++)
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            uint8_t* dst = stage + (32 * ii + lm) * ROWB + (32 * j + 8 * g + 4 * lh) * ES;
                             if constexpr (KIND == 0) {
-                                *reinterpret_cast<float4*>(dst) = make_float4(z[0], z[1], z[2], z[3]);
+                                *reinterpret_cast<float4*>(dst) =
+                                    make_float4(z[ii][g][0], z[ii][g][1], z[ii][g][2], z[ii][g][3]);
                             } else {
                                 // v_cvt_pk_bf16_f32: round to nearest even in hardware
-                                const bf16x4 pk = __builtin_convertvector((f32x4){z[0], z[1], z[2], z[3]}, bf16x4);
+                                const bf16x4 pk = __builtin_convertvector(
+                                    (f32x4){z[ii][g][0], z[ii][g][1], z[ii][g][2], z[ii][g][3]}, bf16x4);
                                 *reinterpret_cast<bf16x4*>(dst) = pk;
                             }
                         }
-                    }
                 }
                 asm volatile("" ::: "memory");
             }

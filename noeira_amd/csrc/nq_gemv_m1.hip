@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
 #pragma unroll
             for (int i = 0; i < CPL; i++) {
                 // Unconditional loads from clamped addresses: a lane whose chunk index runs past the
-                // row re-reads the last chunk, and its contribution vanishes because its x is zero.
+                // row re-reads the last chunk, and its partial product is dropped (one select per chunk).
                 // (A predicated load would become a branch around the load and serialise the batch.)
                 const int c = min(lj + i * lpr, p.nch - 1);
                 wv[r][i] = __builtin_nontemporal_load(&wq[row * p.nch + c]);
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     float xsum[CPL];
 #pragma unroll
     for (int i = 0; i < CPL; i++) {
-        // clamped, unconditional loads; a chunk past the end of the row gets x = 0 afterwards
+        // clamped, unconditional loads; the product of a chunk past the end of the row is dropped below
         const int64_t k0 = (int64_t)min(lj + i * lpr, p.nch - 1) * EPC;
         float s = 0.0f;
         if constexpr (DOT2) {
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
                 const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    xr[i][4 * v + e] = cval[i] ? t[e] : 0u;
+                    xr[i][4 * v + e] = t[e];
                     s += bf16lo(xr[i][4 * v + e]) + bf16hi(xr[i][4 * v + e]);
                 }
             }
@@ -202,9 +202,8 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
             }
 #pragma unroll
             for (int e = 0; e < EPC; e++) {
-                const float fv = cval[i] ? f[e] : 0.0f;
-                xr[i][e] = __float_as_uint(fv);
-                s += fv;
+                xr[i][e] = __float_as_uint(f[e]);
+                s += f[e];
             }
         }
         xsum[i] = s;
@@ -255,17 +254,18 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
                         }
                     }
                     const float zoff = DOT2 ? cz[r][i] + 16.0f : cz[r][i];
-                    acc[r] = fmaf(cs[r][i], fmaf(-zoff, xsum[i], dot), acc[r]);
+                    acc[r] += cval[i] ? cs[r][i] * fmaf(-zoff, xsum[i], dot) : 0.0f;
                 } else if constexpr (FMT == NQ_FMT_W8_CHANNEL) {
 #pragma unroll
                     for (int t = 0; t < 4; t++) {
-                        const uint32_t u = wv[r][i][t] ^ 0x80808080u;  // int8 + 128 as unsigned bytes
-                        dot = fmaf(XF(i, 4 * t + 0), (float)(u & 0xFFu), dot);
-                        dot = fmaf(XF(i, 4 * t + 1), (float)((u >> 8) & 0xFFu), dot);
-                        dot = fmaf(XF(i, 4 * t + 2), (float)((u >> 16) & 0xFFu), dot);
-                        dot = fmaf(XF(i, 4 * t + 3), (float)(u >> 24), dot);
+                        // sign-extending byte -> fp32 conversions (v_cvt_f32_i32 with a byte select)
+                        const uint32_t u = wv[r][i][t];
+                        dot = fmaf(XF(i, 4 * t + 0), (float)(int)(int8_t)(u & 0xFFu), dot);
+                        dot = fmaf(XF(i, 4 * t + 1), (float)(int)(int8_t)((u >> 8) & 0xFFu), dot);
+                        dot = fmaf(XF(i, 4 * t + 2), (float)(int)(int8_t)((u >> 16) & 0xFFu), dot);
+                        dot = fmaf(XF(i, 4 * t + 3), (float)((int)u >> 24), dot);
                     }
-                    acc[r] += fmaf(-128.0f, xsum[i], dot);
+                    acc[r] += cval[i] ? dot : 0.0f;
                 } else {
 #pragma unroll
                     for (int t = 0; t < 4; t++) {
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
                         dot = fmaf(XF(i, 4 * t + 2), b[0], dot);
                         dot = fmaf(XF(i, 4 * t + 3), b[1], dot);
                     }
-                    acc[r] += dot;
+                    acc[r] += cval[i] ? dot : 0.0f;
                 }
             }
         }
