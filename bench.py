@@ -41,6 +41,11 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_PEAK_TOPS = {"fp8": 5000.0, "int8": 5000.0, "bf16": 2500.0}
 SAMPLES, COLD_BYTES = 7, 512 << 20
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (fetched + written), scaled by
+# what the same counters read for a plain copy of known size; None until measured
+HEADLINE_TRAFFIC = 1791744      # mean of the two linears' launches (1.66 MB algorithmic)
+FP8_GEMV_TRAFFIC = 45199360     # K=4096, N=11008 (45.09 MB algorithmic)
+FP8_GEMM_TRAFFIC = 270030438    # M=8192, K=4096, N=4096 (117.4 MB algorithmic; the re-reads hit the Infinity Cache)
 
 
 def ensure_built():
@@ -344,8 +349,50 @@ def sweep(skip_large=False):
         c = max(1, COLD_BYTES // (N * 4096))
         run(f"cfg4 fp8 GEMV K=4096 N={N} M=1 (cold)", make_fp8, "hbm", M=1, N=N, copies=c, calls=max(c, 20))
         if not skip_large:
-            run(f"cfg4 fp8 GEMM M=8192 K=4096 N={N}", make_fp8, "mfma", "fp8", M=8192, N=N, copies=1, calls=3)
+            run(f"cfg4 fp8 GEMM M=8192 K=4096 N={N}", make_fp8, "mfma", "fp8", M=8192, N=N, copies=1, calls=10)
     return out
+
+
+def only_loop(which, steps, warmup):
+    """One kernel, launched call by call `steps` times after `warmup` untimed calls: the loop a
+    rocprofv3 run (kernel trace or one counter pass) is wrapped around."""
+    import torch
+
+    tm = Timer()
+    if which == "copy":
+        n = 256 << 20
+        src = torch.full((n,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        wl = dict(step=lambda i: dst.copy_(src), bytes=2 * n, ops=0, keep=(src, dst))
+        name = "plain device copy, 256 MiB read + 256 MiB written"
+    elif which == "fp8gemv":
+        N = 11008
+        c = max(1, COLD_BYTES // (N * 4096))
+        wl = make_fp8(1, N, copies=c)
+        name = f"cfg4 fp8 GEMV K=4096 N={N} M=1, cold rotation over {c} weight copies"
+    elif which == "mid":
+        wls = [make_act_w8a16(100, 1)]
+        wls += [make_w4g(K, N, 256, 1) for (K, N) in [(960, 960), (960, 2560), (2560, 960)]]
+        wls += [make_q4_0(K, N, 135, 1) for (K, N) in [(960, 960), (960, 320), (960, 2560), (2560, 960)]]
+
+        def step_all(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_all, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "configs 1 (M=100), 2 (M=256) and the reference's Q4_0 shapes at T=135, one call each per step"
+    elif which == "actor":
+        wl = make_actor_fused()
+        name = "cfg3 W8A8 actor 64->256->256->8 M=4096, fused"
+    else:
+        N = 4096
+        wl = make_fp8(8192, N)
+        name = f"cfg4 fp8 GEMM M=8192 K=4096 N={N}"
+    for i in range(warmup):
+        wl["step"](i)
+    sec = tm.run(wl["step"], steps) / steps
+    return {"only": which, "workload": name, "steps": steps, "us_per_call_eager": round(sec * 1e6, 3),
+            "algorithmic_bytes_per_call": wl["bytes"], "ops_per_call": wl["ops"]}
 
 
 def cpu_baseline(budget_s=12.0):
@@ -381,7 +428,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="time only the headline loop (for rocprofv3 runs)")
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy"],
+                    help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
+                         "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
+                         "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
+                         "copy = a plain 256 MiB device copy (the counter calibration kernel)")
+    ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     a = ap.parse_args()
@@ -394,6 +446,9 @@ def main():
     ensure_built()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy"):
+        print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
+        return
 
     per_pair = 2 * 512 * 3200
     copies = -(-COLD_BYTES // per_pair)
@@ -405,9 +460,12 @@ def main():
     # consecutive steps of the rotation (g = the largest divisor of steps that is <= the number
     # of weight copies), a.steps / g replays back to back, bracketed by synchronisations.
     g_steps = max(d for d in range(1, min(a.steps, copies) + 1) if a.steps % d == 0)
-    graph = capture(wl["step"], g_steps)
-    graph.replay()
-    sec = tm.run(lambda i: graph.replay(), a.steps // g_steps)
+    if a.only and a.eager:
+        sec = tm.run(wl["step"], a.steps)
+    else:
+        graph = capture(wl["step"], g_steps)
+        graph.replay()
+        sec = tm.run(lambda i: graph.replay(), a.steps // g_steps)
     ms_per_step = sec / a.steps * 1e3
     value = wl["bytes"] / (sec / a.steps) / 1e9
     launch_s = sec / (a.steps * wl["launches"])
@@ -434,7 +492,7 @@ def main():
         "warm": {"GBps": round(warm["bytes"] / warm_s / 1e9, 2), "us_per_step": round(warm_s * 1e6, 3),
                  "note": "one weight copy, resident in L2 / Infinity Cache (the reference's protocol)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 5), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 5), "traffic": HEADLINE_TRAFFIC,
                      "kernel": "nq::gemv_m1_kernel<W8_CHANNEL>", "avg_launch_us": round(launch_s * 1e6, 3),
                      "note": "1.66 MB per launch: at 8 TB/s the transfer is 0.21 us, less than the 1.4 us an "
                              "empty kernel takes on this GPU, so this workload is launch-latency-bound; the "
@@ -447,10 +505,17 @@ def main():
         line["results"] = sweep()
         mf = [r for r in line["results"] if "fp8 GEMM" in r["workload"]]
         if mf:
-            best = max(mf, key=lambda r: r["TOPS"])
+            best = next((r for r in mf if "N=4096" in r["workload"]), mf[0])  # the shape the traffic figure is for
             line["roofline_mfma"] = {"bound": "mfma", "achieved": best["TOPS"], "peak": MFMA_PEAK_TOPS["fp8"],
                                      "unit": "TFLOP/s", "frac": round(best["TOPS"] / MFMA_PEAK_TOPS["fp8"], 5),
+                                     "traffic": FP8_GEMM_TRAFFIC, "kernel": "nq::gemm8_kernel<fp8>",
                                      "workload": best["workload"]}
+        gv = [r for r in line["results"] if "fp8 GEMV" in r["workload"]]
+        if gv:
+            best = max(gv, key=lambda r: r["GBps"])
+            line["roofline_gemv"] = {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                     "frac": round(best["GBps"] / HBM_PEAK_GBPS, 5), "traffic": FP8_GEMV_TRAFFIC,
+                                     "kernel": "nq::gemv_fp8_row_kernel", "workload": best["workload"]}
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))
