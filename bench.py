@@ -179,6 +179,37 @@ def make_q4_0(IN, OUT, M, copies, seed=3):
                 keep=(layers, x, y))
 
 
+def make_q4_0_fused(IN, OUTS, M, copies, seed=7):
+    """The reference caller's q|k|v or gate|up projections as one row-fused launch."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import FusedRows, QLinear
+
+    rng = np.random.default_rng(seed)
+    fused = []
+    for _ in range(copies):
+        parts = []
+        for OUT in OUTS:
+            nb = OUT * (IN // 32) * 18
+            blocks = rng.integers(0, 256, nb, dtype=np.uint8)
+            sc = rng.uniform(1e-3, 2e-3, OUT * (IN // 32)).astype(np.float16).view(np.uint8).reshape(-1, 2)
+            blocks.reshape(-1, 18)[:, 0:2] = sc
+            ql = QLinear.make(IN, OUT, "gpu")
+            ql.set_blocks(blocks)
+            parts.append(ql)
+        fused.append(FusedRows(parts))  # the parts are copied; they are freed here
+    x = torch.from_numpy(rng.standard_normal((M, IN)).astype(np.float32)).cuda()
+    ys = [torch.empty((M, OUT), dtype=torch.float32, device="cuda") for OUT in OUTS]
+    tot = sum(OUTS)
+
+    def step(i):
+        fused[i % copies].forward(x, outs=ys)
+
+    return dict(step=step, bytes=tot * (IN // 32) * 18 + 4 * IN * M + 4 * tot * M, ops=2 * M * IN * tot, launches=1,
+                keep=(fused, x, ys))
+
+
 def make_w4g(K, N, M, copies, seed=4):
     """configs[2]: asymmetric uint4, group 128, fp16 scales, bf16 activations."""
     import numpy as np
@@ -343,6 +374,12 @@ def sweep(skip_large=False):
         run(f"ref Q4_0 g32 {IN}->{OUT} M=1 fp32 (cold)", make_q4_0, "hbm", IN=IN, OUT=OUT, M=1, copies=c, calls=c)
         run(f"ref Q4_0 g32 {IN}->{OUT} M=135 fp32 (warm)", make_q4_0, "mfma", "bf16", IN=IN, OUT=OUT, M=135,
             copies=1, calls=20)
+    for (name, OUTS) in [("q|k|v 960->960|320|320", [960, 320, 320]), ("gate|up 960->2560|2560", [2560, 2560])]:
+        c = max(1, COLD_BYTES // (sum(OUTS) * 960 * 9 // 16))
+        run(f"ref Q4_0 {name} row-fused M=1 fp32 (cold)", make_q4_0_fused, "hbm", IN=960, OUTS=OUTS, M=1, copies=c,
+            calls=c)
+        run(f"ref Q4_0 {name} row-fused M=135 fp32 (warm)", make_q4_0_fused, "mfma", "bf16", IN=960, OUTS=OUTS,
+            M=135, copies=1, calls=20)
     run("cfg3 W8A8 actor 64->256->256->8 M=4096 (fused, 1 launch)", make_actor_fused, "mfma", "int8", calls=20)
     run("cfg3 W8A8 actor 64->256->256->8 M=4096 (unfused, 6 launches)", make_actor_w8a8, "mfma", "int8", calls=20)
     for N in (4096, 11008):

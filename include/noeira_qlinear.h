@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define NQ_ABI_VERSION 1
+#define NQ_ABI_VERSION 2
 
 /* status codes */
 #define NQ_OK 0
@@ -142,6 +142,33 @@ int32_t nq_keep_only_repacked(nq_handle h);
 int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
                    int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype,
                    int32_t epilogue, void* stream);
+
+/* One layer made of the rows of up to four loaded layers that share their
+ * input (same format, IN, group width; FP8_E4M3: same scale), e.g. q|k|v or
+ * gate|up of a decoder layer: the seven projections the reference's caller
+ * launches one by one (`DecoderLayerWeights.proj_fwd`,
+ * noeira/deep_agents/smolvla/layer_weights.mojo:455-508, called from
+ * fused.mojo:287-363) read the same activations three and two at a time.  The
+ * weights are copied on the device ([OUT, IN] rows are independent, groups
+ * never span rows), so the sources may be destroyed afterwards.  The result
+ * is an ordinary layer (nq_forward writes one [M, sum OUT] y) that also
+ * remembers its parts for nq_forward_fused. */
+int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* stream);
+
+/* Number of parts of a layer made by nq_fuse_rows (1 for any other layer). */
+int32_t nq_fused_parts(nq_handle h);
+
+/* nq_forward of a fused layer with one dense output per part:
+ * ys[t] is [M, OUT_t], what nq_forward of part t alone would write: a row's
+ * arithmetic does not depend on its neighbours (bit for bit at M >= 5; at
+ * M = 1 the number of lanes that share a row, hence the order of its sum, may
+ * follow the total row count).
+ * n_ys must equal nq_fused_parts(h).  bias, if any, is [sum OUT].  One launch
+ * where the kernel for the shape can place rows by part (bf16/fp32
+ * activations at M = 1 and M >= 5), otherwise one launch per part. */
+int32_t nq_forward_fused(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale,
+                         void* const* ys, int32_t n_ys, int32_t y_dtype, int32_t M, const void* bias,
+                         int32_t bias_dtype, int32_t epilogue, void* stream);
 
 /* The device twin of `dequantize_q4_0` (`dequant_q4_0_kernel`,
  * q4_0.mojo:242-266; `QLinear.dequantized`, qlinear.mojo:326-328): deq(W)

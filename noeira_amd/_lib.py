@@ -18,13 +18,14 @@ NQ_OK, NQ_ERR_INVALID, NQ_ERR_NOT_LOADED, NQ_ERR_NO_BLOCKS, NQ_ERR_SIZE, NQ_ERR_
 FMT_Q4_0, FMT_W8_CHANNEL, FMT_W4_GROUP, FMT_FP8_E4M3 = range(4)
 DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
 EPI_NONE, EPI_RELU = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EXPORTS = [
     "nq_abi_version", "nq_last_error", "nq_create", "nq_destroy", "nq_set_blocks", "nq_set_weight_f32",
     "nq_set_weight_i8", "nq_set_weight_w4g", "nq_set_weight_fp8", "nq_blocks_bytes", "nq_get_blocks",
     "nq_keep_only_repacked", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
-    "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward",
+    "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward", "nq_fuse_rows", "nq_fused_parts",
+    "nq_forward_fused",
 ]
 
 
@@ -112,6 +113,12 @@ def lib() -> C.CDLL:
     L.nq_slice_cast_f32.argtypes = [p, p, i32, i32, i32, p]
     L.nq_mlp3_w8a8_forward.restype = i32
     L.nq_mlp3_w8a8_forward.argtypes = [p, p, p, p, p, i32, p, p, p, i32, p]
+    L.nq_fuse_rows.restype = i32
+    L.nq_fuse_rows.argtypes = [C.POINTER(p), C.POINTER(p), i32, p]
+    L.nq_fused_parts.restype = i32
+    L.nq_fused_parts.argtypes = [p]
+    L.nq_forward_fused.restype = i32
+    L.nq_forward_fused.argtypes = [p, p, i32, p, C.POINTER(p), i32, i32, i32, p, i32, i32, p]
     got = L.nq_abi_version()
     if got != ABI_VERSION:
         raise OSError(f"{LIB_NAME}: ABI version {got}, this package binds version {ABI_VERSION}")

@@ -332,21 +332,56 @@ int32_t nq_keep_only_repacked(nq_handle h) {
     return NQ_OK;
 }
 
-int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y, int32_t y_dtype,
-                   int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue, void* stream) {
-    int32_t rc = check_handle(h, "nq_forward");
-    if (rc) return rc;
-    if ((rc = need_loaded(h, "forward"))) return rc;
-    if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward: M must be >= 0");
-    if (M == 0) return NQ_OK;
-    if (!x || !y) return fail(NQ_ERR_INVALID, "nq_forward: null x or y");
-    if (((uintptr_t)x & 15) || ((uintptr_t)y & 3))
-        return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
+namespace {
+
+// a view of rows [r0, r1) of a loaded layer (no ownership; for per-part launches)
+void row_view(const nq_layer* L, int r0, int r1, nq_layer* v) {
+    v->format = L->format, v->in = L->in, v->out = r1 - r0, v->group = L->group, v->groups = L->groups;
+    v->loaded = true, v->has_host_blocks = false, v->device = L->device;
+    v->scale = L->scale, v->row_bytes = L->row_bytes;
+    v->d_codes = L->d_codes + (int64_t)r0 * L->row_bytes;
+    v->d_zps = L->d_zps ? L->d_zps + (int64_t)r0 * L->groups : nullptr;
+    int64_t srow = 0;  // bytes of scale data per row
+    switch (L->format) {
+        case NQ_FMT_Q4_0: srow = (int64_t)(L->in / Q4_GROUP) * 2; break;
+        case NQ_FMT_W4_GROUP: srow = (int64_t)L->groups * 2; break;
+        case NQ_FMT_W8_CHANNEL: srow = 4; break;
+        default: srow = 0;
+    }
+    v->d_scales = L->d_scales ? reinterpret_cast<uint8_t*>(L->d_scales) + r0 * srow : nullptr;
+}
+
+int32_t dispatch(const ForwardArgs& a) {
+    if (a.x_dtype == NQ_DT_I8) {
+        if (gemm8_applicable(a)) return launch_gemm8(a);
+        return launch_gemv_i8(a);
+    }
+    if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
+    if (gemm8_applicable(a)) return launch_gemm8(a);
+    if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
+    if (gemv_m1_applicable(a)) return launch_gemv_m1(a);
+    return launch_gemv(a);
+}
+
+// the kernels that place rows through the part table themselves (one launch for all parts)
+bool places_parts(const ForwardArgs& a) {
+    if (a.x_dtype == NQ_DT_I8) return false;
+    if (gemv_fp8_applicable(a) || gemm8_applicable(a)) return false;
+    return gemm_a16_applicable(a) || gemv_m1_applicable(a);
+}
+
+// argument checks shared by nq_forward and nq_forward_fused, then the launch(es)
+int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, const SegTable& seg,
+                     int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue,
+                     void* stream) {
+    if (((uintptr_t)x & 15)) return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
+    for (int t = 0; t < seg.nseg; t++)
+        if (!seg.y[t] || ((uintptr_t)seg.y[t] & 3))
+            return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
     if (epilogue != NQ_EPI_NONE && epilogue != NQ_EPI_RELU)
         return fail(NQ_ERR_INVALID, "nq_forward: unknown epilogue " + std::to_string(epilogue));
     if (bias && bias_dtype != NQ_DT_F32 && bias_dtype != NQ_DT_BF16)
         return fail(NQ_ERR_INVALID, "nq_forward: bias must be fp32 or bf16");
-    ForwardArgs a{h, x, x_dtype, x_scale, y, y_dtype, M, bias, bias_dtype, epilogue, (hipStream_t)stream};
     if (x_dtype == NQ_DT_I8) {
         if (h->format != NQ_FMT_W8_CHANNEL)
             return fail(NQ_ERR_INVALID, "nq_forward: int8 activations need a W8_CHANNEL layer");
@@ -358,23 +393,151 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
                 return fail(NQ_ERR_INVALID, "nq_forward: y must be fp32, bf16 or int32");
             if (!x_scale) return fail(NQ_ERR_INVALID, "nq_forward: int8 activations need per-row scales");
         }
-        if (gemm8_applicable(a)) return launch_gemm8(a);
-        return launch_gemv_i8(a);
+    } else {
+        if (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16)
+            return fail(NQ_ERR_INVALID, "nq_forward: y must be fp32 or bf16");
+        if (x_dtype == NQ_DT_FP8_E4M3) {
+            if (h->format != NQ_FMT_FP8_E4M3)
+                return fail(NQ_ERR_INVALID, "nq_forward: fp8 activations need an FP8_E4M3 layer");
+            if (!x_scale) return fail(NQ_ERR_INVALID, "nq_forward: fp8 activations need a scale");
+        } else if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16) {
+            return fail(NQ_ERR_INVALID, "nq_forward: unknown x dtype " + std::to_string(x_dtype));
+        }
     }
-    if (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16)
-        return fail(NQ_ERR_INVALID, "nq_forward: y must be fp32 or bf16");
-    if (x_dtype == NQ_DT_FP8_E4M3) {
-        if (h->format != NQ_FMT_FP8_E4M3)
-            return fail(NQ_ERR_INVALID, "nq_forward: fp8 activations need an FP8_E4M3 layer");
-        if (!x_scale) return fail(NQ_ERR_INVALID, "nq_forward: fp8 activations need a scale");
-    } else if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16) {
-        return fail(NQ_ERR_INVALID, "nq_forward: unknown x dtype " + std::to_string(x_dtype));
+    ForwardArgs a{h, x, x_dtype, x_scale, seg.y[0], y_dtype, M, bias, bias_dtype, epilogue, (hipStream_t)stream, seg};
+    if (seg.nseg == 1 || places_parts(a)) return dispatch(a);
+    // one launch per part, each on a view of its rows
+    const int bias_es = bias_dtype == NQ_DT_F32 ? 4 : 2;
+    int r0 = 0;
+    for (int t = 0; t < seg.nseg; t++) {
+        nq_layer view;
+        row_view(h, r0, seg.end[t], &view);
+        ForwardArgs v = a;
+        v.L = &view, v.y = seg.y[t];
+        v.bias = bias ? reinterpret_cast<const uint8_t*>(bias) + (int64_t)r0 * bias_es : nullptr;
+        v.seg.nseg = 1, v.seg.end[0] = view.out, v.seg.y[0] = seg.y[t];
+        const int32_t rc = dispatch(v);
+        if (rc) return rc;
+        r0 = seg.end[t];
     }
-    if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
-    if (gemm8_applicable(a)) return launch_gemm8(a);
-    if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
-    if (gemv_m1_applicable(a)) return launch_gemv_m1(a);
-    return launch_gemv(a);
+    return NQ_OK;
+}
+
+}  // namespace
+
+int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y, int32_t y_dtype,
+                   int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue, void* stream) {
+    int32_t rc = check_handle(h, "nq_forward");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!x || !y) return fail(NQ_ERR_INVALID, "nq_forward: null x or y");
+    SegTable seg{};
+    seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
+    return forward_impl(h, x, x_dtype, x_scale, seg, y_dtype, M, bias, bias_dtype, epilogue, stream);
+}
+
+int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* stream) {
+    if (!out) return fail(NQ_ERR_INVALID, "nq_fuse_rows: null output handle");
+    *out = nullptr;
+    if (!layers || n < 1 || n > 4) return fail(NQ_ERR_INVALID, "nq_fuse_rows: between 1 and 4 layers can be fused");
+    int64_t rows = 0;
+    for (int i = 0; i < n; i++) {
+        int32_t rc = check_handle(layers[i], "nq_fuse_rows");
+        if (rc) return rc;
+        if ((rc = need_loaded(layers[i], "fuse_rows"))) return rc;
+        const nq_layer* a = layers[0];
+        const nq_layer* b = layers[i];
+        if (b->format != a->format || b->in != a->in || b->group != a->group || b->device != a->device)
+            return fail(NQ_ERR_INVALID, "nq_fuse_rows: the layers must share format, IN, group width and device");
+        if (a->format == NQ_FMT_FP8_E4M3 && b->scale != a->scale)
+            return fail(NQ_ERR_INVALID, "nq_fuse_rows: FP8_E4M3 layers must share their per-tensor scale");
+        if (!b->seg_end.empty()) return fail(NQ_ERR_INVALID, "nq_fuse_rows: a fused layer cannot be fused again");
+        rows += b->out;
+    }
+    if (rows > INT32_MAX) return fail(NQ_ERR_INVALID, "nq_fuse_rows: too many rows");
+    const nq_layer* a = layers[0];
+    nq_layer* F = new (std::nothrow) nq_layer();
+    if (!F) return fail(NQ_ERR_INVALID, "nq_fuse_rows: out of host memory");
+    F->format = a->format, F->in = a->in, F->out = (int32_t)rows, F->group = a->group, F->groups = a->groups;
+    F->scale = a->scale, F->row_bytes = a->row_bytes, F->device = a->device;
+    int32_t rc = bind_device(F);
+    if (rc) {
+        delete F;
+        return rc;
+    }
+    int64_t scale_row = 0;
+    switch (a->format) {
+        case NQ_FMT_Q4_0: scale_row = (int64_t)(a->in / Q4_GROUP) * 2; break;
+        case NQ_FMT_W4_GROUP: scale_row = (int64_t)a->groups * 2; break;
+        case NQ_FMT_W8_CHANNEL: scale_row = 4; break;
+        default: scale_row = 0;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e = hipMalloc((void**)&F->d_codes, (size_t)(rows * F->row_bytes) + 128);
+    if (e == hipSuccess && scale_row) e = hipMalloc(&F->d_scales, (size_t)(rows * scale_row) + 128);
+    if (e == hipSuccess && a->d_zps) e = hipMalloc((void**)&F->d_zps, (size_t)(rows * F->groups) + 128);
+    int64_t r0 = 0;
+    bool all_blocks = true;
+    for (int i = 0; i < n && e == hipSuccess; i++) {
+        const nq_layer* b = layers[i];
+        e = hipMemcpyAsync(F->d_codes + r0 * F->row_bytes, b->d_codes, (size_t)(b->out * F->row_bytes),
+                           hipMemcpyDeviceToDevice, s);
+        if (e == hipSuccess && scale_row)
+            e = hipMemcpyAsync(reinterpret_cast<uint8_t*>(F->d_scales) + r0 * scale_row, b->d_scales,
+                               (size_t)(b->out * scale_row), hipMemcpyDeviceToDevice, s);
+        if (e == hipSuccess && a->d_zps)
+            e = hipMemcpyAsync(F->d_zps + r0 * F->groups, b->d_zps, (size_t)((int64_t)b->out * F->groups),
+                               hipMemcpyDeviceToDevice, s);
+        r0 += b->out;
+        F->seg_end.push_back((int32_t)r0);
+        all_blocks = all_blocks && b->has_host_blocks;
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) {
+        free_device(F);
+        delete F;
+        return fail_hip(e, "nq_fuse_rows");
+    }
+    // the logical bytes are row-major over OUT in every format, so the fused layer's are the
+    // concatenation (W4_GROUP's logical form is three arrays: not kept)
+    if (all_blocks && a->format != NQ_FMT_W4_GROUP) {
+        for (int i = 0; i < n; i++)
+            F->host_blocks.insert(F->host_blocks.end(), layers[i]->host_blocks.begin(), layers[i]->host_blocks.end());
+        F->has_host_blocks = true;
+    }
+    F->loaded = true;
+    *out = F;
+    return NQ_OK;
+}
+
+int32_t nq_fused_parts(nq_handle h) {
+    if (!h) return 0;
+    return h->seg_end.empty() ? 1 : (int32_t)h->seg_end.size();
+}
+
+int32_t nq_forward_fused(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* const* ys,
+                         int32_t n_ys, int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype,
+                         int32_t epilogue, void* stream) {
+    int32_t rc = check_handle(h, "nq_forward_fused");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    const int parts = nq_fused_parts(h);
+    if (n_ys != parts)
+        return fail(NQ_ERR_INVALID, "nq_forward_fused: " + std::to_string(n_ys) + " outputs for a layer of " +
+                                        std::to_string(parts) + " fused parts");
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!x || !ys) return fail(NQ_ERR_INVALID, "nq_forward: null x or y");
+    SegTable seg{};
+    seg.nseg = parts;
+    for (int t = 0; t < parts; t++) {
+        seg.end[t] = h->seg_end.empty() ? h->out : h->seg_end[t];
+        seg.y[t] = ys[t];
+        if (!ys[t]) return fail(NQ_ERR_INVALID, "nq_forward: null x or y");
+    }
+    return forward_impl(h, x, x_dtype, x_scale, seg, y_dtype, M, bias, bias_dtype, epilogue, stream);
 }
 
 int32_t nq_dequantize(nq_handle h, float* out_dev, int64_t n_values, void* stream) {

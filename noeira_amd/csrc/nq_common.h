@@ -51,9 +51,27 @@ struct nq_layer {
     uint8_t* d_zps = nullptr;
     float scale = 1.0f;
     int64_t row_bytes = 0;     // bytes of one row of d_codes
+    std::vector<int32_t> seg_end;  // a row-fused layer: the end row of each fused part (else empty)
 };
 
 namespace nq {
+
+// Where the rows of a launch go: part t covers rows [end[t-1], end[t]) and is written dense to
+// y[t] as [M, end[t] - end[t-1]].  An ordinary layer is one part.
+struct SegTable {
+    int32_t nseg;
+    int32_t end[4];
+    void* y[4];
+};
+
+// row n -> (part's y, its width, the column in it)
+__device__ __forceinline__ void seg_lookup(const SegTable& sg, int n, void*& y, int& width, int& col) {
+    int s = 0, base = 0;
+#pragma unroll
+    for (int t = 0; t < 3; t++)
+        if (t + 1 < sg.nseg && n >= sg.end[t]) s = t + 1, base = sg.end[t];
+    y = sg.y[s], width = sg.end[s] - base, col = n - base;
+}
 
 struct ForwardArgs {
     const nq_layer* L;
@@ -67,6 +85,7 @@ struct ForwardArgs {
     int32_t bias_dtype;
     int32_t epilogue;
     hipStream_t stream;
+    SegTable seg;  // seg.y[0] == y and seg.end[0] == OUT for an ordinary call
 };
 
 // nq_q4_0.hip

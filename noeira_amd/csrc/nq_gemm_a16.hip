@@ -57,6 +57,7 @@ struct A16Params {
     int32_t s_pairs;  // Q4_0: scale rows are 4-byte (1) or 8-byte (2) aligned, else 0
     int32_t nch;      // 16-byte chunks per weight row
     int32_t y_dtype, bias_dtype, epilogue;
+    SegTable seg;
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
@@ -435,11 +436,14 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         z += ep_bias[t];
         if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
         if (n < p.N && m < p.M) {
-            const int64_t o = (int64_t)m * p.N + n;
+            void* yp;
+            int width, col;
+            seg_lookup(p.seg, n, yp, width, col);
+            const int64_t o = (int64_t)m * width + col;
             if (p.y_dtype == NQ_DT_F32)
-                reinterpret_cast<float*>(p.y)[o] = z;
+                reinterpret_cast<float*>(yp)[o] = z;
             else
-                reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(z);
+                reinterpret_cast<uint16_t*>(yp)[o] = f32_to_bf16_rne(z);
         }
     }
 }
@@ -490,7 +494,7 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     const bool xf32 = a.x_dtype == NQ_DT_F32;
     A16Params p{};
     p.codes = L->d_codes, p.scales = L->d_scales, p.zps = L->d_zps;
-    p.x = a.x, p.y = a.y, p.bias = a.bias;
+    p.x = a.x, p.y = a.y, p.bias = a.bias, p.seg = a.seg;
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.groups = L->groups;
     p.inv_cpg = L->group ? 32.0f / (float)L->group : 1.0f;

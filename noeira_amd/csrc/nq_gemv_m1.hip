@@ -51,6 +51,7 @@ struct M1Params {
     int32_t lpr_log2;
     int32_t rpw;   // rows per lane group (a multiple of RPL)
     int32_t x_dtype, y_dtype, bias_dtype, epilogue;
+    SegTable seg;
 };
 
 __device__ __forceinline__ float bf16lo(uint32_t pair) { return __uint_as_float(pair << 16); }
@@ -294,10 +295,13 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
                 if (FMT == NQ_FMT_FP8_E4M3) z *= tscale;
                 z += rbias[r];
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                void* yp;
+                int width, col;
+                seg_lookup(p.seg, (int)n, yp, width, col);  // M = 1: the part's row is its only row
                 if (p.y_dtype == NQ_DT_F32)
-                    reinterpret_cast<float*>(p.y)[n] = z;
+                    reinterpret_cast<float*>(yp)[col] = z;
                 else
-                    reinterpret_cast<uint16_t*>(p.y)[n] = to_bf16(z);
+                    reinterpret_cast<uint16_t*>(yp)[col] = to_bf16(z);
             }
         }
         if (rb + RPL < p.rpw) {
@@ -391,7 +395,7 @@ int32_t launch_gemv_m1(const ForwardArgs& a) {
     const bool dot2 = four_bit && a.x_dtype == NQ_DT_BF16;
     M1Params p{};
     p.codes = L->d_codes, p.scales = L->d_scales, p.zps = L->d_zps;
-    p.x = a.x, p.x_scale = a.x_scale, p.y = a.y, p.bias = a.bias;
+    p.x = a.x, p.x_scale = a.x_scale, p.y = a.y, p.bias = a.bias, p.seg = a.seg;
     p.N = L->out, p.K = L->in, p.group = L->group, p.groups = L->groups, p.tscale = L->scale;
     p.nch = L->in / (four_bit ? 32 : 16);
     p.x_dtype = a.x_dtype, p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;

@@ -277,6 +277,65 @@ class FP8Linear(_Layer):
         return self._forward(x_codes, L.DT_FP8_E4M3, x_scale, out, out_dtype, bias, epilogue, "FP8Linear.forward")
 
 
+class FusedRows:
+    """Up to four loaded layers that read the same activations (q|k|v, gate|up
+    of a decoder layer: `DecoderLayerWeights.proj_fwd`, layer_weights.mojo:455-508)
+    as ONE layer: their [OUT, IN] rows are concatenated on the device and
+    `forward` writes one dense [M, OUT_t] output per part, what each part's own
+    forward writes, in one launch where the kernel allows it."""
+
+    def __init__(self, layers):
+        layers = list(layers)
+        arr = (C.c_void_p * len(layers))(*[l._h for l in layers])
+        h = C.c_void_p()
+        L.check(L.lib().nq_fuse_rows(C.byref(h), arr, len(layers), _stream_ptr()))
+        self._h = h
+        self.IN = layers[0].IN
+        self.OUTS = [l.OUT for l in layers]
+        self.OUT = sum(self.OUTS)
+        self._kind = type(layers[0])
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h is not None and h.value:
+            try:
+                L.lib().nq_destroy(h)
+            except Exception:
+                pass
+            self._h = None
+
+    def parts(self) -> int:
+        return int(L.lib().nq_fused_parts(self._h))
+
+    def forward(self, x: torch.Tensor, x_scale: Optional[torch.Tensor] = None, outs=None, bias=None,
+                epilogue: str = "none", out_dtype: torch.dtype = torch.float32):
+        """Returns the list of per-part outputs.  x: fp32/bf16 [M, IN], or e4m3fn
+        codes with `x_scale` for fused FP8Linear layers."""
+        if x.dtype == torch.float8_e4m3fn:
+            x = x.view(torch.uint8)
+        if x.dtype == torch.uint8:
+            x_dt = L.DT_FP8_E4M3
+        elif x.dtype in _TORCH_DT:
+            x_dt = _TORCH_DT[x.dtype]
+        else:
+            raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward: x must be fp32, bf16 or e4m3fn codes")
+        M = _check_x(x, self.IN, "FusedRows.forward")
+        if outs is None:
+            outs = [torch.empty((M, n), dtype=out_dtype, device=x.device) for n in self.OUTS]
+        y_dt = {torch.float32: L.DT_F32, torch.bfloat16: L.DT_BF16}[out_dtype]
+        b_dt = L.DT_F32
+        if bias is not None:
+            if bias.dtype not in _TORCH_DT or bias.numel() != self.OUT or not bias.is_cuda:
+                raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward: bias must be a device fp32/bf16 tensor of "
+                                                  "sum(OUT) values")
+            b_dt = _TORCH_DT[bias.dtype]
+        epi = {"none": L.EPI_NONE, "relu": L.EPI_RELU}[epilogue]
+        ys = (C.c_void_p * len(outs))(*[_dev_ptr(o) for o in outs])
+        L.check(L.lib().nq_forward_fused(self._h, _dev_ptr(x), x_dt, _dev_ptr(x_scale), ys, len(outs), y_dt, M,
+                                         _dev_ptr(bias), b_dt, epi, _stream_ptr()))
+        return outs
+
+
 def quantize_rows_i8(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None):
     """Per-token absmax int8 quantisation on the device: (q int8 [M, K], s fp32 [M])."""
     if x.dtype not in _TORCH_DT or x.dim() != 2 or not x.is_contiguous():
