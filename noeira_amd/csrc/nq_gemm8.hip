@@ -15,9 +15,14 @@
 //
 // K loop.  Stages of BK = 128 bytes: x tile 256 x 128 B and w tile 256 x 128 B
 // (64 KiB), double-buffered in LDS (128 of the CU's 160 KiB).  While a stage is
-// being multiplied, the next stage streams from global memory straight into the
-// other LDS buffer (global_load_lds_dwordx4, 16 per lane per stage): no
-// registers, no ds_write, one wait + one barrier per stage.
+// being multiplied, the stage after next streams from global memory straight
+// into the buffer the previous stage has just freed (global_load_lds_dwordx4, 16
+// per lane per stage): no registers, no ds_write, one wait + one barrier per
+// stage.  What bounds the loop, measured on this GPU with parts of it switched
+// off: the MFMAs alone need 2048 cycles per stage, the transfers alone (64 KiB
+// per CU per stage from L2, ~15 TB/s chip-wide) ~2250 cycles, the LDS fragment
+// reads and their waits nothing (the LDS sustains > 500 B/clk per CU); together
+// the stage takes ~2600 cycles.
 //
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= (row >> 1) & 7.  Rows r and r + 1 then sit 128 B apart in
@@ -52,8 +57,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 
-constexpr int BM = 256, BN = 256, BK = 128;
-constexpr int STAGE_BYTES = (BM + BN) * BK;  // 64 KiB
+constexpr int BM = 256;  // rows of x per workgroup tile (2 wavefronts x 128)
 
 struct Gemm8Params {
     const uint8_t* a;  // x [M][K]
@@ -74,16 +78,20 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float v) {
     return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
 }
 
-__device__ __forceinline__ int lds_off(int row, int slot) {
-    return row * BK + ((slot ^ ((row >> 1) & 7)) << 4);
-}
-
-template <bool FP8>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void gemm8_kernel(const Gemm8Params p) {
+// BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with
+// BK = 128 (a 256 x 128, BK = 64 variant with two workgroups per CU measured slower: its stage is
+// too short for a transfer to land in).
+template <bool FP8, int BN, int BK>
+__device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
+    constexpr int STAGE_BYTES = (BM + BN) * BK;
+    constexpr int SLOTS = BK / 16;     // 16-byte slots per LDS row
+    constexpr int SWZ = SLOTS - 1;     // slot ^= (row >> 1) & SWZ
+    constexpr int WN = BN / 2;         // channels per wavefront
+    constexpr int TJ = WN / 32;        // weight fragments (MFMA tiles along N) per wavefront
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
     const int wm = wave >> 1, wn = wave & 1;
 
     // ---- XCD-aware tile assignment
@@ -102,36 +110,62 @@ void gemm8_kernel(const Gemm8Params p) {
     const int m0 = tm * BM, n0 = tn * BN;
 
     // ---- global -> LDS, direct (global_load_lds_dwordx4): no register round trip.  One
-    // instruction fills 1 KiB of LDS, lane l at byte 16 l, i.e. 8 rows of 128 B; wavefront w owns
-    // rows [64 w, 64 w + 64) of both tiles.  The slot swizzle is applied on the global side: the
-    // lane that lands in physical slot l % 8 of its row fetches logical slot (l % 8) ^ swz(row).
+    // instruction fills 1 KiB of LDS, lane l at byte 16 l, i.e. 1024 / BK rows; wavefront w owns
+    // a quarter of the rows of both tiles.  The slot swizzle is applied on the global side: the
+    // lane that lands in physical slot s of its row fetches logical slot s ^ swz(row).
     typedef __attribute__((address_space(1))) const void gptr_t;
     typedef __attribute__((address_space(3))) void lptr_t;
-    const uint8_t* da[8];
-    const uint8_t* db[8];
+    constexpr int DROWS = 1024 / BK;           // rows per instruction
+    constexpr int DA = BM / 4 / DROWS;         // instructions per wavefront and stage, x tile
+    constexpr int DB = BN / 4 / DROWS;         // ... w tile
+    // addresses as a uniform 64-bit tile base (advanced by k0) plus a 32-bit per-lane offset, and
+    // the LDS destination as a scalar: two instructions per transfer (set M0, issue)
+    const uint8_t* const abase = p.a + (int64_t)m0 * p.K;
+    const uint8_t* const bbase = p.b + (int64_t)n0 * p.K;
+    uint32_t doff[DA + DB];
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
-        const int row = wave * 64 + t * 8 + (lane >> 3);
-        const int slot = (lane & 7) ^ ((row >> 1) & 7);
-        da[t] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.K + slot * 16;
-        db[t] = p.b + (int64_t)min(n0 + row, p.N - 1) * p.K + slot * 16;
+    for (int t = 0; t < DA; t++) {
+        const int row = wave * (BM / 4) + t * DROWS + lane / SLOTS;
+        const int slot = (lane % SLOTS) ^ ((row >> 1) & SWZ);
+        doff[t] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.K + slot * 16;
     }
-    auto dma = [&](int k0, int buf) {
-        uint8_t* base = lds + buf * STAGE_BYTES + wave * 64 * BK;
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
-            __builtin_amdgcn_global_load_lds((gptr_t*)(da[t] + k0), (lptr_t*)(base + t * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t*)(db[t] + k0), (lptr_t*)(base + BM * BK + t * 1024), 16, 0, 0);
-        }
-    };
+    for (int t = 0; t < DB; t++) {
+        const int row = wave * (BN / 4) + t * DROWS + lane / SLOTS;
+        const int slot = (lane % SLOTS) ^ ((row >> 1) & SWZ);
+        doff[DA + t] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.K + slot * 16;
+    }
+    // transfer t (0 .. DA+DB-1) of a stage: M0 = the LDS address of the 1 KiB the instruction
+    // fills (a scalar base of the buffer half plus t KiB), global address = scalar base + lane
+    // offset.  Three instructions per transfer.
+    const uint32_t lds_addr0 = (uint32_t)(uintptr_t)(lptr_t*)lds;
+    uint32_t dbase[2][2];  // [buffer][x tile, w tile]: this wavefront's first destination
+#pragma unroll
+    for (int buf = 0; buf < 2; buf++) {
+        dbase[buf][0] = lds_addr0 + buf * STAGE_BYTES + wave * (BM / 4) * BK;
+        dbase[buf][1] = lds_addr0 + buf * STAGE_BYTES + BM * BK + wave * (BN / 4) * BK;
+    }
+#define NQ_DMA(t, buf, srca, srcb)                                                                     \
+    do {                                                                                               \
+        if constexpr ((t) < DA)                                                                        \
+            asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"           \
+                         :                                                                             \
+                         : "s"(dbase[buf][0]), "v"(doff[(t)]), "s"(srca), "n"((t) * 1024)              \
+                         : "memory", "m0");                                                            \
+        else                                                                                           \
+            asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"           \
+                         :                                                                             \
+                         : "s"(dbase[buf][1]), "v"(doff[(t)]), "s"(srcb), "n"(((t) - DA) * 1024)       \
+                         : "memory", "m0");                                                            \
+    } while (0)
     const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;  // requested now, used in the epilogue
 
     typedef typename std::conditional<FP8, f32x16, i32x16>::type acc_t;
-    acc_t acc[4][4];
+    acc_t acc[4][TJ];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
@@ -141,95 +175,225 @@ void gemm8_kernel(const Gemm8Params p) {
     // term depends on the row within the tile only.
     const int frow = lane & 31;
     const int fh = lane >> 5;
-    const int fsw = (frow >> 1) & 7;
+    const int fsw = (frow >> 1) & SWZ;
 
-    // ---- main loop, software-pipelined by hand.  A wavefront has its SIMD to itself (the
-    // 128 x 128 accumulator leaves room for one), so nothing hides an LDS round trip unless
-    // the program order does: every fragment is read one MFMA group (4 MFMAs, ~256 cycles)
-    // before the group that consumes it, the next sub-step's weight fragments are spread over
-    // the four groups of the current one, and the one barrier of a K step sits before its LAST
-    // group, followed at once by the first reads of the next stage, so that barrier skew and
-    // read latency are both covered by matrix-core work already queued.
-    // __builtin_amdgcn_sched_barrier(0) pins that order against the instruction scheduler.
-    constexpr int NS = FP8 ? 2 : 4;  // sub-steps (one MFMA k-extent each) per K step
-    typedef typename std::conditional<FP8, i32x8, i32x4>::type frag_t;
-    auto read_frag = [&](const uint8_t* base, int sub, int t) -> frag_t {
-        if constexpr (FP8) {
-            const int o0 = ((4 * sub + 2 * fh) ^ fsw) << 4, o1 = ((4 * sub + 2 * fh + 1) ^ fsw) << 4;
-            const i32x4 lo = *reinterpret_cast<const i32x4*>(base + t * 32 * BK + o0);
-            const i32x4 hi = *reinterpret_cast<const i32x4*>(base + t * 32 * BK + o1);
-            return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        } else {
-            const int o0 = ((2 * sub + fh) ^ fsw) << 4;
-            return *reinterpret_cast<const i32x4*>(base + t * 32 * BK + o0);
+    // ---- main loop, software-pipelined by hand, with the LDS reads and their waits written out.
+    // Measured on this GPU: an MFMA 32x32x64 occupies the matrix core for 64 cycles and other
+    // instructions of the same wavefront issue in its shadow, about seven of them; past that
+    // every extra instruction delays the next MFMA.  With one wavefront per SIMD the loop is
+    // therefore laid out so that no gap between two MFMAs holds more than a handful of
+    // instructions, and nothing in it waits longer than it must:
+    //   - the compiler's own s_waitcnt before a use of loaded data is lgkmcnt(0) here (it waits
+    //     for every read in flight), so the fragment reads are inline-asm ds_read_b128 whose
+    //     latency the compiler does not see, and each MFMA is preceded by s_waitcnt lgkmcnt(N)
+    //     with N from a compile-time model of the issue order (Sched): "all but the N youngest
+    //     reads have landed";
+    //   - per stage of G = 4 SPS groups (a group = the TJ MFMAs of one x fragment): the x
+    //     fragment of group g+2 is requested in group g (four register sets in rotation), the
+    //     w fragments of the next sub-step in the first two groups of the current one (two
+    //     sets), each after the group's first MFMA;
+    //   - the stage's only barrier sits at the start of its last-but-one group, with vmcnt(0)
+    //     (this wavefront's part of the next stage has landed) and lgkmcnt(0) (its reads of
+    //     this stage are done: the buffer may be overwritten); the two groups after it request
+    //     the next stage's first fragments and issue the global -> LDS transfers of the stage
+    //     after next into the buffer just freed, two or three between consecutive MFMAs, so a
+    //     transfer has a whole stage to land;
+    //   - the K loop is unrolled by two stages so that buffer addresses are loop invariants.
+    // __builtin_amdgcn_sched_barrier(0) pins the order against the instruction scheduler.
+    constexpr int KE = FP8 ? 64 : 32;       // bytes of K one MFMA consumes
+    constexpr int SPS = BK / KE;             // sub-steps (one MFMA k-extent each) per stage
+    constexpr int G = 4 * SPS;               // groups per stage
+    constexpr int R = FP8 ? 2 : 1;           // 128-bit reads per fragment
+    constexpr int HB = TJ / 2;               // w fragments requested per group (in the groups that request any)
+    static_assert(SPS % 2 == 0 && TJ == 4, "register-set rotation and transfer slots assume this tile");
+
+    struct Sched {
+        // reads requested in group g (after its first MFMA): the x fragment of group g+2, then w fragments
+        static constexpr int wfrags(int g) {
+            const int sub = g / 4, i = g % 4;
+            return (sub < SPS - 1) ? (i < 2 ? HB : 0) : (i >= 2 ? HB : 0);
+        }
+        static constexpr int reads(int g) { return R * (1 + wfrags(g)); }
+        static constexpr int before(int g) {  // reads requested in groups 0..g-1 of a stage
+            int n = 0;
+            for (int t = 0; t < g; t++) n += reads(t);
+            return n;
+        }
+        static constexpr int total() { return before(G); }
+        // position (reads since the start of the stage, negative = previous stage) of the LAST read of ...
+        static constexpr int pos_a(int g) {  // ... the x fragment group g consumes
+            return g >= 2 ? before(g - 2) + R - 1 : before(G + g - 2) + R - 1 - total();
+        }
+        static constexpr int pos_b(int sub, int j) {  // ... w fragment j of sub-step sub
+            const int g = sub >= 1 ? (sub - 1) * 4 + j / HB : (SPS - 1) * 4 + 2 + j / HB;
+            const int pos = before(g) + R + (j % HB) * R + R - 1;
+            return sub >= 1 ? pos : pos - total();
+        }
+        // reads that may still be in flight when MFMA j of group g issues
+        static constexpr int allow(int g, int j) {
+            const int issued = before(g) + (j >= 1 ? reads(g) : 0);
+            const int pa = pos_a(g), pb = pos_b(g / 4, j);
+            const int n = issued - 1 - (pa > pb ? pa : pb);
+            return n > 15 ? 15 : n;
         }
     };
-    auto stage_a = [&](int kt) { return lds + (kt & 1) * STAGE_BYTES + (wm * 128 + frow) * BK; };
-    auto stage_b = [&](int kt) { return lds + (kt & 1) * STAGE_BYTES + BM * BK + (wn * 128 + frow) * BK; };
+
+    // LDS byte addresses (32-bit) of this lane's reads: [buffer][sub-step][half of the fragment];
+    // the fragment index t is the instruction's immediate offset
+    uint32_t aaddr[2][SPS][R], baddr[2][SPS][R];
+#pragma unroll
+    for (int buf = 0; buf < 2; buf++)
+#pragma unroll
+        for (int sub = 0; sub < SPS; sub++)
+#pragma unroll
+            for (int e = 0; e < R; e++) {
+                const uint32_t so = FP8 ? (uint32_t)(((4 * sub + 2 * fh + e) ^ fsw) << 4)
+                                        : (uint32_t)(((2 * sub + fh) ^ fsw) << 4);
+                aaddr[buf][sub][e] = lds_addr0 + buf * STAGE_BYTES + (wm * 128 + frow) * BK + so;
+                baddr[buf][sub][e] = lds_addr0 + buf * STAGE_BYTES + BM * BK + (wn * WN + frow) * BK + so;
+            }
+
+    i32x4 af[4][R], bf[2][TJ][R];
+#define NQ_LDS_READ(dst, addr, imm) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm))
+#define NQ_LDS_WAIT(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n))
+    auto mma = [&](int i, int j, const i32x4(&a)[R], const i32x4(&b)[R]) {
+        if constexpr (FP8) {
+            const i32x8 av = {a[0][0], a[0][1], a[0][2], a[0][3], a[1][0], a[1][1], a[1][2], a[1][3]};
+            const i32x8 bv = {b[0][0], b[0][1], b[0][2], b[0][3], b[1][0], b[1][1], b[1][2], b[1][3]};
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[i][j], 0, 0, 0, 0, 0, 0);
+        } else {
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], acc[i][j], 0, 0, 0);
+        }
+    };
+    // the requests of group g of the stage in buffer BUF, in Sched's order (a request that would
+    // belong to a stage past K reads stale LDS into registers nobody uses)
+    auto requests = [&](auto gc, auto bufc) {
+        constexpr int g = decltype(gc)::value, BUF = decltype(bufc)::value;
+        auto& afr = af;  // (named outside the asm statements so that the lambda captures them)
+        auto& bfr = bf;
+        constexpr int sub = g / 4, i = g % 4;
+        constexpr int g2 = (g + 2) % G;                       // the group whose x fragment is requested
+        constexpr int abuf = (g + 2 >= G) ? BUF ^ 1 : BUF;    // ... in the next stage's buffer when it wraps
+#pragma unroll
+        for (int e = 0; e < R; e++) {
+            const uint32_t addr = aaddr[abuf][g2 / 4][e];
+            NQ_LDS_READ(afr[(g + 2) % 4][e], addr, (g2 % 4) * 32 * BK);
+        }
+        if constexpr (Sched::wfrags(g) > 0) {
+            constexpr bool nb = sub == SPS - 1;  // the w fragments are the next stage's first sub-step
+            constexpr int first = (nb ? i - 2 : i) * HB;
+            constexpr int set = (sub + 1) & 1, bsub = nb ? 0 : sub + 1, bbuf = nb ? BUF ^ 1 : BUF;
+#pragma unroll
+            for (int f = 0; f < HB; f++)
+#pragma unroll
+                for (int e = 0; e < R; e++) {
+                    const uint32_t addr = baddr[bbuf][bsub][e];
+                    NQ_LDS_READ(bfr[set][first + f][e], addr, (first + f) * 32 * BK);
+                }
+        }
+    };
+    // transfers of the stage after next, issued from groups G-2 and G-1 in three slots each
+    constexpr int ND = DA + DB, DPG = ND / 2;
+    static_assert(ND == 16, "transfer slots below are written for 16 transfers per wavefront and stage");
+#define NQ_DMA_SLOT(g, slot, buf, srca, srcb)                                                      \
+    if constexpr ((g) >= G - 2) {                                                                  \
+        if (have2) {                                                                               \
+            constexpr int t0 = ((g) - (G - 2)) * DPG + (slot) * 3;                                 \
+            NQ_DMA(t0, buf, srca, srcb);                                                           \
+            NQ_DMA(t0 + 1, buf, srca, srcb);                                                       \
+            if constexpr ((slot) < 2) NQ_DMA(t0 + 2, buf, srca, srcb);                             \
+        }                                                                                          \
+    }
+#define NQ_GROUP(g, BUF)                                                                           \
+    if constexpr ((g) < G) {                                                                       \
+        constexpr int sub_ = (g) / 4, i_ = (g) % 4, set_ = sub_ & 1;                               \
+        constexpr int w0_ = ((g) == G - 2) ? 0 : Sched::allow((g), 0);                             \
+        if constexpr ((g) == G - 2) {                                                              \
+            /* this wavefront's share of the next stage has landed and its reads of this stage */ \
+            /* are done; past the barrier that holds for every wavefront */                        \
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                            \
+            __builtin_amdgcn_s_barrier();                                                          \
+        } else {                                                                                   \
+            NQ_LDS_WAIT(w0_);                                                                      \
+        }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        mma(i_, 0, af[(g) % 4], bf[set_][0]);                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        requests(std::integral_constant<int, (g)>{}, std::integral_constant<int, BUF>{});          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        /* later MFMAs of the group wait again only where their w fragment is younger */           \
+        constexpr int b1_ = w0_ + Sched::reads((g));                                               \
+        constexpr int w1_ = Sched::allow((g), 1) < b1_ ? Sched::allow((g), 1) : b1_;               \
+        if constexpr (w1_ < b1_) NQ_LDS_WAIT(w1_);                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        mma(i_, 1, af[(g) % 4], bf[set_][1]);                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        NQ_DMA_SLOT((g), 0, BUF, srca, srcb)                                                       \
+        constexpr int w2_ = Sched::allow((g), 2) < w1_ ? Sched::allow((g), 2) : w1_;               \
+        if constexpr (w2_ < w1_) NQ_LDS_WAIT(w2_);                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        mma(i_, 2, af[(g) % 4], bf[set_][2]);                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        NQ_DMA_SLOT((g), 1, BUF, srca, srcb)                                                       \
+        constexpr int w3_ = Sched::allow((g), 3) < w2_ ? Sched::allow((g), 3) : w2_;               \
+        if constexpr (w3_ < w2_) NQ_LDS_WAIT(w3_);                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        mma(i_, 3, af[(g) % 4], bf[set_][3]);                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        NQ_DMA_SLOT((g), 2, BUF, srca, srcb)                                                       \
+    }
+    // one stage, read from buffer BUF; its groups G-2 and G-1 refill BUF with stage st+2
+#define NQ_STAGE(BUF)                                                                              \
+    {                                                                                              \
+        const bool have2 = st + 2 < KT;                                                            \
+        const uint8_t* const srca = abase + (int64_t)(st + 2) * BK;                                \
+        const uint8_t* const srcb = bbase + (int64_t)(st + 2) * BK;                                \
+        NQ_GROUP(0, BUF) NQ_GROUP(1, BUF) NQ_GROUP(2, BUF) NQ_GROUP(3, BUF) NQ_GROUP(4, BUF)       \
+        NQ_GROUP(5, BUF) NQ_GROUP(6, BUF) NQ_GROUP(7, BUF) NQ_GROUP(8, BUF) NQ_GROUP(9, BUF)       \
+        NQ_GROUP(10, BUF) NQ_GROUP(11, BUF) NQ_GROUP(12, BUF) NQ_GROUP(13, BUF) NQ_GROUP(14, BUF)  \
+        NQ_GROUP(15, BUF)                                                                          \
+    }
 
     const int KT = p.K / BK;
-    dma(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    // Fragment registers are two named sets used in turn (groups alternate between af[0] and
-    // af[1], sub-steps between bf[0] and bf[1]); a K step has an even number of both, so the
-    // sets line up again at the loop's back edge and nothing is copied.
-    frag_t af[2], bf[2][4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) bf[0][j] = read_frag(stage_b(0), 0, j);
-    af[0] = read_frag(stage_a(0), 0, 0);
-    for (int kt = 0; kt < KT; kt++) {
-        // stage kt+1 streams into the other buffer while stage kt is multiplied; the barrier
-        // inside the previous iteration guarantees nobody still reads that buffer
-        if (kt + 1 < KT) dma((kt + 1) * BK, (kt + 1) & 1);
-        const uint8_t* sa = stage_a(kt);
-        const uint8_t* sb = stage_b(kt);
-#pragma unroll
-        for (int sub = 0; sub < NS; sub++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int g = sub * 4 + i;  // group index within the K step
-                const bool last = (sub == NS - 1 && i == 3);
-                frag_t& acur = af[g & 1];
-                frag_t& anext = af[(g + 1) & 1];
-                frag_t(&bcur)[4] = bf[sub & 1];
-                frag_t(&bnext)[4] = bf[(sub + 1) & 1];
-                if (last) {
-                    // every read of stage kt has been issued and waited for; once all wavefronts
-                    // are here stage kt+1 is complete and stage kt's buffer may be overwritten
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                    __syncthreads();
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                // the first MFMA of the group goes ahead of the prefetch so that the reads are
-                // issued while the matrix core is busy and have the rest of the group to land
-                if constexpr (FP8)
-                    acc[i][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bcur[0], acur, acc[i][0], 0, 0, 0, 0,
-                                                                                 0, 0);
-                else
-                    acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bcur[0], acur, acc[i][0], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                if (!last) {
-                    anext = (i < 3) ? read_frag(sa, sub, i + 1) : read_frag(sa, sub + 1, 0);
-                    if (sub + 1 < NS) bnext[i] = read_frag(sb, sub + 1, i);
-                } else if (kt + 1 < KT) {
-                    anext = read_frag(stage_a(kt + 1), 0, 0);
-#pragma unroll
-                    for (int j = 0; j < 4; j++) bnext[j] = read_frag(stage_b(kt + 1), 0, j);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 1; j < 4; j++) {
-                    if constexpr (FP8)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bcur[j], acur, acc[i][j], 0, 0, 0,
-                                                                                     0, 0, 0);
-                    else
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bcur[j], acur, acc[i][j], 0, 0, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
+    {
+        // stage 0 now, stage 1 on its way during all of stage 0
+        const bool have2 = true;
+        (void)have2;
+        const uint8_t* srca = abase;
+        const uint8_t* srcb = bbase;
+#define NQ_DMA_ALL(buf)                                                                            \
+    NQ_DMA(0, buf, srca, srcb); NQ_DMA(1, buf, srca, srcb); NQ_DMA(2, buf, srca, srcb);            \
+    NQ_DMA(3, buf, srca, srcb); NQ_DMA(4, buf, srca, srcb); NQ_DMA(5, buf, srca, srcb);            \
+    NQ_DMA(6, buf, srca, srcb); NQ_DMA(7, buf, srca, srcb); NQ_DMA(8, buf, srca, srcb);            \
+    NQ_DMA(9, buf, srca, srcb); NQ_DMA(10, buf, srca, srcb); NQ_DMA(11, buf, srca, srcb);          \
+    NQ_DMA(12, buf, srca, srcb); NQ_DMA(13, buf, srca, srcb); NQ_DMA(14, buf, srca, srcb);         \
+    NQ_DMA(15, buf, srca, srcb);
+        NQ_DMA_ALL(0)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (KT > 1) {
+            srca = abase + BK, srcb = bbase + BK;
+            NQ_DMA_ALL(1)
         }
+#undef NQ_DMA_ALL
     }
+    // what groups G-2 and G-1 of a previous stage (in buffer 1) would have requested
+    requests(std::integral_constant<int, G - 2>{}, std::integral_constant<int, 1>{});
+    requests(std::integral_constant<int, G - 1>{}, std::integral_constant<int, 1>{});
+    int st = 0;
+    for (; st + 1 < KT; st++) {
+        NQ_STAGE(0)
+        st++;
+        NQ_STAGE(1)
+    }
+    if (st < KT) NQ_STAGE(0)  // an odd number of stages: the last one, in buffer 0 again
+    NQ_LDS_WAIT(0);  // requests past the last stage still target registers: let them land
+#undef NQ_STAGE
+#undef NQ_GROUP
+#undef NQ_DMA_SLOT
+#undef NQ_DMA
+#undef NQ_LDS_READ
+#undef NQ_LDS_WAIT
 
     // ---- epilogue.  The MFMA was issued with the weight tile as its first operand, so in
     // acc[i][j] a lane holds ONE token m = 32 i + lane % 32 (MFMA column) and, for g = 0..3, the
@@ -238,7 +402,7 @@ void gemm8_kernel(const Gemm8Params p) {
     // stages its results through its own LDS region (free now: the loop ended on a barrier) as
     // [token][channel] rows, and writes them out as 128-bit stores, 256 B (bf16) or 512 B (fp32 /
     // int32) contiguous per row of y.
-    const int wm0 = m0 + wm * 128, wn0 = n0 + wn * 128;
+    const int wm0 = m0 + wm * 128, wn0 = n0 + wn * WN;
     const int lm = lane & 31, lh = lane >> 5;
     const bool full_tile = (m0 + BM <= p.M) && (n0 + BN <= p.N) && (p.N % 8 == 0);
 
@@ -260,7 +424,7 @@ void gemm8_kernel(const Gemm8Params p) {
         constexpr int KIND = decltype(kind)::value;  // 0: fp32, 1: bf16, 2: raw int32
         constexpr int ES = (KIND == 1) ? 2 : 4;      // bytes per output element
         constexpr int IP = (KIND == 1) ? 2 : 1;      // token tiles (of 32) staged per pass
-        constexpr int ROWB = 128 * ES + 16;          // staged row: 128 channels + pad (bank spread)
+        constexpr int ROWB = WN * ES + 16;           // staged row: the wavefront's channels + pad (bank spread)
         uint8_t* stage = lds + wave * (32 * IP * ROWB);
 #pragma unroll
         for (int ip = 0; ip < 4; ip += IP) {
@@ -274,7 +438,7 @@ void gemm8_kernel(const Gemm8Params p) {
                 if constexpr (!FP8 && KIND != 2) rscale[ii] = p.row_scale[min(wm0 + 32 * (ip + ii) + lm, p.M - 1)];
             }
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < TJ; j++) {
                 float cs[4][4], cb[4][4];
                 if constexpr (KIND != 2) {
 #pragma unroll
@@ -338,7 +502,7 @@ void gemm8_kernel(const Gemm8Params p) {
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             // ---- LDS -> global: 16 bytes per lane, rows of y contiguous
-            constexpr int LPRW = 128 * ES / 16;          // lanes per staged row (16 or 32)
+            constexpr int LPRW = WN * ES / 16;           // lanes per staged row (8, 16 or 32)
             constexpr int RPI = 64 / LPRW;               // rows per wavefront instruction
 #pragma unroll
             for (int t = 0; t < 32 * IP / RPI; t++) {
@@ -375,13 +539,33 @@ void gemm8_kernel(const Gemm8Params p) {
         emit(std::integral_constant<int, 2>{});
 }
 
+template <bool FP8>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm8_kernel(const Gemm8Params p) {
+    gemm8_body<FP8, 256, 128>(p);
+}
+
+template <typename K>
+int32_t launch_cfg(K kernel, bool* attr_set, const Gemm8Params& p, int bn, int bk, hipStream_t s) {
+    const size_t lds = (size_t)2 * (BM + bn) * bk;
+    if (!*attr_set) {
+        NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)lds));
+        *attr_set = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(p.tiles_m * p.tiles_n), dim3(256), lds, s, p);
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
 }  // namespace
 
 bool gemm8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     const bool fp8 = (a.x_dtype == NQ_DT_FP8_E4M3 && L->format == NQ_FMT_FP8_E4M3);
     const bool i8 = (a.x_dtype == NQ_DT_I8 && L->format == NQ_FMT_W8_CHANNEL);
-    return (fp8 || i8) && (L->in % BK == 0) && a.M >= 64;
+    // the kernel addresses a tile's rows with 32-bit offsets from the tile's base
+    return (fp8 || i8) && (L->in % 128 == 0) && a.M >= 64 && (int64_t)L->in * 256 < ((int64_t)1 << 32);
 }
 
 int32_t launch_gemm8(const ForwardArgs& a) {
@@ -394,28 +578,11 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     p.col_scale = reinterpret_cast<const float*>(L->d_scales);
     p.tscale = L->scale;
     p.M = a.M, p.N = L->out, p.K = L->in;
-    p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + BN - 1) / BN;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
-    const dim3 grid(p.tiles_m * p.tiles_n);
-    const size_t lds = 2 * STAGE_BYTES;
+    p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + 255) / 256;
     static bool attr_set[2] = {false, false};
-    if (a.x_dtype == NQ_DT_FP8_E4M3) {
-        if (!attr_set[0]) {
-            NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            attr_set[0] = true;
-        }
-        hipLaunchKernelGGL(gemm8_kernel<true>, grid, dim3(256), lds, a.stream, p);
-    } else {
-        if (!attr_set[1]) {
-            NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_kernel<false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            attr_set[1] = true;
-        }
-        hipLaunchKernelGGL(gemm8_kernel<false>, grid, dim3(256), lds, a.stream, p);
-    }
-    NQ_HIP(hipGetLastError());
-    return NQ_OK;
+    if (a.x_dtype == NQ_DT_FP8_E4M3) return launch_cfg(gemm8_kernel<true>, &attr_set[0], p, 256, 128, a.stream);
+    return launch_cfg(gemm8_kernel<false>, &attr_set[1], p, 256, 128, a.stream);
 }
 
 }  // namespace nq
