@@ -151,12 +151,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"           \
                          :                                                                             \
                          : "s"(dbase[buf][0]), "v"(doff[(t)]), "s"(srca), "n"((t) * 1024)              \
-                         : "memory", "m0");                                                            \
+                         : "memory", "m0", "scc");                                                            \
         else                                                                                           \
             asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"           \
                          :                                                                             \
                          : "s"(dbase[buf][1]), "v"(doff[(t)]), "s"(srcb), "n"(((t) - DA) * 1024)       \
-                         : "memory", "m0");                                                            \
+                         : "memory", "m0", "scc");                                                            \
     } while (0)
     const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;  // requested now, used in the epilogue
 
