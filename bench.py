@@ -337,6 +337,29 @@ def make_fp8(M, N, K=4096, copies=1, seed=6):
     return dict(step=step, bytes=N * K + M * K + 2 * M * N + 8, ops=2 * M * N * K, launches=1, keep=(layers, a, sa, y))
 
 
+def make_w8a8_gemm(M, N, K=4096, seed=8):
+    """The large-M W8A8 GEMM of the north star: int8 x int8 -> int32 on the matrix cores, per-token and
+    per-channel scales and bias in the epilogue, bf16 out."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import W8Linear
+
+    rng = np.random.default_rng(seed)
+    lin = W8Linear(K, N)
+    lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+    xq = torch.from_numpy(rng.integers(-127, 128, (M, K), dtype=np.int8)).cuda()
+    xs = torch.from_numpy(rng.uniform(1e-2, 2e-2, M).astype(np.float32)).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def step(i):
+        lin.forward_a8(xq, xs, bias=bias, out=y, out_dtype=torch.bfloat16)
+
+    return dict(step=step, bytes=N * K + M * K + 2 * M * N + 4 * (M + 2 * N), ops=2 * M * N * K, launches=1,
+                keep=(lin, xq, xs, bias, y))
+
+
 def report(name, wl, seconds, bound, peak_key=None):
     gbps = wl["bytes"] / seconds / 1e9
     tops = wl["ops"] / seconds / 1e12
@@ -387,6 +410,9 @@ def sweep(skip_large=False):
         run(f"cfg4 fp8 GEMV K=4096 N={N} M=1 (cold)", make_fp8, "hbm", M=1, N=N, copies=c, calls=max(c, 20))
         if not skip_large:
             run(f"cfg4 fp8 GEMM M=8192 K=4096 N={N}", make_fp8, "mfma", "fp8", M=8192, N=N, copies=1, calls=10)
+    if not skip_large:
+        run("W8A8 int8 GEMM M=8192 K=4096 N=4096 (scales + bias epilogue, bf16 out)", make_w8a8_gemm, "mfma", "int8",
+            M=8192, N=4096, calls=10)
     return out
 
 

@@ -81,7 +81,9 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float v) {
 // BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with
 // BK = 128 (a 256 x 128, BK = 64 variant with two workgroups per CU measured slower: its stage is
 // too short for a transfer to land in).
-template <bool FP8, int BN, int BK>
+// KIND: the output type the epilogue is built for (0 fp32, 1 bf16, 2 raw int32 accumulators); one
+// kernel per kind, because with all three in one function the register allocator spills.
+template <bool FP8, int KIND_, int BN, int BK>
 __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int STAGE_BYTES = (BM + BN) * BK;
     constexpr int SLOTS = BK / 16;     // 16-byte slots per LDS row
@@ -531,18 +533,13 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     };
-    if (p.y_dtype == NQ_DT_F32)
-        emit(std::integral_constant<int, 0>{});
-    else if (p.y_dtype == NQ_DT_BF16)
-        emit(std::integral_constant<int, 1>{});
-    else if constexpr (!FP8)
-        emit(std::integral_constant<int, 2>{});
+    emit(std::integral_constant<int, KIND_>{});
 }
 
-template <bool FP8>
+template <bool FP8, int KIND>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm8_kernel(const Gemm8Params p) {
-    gemm8_body<FP8, 256, 128>(p);
+    gemm8_body<FP8, KIND, 256, 128>(p);
 }
 
 template <typename K>
@@ -580,9 +577,14 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + 255) / 256;
-    static bool attr_set[2] = {false, false};
-    if (a.x_dtype == NQ_DT_FP8_E4M3) return launch_cfg(gemm8_kernel<true>, &attr_set[0], p, 256, 128, a.stream);
-    return launch_cfg(gemm8_kernel<false>, &attr_set[1], p, 256, 128, a.stream);
+    static bool attr_set[5] = {false, false, false, false, false};
+    const bool f32 = a.y_dtype == NQ_DT_F32;
+    if (a.x_dtype == NQ_DT_FP8_E4M3)
+        return f32 ? launch_cfg(gemm8_kernel<true, 0>, &attr_set[0], p, 256, 128, a.stream)
+                   : launch_cfg(gemm8_kernel<true, 1>, &attr_set[1], p, 256, 128, a.stream);
+    if (a.y_dtype == NQ_DT_I32) return launch_cfg(gemm8_kernel<false, 2>, &attr_set[4], p, 256, 128, a.stream);
+    return f32 ? launch_cfg(gemm8_kernel<false, 0>, &attr_set[2], p, 256, 128, a.stream)
+               : launch_cfg(gemm8_kernel<false, 1>, &attr_set[3], p, 256, 128, a.stream);
 }
 
 }  // namespace nq
