@@ -8,10 +8,9 @@
 // Tiling.  One workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 tile of y;
 // each wavefront owns 128 x 128 of it as 4 x 4 MFMA tiles of 32 x 32, i.e. 256
 // fp32/int32 accumulators per lane (the AGPR half of the unified register
-// file), one workgroup per CU.  A wavefront tile this large is what keeps the
-// kernel MFMA-bound: per 64-byte k-step a wavefront issues 16 MFMAs (1024
-// cycles) for 16 KiB of LDS reads, half the LDS bandwidth; at 64 x 64 the LDS
-// would be the limit.
+// file), one workgroup per CU.  A tile this large is what keeps operand traffic
+// down: a stage moves 64 KiB from L2 into a CU for 2048 cycles of MFMA work, and
+// that delivery is already the nearer bound (below).
 //
 // K loop.  Stages of BK = 128 bytes: x tile 256 x 128 B and w tile 256 x 128 B
 // (64 KiB), double-buffered in LDS (128 of the CU's 160 KiB).  While a stage is

@@ -4,20 +4,24 @@
 // This is the regime of the reference's real caller, the SmolVLA prefill at
 // T = 135 tokens (noeira/deep_agents/smolvla/fused.mojo:255-384), and of
 // BASELINE's M = 100 / 256 configs: the weights are ~1 MB, so the call is
-// latency- and occupancy-bound, not MFMA-bound.  The kernel therefore has no
-// LDS staging and no block-wide barrier in its K loop: every wavefront pulls
-// its own operand fragments straight from global memory (x is L2-resident, W
-// is read exactly once per M tile) and the only synchronisation is the final
-// fixed-order reduction of the four K-slices through LDS.
+// bound by instruction issue per wavefront and by L1 look-ups, not by MFMA or
+// bytes.  The kernel therefore has no LDS staging and no block-wide barrier in
+// its K loop: every wavefront pulls its own operand fragments straight from
+// global memory (x is L2-resident, W is read once per M tile) and the only
+// synchronisation is the final fixed-order reduction of the K-slices through
+// LDS.
 //
 // Exactness.  Weights enter the MFMA as the integer codes, converted to bf16
 // exactly: a 4-bit code q becomes 16 + q by OR-ing it into the mantissa of
 // bf16 16.0 (one shift and one and-or per pair), an int8 code becomes q + 128.
 // The offset is removed in fp32 with X = sum_k x_k, which a second MFMA against
 // an all-ones operand provides in the same lane layout:
-//     sum_k x_k (q_k - z) = P - (offset + z) X.
-// Scales are applied in fp32 after the MFMA, per 32-wide chunk for the 4-bit
-// formats (one chunk = one Q4_0 group = one MFMA), once at the end for W8.
+//     sum_k x_k (q_k - z) = P - (offset + z) X,
+// and -(offset + z) X is handed to the product MFMA as its C operand.  Scales
+// are applied in fp32 after the MFMA: per 32-wide chunk (one chunk = one Q4_0
+// group = one MFMA), per 128-wide k-step where a k-step lies in one group
+// (W4_GROUP with a group width that is a multiple of 128), once at the end for
+// W8.
 // bf16 activations are exact operands; fp32 activations are split into three
 // bf16 terms hi + mid + lo that add up to the fp32 value exactly, so every
 // product the matrix core forms is exact and only the fp32 accumulation rounds

@@ -7,9 +7,16 @@
 // the 16-byte chunks j, j + lpr, ... (CPL of them), and the x values under
 // those chunks are loaded once, up front, together with the first weights -
 // one round trip to memory, no LDS, no barrier.  A lane group then walks its
-// rows RPL at a time (RPL x CPL independent loads in flight per lane).
+// rows RPL at a time (RPL x CPL independent loads in flight per lane); the
+// host picks one row per lane group and as many lanes per row as it takes to
+// launch ~1k wavefronts, which measured best from 68 KB to 45 MB of weights.
+// Every load is unconditional from a clamped address (a predicated load
+// becomes a branch and serialises the batch); the product of a chunk past the
+// end of a row is dropped with one select.
 //
-//   8-bit weights (int8, fp8):  x held as fp32, one v_cvt per code + one FMA.
+//   8-bit weights (int8, fp8):  x held as fp32, one v_cvt per code (for int8
+//       the sign-extending byte form of v_cvt_f32_i32) + one FMA.  fp8
+//       weights with fp8 activations go to nq_gemv_fp8.hip instead.
 //   4-bit weights, bf16 x:      x held as packed bf16 pairs; a word of eight
 //       codes becomes four bf16 pairs (16 + q) with a shift and an and-or each
 //       (device nibble order, nq_nib.h) and goes through v_dot2_f32_bf16:

@@ -108,3 +108,15 @@ def test_mirror_refuses_cpu_target():
     from noeira_amd.qlinear import QLinear
     with pytest.raises(L.NQError, match="no CPU path"):
         QLinear.make(64, 4, target="cpu")
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path runs on one GPU: `bench.py --gpus N` with N > 1 exits with a message saying so."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr
