@@ -480,8 +480,21 @@ def cpu_baseline(budget_s=12.0):
         dt = time.perf_counter() - t0
         if dt >= budget_s and n >= 3:
             break
+    # the reference's own layer on its own shapes (Q4_0, fp32 x), same CPU path, a few calls each
+    q4 = []
+    for (IN, OUT) in [(960, 960), (960, 320), (960, 2560), (2560, 960)]:
+        blocks = rng.integers(0, 256, OUT * (IN // 32) * 18, dtype=np.uint8)
+        sc = rng.uniform(1e-3, 2e-3, OUT * (IN // 32)).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        blocks.reshape(-1, 18)[:, 0:2] = sc
+        for M, calls in ((1, 5), (135, 1)):
+            x = rng.standard_normal((M, IN)).astype(np.float32)
+            O.qlinear_forward_cpu(blocks, IN, OUT, x)
+            t1 = time.perf_counter()
+            for _ in range(calls):
+                O.qlinear_forward_cpu(blocks, IN, OUT, x)
+            q4.append({"layer": f"Q4_0 {IN}->{OUT}", "M": M, "ms_per_call": round((time.perf_counter() - t1) / calls * 1e3, 3)})
     return {"value": round(nbytes * n / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "ms_per_step": round(dt / n * 1e3, 3),
+            "ms_per_step": round(dt / n * 1e3, 3), "q4_0_reference_shapes": q4,
             "sample": f"{n} steps of the headline workload (both W8 linears at M=1): a fresh dequantize to an "
                       f"fp32 [OUT, IN] scratch then the serial triple loop, single thread, {dt:.1f} s"}
 
