@@ -160,12 +160,12 @@ int32_t nq_fused_parts(nq_handle h);
 
 /* nq_forward of a fused layer with one dense output per part:
  * ys[t] is [M, OUT_t], what nq_forward of part t alone would write: a row's
- * arithmetic does not depend on its neighbours (bit for bit at M >= 5; at
+ * arithmetic does not depend on its neighbours (bit for bit at M >= 2; at
  * M = 1 the number of lanes that share a row, hence the order of its sum, may
  * follow the total row count).
  * n_ys must equal nq_fused_parts(h).  bias, if any, is [sum OUT].  One launch
  * where the kernel for the shape can place rows by part (bf16/fp32
- * activations at M = 1 and M >= 5), otherwise one launch per part. */
+ * activations at any M), otherwise one launch per part. */
 int32_t nq_forward_fused(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale,
                          void* const* ys, int32_t n_ys, int32_t y_dtype, int32_t M, const void* bias,
                          int32_t bias_dtype, int32_t epilogue, void* stream);

@@ -1,4 +1,4 @@
-// fp8 x fp8 GEMV for 1..16 activation rows on the matrix cores:
+// fp8 x fp8 GEMV for 1..63 activation rows on the matrix cores:
 //     y[M, N] = epi( (x[M, K] @ W[N, K]^T) * s_w * s_x + bias ),  x and W in e4m3.
 //
 // The call is bound by the weight stream (K = 4096, N = 11008 is 45 MB), and what a
@@ -11,8 +11,9 @@
 //   - lane (n = lane % 16, kb = lane / 16) loads the 32 bytes of row n under k-block kb of a
 //     step (two 128-bit loads, 128 contiguous bytes per row across the four lanes) - this is
 //     exactly its share of the MFMA's B operand, so nothing is shuffled or converted;
-//   - the activations are the A operand: row m = lane % 16 (clamped to M - 1), same k-block;
-//     they are 16 x K bytes at most and stay in L1/L2;
+//   - the activations are the A operand: row m = lane % 16 of the workgroup's 16-row M tile
+//     (clamped to M - 1), same k-block; they stay in L1/L2, and more than 16 rows take one
+//     workgroup per M tile, re-reading the weights from L2;
 //   - all of a wavefront's loads are issued before its first MFMA (SPW x 32 bytes per lane,
 //     up to 16 KB per wavefront in flight);
 //   - the KW partial 16 x 16 tiles are summed through LDS in wave order (fixed, so a repeated
@@ -62,9 +63,10 @@ __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kb = lane >> 4;
     const int n_base = blockIdx.x * 16;
+    const int m_base = blockIdx.y * 16;
 
     const int64_t wrow = (int64_t)min(n_base + ln, p.N - 1) * p.K;
-    const int64_t xrow = (int64_t)min(ln, p.M - 1) * p.K;
+    const int64_t xrow = (int64_t)min(m_base + ln, p.M - 1) * p.K;
 
     f32x4 acc = {0, 0, 0, 0};
     for (int s0 = wave * SPW; s0 < p.nsteps; s0 += KW * SPW) {
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p
     __syncthreads();
     const int t = threadIdx.x;
     if (t < 256) {
-        const int m = t >> 4, n = n_base + (t & 15);
+        const int m = m_base + (t >> 4), n = n_base + (t & 15);
         if (m < p.M && n < p.N) {
             float z = red[0][t];
 #pragma unroll
@@ -239,7 +241,7 @@ int32_t launch_kw(const Fp8GemvParams& p, int kw, dim3 grid, hipStream_t s) {
 }  // namespace
 
 // a row of 768..8192 codes takes the one-row kernel (M = 1, K a multiple of 16); otherwise the
-// 16-row tile kernel needs whole MFMA steps (K a multiple of 128)
+// 16-row tile kernel (M < 64) needs whole MFMA steps (K a multiple of 128)
 static bool row_kernel_fits(const ForwardArgs& a) {
     return a.M == 1 && a.L->in % 16 == 0 && a.L->in >= 768 && a.L->in <= 8192;
 }
@@ -247,7 +249,7 @@ static bool row_kernel_fits(const ForwardArgs& a) {
 bool gemv_fp8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (L->format != NQ_FMT_FP8_E4M3 || a.x_dtype != NQ_DT_FP8_E4M3 || a.x_scale == nullptr) return false;
-    return row_kernel_fits(a) || (a.M >= 1 && a.M <= 16 && L->in % 128 == 0);
+    return row_kernel_fits(a) || (a.M >= 1 && a.M < 64 && L->in % 128 == 0);
 }
 
 int32_t launch_gemv_fp8(const ForwardArgs& a) {
@@ -282,7 +284,7 @@ int32_t launch_gemv_fp8(const ForwardArgs& a) {
     while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
     if (kw == 16 && spw > 4) spw = 4;
     kw = env_int("NQ_FP8V_KW", kw), spw = env_int("NQ_FP8V_SPW", spw);
-    const dim3 grid((unsigned)wgs);
+    const dim3 grid((unsigned)wgs, (unsigned)((a.M + 15) / 16));
     switch (spw) {
         case 1: return launch_kw<1>(p, kw, grid, a.stream);
         case 2: return launch_kw<2>(p, kw, grid, a.stream);

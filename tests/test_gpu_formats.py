@@ -190,10 +190,10 @@ def test_encode_e4m3_host_matches_oracle():
     assert np.array_equal(F.encode_e4m3(x), O.e4m3_encode(np.clip(x, -448, 448)))
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 17, 64])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 40, 63, 64])
 def test_config5_fp8_reduced_size_vs_oracle(M):
     rng = np.random.default_rng(5 + M)
-    N, K = (504 if M in (7, 17) else 512), 4096  # 504 = 31.5 row tiles of 16
+    N, K = (504 if M in (7, 17, 63) else 512), 4096  # 504 = 31.5 row tiles of 16
     a, b = fp8_operands(rng, M, N, K)
     sa, sb = np.float32(0.731), np.float32(1.37)
     lin = FP8Linear(K, N)

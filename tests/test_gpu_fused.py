@@ -36,7 +36,7 @@ def test_q4_0_qkv_fused_equals_parts(M, xdt):
     for l, y, b, n in zip(layers, ys, blocks, outs):
         own = l.forward(x)
         assert y.shape == (M, n)
-        if M >= 5:
+        if M >= 2:
             assert torch.equal(y, own)
         else:
             scale = own.abs().max().item()
@@ -83,7 +83,7 @@ def test_w8_fused_with_bias_and_relu(M):
     r0 = 0
     for l, y, n in zip(layers, ys, outs):
         own = l.forward(x, bias=bias[r0:r0 + n].contiguous(), epilogue="relu")
-        if M >= 5:
+        if M >= 2:
             assert torch.equal(y, own)
         else:
             assert (y - own).abs().max().item() <= 2e-6 * max(own.abs().max().item(), 1e-30)
@@ -106,7 +106,7 @@ def test_w4g_fused(M):
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(torch.bfloat16)
     for l, y in zip(layers, fused.forward(x)):
         own = l.forward(x)
-        if M >= 5:
+        if M >= 2:
             assert torch.equal(y, own)
         else:
             assert (y - own).abs().max().item() <= 2e-6 * own.abs().max().item()
