@@ -114,7 +114,6 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     // instruction fills 1 KiB of LDS, lane l at byte 16 l, i.e. 1024 / BK rows; wavefront w owns
     // a quarter of the rows of both tiles.  The slot swizzle is applied on the global side: the
     // lane that lands in physical slot s of its row fetches logical slot s ^ swz(row).
-    typedef __attribute__((address_space(1))) const void gptr_t;
     typedef __attribute__((address_space(3))) void lptr_t;
     constexpr int DROWS = 1024 / BK;           // rows per instruction
     constexpr int DA = BM / 4 / DROWS;         // instructions per wavefront and stage, x tile
@@ -138,7 +137,8 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     }
     // transfer t (0 .. DA+DB-1) of a stage: M0 = the LDS address of the 1 KiB the instruction
     // fills (a scalar base of the buffer half plus t KiB), global address = scalar base + lane
-    // offset.  Three instructions per transfer.
+    // offset.  Three instructions per transfer.  (M0 is a reserved register the compiler sets itself
+    // right before each of its own uses, so writing it here needs no clobber; SCC does.)
     const uint32_t lds_addr0 = (uint32_t)(uintptr_t)(lptr_t*)lds;
     uint32_t dbase[2][2];  // [buffer][x tile, w tile]: this wavefront's first destination
 #pragma unroll
@@ -152,12 +152,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"           \
                          :                                                                             \
                          : "s"(dbase[buf][0]), "v"(doff[(t)]), "s"(srca), "n"((t) * 1024)              \
-                         : "memory", "m0", "scc");                                                            \
+                         : "memory", "scc");                                                            \
         else                                                                                           \
             asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"           \
                          :                                                                             \
                          : "s"(dbase[buf][1]), "v"(doff[(t)]), "s"(srcb), "n"(((t) - DA) * 1024)       \
-                         : "memory", "m0", "scc");                                                            \
+                         : "memory", "scc");                                                            \
     } while (0)
     const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;  // requested now, used in the epilogue
 
