@@ -9,19 +9,35 @@
 // each wavefront owns 128 x 128 of it as 4 x 4 MFMA tiles of 32 x 32, i.e. 256
 // fp32/int32 accumulators per lane (the AGPR half of the unified register
 // file), one workgroup per CU.  A tile this large is what keeps operand traffic
-// down: a stage moves 64 KiB from L2 into a CU for 2048 cycles of MFMA work, and
-// that delivery is already the nearer bound (below).
+// down: a stage moves 64 KiB from L2 into a CU for 2048 cycles of MFMA work.
 //
 // K loop.  Stages of BK = 128 bytes: x tile 256 x 128 B and w tile 256 x 128 B
 // (64 KiB), double-buffered in LDS (128 of the CU's 160 KiB).  While a stage is
 // being multiplied, the stage after next streams from global memory straight
 // into the buffer the previous stage has just freed (global_load_lds_dwordx4, 16
 // per lane per stage): no registers, no ds_write, one wait + one barrier per
-// stage.  What bounds the loop, measured on this GPU with parts of it switched
-// off: the MFMAs alone need 2048 cycles per stage, the transfers alone (64 KiB
-// per CU per stage from L2, ~15 TB/s chip-wide) ~2250 cycles, the LDS fragment
-// reads and their waits nothing (the LDS sustains > 500 B/clk per CU); together
-// the stage takes ~2600 cycles.
+// stage.
+//
+// What bounds the loop, measured on this GPU (8192 x 4096 x 4096 fp8, stamps of the
+// cycle counter around the loop, parts switched off one at a time).  In cycles, with
+// N(0,1) data: the whole stage 2610 at a clock of 1.82 GHz; without the barrier 2340;
+// without the transfers 2280; MFMAs alone 2230 (2048 + the switches' own branches).
+// Barrier and transfers cost little each and ~450 cycles together: right after the
+// barrier all four wavefronts ask the CU's address unit for their 16 KiB at once, the
+// issue blocks, and the MFMAs queue up behind it.  Neither L2 nor LDS is near a limit:
+// the same transfers alone, two stages in flight, land in 1390 cycles (47 B/clk per
+// CU, 26 TB/s over the chip), from one CU alone in 1030 (the 64 B/clk of the L1 path),
+// and the LDS serves the stage's 128 KiB of fragment reads in 517 cycles (253 B/clk)
+// while taking the transfers' writes at full rate.
+// But cycles are not what the time is made of here.  A variant with four 32 KiB
+// buffers that spreads each refill over a whole stage takes 2390 cycles per stage -
+// and runs at 1.67 GHz instead of 1.82: 1.43 us per stage either way.  With all-zero
+// or constant activations the same two kernels run at 2.24 - 2.38 GHz and the call
+// takes 93 - 98 us instead of 114 - 121.  On data that toggles the multipliers the
+// loop sits on the board's power limit: the governor trades every cycle saved for
+// clock, so what is left to gain is energy per stage (bytes moved, instructions
+// issued), not issue slots.  MFMAs alone, on random data, are held to 3.7 - 3.9
+// PFLOP/s by the same limit; this loop delivers 2.4 of them.
 //
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= (row >> 1) & 7.  Rows r and r + 1 then sit 128 B apart in
