@@ -1,0 +1,128 @@
+"""Randomised shapes for every format and activation type, through the C ABI.
+
+Each case draws a format, M (1 .. 1000, dense around the kernel-selection
+thresholds), IN, OUT (ragged on purpose: OUT = 1 .. 3000, IN any legal
+multiple), activation and output dtypes, bias kind and epilogue, and checks
+the result against an fp64 product of the layer's dequantised weights.  Those
+weights come from the library's own dequantise call, which
+tests/test_gpu_qlinear.py and tests/test_gpu_formats.py pin bit for bit
+against the CPU oracle; the int8 x int8 accumulators are compared exactly.
+Bars as everywhere: 1e-3 * RMS (fp8: 1e-2), plus half a bf16 step when the
+output is bf16.
+"""
+import numpy as np
+import pytest
+import torch
+
+from noeira_amd import formats as F
+from noeira_amd.qlinear import FP8Linear, QLinear, W4GroupLinear, W8Linear, quantize_rows_i8
+
+pytestmark = pytest.mark.gpu
+
+MS = [1, 1, 1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 127, 128, 135, 255, 256, 257, 300, 513, 1000]
+
+
+def _pick_k(rng, mult, hi=4096):
+    c = rng.integers(0, 4)
+    if c == 0:
+        return int(mult * rng.integers(1, 9))
+    if c == 1:
+        return int(rng.choice([256, 512, 960, 1024, 2560, 3200, 4096]) // mult * mult)
+    return int(mult * rng.integers(1, hi // mult + 1))
+
+
+def _pick_n(rng):
+    c = rng.integers(0, 4)
+    if c == 0:
+        return int(rng.integers(1, 40))
+    if c == 1:
+        return int(rng.choice([8, 256, 320, 512, 960, 2560, 3200, 4096]))
+    return int(rng.integers(1, 3000))
+
+
+def _check(tag, y, exact, out_bf16, tol=1e-3):
+    y = y.double()
+    rms = max(float(exact.pow(2).mean().sqrt()), 1e-30)
+    err = (y - exact).abs()
+    allow = tol * rms + (2.0 ** -8) * exact.abs() * (1 if out_bf16 else 0)
+    assert not bool(torch.isnan(y).any()), tag
+    assert not bool((err > allow).any()), (tag, float(err.max()) / rms)
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_shapes(seed):
+    rng = np.random.default_rng(seed)
+    for case in range(150):
+        fmt = ["q4_0", "w8", "w4g", "fp8", "w8a8"][case % 5]
+        M = int(rng.choice(MS))
+        N = _pick_n(rng)
+        xdt = torch.float32 if rng.integers(0, 2) else torch.bfloat16
+        odt = torch.float32 if rng.integers(0, 3) else torch.bfloat16
+        use_bias = int(rng.integers(0, 3))  # 0 none, 1 fp32, 2 bf16
+        epi = "relu" if rng.integers(0, 3) == 0 else "none"
+        w = None
+        if fmt == "q4_0":
+            K = _pick_k(rng, 32)
+            lin = QLinear(K, N)
+            blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0] = sc & 0xFF
+            blocks[:, :, 1] = sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+            use_bias, epi, odt = 0, "none", torch.float32
+        elif fmt in ("w8", "w8a8"):
+            K = _pick_k(rng, 128 if (fmt == "w8a8" and rng.integers(0, 2)) else 16)
+            lin = W8Linear(K, N)
+            w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+            lin.set_weight(w, rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        elif fmt == "w4g":
+            group = int(rng.choice([128, 128, 64, 32]))
+            K = _pick_k(rng, 32)
+            G = -(-K // group)
+            q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+            z = rng.integers(0, 16, (N, G), dtype=np.uint8)
+            codes, zps = F.pack_w4g(q, z)
+            lin = W4GroupLinear(K, N, group)
+            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+        else:
+            K = _pick_k(rng, 16)
+            lin = FP8Linear(K, N)
+            wt = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).to(torch.float8_e4m3fn)
+            lin.set_weight(wt.view(torch.uint8).numpy(), 1.0 / 16)
+        tag = "%s M=%d K=%d N=%d x=%s y=%s bias=%d %s" % (fmt, M, K, N, str(xdt)[6:], str(odt)[6:], use_bias, epi)
+        deq = lin.dequantized_dev().double()
+        bias = None
+        if use_bias:
+            bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+            if use_bias == 2:
+                bias = bias.to(torch.bfloat16)
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
+
+        def fin(e):
+            if bias is not None:
+                e = e + bias.double()
+            return e.clamp_min(0) if epi == "relu" else e
+
+        if fmt == "q4_0":
+            _check(tag, lin.forward(x), x.double() @ deq.T, False)
+        elif fmt in ("w8", "w4g"):
+            y = lin.forward(x, bias=bias, epilogue=epi, out_dtype=odt)
+            _check(tag, y, fin(x.double() @ deq.T), odt == torch.bfloat16)
+        elif fmt == "fp8":
+            xc = x.float().to(torch.float8_e4m3fn)
+            sa = torch.tensor([0.125], dtype=torch.float32, device="cuda")
+            y = lin.forward(xc.view(torch.uint8), sa, bias=bias, epilogue=epi, out_dtype=odt)
+            _check(tag, y, fin(0.125 * (xc.double() @ deq.T)), odt == torch.bfloat16, 1e-2)
+        else:
+            xq, sx = quantize_rows_i8(x.float().contiguous())
+            wd = torch.from_numpy(w).cuda().double()
+            acc_exact = xq.double() @ wd.T  # exact: |acc| < 2^53
+            acc = lin.forward_a8(xq, sx, out_dtype=torch.int32)
+            assert bool((acc.double() == acc_exact).all()), tag + ": int32 accumulators differ"
+            # the channel scale, read back through the dequantised weights at a nonzero code
+            nz = wd.abs().argmax(dim=1)
+            rows = torch.arange(N, device="cuda")
+            sw = deq[rows, nz] / wd[rows, nz]
+            y = lin.forward_a8(xq, sx, bias=bias, epilogue=epi, out_dtype=odt)
+            _check(tag, y, fin(acc_exact * sx.double()[:, None] * sw[None, :]), odt == torch.bfloat16)
+        del lin
