@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define NQ_ABI_VERSION 2
+#define NQ_ABI_VERSION 3
 
 /* status codes */
 #define NQ_OK 0
@@ -206,6 +206,47 @@ int32_t nq_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int32_t
 int32_t nq_mlp3_w8a8_forward(nq_handle l1, nq_handle l2, nq_handle l3, const float* x, float* y,
                              int32_t M, const float* b1, const float* b2, const float* b3,
                              int32_t final_epilogue, void* stream);
+
+/* ---- GPTQ onto the Q4_0 grid (load time; noeira/nn/quant/gptq.mojo) ------------------------ */
+
+/* The calibration Hessian of one linear's inputs, H = sum x x^T in fp64, kept on the device:
+ * `HessianAccumulator` (noeira/nn/quant/hessian.mojo:24-77). */
+typedef struct nq_hessian_s* nq_hessian;
+
+/* An all-zero [n, n] Hessian (hessian.mojo:34-37). */
+int32_t nq_hessian_create(nq_hessian* out, int32_t n);
+int32_t nq_hessian_destroy(nq_hessian h);
+
+/* H += X^T X over the first `rows` rows of the device slab x [rows, n] (fp32 or bf16), the rows
+ * added in ascending order: `HessianAccumulator.add` (hessian.mojo:41-77) without the download. */
+int32_t nq_hessian_add(nq_hessian h, const void* x, int32_t x_dtype, int32_t rows, void* stream);
+
+/* Rows added so far (`HessianAccumulator.rows`). */
+int64_t nq_hessian_rows(nq_hessian h);
+
+/* Copy H out to / in from host memory ([n, n] fp64 row-major; `count` must be n * n).  `set` also
+ * sets the row count (a Hessian computed elsewhere, e.g. read from a fixture). */
+int32_t nq_hessian_get(nq_hessian h, double* out_host, int64_t count);
+int32_t nq_hessian_set(nq_hessian h, const double* h_host, int64_t count, int64_t rows);
+
+/* U, upper triangular with U^T U = h^-1, for h symmetric positive definite ([n, n] fp64 on the
+ * host, not modified), computed on the device: `hinv_upper_f64` (noeira/nn/quant/dense.mojo:355-363).
+ * Fails with NQ_ERR_INVALID and the pivot's index when h is not positive definite
+ * (dense.mojo:229-236). */
+int32_t nq_hinv_upper_f64(const double* h_host, int32_t n, double* u_host, void* stream);
+
+/* `gptq_q4_0` (noeira/nn/quant/gptq.mojo:62-150) followed by `pack_q4_0` and the upload: quantizes
+ * the host fp32 weight w [OUT, IN] of a Q4_0 layer column by column against the Hessian of the
+ * layer's inputs (not modified), and loads the layer with the result, as nq_set_weight_f32 does
+ * with round-to-nearest.  damp_frac: the damping as a fraction of mean(diag H) (the reference's
+ * default is 0.01).  dead_out / damp_out (may be NULL): `GPTQStats`. */
+int32_t nq_set_weight_gptq(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess,
+                           double damp_frac, int64_t* dead_out, double* damp_out, void* stream);
+
+/* `q4_0_objective` (gptq.mojo:152-189): tr((W - What) H (W - What)^T) in fp64 for the layer's
+ * current weights What against the host fp32 weight w [OUT, IN] they were quantized from. */
+int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess,
+                          double* out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -18,14 +18,15 @@ NQ_OK, NQ_ERR_INVALID, NQ_ERR_NOT_LOADED, NQ_ERR_NO_BLOCKS, NQ_ERR_SIZE, NQ_ERR_
 FMT_Q4_0, FMT_W8_CHANNEL, FMT_W4_GROUP, FMT_FP8_E4M3 = range(4)
 DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
 EPI_NONE, EPI_RELU = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 EXPORTS = [
     "nq_abi_version", "nq_last_error", "nq_create", "nq_destroy", "nq_set_blocks", "nq_set_weight_f32",
     "nq_set_weight_i8", "nq_set_weight_w4g", "nq_set_weight_fp8", "nq_blocks_bytes", "nq_get_blocks",
     "nq_keep_only_repacked", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
     "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward", "nq_fuse_rows", "nq_fused_parts",
-    "nq_forward_fused",
+    "nq_forward_fused", "nq_hessian_create", "nq_hessian_destroy", "nq_hessian_add", "nq_hessian_rows",
+    "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_set_weight_gptq", "nq_q4_0_objective",
 ]
 
 
@@ -119,6 +120,25 @@ def lib() -> C.CDLL:
     L.nq_fused_parts.argtypes = [p]
     L.nq_forward_fused.restype = i32
     L.nq_forward_fused.argtypes = [p, p, i32, p, C.POINTER(p), i32, i32, i32, p, i32, i32, p]
+    f64 = C.c_double
+    L.nq_hessian_create.restype = i32
+    L.nq_hessian_create.argtypes = [C.POINTER(p), i32]
+    L.nq_hessian_destroy.restype = i32
+    L.nq_hessian_destroy.argtypes = [p]
+    L.nq_hessian_add.restype = i32
+    L.nq_hessian_add.argtypes = [p, p, i32, i32, p]
+    L.nq_hessian_rows.restype = i64
+    L.nq_hessian_rows.argtypes = [p]
+    L.nq_hessian_get.restype = i32
+    L.nq_hessian_get.argtypes = [p, p, i64]
+    L.nq_hessian_set.restype = i32
+    L.nq_hessian_set.argtypes = [p, p, i64, i64]
+    L.nq_hinv_upper_f64.restype = i32
+    L.nq_hinv_upper_f64.argtypes = [p, i32, p, p]
+    L.nq_set_weight_gptq.restype = i32
+    L.nq_set_weight_gptq.argtypes = [p, p, i64, p, f64, C.POINTER(i64), C.POINTER(f64), p]
+    L.nq_q4_0_objective.restype = i32
+    L.nq_q4_0_objective.argtypes = [p, p, i64, p, C.POINTER(f64), p]
     got = L.nq_abi_version()
     if got != ABI_VERSION:
         raise OSError(f"{LIB_NAME}: ABI version {got}, this package binds version {ABI_VERSION}")

@@ -23,7 +23,7 @@ OBJ = os.path.join(HERE, "csrc", "_obj")
 LIB = os.path.join(HERE, "libnoeira_qlinear.so")
 ROOT = os.path.dirname(HERE)
 
-SOURCES = ["nq_api.hip", "nq_q4_0.hip", "nq_gemv.hip", "nq_quant.hip", "nq_gemm8.hip", "nq_gemm_a16.hip", "nq_mlp.hip", "nq_gemv_m1.hip", "nq_gemv_fp8.hip"]
+SOURCES = ["nq_api.hip", "nq_q4_0.hip", "nq_gemv.hip", "nq_quant.hip", "nq_gemm8.hip", "nq_gemm_a16.hip", "nq_mlp.hip", "nq_gemv_m1.hip", "nq_gemv_fp8.hip", "nq_gptq.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -31,6 +31,9 @@ FLAGS = [
     # packed-fp32 code generation is switched off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# GPTQ's codes depend on the last bit of every sum: its sums are written as separate multiplications and
+# additions, and must stay that way
+EXTRA_FLAGS = {"nq_gptq.hip": ["-ffp-contract=off"]}
 
 
 def _deps():
@@ -45,7 +48,7 @@ def _compile(src: str, force: bool) -> str:
     newest = max(os.path.getmtime(p) for p in [path] + _deps())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj
-    cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
+    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")

@@ -563,6 +563,184 @@ int32_t nq_grad_input(nq_handle h, const float* gy, float* gx, int32_t M, void* 
     return launch_grad_input_q4_0(h, gy, gx, M, (hipStream_t)stream);
 }
 
+// ---- GPTQ (load time) ------------------------------------------------------------------------
+struct nq_hessian_s {
+    uint32_t magic = 0x4E514853u;  // "NQHS"
+    int32_t n = 0;
+    int64_t rows = 0;
+    int device = -1;
+    double* d_h = nullptr;
+};
+
+static int32_t check_hessian(nq_hessian h, const char* what) {
+    if (!h || h->magic != 0x4E514853u) return fail(NQ_ERR_INVALID, std::string(what) + ": not a Hessian handle");
+    int dev = 0;
+    NQ_HIP(hipGetDevice(&dev));
+    if (dev != h->device)
+        return fail(NQ_ERR_INVALID, std::string(what) + ": the Hessian lives on device " + std::to_string(h->device) +
+                                        " but the current device is " + std::to_string(dev));
+    return NQ_OK;
+}
+
+int32_t nq_hessian_create(nq_hessian* out, int32_t n) {
+    if (!out) return fail(NQ_ERR_INVALID, "nq_hessian_create: null output handle");
+    *out = nullptr;
+    if (n <= 0) return fail(NQ_ERR_INVALID, "nq_hessian_create: n must be positive");
+    nq_hessian h = new (std::nothrow) nq_hessian_s();
+    if (!h) return fail(NQ_ERR_HIP, "nq_hessian_create: out of host memory");
+    h->n = n;
+    hipError_t e = hipGetDevice(&h->device);
+    if (e == hipSuccess) e = hipMalloc((void**)&h->d_h, (size_t)n * n * 8);
+    if (e == hipSuccess) e = hipMemset(h->d_h, 0, (size_t)n * n * 8);
+    if (e != hipSuccess) {
+        (void)hipFree(h->d_h);
+        delete h;
+        return fail_hip(e, "nq_hessian_create");
+    }
+    *out = h;
+    return NQ_OK;
+}
+
+int32_t nq_hessian_destroy(nq_hessian h) {
+    if (!h) return NQ_OK;
+    if (h->magic != 0x4E514853u) return fail(NQ_ERR_INVALID, "nq_hessian_destroy: not a Hessian handle");
+    (void)hipFree(h->d_h);
+    h->magic = 0;
+    delete h;
+    return NQ_OK;
+}
+
+int32_t nq_hessian_add(nq_hessian h, const void* x, int32_t x_dtype, int32_t rows, void* stream) {
+    int32_t rc = check_hessian(h, "HessianAccumulator.add");
+    if (rc) return rc;
+    if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "HessianAccumulator.add: the slab must be fp32 or bf16");
+    if (rows < 0) return fail(NQ_ERR_INVALID, "HessianAccumulator.add: rows must be >= 0");
+    if (rows == 0) return NQ_OK;
+    if (!x) return fail(NQ_ERR_INVALID, "HessianAccumulator.add: null slab");
+    rc = launch_hessian_add(h->d_h, h->n, x, x_dtype, rows, (hipStream_t)stream);
+    if (rc == NQ_OK) h->rows += rows;
+    return rc;
+}
+
+int64_t nq_hessian_rows(nq_hessian h) { return (h && h->magic == 0x4E514853u) ? h->rows : -1; }
+
+int32_t nq_hessian_get(nq_hessian h, double* out_host, int64_t count) {
+    int32_t rc = check_hessian(h, "nq_hessian_get");
+    if (rc) return rc;
+    if (!out_host || count != (int64_t)h->n * h->n)
+        return fail(NQ_ERR_SIZE, "nq_hessian_get: the buffer must hold n * n = " +
+                                     std::to_string((int64_t)h->n * h->n) + " values");
+    NQ_HIP(hipDeviceSynchronize());
+    NQ_HIP(hipMemcpy(out_host, h->d_h, (size_t)count * 8, hipMemcpyDeviceToHost));
+    return NQ_OK;
+}
+
+int32_t nq_hessian_set(nq_hessian h, const double* h_host, int64_t count, int64_t rows) {
+    int32_t rc = check_hessian(h, "nq_hessian_set");
+    if (rc) return rc;
+    if (!h_host || count != (int64_t)h->n * h->n)
+        return fail(NQ_ERR_SIZE, "nq_hessian_set: expected n * n = " + std::to_string((int64_t)h->n * h->n) +
+                                     " values");
+    NQ_HIP(hipDeviceSynchronize());
+    NQ_HIP(hipMemcpy(h->d_h, h_host, (size_t)count * 8, hipMemcpyHostToDevice));
+    h->rows = rows;
+    return NQ_OK;
+}
+
+int32_t nq_hinv_upper_f64(const double* h_host, int32_t n, double* u_host, void* stream) {
+    if (!h_host || !u_host || n <= 0) return fail(NQ_ERR_INVALID, "hinv_upper_f64: null matrix or n <= 0");
+    hipStream_t s = (hipStream_t)stream;
+    const size_t bytes = (size_t)n * n * 8;
+    double *hd = nullptr, *ud = nullptr;
+    int* status = nullptr;
+    hipError_t e = hipMalloc((void**)&hd, bytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&ud, bytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&status, 4);
+    const int big = 0x7FFFFFFF;
+    int pivot = big;
+    int32_t rc = NQ_OK;
+    if (e == hipSuccess) e = hipMemcpyAsync(hd, h_host, bytes, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(status, &big, 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) rc = launch_hinv_upper_f64(hd, n, ud, status, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipMemcpyAsync(u_host, ud, bytes, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipMemcpyAsync(&pivot, status, 4, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
+    (void)hipFree(hd), (void)hipFree(ud), (void)hipFree(status);
+    if (e != hipSuccess) return fail_hip(e, "hinv_upper_f64");
+    if (rc) return rc;
+    if (pivot != big)  // the factorization runs on the index-reversed matrix
+        return fail(NQ_ERR_INVALID, "cholesky_f64: not positive definite (pivot " + std::to_string(pivot) + ")");
+    return NQ_OK;
+}
+
+int32_t nq_set_weight_gptq(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess, double damp_frac,
+                           int64_t* dead_out, double* damp_out, void* stream) {
+    int32_t rc = check_handle(h, "nq_set_weight_gptq");
+    if (rc) return rc;
+    if (h->format != NQ_FMT_Q4_0) return fail(NQ_ERR_INVALID, "nq_set_weight_gptq: the layer's format is not Q4_0");
+    if ((rc = check_hessian(hess, "gptq_q4_0"))) return rc;
+    const int64_t want = (int64_t)h->in * h->out;
+    if (n_values < want || hess->n != h->in)  // gptq.mojo:80-83
+        return fail(NQ_ERR_SIZE, "gptq_q4_0: w or h is smaller than [n, k] / [k, k] (w holds " +
+                                     std::to_string(n_values) + " values, h is " + std::to_string(hess->n) + " x " +
+                                     std::to_string(hess->n) + ", the layer is [" + std::to_string(h->out) + ", " +
+                                     std::to_string(h->in) + "])");
+    if (!w_host) return fail(NQ_ERR_INVALID, "nq_set_weight_gptq: null weight");
+    if (!(damp_frac >= 0)) return fail(NQ_ERR_INVALID, "nq_set_weight_gptq: damp_frac must be >= 0");
+    hipStream_t s = (hipStream_t)stream;
+    h->loaded = false;
+    if ((rc = bind_device(h))) return rc;
+    const int64_t nbytes = logical_bytes(h);
+    const size_t hbytes = (size_t)h->in * h->in * 8;
+    float* wd = nullptr;
+    uint8_t* raw = nullptr;
+    double* hd = nullptr;
+    hipError_t e = hipMalloc((void**)&wd, (size_t)want * 4);
+    if (e == hipSuccess) e = hipMalloc((void**)&raw, (size_t)nbytes + 16);
+    if (e == hipSuccess) e = hipMalloc((void**)&hd, hbytes);
+    double stats[2] = {0, 0};
+    if (e == hipSuccess) e = hipMemcpyAsync(wd, w_host, (size_t)want * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(hd, hess->d_h, hbytes, hipMemcpyDeviceToDevice, s);  // gptq consumes its copy
+    if (e == hipSuccess) rc = run_gptq_q4_0(wd, h->out, h->in, hd, damp_frac, raw, stats, s);
+    if (e == hipSuccess && rc == NQ_OK) {
+        h->host_blocks.resize((size_t)nbytes);
+        e = hipMemcpyAsync(h->host_blocks.data(), raw, (size_t)nbytes, hipMemcpyDeviceToHost, s);
+    }
+    if (e == hipSuccess && rc == NQ_OK) rc = adopt_q4_0_blocks(h, raw, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
+    (void)hipFree(wd), (void)hipFree(raw), (void)hipFree(hd);
+    if (e != hipSuccess) return fail_hip(e, "nq_set_weight_gptq");
+    if (rc) return rc;
+    if (dead_out) *dead_out = (int64_t)stats[0];
+    if (damp_out) *damp_out = stats[1];
+    h->has_host_blocks = true;
+    h->loaded = true;
+    return NQ_OK;
+}
+
+int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess, double* out,
+                          void* stream) {
+    int32_t rc = check_handle(h, "nq_q4_0_objective");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "q4_0_objective"))) return rc;
+    if (h->format != NQ_FMT_Q4_0) return fail(NQ_ERR_INVALID, "nq_q4_0_objective: the layer's format is not Q4_0");
+    if ((rc = check_hessian(hess, "q4_0_objective"))) return rc;
+    const int64_t want = (int64_t)h->in * h->out;
+    if (n_values < want || hess->n != h->in || !w_host || !out)
+        return fail(NQ_ERR_SIZE, "q4_0_objective: w must hold [OUT, IN] values and h be [IN, IN]");
+    hipStream_t s = (hipStream_t)stream;
+    float *wd = nullptr, *deq = nullptr;
+    hipError_t e = hipMalloc((void**)&wd, (size_t)want * 4);
+    if (e == hipSuccess) e = hipMalloc((void**)&deq, (size_t)want * 4);
+    if (e == hipSuccess) e = hipMemcpyAsync(wd, w_host, (size_t)want * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) rc = launch_dequantize(h, deq, s);
+    if (e == hipSuccess && rc == NQ_OK) rc = run_q4_0_objective(wd, deq, h->out, h->in, hess->d_h, out, s);
+    (void)hipFree(wd), (void)hipFree(deq);
+    if (e != hipSuccess) return fail_hip(e, "nq_q4_0_objective");
+    return rc;
+}
+
 int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M, int32_t K,
                             void* stream) {
     if (M < 0 || K <= 0 || K % 4 != 0)

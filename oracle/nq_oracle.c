@@ -12,9 +12,11 @@
  *     noeira/io/safetensors.mojo:578   fp32 -> bf16 bits, ties to even
  *     noeira/nn/core/cpu_gemm.mojo:88  the Linux CPU GEMM (a triple loop)
  *     noeira/nn/quant/qlinear.mojo:416 QLinear.forward["cpu"] and vjp["cpu"]
+ *     noeira/nn/quant/gptq.mojo,       GPTQ onto the Q4_0 grid, the factor of H^-1 it
+ *       dense.mojo, hessian.mojo       reads, the calibration Hessian (load time)
  * and is pinned by the reference's own golden vectors
- * (tests/fixtures/quant/q4_0_rtn.safetensors) and by closed forms; see
- * tests/test_oracle_*.py.
+ * (tests/fixtures/quant/q4_0_rtn.safetensors, gptq_q4_0.safetensors) and by
+ * closed forms; see tests/test_oracle_*.py.
  *
  * Part 2 defines the formats BASELINE names that the reference does not
  * implement (int8 per-channel, int8 per-token activations, uint4 group-wise
@@ -336,6 +338,210 @@ void nqo_slice_cast_f32(const uint16_t* src, int64_t rows, int64_t cols, int64_t
     for (int64_t r = 0; r < rows; r++)
         for (int64_t c = 0; c < cols; c++)
             dst[r * cols + c] = nqo_bf16_bits_value(src[r * cols_pad + c]);
+}
+
+/* ------------------------------------------------------------------------ */
+/* GPTQ onto the Q4_0 grid (load time, off the forward path)                 */
+/* ------------------------------------------------------------------------ */
+
+/* dense.mojo:212-289: a (n x n row-major, symmetric positive definite, lower
+ * triangle read) becomes L with L L^T = a, upper triangle zeroed.  Returns 0,
+ * or 1 + the index of the first non-positive pivot.  Right-looking and blocked
+ * like the reference's (by CHOL_BLOCK columns: factor the diagonal block, solve
+ * the panel below it, subtract the panel's outer product from the trailing
+ * matrix), with every sum in one stated order: a dot product runs over the
+ * block's columns ascending from 0 and is subtracted once; the trailing update
+ * is c + (-1 * dot) (gemm_acc with alpha = -1, dense.mojo:54-124). */
+#define CHOL_BLOCK 64
+int64_t nqo_cholesky_f64(double* a, int64_t n) {
+    for (int64_t k0 = 0; k0 < n; k0 += CHOL_BLOCK) {
+        int64_t k1 = k0 + CHOL_BLOCK < n ? k0 + CHOL_BLOCK : n;
+        for (int64_t j = k0; j < k1; j++) {
+            double dot = 0;
+            for (int64_t t = k0; t < j; t++) dot += a[j * n + t] * a[j * n + t];
+            double s = a[j * n + j] - dot;
+            if (!(s > 0)) return j + 1;
+            double d = sqrt(s);
+            a[j * n + j] = d;
+            for (int64_t i = j + 1; i < k1; i++) {
+                dot = 0;
+                for (int64_t t = k0; t < j; t++) dot += a[i * n + t] * a[j * n + t];
+                a[i * n + j] = (a[i * n + j] - dot) / d;
+            }
+        }
+        for (int64_t i = k1; i < n; i++)
+            for (int64_t j = k0; j < k1; j++) {
+                double dot = 0;
+                for (int64_t t = k0; t < j; t++) dot += a[i * n + t] * a[j * n + t];
+                a[i * n + j] = (a[i * n + j] - dot) / a[j * n + j];
+            }
+        for (int64_t i = k1; i < n; i++)
+            for (int64_t j = k1; j <= i; j++) {
+                double dot = 0;
+                for (int64_t t = k0; t < k1; t++) dot += a[i * n + t] * a[j * n + t];
+                a[i * n + j] = a[i * n + j] + -1.0 * dot;
+            }
+    }
+    for (int64_t i = 0; i < n; i++)
+        for (int64_t j = i + 1; j < n; j++) a[i * n + j] = 0;
+    return 0;
+}
+
+/* dense.mojo:291-352: X = L^-1 by blocked forward substitution of L X = I:
+ * block row k is solved against L's diagonal block (each term subtracted in
+ * turn, q ascending, then the division), then subtracted from every row below
+ * as c + (-1 * dot over the block). */
+void nqo_tri_inv_lower_f64(const double* l, int64_t n, double* x) {
+    for (int64_t i = 0; i < n * n; i++) x[i] = 0;
+    for (int64_t i = 0; i < n; i++) x[i * n + i] = 1.0;
+    for (int64_t k0 = 0; k0 < n; k0 += CHOL_BLOCK) {
+        int64_t k1 = k0 + CHOL_BLOCK < n ? k0 + CHOL_BLOCK : n;
+        for (int64_t i = k0; i < k1; i++) {
+            for (int64_t q = k0; q < i; q++) {
+                double f = l[i * n + q];
+                for (int64_t j = 0; j < k1; j++) x[i * n + j] = x[i * n + j] - f * x[q * n + j];
+            }
+            double d = l[i * n + i];
+            for (int64_t j = 0; j < k1; j++) x[i * n + j] = x[i * n + j] / d;
+        }
+        for (int64_t i = k1; i < n; i++)
+            for (int64_t j = 0; j < k1; j++) {
+                double dot = 0;
+                for (int64_t q = k0; q < k1; q++) dot += l[i * n + q] * x[q * n + j];
+                x[i * n + j] = x[i * n + j] + -1.0 * dot;
+            }
+    }
+}
+
+static void reverse_f64(double* v, int64_t n) {
+    for (int64_t i = 0; i < n / 2; i++) {
+        double t = v[i];
+        v[i] = v[n - 1 - i];
+        v[n - 1 - i] = t;
+    }
+}
+
+/* dense.mojo:355-363: U upper triangular with U^T U = h^-1, as J chol(J h J)^-1 J
+ * (J reverses the indices: on a row-major n x n array, reversing the flat
+ * array).  h is consumed.  Returns nqo_cholesky_f64's status. */
+int64_t nqo_hinv_upper_f64(double* h, int64_t n, double* u) {
+    reverse_f64(h, n * n);
+    int64_t rc = nqo_cholesky_f64(h, n);
+    if (rc) return rc;
+    nqo_tri_inv_lower_f64(h, n, u);
+    reverse_f64(u, n * n);
+    return 0;
+}
+
+/* gptq.mojo:62-150.  w [n, k] fp32, h [k, k] fp64 (consumed) -> codes q [n, k],
+ * scales d [n, k/32] (bf16-rounded fp32).  Dead inputs (h_ii == 0): weights
+ * zeroed, diagonal 1.  Damping damp_frac * mean(diag).  U in fp64, rounded to
+ * fp32; the column loop in fp32, blocks of 128 columns, each row on its own:
+ *   at c % 32 == 0 the group's scale from the current weights; the code;
+ *   e = (w_c - deq) / U[c,c];  w[c .. block end) -= e * U[c, c .. block end);
+ *   after the block  w[block end ..) -= E @ U[block, block end ..)
+ * (dense.mojo:54-124 with alpha = -1: the sum over the block's columns in
+ * ascending order, then c + (-1 * sum)).  Multiplications and additions are
+ * separate roundings here (the file is compiled with -ffp-contract=off), as in
+ * the numpy transcription the reference's fixture was written by
+ * (tools/quant/gptq_q4_0_reference.py:57-86). */
+#define GPTQ_BLOCK 128
+int nqo_gptq_q4_0(const float* w, int64_t n, int64_t k, double* h, uint8_t* q, float* d, double damp_frac,
+                  int64_t* dead_out, double* damp_out) {
+    if (k % Q4_GROUP != 0) return NQO_ESIZE;
+    float* ww = (float*)malloc((size_t)(n * k) * sizeof(float));
+    double* u64 = (double*)malloc((size_t)(k * k) * sizeof(double));
+    float* u = (float*)malloc((size_t)(k * k) * sizeof(float));
+    float* err = (float*)malloc((size_t)GPTQ_BLOCK * sizeof(float));
+    if (!ww || !u64 || !u || !err) {
+        free(ww), free(u64), free(u), free(err);
+        return NQO_ESIZE;
+    }
+    for (int64_t i = 0; i < n * k; i++) ww[i] = w[i];
+    int64_t dead = 0;
+    double mean = 0;
+    for (int64_t i = 0; i < k; i++) {
+        if (h[i * k + i] == 0) {
+            dead++;
+            h[i * k + i] = 1.0;
+            for (int64_t r = 0; r < n; r++) ww[r * k + i] = 0;
+        }
+        mean += h[i * k + i];
+    }
+    double damp = damp_frac * mean / (double)k;
+    for (int64_t i = 0; i < k; i++) h[i * k + i] += damp;
+    if (dead_out) *dead_out = dead;
+    if (damp_out) *damp_out = damp;
+    if (nqo_hinv_upper_f64(h, k, u64)) {
+        free(ww), free(u64), free(u), free(err);
+        return NQO_ESIZE + 1; /* not positive definite */
+    }
+    for (int64_t i = 0; i < k * k; i++) u[i] = (float)u64[i];
+    int64_t groups = k / Q4_GROUP;
+    for (int64_t r = 0; r < n; r++) {
+        float* row = ww + r * k;
+        for (int64_t i1 = 0; i1 < k; i1 += GPTQ_BLOCK) {
+            int64_t i2 = i1 + GPTQ_BLOCK < k ? i1 + GPTQ_BLOCK : k;
+            float dg = 0;
+            for (int64_t c = i1; c < i2; c++) {
+                if (c % Q4_GROUP == 0) {
+                    dg = nqo_q4_0_group_scale(row + c);
+                    d[r * groups + c / Q4_GROUP] = dg;
+                }
+                float x = row[c];
+                uint8_t code = nqo_q4_0_code(x, dg);
+                q[r * k + c] = code;
+                float deq = ((float)(int)code - 8.0f) * dg;
+                float e = (x - deq) / u[c * k + c];
+                for (int64_t j = c; j < i2; j++) {
+                    float t = e * u[c * k + j];
+                    row[j] = row[j] - t;
+                }
+                err[c - i1] = e;
+            }
+            for (int64_t j = i2; j < k; j++) {
+                float acc = 0;
+                for (int64_t c = i1; c < i2; c++) {
+                    float t = err[c - i1] * u[c * k + j];
+                    acc = acc + t;
+                }
+                float t = -1.0f * acc;
+                row[j] = row[j] + t;
+            }
+        }
+    }
+    free(ww), free(u64), free(u), free(err);
+    return NQO_OK;
+}
+
+/* gptq.mojo:152-189: tr((W - What) H (W - What)^T) in fp64, What = (q - 8) d, H undamped. */
+double nqo_q4_0_objective(const float* w, const uint8_t* q, const float* d, int64_t n, int64_t k, const double* h) {
+    int64_t groups = k / Q4_GROUP;
+    double* delta = (double*)malloc((size_t)k * sizeof(double));
+    double s = 0;
+    for (int64_t r = 0; r < n; r++) {
+        for (int64_t c = 0; c < k; c++) {
+            double deq = ((double)(int)q[r * k + c] - 8.0) * (double)d[r * groups + c / Q4_GROUP];
+            delta[c] = (double)w[r * k + c] - deq;
+        }
+        for (int64_t j = 0; j < k; j++) {
+            double acc = 0;
+            for (int64_t c = 0; c < k; c++) acc += delta[c] * h[c * k + j];
+            s += acc * delta[j];
+        }
+    }
+    free(delta);
+    return s;
+}
+
+/* hessian.mojo:24-77: H += X^T X in fp64 over the first `rows` rows of x [rows, n] fp32. */
+void nqo_hessian_add(double* h, int64_t n, const float* x, int64_t rows) {
+    for (int64_t r = 0; r < rows; r++)
+        for (int64_t i = 0; i < n; i++) {
+            double xi = (double)x[r * n + i];
+            if (xi == 0) continue;
+            for (int64_t j = 0; j < n; j++) h[i * n + j] += xi * (double)x[r * n + j];
+        }
 }
 
 /* ======================================================================== */

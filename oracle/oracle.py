@@ -105,6 +105,18 @@ def lib() -> C.CDLL:
         for name in ("nqo_e4m3_encode_array", "nqo_f16_bits_array", "nqo_f16_value_array"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [p, i64, p]
+        L.nqo_cholesky_f64.restype = i64
+        L.nqo_cholesky_f64.argtypes = [p, i64]
+        L.nqo_tri_inv_lower_f64.restype = None
+        L.nqo_tri_inv_lower_f64.argtypes = [p, i64, p]
+        L.nqo_hinv_upper_f64.restype = i64
+        L.nqo_hinv_upper_f64.argtypes = [p, i64, p]
+        L.nqo_gptq_q4_0.restype = C.c_int
+        L.nqo_gptq_q4_0.argtypes = [p, i64, i64, p, p, p, C.c_double, p, p]
+        L.nqo_q4_0_objective.restype = C.c_double
+        L.nqo_q4_0_objective.argtypes = [p, p, p, i64, i64, p]
+        L.nqo_hessian_add.restype = None
+        L.nqo_hessian_add.argtypes = [p, i64, p, i64]
         _lib = L
     return _lib
 
@@ -202,6 +214,70 @@ def rtn_q4_0_blocks(w):
     if rc:
         raise ValueError("rtn_q4_0_blocks failed")
     return out
+
+
+# ── GPTQ (gptq.mojo, dense.mojo, hessian.mojo) ─────────────────────────────
+def cholesky_f64(a):
+    """L (lower, L L^T = a); raises at a non-positive pivot like dense.mojo:229-236."""
+    a = np.array(a, dtype=np.float64, order="C")
+    n = a.shape[0]
+    rc = lib().nqo_cholesky_f64(_ptr(a), n)
+    if rc:
+        raise ValueError(f"cholesky_f64: not positive definite (pivot {rc - 1})")
+    return a
+
+
+def tri_inv_lower_f64(l):
+    l = _c(l, np.float64)
+    x = np.empty_like(l)
+    lib().nqo_tri_inv_lower_f64(_ptr(l), l.shape[0], _ptr(x))
+    return x
+
+
+def hinv_upper_f64(h):
+    """U upper triangular with U^T U = h^-1 (dense.mojo:355-363)."""
+    h = np.array(h, dtype=np.float64, order="C")
+    u = np.empty_like(h)
+    rc = lib().nqo_hinv_upper_f64(_ptr(h), h.shape[0], _ptr(u))
+    if rc:
+        raise ValueError(f"hinv_upper_f64: not positive definite (pivot {rc - 1})")
+    return u
+
+
+def gptq_q4_0(w, h, damp_frac=0.01):
+    """(codes [n, k] u8, scales [n, k/32] f32, dead, damp) as gptq.mojo:62-150."""
+    w = _c(w, np.float32)
+    n, k = w.shape
+    if k % Q4_GROUP != 0:
+        raise ValueError(f"gptq_q4_0: k = {k} is not a multiple of 32")
+    h = np.array(h, dtype=np.float64, order="C")
+    if h.size < k * k:
+        raise ValueError("gptq_q4_0: w or h is smaller than [n, k] / [k, k]")
+    q = np.zeros((n, k), np.uint8)
+    d = np.zeros((n, k // Q4_GROUP), np.float32)
+    dead = C.c_int64(0)
+    damp = C.c_double(0)
+    rc = lib().nqo_gptq_q4_0(_ptr(w), n, k, _ptr(h), _ptr(q), _ptr(d), damp_frac, C.byref(dead), C.byref(damp))
+    if rc:
+        raise ValueError("gptq_q4_0: the damped Hessian is not positive definite")
+    return q, d, dead.value, damp.value
+
+
+def q4_0_objective(w, q, d, h) -> float:
+    w = _c(w, np.float32)
+    q = _c(q, np.uint8)
+    d = _c(d, np.float32)
+    h = _c(h, np.float64)
+    n, k = w.shape
+    return float(lib().nqo_q4_0_objective(_ptr(w), _ptr(q), _ptr(d), n, k, _ptr(h)))
+
+
+def hessian_add(h, x):
+    """h [n, n] f64 += x^T x for x [rows, n] f32, in place (hessian.mojo:41-77)."""
+    x = _c(x, np.float32)
+    assert h.dtype == np.float64 and h.flags.c_contiguous
+    lib().nqo_hessian_add(_ptr(h), h.shape[0], _ptr(x), x.shape[0])
+    return h
 
 
 def dequantize_q4_0(blocks, n, k):

@@ -1,0 +1,154 @@
+"""Pins the CPU oracle's GPTQ half (gptq.mojo, dense.mojo, hessian.mojo).
+
+Gates as the reference's own (tests/nn/quant/test_gptq.mojo [1]-[5],
+tests/nn/quant/test_cholesky.mojo), on the reference's own fixture
+(tests/fixtures/quant/gptq_q4_0.safetensors: two cases with w, h and the
+numpy transcription's q, d and objectives), plus numpy's LAPACK routines as the
+independent checker for the factorizations.
+"""
+import hashlib
+import os
+
+import numpy as np
+import pytest
+
+from noeira_amd.safetensors_io import SafeTensors
+from oracle import oracle as O
+
+FIX = "gptq_q4_0.safetensors"
+FIX_SHA256_PREFIX = "0d47dee5"
+
+
+@pytest.fixture(scope="module")
+def fix(golden_dir):
+    path = os.path.join(golden_dir, FIX)
+    digest = hashlib.sha256(open(path, "rb").read()).hexdigest()
+    assert digest.startswith(FIX_SHA256_PREFIX) and digest.endswith("c010a1")
+    f = SafeTensors(path)
+    return {c: dict(w=f.read_f32(c + ".w"), h=f.read_f32(c + ".h"), q=f.read(c + ".q"), d=f.read_f32(c + ".d"),
+                    obj=f.read_f32(c + ".obj")) for c in "ab"}
+
+
+def spd(rng, n, cond=1e4):
+    x = rng.standard_normal((3 * n, n)) * np.geomspace(1.0, np.sqrt(cond), n)[rng.permutation(n)]
+    return x.T @ x + 1e-3 * np.eye(n)
+
+
+# ── the factorizations against LAPACK (test_cholesky.mojo) ─────────────────
+@pytest.mark.parametrize("n", [1, 2, 7, 128, 129, 300])
+def test_cholesky_and_inverse_against_numpy(n):
+    rng = np.random.default_rng(n)
+    a = spd(rng, n)
+    l = O.cholesky_f64(a)
+    ref = np.linalg.cholesky(a)
+    assert np.array_equal(np.triu(l, 1), np.zeros_like(l))
+    assert np.abs(l - ref).max() <= 1e-11 * np.abs(ref).max()
+    x = O.tri_inv_lower_f64(l)
+    assert np.array_equal(np.triu(x, 1), np.zeros_like(x))
+    assert np.abs(x @ l - np.eye(n)).max() < 1e-9
+    u = O.hinv_upper_f64(a)
+    assert np.array_equal(np.tril(u, -1), np.zeros_like(u)) and (np.diag(u) > 0).all()
+    # U^T U = a^-1, and U is THE upper Cholesky factor of a^-1 (unique): numpy's chol(inv(a))^T
+    assert np.abs(u.T @ u @ a - np.eye(n)).max() < 1e-7
+    want = np.linalg.cholesky(np.linalg.inv(a)).T
+    assert np.abs(u - want).max() <= 1e-8 * np.abs(want).max()
+
+
+def test_cholesky_rejects_indefinite():
+    a = np.array([[1.0, 2.0], [2.0, 1.0]])
+    with pytest.raises(ValueError, match="pivot 1"):
+        O.cholesky_f64(a)
+
+
+def test_hinv_upper_diagonal_is_exact():
+    d = np.array([0.25, 4.0, 16.0, 1.0])
+    u = O.hinv_upper_f64(np.diag(d))
+    assert np.array_equal(u, np.diag(1.0 / np.sqrt(d)))
+
+
+def test_hessian_add_against_numpy():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((50, 24)).astype(np.float32)
+    x[:, 5] = 0
+    h = np.zeros((24, 24))
+    O.hessian_add(h, x[:20])
+    O.hessian_add(h, x[20:])
+    want = x.astype(np.float64).T @ x.astype(np.float64)
+    assert np.abs(h - want).max() <= 1e-12 * np.abs(want).max()
+    assert h[5, 5] == 0
+
+
+# ── [1] parity with the reference's fixture (test_gptq.mojo:47-82) ─────────
+@pytest.mark.parametrize("case", ["a", "b"])
+def test_gptq_parity_with_reference_fixture(fix, case):
+    c = fix[case]
+    w, h = c["w"], c["h"].astype(np.float64)
+    n, k = w.shape
+    q, d, dead, damp = O.gptq_q4_0(w, h)
+    assert dead == {"a": 3, "b": 2}[case]
+    assert damp == pytest.approx(0.01 * (np.trace(h) + dead) / k, rel=1e-12)
+    rows_same = (q == c["q"]).all(axis=1)
+    scale_bad = (d.view(np.uint32) != c["d"].view(np.uint32))[rows_same].sum()
+    obj = O.q4_0_objective(w, q, d, h)
+    rel = abs(obj - float(c["obj"][0])) / float(c["obj"][0])
+    # the reference's gate: objective within 1 %, >= 90 % of rows identical code for code, every scale
+    # identical in those rows
+    assert rel < 0.01, rel
+    assert rows_same.sum() * 10 >= n * 9, (int(rows_same.sum()), n)
+    assert scale_bad == 0
+
+
+# ── [2] a diagonal Hessian propagates nothing: GPTQ is RTN, bit for bit (test_gptq.mojo:90-113)
+def test_gptq_with_diagonal_hessian_is_rtn():
+    rng = np.random.default_rng(5)
+    n, k = 70, 288
+    w = ((rng.random((n, k)) - 0.5) * 0.3).astype(np.float32)
+    h = np.diag(0.1 + 10.0 * rng.random(k))
+    q, d, dead, _ = O.gptq_q4_0(w, h)
+    qr, dr = O.quantize_rtn_q4_0(w)
+    assert dead == 0
+    assert np.array_equal(q, qr) and np.array_equal(d.view(np.uint32), dr.view(np.uint32))
+
+
+# ── [3] objectives (test_gptq.mojo:115-135) ────────────────────────────────
+@pytest.mark.parametrize("case", ["a", "b"])
+def test_objectives(fix, case):
+    c = fix[case]
+    w, h = c["w"], c["h"].astype(np.float64)
+    qr, dr = O.quantize_rtn_q4_0(w)
+    o_rtn = O.q4_0_objective(w, qr, dr, h)
+    assert abs(o_rtn - float(c["obj"][1])) / float(c["obj"][1]) < 1e-6
+    # the objective itself against numpy, from the fixture's own codes
+    deq = (c["q"].astype(np.float64) - 8.0) * np.repeat(c["d"].astype(np.float64), 32, axis=1)
+    delta = w.astype(np.float64) - deq
+    want = float(np.sum((delta @ h) * delta))
+    assert O.q4_0_objective(w, c["q"], c["d"], h) == pytest.approx(want, rel=1e-12)
+    q, d, _, _ = O.gptq_q4_0(w, h)
+    assert O.q4_0_objective(w, q, d, h) < 0.85 * o_rtn
+
+
+# ── [4] rows are independent; runs repeat (test_gptq.mojo:137-163) ─────────
+def test_rows_independent_and_repeatable(fix):
+    w, h = fix["b"]["w"], fix["b"]["h"].astype(np.float64)
+    qa, da, _, _ = O.gptq_q4_0(w, h)
+    qb, db, _, _ = O.gptq_q4_0(w, h)
+    qs, ds, _, _ = O.gptq_q4_0(w[:40], h)
+    assert np.array_equal(qa, qb) and np.array_equal(da, db)
+    assert np.array_equal(qa[:40], qs) and np.array_equal(da[:40].view(np.uint32), ds.view(np.uint32))
+
+
+# ── [5] k not a multiple of 32 raises (test_gptq.mojo:165-173) ─────────────
+def test_k_not_multiple_of_32_raises():
+    with pytest.raises(ValueError, match="not a multiple of 32"):
+        O.gptq_q4_0(np.zeros((1, 40), np.float32), np.ones((40, 40)))
+
+
+def test_dead_inputs_are_zeroed_and_damping_is_relative(fix):
+    """Scaling H changes nothing (the damping is relative to it); a dead column's codes are the grid's zero."""
+    w, h = fix["a"]["w"], fix["a"]["h"].astype(np.float64)
+    q1, d1, dead, _ = O.gptq_q4_0(w, h)
+    q2, d2, _, _ = O.gptq_q4_0(w, h * 1024.0)   # a power of two: every quotient is unchanged, up to the dead 1s
+    dead_cols = np.diag(h) == 0
+    assert dead == dead_cols.sum() == 3
+    assert (q1[:, dead_cols] == 8).all()
+    assert (q1 == q2).mean() > 0.99
