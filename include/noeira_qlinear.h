@@ -207,6 +207,16 @@ int32_t nq_mlp3_w8a8_forward(nq_handle l1, nq_handle l2, nq_handle l3, const flo
                              int32_t M, const float* b1, const float* b2, const float* b3,
                              int32_t final_epilogue, void* stream);
 
+/* A frozen LoRA adapter's share, added into the base layer's output right after its forward:
+ *     y[T, OUT] += scale * (x[T, IN] @ A[IN, R_PAD]) @ B[R_PAD, OUT]
+ * `LoRAAdapter.forward_add` (noeira/nn/peft/lora.mojo:292-349).  a, b: the adapter's device
+ * parameters (`lora_A.val`, `lora_B.val`: fp32 row-major, rank-padded with zeros); scale:
+ * `LoRAAdapter.scale()` (alpha / R, or alpha / sqrt(R)); x: the base layer's own input, fp32 or
+ * bf16; y: its fp32 output.  One launch, no scratch; a merged adapter simply does not call it. */
+int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features, int32_t out_features,
+                            int32_t r_pad, float scale, const void* x, int32_t x_dtype, float* y, int32_t T,
+                            void* stream);
+
 /* ---- GPTQ onto the Q4_0 grid (load time; noeira/nn/quant/gptq.mojo) ------------------------ */
 
 /* The calibration Hessian of one linear's inputs, H = sum x x^T in fp64, kept on the device:

@@ -563,6 +563,18 @@ int32_t nq_grad_input(nq_handle h, const float* gy, float* gx, int32_t M, void* 
     return launch_grad_input_q4_0(h, gy, gx, M, (hipStream_t)stream);
 }
 
+int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features, int32_t out_features, int32_t r_pad,
+                            float scale, const void* x, int32_t x_dtype, float* y, int32_t T, void* stream) {
+    if (in_features <= 0 || out_features <= 0 || r_pad <= 0)
+        return fail(NQ_ERR_INVALID, "LoRAAdapter.forward_add: IN, OUT and R_PAD must be positive");
+    if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "LoRAAdapter.forward_add: x must be fp32 or bf16");
+    if (T < 0) return fail(NQ_ERR_INVALID, "LoRAAdapter.forward_add: T must be >= 0");
+    if (T == 0) return NQ_OK;
+    if (!a || !b || !x || !y) return fail(NQ_ERR_INVALID, "LoRAAdapter.forward_add: null pointer");
+    return launch_lora_add(x, x_dtype, a, b, y, T, in_features, out_features, r_pad, scale, (hipStream_t)stream);
+}
+
 // ---- GPTQ (load time) ------------------------------------------------------------------------
 struct nq_hessian_s {
     uint32_t magic = 0x4E514853u;  // "NQHS"

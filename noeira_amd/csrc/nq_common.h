@@ -132,6 +132,10 @@ int32_t launch_cast_pad_bf16(const float* src, uint16_t* dst, int32_t rows, int3
 int32_t launch_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int32_t cols,
                               int32_t cols_pad, hipStream_t s);
 
+// nq_lora.hip: y += s (x A) B
+int32_t launch_lora_add(const void* x, int32_t x_dtype, const float* A, const float* B, float* y, int32_t T, int32_t IN,
+                        int32_t OUT, int32_t R, float s, hipStream_t stream);
+
 // nq_gptq.hip: the calibration Hessian, the factor of its inverse, GPTQ's column loop, its objective
 int32_t launch_hessian_add(double* H, int n, const void* x, int32_t x_dtype, int rows, hipStream_t s);
 int32_t launch_hinv_upper_f64(double* h, int n, double* u, int* status_dev, hipStream_t s);

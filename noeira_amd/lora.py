@@ -1,0 +1,65 @@
+"""Host-side mirror of the reference's LoRA adapter for inference, over the C ABI.
+
+``LoRAAdapter`` keeps what `LoRAAdapter[IN, OUT, R, PAD_R, RSLORA]`
+(noeira/nn/peft/lora.mojo:152-349) needs to serve a frozen adapter beside a
+quantized linear: the rank-padded parameters on the device, ``alpha``,
+``scale()``, ``merged`` and ``forward_add``.  Training (``vjp_add``, the
+optimizer walks) and merging into an fp32 base weight are not part of the
+inference path and are not here.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from .qlinear import _TORCH_DT, _dev_ptr, _stream_ptr
+
+
+class LoRAAdapter:
+    """``s * (x A) B`` beside a linear [IN -> OUT]; A [IN, R_PAD], B [R_PAD, OUT] fp32, the logical R
+    columns / rows first and zeros after (lora.mojo:28-41)."""
+
+    def __init__(self, IN: int, OUT: int, R: int, PAD_R: int = 16, RSLORA: bool = False, alpha: float | None = None):
+        if R < 1 or PAD_R < 1:  # the comptime asserts of lora.mojo:198-199
+            raise L.NQError(L.NQ_ERR_INVALID, "LoRA rank must be at least 1" if R < 1 else "PAD_R must be at least 1")
+        self.IN, self.OUT, self.R, self.RSLORA = IN, OUT, R, RSLORA
+        self.R_PAD = (R + PAD_R - 1) // PAD_R * PAD_R
+        self.alpha = float(R if alpha is None else alpha)
+        self.merged = False
+        self.lora_A = torch.zeros((IN, self.R_PAD), dtype=torch.float32, device="cuda")
+        self.lora_B = torch.zeros((self.R_PAD, OUT), dtype=torch.float32, device="cuda")
+
+    def scale(self) -> float:
+        return self.alpha / math.sqrt(self.R) if self.RSLORA else self.alpha / self.R
+
+    def set_params(self, a, b):
+        """Load the logical blocks: a [IN, R], b [R, OUT] (the pad stays zero)."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        if a.shape != (self.IN, self.R) or b.shape != (self.R, self.OUT):
+            raise L.NQError(L.NQ_ERR_SIZE, f"LoRAAdapter.set_params: expected A [{self.IN}, {self.R}] and "
+                                           f"B [{self.R}, {self.OUT}]")
+        self.lora_A.zero_()
+        self.lora_B.zero_()
+        self.lora_A[:, :self.R] = torch.from_numpy(a).cuda()
+        self.lora_B[:self.R] = torch.from_numpy(b).cuda()
+
+    def forward_add(self, x: torch.Tensor, y: torch.Tensor):
+        """``y[T, OUT] += s * (x[T, IN] A) B``, called with the base linear's own input and output right
+        after its forward.  Nothing once merged (lora.mojo:292-303)."""
+        if self.merged:
+            return y
+        if x.dtype not in _TORCH_DT or not x.is_cuda or not x.is_contiguous() or x.numel() % self.IN:
+            raise L.NQError(L.NQ_ERR_INVALID, "LoRAAdapter.forward_add: x must be a contiguous fp32/bf16 device "
+                                              "tensor of [T, IN] values")
+        T = x.numel() // self.IN
+        if y.dtype != torch.float32 or not y.is_cuda or not y.is_contiguous() or y.numel() != T * self.OUT:
+            raise L.NQError(L.NQ_ERR_INVALID, "LoRAAdapter.forward_add: y must be the base layer's fp32 [T, OUT] output")
+        L.check(L.lib().nq_lora_forward_add(_dev_ptr(self.lora_A), _dev_ptr(self.lora_B), self.IN, self.OUT,
+                                            self.R_PAD, C.c_float(self.scale()), _dev_ptr(x), _TORCH_DT[x.dtype],
+                                            _dev_ptr(y), T, _stream_ptr()))
+        return y

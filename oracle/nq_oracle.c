@@ -12,6 +12,7 @@
  *     noeira/io/safetensors.mojo:578   fp32 -> bf16 bits, ties to even
  *     noeira/nn/core/cpu_gemm.mojo:88  the Linux CPU GEMM (a triple loop)
  *     noeira/nn/quant/qlinear.mojo:416 QLinear.forward["cpu"] and vjp["cpu"]
+ *     noeira/nn/peft/lora.mojo:292     LoRAAdapter.forward_add["cpu"]
  *     noeira/nn/quant/gptq.mojo,       GPTQ onto the Q4_0 grid, the factor of H^-1 it
  *       dense.mojo, hessian.mojo       reads, the calibration Hessian (load time)
  * and is pinned by the reference's own golden vectors
@@ -338,6 +339,20 @@ void nqo_slice_cast_f32(const uint16_t* src, int64_t rows, int64_t cols, int64_t
     for (int64_t r = 0; r < rows; r++)
         for (int64_t c = 0; c < cols; c++)
             dst[r * cols + c] = nqo_bf16_bits_value(src[r * cols_pad + c]);
+}
+
+/* noeira/nn/peft/lora.mojo:292-318 (the CPU branch of LoRAAdapter.forward_add):
+ * h[T, R] = x[T, IN] @ A[IN, R] (gemm_cpu, beta = 0), then
+ * y[T, OUT] = s * (h @ B[R, OUT]) + 1 * y (gemm_cpu with alpha = s, beta = 1).
+ * R is the padded rank the parameters hold; s the adapter's scale. */
+int nqo_lora_forward_add(const float* x, const float* a, const float* b, int64_t T, int64_t in, int64_t out,
+                         int64_t r, float s, float* y) {
+    float* h = (float*)malloc((size_t)(T * r > 0 ? T * r : 1) * sizeof(float));
+    if (!h) return NQO_ESIZE;
+    nqo_gemm_cpu(0, 0, T, r, in, 1.0f, x, in, a, r, 0.0f, h, r);
+    nqo_gemm_cpu(0, 0, T, out, r, s, h, r, b, out, 1.0f, y, out);
+    free(h);
+    return NQO_OK;
 }
 
 /* ------------------------------------------------------------------------ */

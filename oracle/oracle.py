@@ -105,6 +105,8 @@ def lib() -> C.CDLL:
         for name in ("nqo_e4m3_encode_array", "nqo_f16_bits_array", "nqo_f16_value_array"):
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [p, i64, p]
+        L.nqo_lora_forward_add.restype = C.c_int
+        L.nqo_lora_forward_add.argtypes = [p, p, p, i64, i64, i64, i64, f32, p]
         L.nqo_cholesky_f64.restype = i64
         L.nqo_cholesky_f64.argtypes = [p, i64]
         L.nqo_tri_inv_lower_f64.restype = None
@@ -214,6 +216,17 @@ def rtn_q4_0_blocks(w):
     if rc:
         raise ValueError("rtn_q4_0_blocks failed")
     return out
+
+
+def lora_forward_add(x, a, b, s, y):
+    """y[T, OUT] += s * (x[T, IN] @ a[IN, R]) @ b[R, OUT], in place, as lora.mojo:305-318."""
+    x, a, b = _c(x, np.float32), _c(a, np.float32), _c(b, np.float32)
+    assert y.dtype == np.float32 and y.flags.c_contiguous
+    T, IN = x.shape
+    R, OUT = b.shape
+    assert a.shape == (IN, R) and y.shape == (T, OUT)
+    lib().nqo_lora_forward_add(_ptr(x), _ptr(a), _ptr(b), T, IN, OUT, R, float(s), _ptr(y))
+    return y
 
 
 # ── GPTQ (gptq.mojo, dense.mojo, hessian.mojo) ─────────────────────────────

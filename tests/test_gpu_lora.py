@@ -1,0 +1,90 @@
+"""A frozen LoRA adapter beside a quantized linear (QLoRA inference), on the GPU
+through the C ABI, against the CPU oracle.
+
+Gates as the reference's tests/nn/quant/test_qlora.mojo and
+tests/nn/peft/test_lora.mojo [1]: B = 0 leaves the base layer's output bit for
+bit; with a nonzero B the result equals LoRA over deq(W) within the fp32 band
+(1e-5 of the largest reference value); rank padding is exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from noeira_amd import _lib as L
+from noeira_amd.lora import LoRAAdapter
+from noeira_amd.qlinear import QLinear
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+BAND = 1e-5
+
+
+def make(rng, IN, OUT, R, pad=16, zero_b=False):
+    ad = LoRAAdapter(IN, OUT, R, PAD_R=pad, alpha=2.0 * R)
+    bound = 1.0 / np.sqrt(IN)
+    a = ((rng.random((IN, R)) * 2 - 1) * bound).astype(np.float32)       # PEFT's init (lora.mojo:232-237)
+    b = np.zeros((R, OUT), np.float32) if zero_b else (rng.standard_normal((R, OUT)) * 0.05).astype(np.float32)
+    ad.set_params(a, b)
+    return ad, a, b
+
+
+# the reference's shapes (test_qlora.mojo:15-19): small, k / v, down; T = 7; plus one token and a prefill
+@pytest.mark.parametrize("IN,OUT,T,R", [(64, 96, 7, 4), (960, 320, 7, 16), (2560, 960, 7, 16),
+                                          (960, 2560, 1, 16), (960, 960, 135, 8), (64, 300, 33, 40)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_qlora_forward(IN, OUT, T, R, xdt):
+    rng = np.random.default_rng(IN + OUT + T + R)
+    w = (rng.standard_normal((OUT, IN)) * 0.05).astype(np.float32)
+    base = QLinear(IN, OUT)
+    base.set_weight(w)
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).to(xdt).cuda()
+    y_base = base.forward(x)
+    # B = 0: bit for bit the bare QLinear
+    ad0, _, _ = make(rng, IN, OUT, R, zero_b=True)
+    y0 = ad0.forward_add(x, y_base.clone())
+    assert torch.equal(y0, y_base)
+    # nonzero B: LoRA over deq(W) (qlora_common.mojo), oracle on the same inputs
+    ad, a, b = make(rng, IN, OUT, R)
+    assert ad.scale() == 2.0
+    y = ad.forward_add(x, y_base.clone()).cpu().numpy()
+    xf = x.float().cpu().numpy()
+    want = O.qlinear_forward_cpu(base.blocks(), IN, OUT, xf)
+    want = O.lora_forward_add(xf, a, b, ad.scale(), want)
+    assert O.rel_max(y, want) < BAND, O.rel_max(y, want)
+    # the adapter's share alone, against fp64
+    share = 2.0 * (xf.astype(np.float64) @ a.astype(np.float64)) @ b.astype(np.float64)
+    got = y.astype(np.float64) - y_base.cpu().numpy().astype(np.float64)
+    assert np.abs(got - share).max() <= 2e-6 * max(np.abs(share).max(), np.abs(y).max())
+
+
+def test_rank_padding_is_exact_and_rslora_scale():
+    rng = np.random.default_rng(3)
+    IN, OUT, T, R = 96, 70, 5, 3
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).cuda()
+    y0 = torch.from_numpy(rng.standard_normal((T, OUT)).astype(np.float32)).cuda()
+    padded, a, b = make(rng, IN, OUT, R, pad=16)
+    bare = LoRAAdapter(IN, OUT, R, PAD_R=1, alpha=2.0 * R)
+    bare.set_params(a, b)
+    assert padded.R_PAD == 16 and bare.R_PAD == 3
+    assert torch.equal(padded.forward_add(x, y0.clone()), bare.forward_add(x, y0.clone()))
+    rs = LoRAAdapter(IN, OUT, 4, RSLORA=True, alpha=8.0)
+    assert rs.scale() == 4.0 and LoRAAdapter(IN, OUT, 4, alpha=8.0).scale() == 2.0
+
+
+def test_merged_adapter_adds_nothing_and_errors():
+    rng = np.random.default_rng(4)
+    ad, _, _ = make(rng, 64, 32, 4)
+    x = torch.from_numpy(rng.standard_normal((2, 64)).astype(np.float32)).cuda()
+    y = torch.ones((2, 32), device="cuda")
+    ad.merged = True
+    assert torch.equal(ad.forward_add(x, y.clone()), y)
+    ad.merged = False
+    with pytest.raises(L.NQError, match="fp32"):
+        ad.forward_add(x, y.to(torch.bfloat16))
+    with pytest.raises(L.NQError, match=r"\[T, IN\]"):
+        ad.forward_add(x[:, :63].contiguous(), y)
+    with pytest.raises(L.NQError, match="rank"):
+        LoRAAdapter(64, 32, 0)
+    with pytest.raises(L.NQError, match="expected A"):
+        ad.set_params(np.zeros((64, 5), np.float32), np.zeros((4, 32), np.float32))

@@ -148,3 +148,23 @@ def test_fp8_forward_vs_numpy():
     assert np.abs(y64 - want).max() <= 1e-12 * np.abs(want).max()
     want_bf = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     assert np.array_equal(ybf, want_bf)
+
+
+# ── LoRA forward_add (lora.mojo:292-318) ───────────────────────────────────
+def test_lora_forward_add_against_numpy():
+    rng = np.random.default_rng(12)
+    T, IN, OUT, R = 4, 13, 7, 5
+    x = rng.standard_normal((T, IN)).astype(np.float32)
+    a = rng.standard_normal((IN, R)).astype(np.float32)
+    b = rng.standard_normal((R, OUT)).astype(np.float32)
+    y0 = rng.standard_normal((T, OUT)).astype(np.float32)
+    y = O.lora_forward_add(x, a, b, 0.4, y0.copy())
+    want = y0.astype(np.float64) + 0.4 * (x.astype(np.float64) @ a.astype(np.float64)) @ b.astype(np.float64)
+    assert np.abs(y - want).max() <= 1e-6 * np.abs(want).max()
+    # B = 0 is a no-op, bit for bit (test_lora.mojo [1]); a swapped A / B or a dropped scale is not
+    assert np.array_equal(O.lora_forward_add(x, a, np.zeros_like(b), 0.4, y0.copy()), y0)
+    assert np.abs(O.lora_forward_add(x, a, b, 1.0, y0.copy()) - want).max() > 1e-2
+    # rank padding is exact: zero columns of A / rows of B change nothing (lora.mojo:28-41)
+    ap = np.concatenate([a, np.zeros((IN, 11), np.float32)], axis=1)
+    bp = np.concatenate([b, np.zeros((11, OUT), np.float32)], axis=0)
+    assert np.array_equal(O.lora_forward_add(x, ap, bp, 0.4, y0.copy()), y)
