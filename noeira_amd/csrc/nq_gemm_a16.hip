@@ -35,7 +35,6 @@
 // the B operand of four MFMAs.
 #include <hip/hip_fp16.h>
 
-#include <cstdlib>
 
 #include "nq_common.h"
 
@@ -473,11 +472,6 @@ int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipSt
     return fail(NQ_ERR_INVALID, "nq_forward: no medium-M kernel of that tile shape");
 }
 
-int env_int(const char* name, int dflt) {
-    const char* v = std::getenv(name);
-    return v ? std::atoi(v) : dflt;
-}
-
 }  // namespace
 
 bool gemm_a16_applicable(const ForwardArgs& a) {
@@ -520,12 +514,10 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
         const int64_t wgs = (int64_t)((mt + mw - 1) / mw) * ((L->out + 16 * nw - 1) / (16 * nw));
         if (wgs >= (mw * nw == 8 ? 2048 : 128)) break;
     }
-    mw = env_int("NQ_A16_MW", mw), nw = env_int("NQ_A16_NW", nw);
     // K split: 8 wavefronts when there are more than 4 k-steps
     const int kstep = four_bit ? 128 : 64;
     const int nsteps = (L->in + kstep - 1) / kstep;
-    int kw = nsteps > 4 ? 8 : 4;
-    kw = env_int("NQ_A16_KW", kw);
+    const int kw = nsteps > 4 ? 8 : 4;
     dim3 grid((L->out + 16 * nw - 1) / (16 * nw), (a.M + 16 * mw - 1) / (16 * mw));
     switch (L->format) {
         case NQ_FMT_Q4_0:

@@ -23,7 +23,6 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
-#include <cstdlib>
 
 #include "nq_common.h"
 
@@ -340,11 +339,6 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(const GemvParams p) {
     }
 }
 
-int env_int(const char* name, int dflt) {
-    const char* v = std::getenv(name);
-    return v ? std::atoi(v) : dflt;
-}
-
 // lanes per row: the power of two that wastes the fewest lane slots, larger
 // (more rows in flight per byte) on ties broken towards more parallel waves.
 void choose_split(int nch, int N, int rpl_max, int* lpr_out, int* rpl_out, int* ri_out) {
@@ -415,9 +409,6 @@ int32_t launch_gemv(const ForwardArgs& a) {
                                             " exceeds the GEMV kernel's LDS tile (15360)");
     int lpr, rpl, ri;
     choose_split(p.nch, p.N, mt == 1 ? 4 : (mt == 2 ? 2 : 2), &lpr, &rpl, &ri);
-    lpr = env_int("NQ_GEMV_LPR", lpr);
-    rpl = env_int("NQ_GEMV_RPL", rpl);
-    ri = env_int("NQ_GEMV_RI", ri);
     p.lpr = lpr, p.ri = ri;
     const int qpc = epc / 4;
     p.psq = p.nch + ((9 - (p.nch % 8)) % 8);  // plane stride = 1 (mod 8) float4s: conflict-free staging

@@ -29,7 +29,6 @@
 // instructions per KB-row and the kernel issues little besides its loads.
 #include "nq_common.h"
 
-#include <cstdlib>
 
 namespace nq {
 
@@ -124,11 +123,6 @@ __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p
     }
 }
 
-
-int env_int(const char* name, int dflt) {
-    const char* v = std::getenv(name);
-    return v ? std::atoi(v) : dflt;
-}
 
 // ---- M = 1: one wavefront per weight row, coalesced loads, trace of the MFMA tile
 template <int CPL, int WAVES>
@@ -262,8 +256,8 @@ int32_t launch_gemv_fp8(const ForwardArgs& a) {
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     // one row: a wavefront per weight row once a row fills most of its 64 lanes (K >= 768)
     const int cpl = (L->in / 16 + 63) / 64;
-    if (row_kernel_fits(a) && (L->in % 128 != 0 || env_int("NQ_FP8V_ROW", 1))) {
-        const int waves = env_int("NQ_FP8V_WAVES", 8);
+    if (row_kernel_fits(a)) {
+        const int waves = 8;
         switch (cpl) {
             case 1: return launch_row<1>(p, waves, a.stream);
             case 2: return launch_row<2>(p, waves, a.stream);
@@ -283,7 +277,6 @@ int32_t launch_gemv_fp8(const ForwardArgs& a) {
     if (wgs < 128) kw = 16;
     while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
     if (kw == 16 && spw > 4) spw = 4;
-    kw = env_int("NQ_FP8V_KW", kw), spw = env_int("NQ_FP8V_SPW", spw);
     const dim3 grid((unsigned)wgs, (unsigned)((a.M + 15) / 16));
     switch (spw) {
         case 1: return launch_kw<1>(p, kw, grid, a.stream);

@@ -30,7 +30,6 @@
 // bits (tests/nn/quant/test_qlinear_gpu.mojo:96,128).
 #include <hip/hip_fp16.h>
 
-#include <cstdlib>
 
 #include "nq_common.h"
 
@@ -324,11 +323,6 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
 
 #undef XF
 
-int env_int(const char* name, int dflt) {
-    const char* v = std::getenv(name);
-    return v ? std::atoi(v) : dflt;
-}
-
 // Only the combinations the host picks are instantiated: at most 8 loads in flight per lane
 // (RPL x CPL), and at most 96 registers of x (CPL <= 3 when a chunk of x takes 32 registers).
 template <int FMT, int XDT, bool DOT2, int CPL>
@@ -417,10 +411,8 @@ int32_t launch_gemv_m1(const ForwardArgs& a) {
     // One row per lane group and one batch per wavefront: the most wavefronts, the shortest
     // dependency chain.  Measured best from 68 KB to 45 MB of weights (memory-level parallelism
     // comes from occupancy, not from rows per lane).
-    int rpl = 1, mult = 1;
-    lpr = env_int("NQ_M1_LPR", lpr);
-    rpl = env_int("NQ_M1_RPL", rpl);
-    mult = env_int("NQ_M1_MULT", mult);
+    int rpl = 1;
+    const int mult = 1;
     cpl = (p.nch + lpr - 1) / lpr;
     rpl = cpl <= 2 ? (rpl >= 4 ? 4 : (rpl >= 2 ? 2 : 1)) : (cpl <= 4 ? (rpl >= 2 ? 2 : 1) : 1);
     p.lpr = lpr;
