@@ -1,0 +1,113 @@
+"""The single-row GEMV over large 4-bit weights (megabytes of codes), through the C ABI,
+against fp64 products of the layer's dequantised weights (pinned bit for bit against the CPU
+oracle in tests/test_gpu_qlinear.py and tests/test_gpu_formats.py) and, at a size the oracle
+finishes in seconds, against the oracle's own forward.
+
+Bars: the reference's fp32 band for Q4_0 with fp32 activations (1e-5 of the largest reference
+value, tests/nn/quant/qlinear_common.mojo:39-45), 1e-3 of the output RMS otherwise; repeated
+calls return the same bits (test_qlinear_gpu.mojo:96,128).
+"""
+import numpy as np
+import pytest
+import torch
+
+from noeira_amd import formats as F
+from noeira_amd.qlinear import FusedRows, QLinear, W4GroupLinear
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def q4_layer(rng, K, N, scale_kind="uniform"):
+    lin = QLinear(K, N)
+    blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+    sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16)
+    if scale_kind == "signed":
+        sc *= rng.choice([-1.0, 1.0], sc.shape).astype(np.float16)
+    bits = sc.view(np.uint16)
+    blocks[:, :, 0] = bits & 0xFF
+    blocks[:, :, 1] = bits >> 8
+    lin.set_blocks(blocks.reshape(-1))
+    return lin
+
+
+# rows of 1 .. 8 KiB of codes; 11008 = 5.375 loads of a wavefront (a ragged last one); N off every tile size
+@pytest.mark.parametrize("K,N", [(2048, 2051), (4096, 1100), (4096, 4096), (11008, 777), (16384, 300), (8192, 1031)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_q4_0_large_single_row(K, N, xdt):
+    rng = np.random.default_rng(K + N)
+    lin = q4_layer(rng, K, N, "signed")
+    deq = lin.dequantized_dev().double()
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
+    y = lin.forward(x)
+    exact = x.double() @ deq.T
+    rel = float((y.double() - exact).abs().max() / exact.abs().max())
+    assert rel < 1e-5, rel
+    assert torch.equal(lin.forward(x), y)
+
+
+def test_q4_0_large_against_oracle_forward():
+    rng = np.random.default_rng(7)
+    K, N = 4096, 1024
+    lin = q4_layer(rng, K, N)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    y = lin.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    want = O.qlinear_forward_cpu(lin.blocks(), K, N, x)
+    assert O.rel_max(y, want) < 1e-5
+    exact = O.dense_forward_f64(O.dequantize_q4_0(lin.blocks().reshape(N, -1), N, K), x)
+    assert O.rel_max(y, exact.astype(np.float32)) < 1e-5
+
+
+@pytest.mark.parametrize("K,N,group", [(4096, 1500, 128), (2048, 2100, 64), (11008, 600, 128), (4096, 1030, 32),
+                                         (8192, 520, 256)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_w4_group_large_single_row(K, N, group, xdt):
+    rng = np.random.default_rng(K + N + group)
+    G = -(-K // group)
+    q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+    z = rng.integers(0, 16, (N, G), dtype=np.uint8)
+    codes, zps = F.pack_w4g(q, z)
+    lin = W4GroupLinear(K, N, group)
+    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+    deq = lin.dequantized_dev().double()
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    exact = x.double() @ deq.T + bias.double()
+    rms = float(exact.pow(2).mean().sqrt())
+    y = lin.forward(x, bias=bias)
+    assert float((y.double() - exact).abs().max()) < 1e-3 * rms
+    yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16)
+    want = (x.double() @ deq.T + bias.to(torch.bfloat16).double()).clamp_min(0)
+    assert float((yr.double() - want).abs().max()) <= 1e-3 * rms + 2.0 ** -8 * float(want.abs().max())
+
+
+def test_large_fused_rows_single_row():
+    """q | k | v of a 4096-wide model as one row-fused layer: every part equals its own forward."""
+    rng = np.random.default_rng(11)
+    K = 4096
+    parts = [q4_layer(rng, K, n) for n in (1024, 256, 260)]
+    fused = FusedRows(parts)
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).cuda()
+    outs = fused.forward(x)
+    for lin, y in zip(parts, outs):
+        want = lin.forward(x)
+        assert float((y - want).abs().max()) <= 2e-6 * float(want.abs().max())
+
+
+def test_nan_and_zero_scales_stay_local():
+    """A zero scale silences its group whatever the codes (qlinear.mojo:32-34); a NaN scale poisons its own
+    row only."""
+    rng = np.random.default_rng(13)
+    K, N = 4096, 1024
+    lin = QLinear(K, N)
+    blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+    bits = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+    bits[5, :] = 0          # row 5: all groups silent
+    bits[9, 17] = 0x7E01    # row 9: one NaN scale
+    blocks[:, :, 0] = bits & 0xFF
+    blocks[:, :, 1] = bits >> 8
+    lin.set_blocks(blocks.reshape(-1))
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).cuda()
+    y = lin.forward(x).cpu().numpy()[0]
+    assert y[5] == 0.0
+    assert np.isnan(y[9]) and np.isnan(y).sum() == 1
