@@ -115,6 +115,10 @@ int32_t launch_gemv_m1(const ForwardArgs& a);
 bool gemv_row4_applicable(const ForwardArgs& a);
 int32_t launch_gemv_row4(const ForwardArgs& a);
 
+// nq_gemv_row8.hip: 8-bit GEMV for one bf16 / fp32 activation row over a large weight, x staged in LDS
+bool gemv_row8_applicable(const ForwardArgs& a);
+int32_t launch_gemv_row8(const ForwardArgs& a);
+
 // nq_gemv_fp8.hip: fp8 x fp8 GEMV for 1..16 activation rows on the matrix cores
 bool gemv_fp8_applicable(const ForwardArgs& a);
 int32_t launch_gemv_fp8(const ForwardArgs& a);

@@ -111,3 +111,42 @@ def test_nan_and_zero_scales_stay_local():
     y = lin.forward(x).cpu().numpy()[0]
     assert y[5] == 0.0
     assert np.isnan(y[9]) and np.isnan(y).sum() == 1
+
+
+# ── 8-bit weights (int8 per-channel; fp8 is reached through the C ABI with bf16 / fp32 x only) ──
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4112, 1030), (8192, 600), (11008, 400), (16384, 260), (5120, 1500)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_w8_large_single_row(K, N, xdt):
+    from noeira_amd.qlinear import W8Linear
+    rng = np.random.default_rng(K * 7 + N)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    w[3, :] = -128  # the one code the symmetric range leaves out
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    lin = W8Linear(K, N)
+    lin.set_weight(w, s)
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    y = lin.forward(x, bias=bias)
+    exact = O.w8_forward_f64(w, s, x.float().cpu().numpy(), bias.cpu().numpy())
+    rms = np.sqrt((exact ** 2).mean())
+    assert np.abs(y.cpu().numpy() - exact).max() < 1e-3 * rms
+    assert torch.equal(lin.forward(x, bias=bias), y)
+    yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16).float().cpu().numpy()
+    want = np.maximum(O.w8_forward_f64(w, s, x.float().cpu().numpy(), bias.to(torch.bfloat16).float().cpu().numpy()), 0)
+    assert np.abs(yr - want).max() <= 1e-3 * rms + 2.0 ** -8 * np.abs(want).max()
+
+
+def test_w8_large_fused_rows_single_row():
+    from noeira_amd.qlinear import W8Linear
+    rng = np.random.default_rng(21)
+    K = 8192
+    parts = []
+    for n in (1024, 300, 260):
+        lin = W8Linear(K, n)
+        lin.set_weight(rng.integers(-127, 128, (n, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, n).astype(np.float32))
+        parts.append(lin)
+    fused = FusedRows(parts)
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    for lin, y in zip(parts, fused.forward(x)):
+        want = lin.forward(x)  # (the small parts alone take another kernel: same products, another order of sums)
+        assert float((y - want).abs().max()) <= 2e-6 * float(want.abs().max())
