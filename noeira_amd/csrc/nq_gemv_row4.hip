@@ -291,10 +291,11 @@ int32_t launch_one(const Row4Params& p, hipStream_t s) {
     return NQ_OK;
 }
 
-// One row per wavefront and eight wavefronts per workgroup measured best on every shape tried (more rows
-// per wavefront amortise the staging of x but leave fewer wavefronts to hide each other's waits).
+// One row per wavefront measured best on every shape tried (more rows per wavefront amortise the staging
+// of x but leave fewer wavefronts to hide each other's waits); 8 wavefronts per workgroup, 16 for fp32 x.
 template <int FMT, bool XF32, int CPL>
 int32_t launch_rpw(const Row4Params& p, hipStream_t s) {
+    if constexpr (XF32) return launch_one<FMT, XF32, CPL, 16, 1>(p, s);  // the three-term split of x: 16 rows share it
     return launch_one<FMT, XF32, CPL, 8, 1>(p, s);
 }
 
