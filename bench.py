@@ -152,6 +152,30 @@ def make_act_w8a16(M, copies, seed=2):
     return dict(step=step, bytes=nbytes, ops=ops, launches=2, keep=(sets, xs, bs, ys))
 
 
+def make_w8a16_one(K, N, copies, seed=9):
+    """One W8A16 linear at M = 1 (int8 weights, per-channel scales, bf16 activations, fp32 out)."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import W8Linear
+
+    rng = np.random.default_rng(seed)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    layers = []
+    for _ in range(copies):
+        lin = W8Linear(K, N)
+        lin.set_weight(w, s)
+        layers.append(lin)
+    x = bf16_t(rng.standard_normal((1, K))).cuda()
+    y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+
+    def step(i):
+        layers[i % copies].forward(x, out=y)
+
+    return dict(step=step, bytes=N * K + 4 * N + 2 * K + 4 * N, ops=2 * N * K, launches=1, keep=(layers, x, y))
+
+
 def make_q4_0(IN, OUT, M, copies, seed=3):
     """The reference's own layer: Q4_0 group 32, fp32 activations, fp32 out."""
     import numpy as np
@@ -413,6 +437,12 @@ def sweep(skip_large=False):
     if not skip_large:
         run("W8A8 int8 GEMM M=8192 K=4096 N=4096 (scales + bias epilogue, bf16 out)", make_w8a8_gemm, "mfma", "int8",
             M=8192, N=4096, calls=10)
+        # the dequant-GEMVs at a size where the HBM fraction means something (22 - 45 MB of codes)
+        c = max(1, COLD_BYTES // (4096 * 11008 // 2))
+        run("W4A16 g128 4096->11008 M=1 (cold)", make_w4g, "hbm", K=4096, N=11008, M=1, copies=c, calls=c)
+        run("ref Q4_0 g32 4096->11008 M=1 fp32 (cold)", make_q4_0, "hbm", IN=4096, OUT=11008, M=1, copies=c, calls=c)
+        run("W8A16 4096->11008 M=1 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, copies=max(1, c // 2),
+            calls=max(1, c // 2))
     return out
 
 
@@ -444,6 +474,18 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_all, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "configs 1 (M=100), 2 (M=256) and the reference's Q4_0 shapes at T=135, one call each per step"
+    elif which == "biggemv":
+        K, N = 4096, 11008
+        c = max(1, COLD_BYTES // (N * K // 2))
+        wls = [make_w4g(K=K, N=N, M=1, copies=c), make_q4_0(IN=K, OUT=N, M=1, copies=c),
+               make_w8a16_one(K=K, N=N, copies=max(1, c // 2))]
+
+        def step_big(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_big, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "W4A16 g128, Q4_0 (fp32 x) and W8A16 at 4096->11008, M=1, cold rotation, one call each per step"
     elif which == "actor":
         wl = make_actor_fused()
         name = "cfg3 W8A8 actor 64->256->256->8 M=4096, fused"
@@ -504,7 +546,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
@@ -522,7 +564,7 @@ def main():
     ensure_built()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy"):
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 

@@ -25,8 +25,10 @@
 //   - x is staged once per workgroup into LDS as bf16: bf16 input as it is, fp32 input as the
 //     three-term split hi + mid + lo (each term exact, together the fp32 value), one MFMA per
 //     term, so the products are the exact fp32 x times the exact code (the 1e-5 band of the
-//     reference's fp32 path).  Within a block of 64 chunks the chunk 4 c + m sits in slot
-//     16 m + c, which makes the operand reads of an MFMA one contiguous KiB (no bank conflicts).
+//     reference's fp32 path).  Within a block of 64 chunks the eight values lane (c, q) needs
+//     for MFMA m sit at byte 1024 m + 16 (c + 16 q): an MFMA's operand read is one KiB with lane l
+//     at byte 16 l, the only pattern a 128-bit LDS read serves without bank conflicts (a stride
+//     of 64 bytes between neighbouring lanes measured 46 % conflict cycles).
 //     Chunks past K read zeros of x; their scale is forced to 0.
 // Every load is unconditional from a clamped address and is requested before x is staged.  The cross-lane
 // sum is a fixed butterfly.
@@ -121,13 +123,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row4_kernel(const Row4Params 
 #pragma unroll
     for (int rr = 0; rr < RPW; rr++) fetch(row_first + rr, wv[rr], meta[rr]);
 
-    // ---- x -> LDS: 8 values per thread and step; 4 consecutive threads cover one chunk.  Chunk ch of a
-    // block of 64 goes to slot 16 (ch % 4) + ch / 4.
+    // ---- x -> LDS: 8 values per thread and step; 4 consecutive threads cover one chunk
     for (int e = tid; e < KPAD / 8; e += NTHR) {
         const int k0 = e * 8, kc = min(k0, p.K - 8);
         const uint32_t keep = k0 < p.K ? ~0u : 0u;
         const int ch = e >> 2, blk = ch >> 6, cin = ch & 63;
-        const int at = ((blk * 64 + 16 * (cin & 3) + (cin >> 2)) * 32 + 8 * (e & 3)) * 2;  // byte offset in a plane
+        // byte offset in a plane: MFMA m = cin % 4 of the block reads one KiB, lane (c = cin / 4, q = e % 4) its 16 bytes
+        const int at = blk * 4096 + (cin & 3) * 1024 + ((cin >> 2) + 16 * (e & 3)) * 16;
         float part;
         if constexpr (XF32) {
             const u32x4 r0 = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc);
@@ -219,13 +221,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row4_kernel(const Row4Params 
             f32x4 dd = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int m = 0; m < 4; m++) {
-                // chunk 64 j + 4 c + m sits in slot 64 j + 16 m + c: the lanes of an MFMA read one contiguous KiB
-                const int slot = j * 64 + 16 * m + c;
                 const u32x4 bop = nib_word_to_bf16(tw[m], magic);
                 if constexpr (!G128) dd = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
-                    const u32x4 aop = *reinterpret_cast<const u32x4*>(plane + t * KPAD * 2 + (slot * 32 + 8 * kq) * 2);
+                    // x under chunk 64 j + 4 c + m, values 8 q .. 8 q + 7: lane l reads bytes 16 l of the MFMA's KiB
+                    const u32x4 aop = *reinterpret_cast<const u32x4*>(plane + t * KPAD * 2 + j * 4096 + m * 1024 + lane * 16);
                     dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop), as_bf16x8(bop), dd, 0, 0, 0);
                 }
                 if constexpr (!G128) {
