@@ -27,8 +27,7 @@
 //     term, so the products are the exact fp32 x times the exact code (the 1e-5 band of the
 //     reference's fp32 path).  Within a block of 64 chunks the eight values lane (c, q) needs
 //     for MFMA m sit at byte 1024 m + 16 (c + 16 q): an MFMA's operand read is one KiB with lane l
-//     at byte 16 l, the only pattern a 128-bit LDS read serves without bank conflicts (a stride
-//     of 64 bytes between neighbouring lanes measured 46 % conflict cycles).
+//     at byte 16 l, the pattern a 128-bit LDS read serves without bank conflicts.
 //     Chunks past K read zeros of x; their scale is forced to 0.
 // Every load is unconditional from a clamped address and is requested before x is staged.  The cross-lane
 // sum is a fixed butterfly.
