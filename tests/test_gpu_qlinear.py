@@ -125,6 +125,22 @@ def test_forward_vs_oracle(layers, IN, OUT, T):
     assert np.array_equal(y.view(np.uint32), y2.view(np.uint32))
 
 
+@pytest.mark.parametrize("T", [48, 140, 1120])
+@pytest.mark.parametrize("IN,OUT", SHAPES)
+def test_forward_at_the_reference_bench_row_counts(layers, IN, OUT, T):
+    """The row counts of benchmarks/quant/bench_qint4_smolvla_shapes.mojo:64-70 (1, 5 and 40 observations of
+    28 tokens): every output element against an fp64 product, as that bench checks its kernel (its band is
+    2e-2, :81-83; this path meets the fp32 band)."""
+    ql, _, _, deq = layers[(IN, OUT)]
+    rng = np.random.default_rng(77 * T + IN + OUT)
+    xd = torch.from_numpy(gaussian(rng, (T, IN), 1.0)).cuda()
+    y = ql.forward(xd)
+    exact = xd.double() @ torch.from_numpy(deq).cuda().double().T
+    assert not bool(torch.isnan(y).any())
+    assert float((y.double() - exact).abs().max() / exact.abs().max()) < TOL_REF
+    assert torch.equal(ql.forward(xd), y)
+
+
 @pytest.mark.parametrize("IN,OUT", [(960, 960), (2560, 960)])
 def test_forward_bf16_activations(layers, IN, OUT):
     """bf16 x (W4A16): the products are still exact, so the fp32 band holds
