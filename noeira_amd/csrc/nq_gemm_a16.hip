@@ -35,6 +35,8 @@
 // the B operand of four MFMAs.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
+
 
 #include "nq_common.h"
 
@@ -85,13 +87,15 @@ __device__ __forceinline__ uint32_t ld1(const void* base, uint32_t off) {
     return *reinterpret_cast<const uint8_t*>(reinterpret_cast<const char*>(base) + off);
 }
 
-// eight 4-bit codes of one word (pair s = elements 2s, 2s+1 in nibbles s and s+4) -> bf16 16+q
-__device__ __forceinline__ u32x4 nib_word_to_bf16(uint32_t w) {
+// eight 4-bit codes of one word (pair s = elements 2s, 2s+1 in nibbles s and s+4) -> bf16 16+q.
+// `magic` is 0x41804180 (bf16 16.0 twice) held in a vector register whose value the compiler
+// cannot see, which makes it fuse the mask and the OR into one v_and_or_b32.
+__device__ __forceinline__ u32x4 nib_word_to_bf16(uint32_t w, uint32_t magic) {
     u32x4 r;
-    r[0] = ((w << 3) & 0x00780078u) | 0x41804180u;
-    r[1] = ((w >> 1) & 0x00780078u) | 0x41804180u;
-    r[2] = ((w >> 5) & 0x00780078u) | 0x41804180u;
-    r[3] = ((w >> 9) & 0x00780078u) | 0x41804180u;
+    r[0] = ((w << 3) & 0x00780078u) | magic;
+    r[1] = ((w >> 1) & 0x00780078u) | magic;
+    r[2] = ((w >> 5) & 0x00780078u) | magic;
+    r[3] = ((w >> 9) & 0x00780078u) | magic;
     return r;
 }
 
@@ -130,37 +134,56 @@ __device__ __forceinline__ void make_terms(const u32x4 (&raw)[XF32 ? 2 : 1], u32
 
 // One workgroup computes a [16 MW] x [16 NW] output tile; its KW wavefronts split K by
 // k-steps (wave w takes k-steps w, w + KW, ...).  Calls of this size are bound by how many
-// instructions one wavefront executes back to back and by how many cache lines its loads
-// touch, not by the matrix cores or by bytes, which shapes the kernel:
+// instructions one wavefront executes back to back and by what its loads cost in the L1
+// (a load instruction is priced by the number of separate pieces of cache line its lanes
+// touch, not by its bytes: 64 lanes reading 16 bytes each from 16 rows, the four lanes of a
+// row 16 lanes apart, take about 100 cycles of the L1; the same bytes with a row's lanes
+// adjacent about 45; two-byte loads cost as much as 16-byte ones), which shapes the kernel:
+//   - operands are loaded row-contiguously (a run of lanes per row) into registers one k-step
+//     ahead, and reach the MFMA operand layout through a private piece of LDS per wavefront:
+//     one 128-bit store and one 128-bit read per register quad, both free of bank conflicts
+//     (XOR swizzle of the 16-byte slot by the row), no barrier (LDS executes one wavefront's
+//     accesses in order);
 //   - a wavefront's activations are the large operand (2 or 4 bytes an element against half
 //     a byte or one byte of weight), so the tile is wide in N: every activation fragment,
 //     and for fp32 input its three-term split, is formed once for NW weight tiles;
-//   - all loads are issued one k-step ahead from clamped addresses (a fragment register is
-//     refilled as soon as it has been read), so a wavefront waits for memory once;
-//   - scale records come in as few loads as their alignment allows, since every load costs
-//     one cache-line look-up per weight row whatever its width;
+//   - scale records come in as few loads as their alignment allows;
 //   - the zero-point term enters the MFMA as its C operand, and where a whole k-step lies in
 //     one group (WHOLE) the scale is applied once per k-step instead of once per chunk.
 template <int FMT, bool XF32, int MW, int NW, int KW, bool WHOLE>
 __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL);
     constexpr int NT = XF32 ? 3 : 1;            // bf16 terms per activation
-    constexpr int NL = XF32 ? 2 : 1;            // 16-byte loads per activation fragment
+    constexpr int NL = XF32 ? 2 : 1;            // 16-byte pieces per activation fragment
     constexpr int ES = XF32 ? 4 : 2;            // bytes per activation
-    constexpr int KSTEP = FOUR_BIT ? 128 : 64;  // k covered by one 16-byte weight load per lane x 4 lanes
+    constexpr int KSTEP = FOUR_BIT ? 128 : 64;  // k covered by 64 bytes of a weight row
     constexpr int NMF = FOUR_BIT ? 4 : 2;       // MFMAs (32 k each) per k-step
     constexpr int NS = WHOLE ? 1 : 4;           // scale records per k-step and weight row
     constexpr int TA = MW * NW * 4;             // accumulator registers per lane
     constexpr int RED = TA * 64;                // floats one wavefront contributes to the reduction
     constexpr int EPW = (TA + KW - 1) / KW;     // accumulators one wavefront finishes
-    extern __shared__ float red[];              // [KW][RED]
+    // activations travel in units of 16 rows x XB bytes: NI loads, each RPI rows x XB bytes
+    constexpr int XB = (!FOUR_BIT && !XF32) ? 128 : 256;
+    constexpr int NU = KSTEP * ES / XB;  // units per k-step
+    constexpr int QU = NMF / NU;         // MFMA fragments per unit
+    constexpr int PPR = XB / 16;         // 16-byte pieces per row of a unit
+    constexpr int RPI = 64 / PPR;        // rows per load instruction
+    constexpr int NI = 16 / RPI;         // load instructions per unit
+    constexpr int KU = XB / ES;          // k per unit
+    constexpr int XS = 16 * XB;          // bytes of the activation staging area
+    constexpr int SCR = XS + NW * 1024;  // staging bytes per wavefront
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // max(KW SCR, KW RED floats)
+    float* red = reinterpret_cast<float*>(smem);                    // [KW][RED], after the K loop
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ln = lane & 15, kb = lane >> 4;
     const int n_base = blockIdx.x * (16 * NW);
     const int m_base = blockIdx.y * (16 * MW);
+    uint8_t* scr = smem + wave * SCR;
 
     const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    uint32_t magic = 0x41804180u;
+    asm volatile("" : "+v"(magic));
 
     f32x4 acc[MW][NW];
     f32x4 xacc[MW];  // W8 only: sum_k x_k over the wave's k-steps
@@ -171,14 +194,43 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         for (int j = 0; j < NW; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
     }
 
-    // byte offsets of this lane's rows (the host has checked that every operand is < 4 GiB)
-    uint32_t xoff[MW], woff[NW], soff[NW];
+    // ---- the lane's place in a load (row-contiguous) and in a fragment (MFMA layout)
+    // weights: lane -> row lane/4 of a 16-row tile, 16-byte piece lane%4 of the k-step's 64 bytes;
+    // staged at row * 64 + (piece ^ row/4) * 16 and read back as (row ln, piece kb)
+    const int wrow = lane >> 2, wpc = lane & 3;
+    const uint32_t w_st = XS + wrow * 64 + ((wpc ^ (wrow >> 2)) & 3) * 16;
+    const uint32_t w_rd = XS + ln * 64 + ((kb ^ (ln >> 2)) & 3) * 16;
+    // activations: lane -> row lane/PPR of the instruction's RPI rows, piece lane%PPR;
+    // staged at row * XB + (piece ^ f(row)) * 16 with f(row) = row (XB = 256) or row/2 (XB = 128)
+    const int trow = lane / PPR, tpc = lane % PPR;
+    auto swz = [](int row) { return XB == 256 ? row : (row >> 1); };
+    uint32_t x_st[NI], x_rd[QU][NL];
 #pragma unroll
-    for (int i = 0; i < MW; i++) xoff[i] = (uint32_t)min(m_base + 16 * i + ln, p.M - 1) * (uint32_t)p.K * ES;
+    for (int ii = 0; ii < NI; ii++) {
+        const int row = ii * RPI + trow;
+        x_st[ii] = row * XB + ((tpc ^ swz(row)) & (PPR - 1)) * 16;
+    }
+#pragma unroll
+    for (int qq = 0; qq < QU; qq++)
+#pragma unroll
+        for (int h = 0; h < NL; h++) {
+            // the piece that holds the first 8 k of fragment q of this lane (second half: + 4) within its unit
+            const int piece = FOUR_BIT ? (XF32 ? 8 * qq + 2 * kb + h : 4 * qq + kb)
+                                       : (XF32 ? 4 * kb + 2 * qq + h : 2 * kb + qq);
+            x_rd[qq][h] = ln * XB + ((piece ^ swz(ln)) & (PPR - 1)) * 16;
+        }
+
+    // byte offsets of the rows this lane loads (the host has checked that every operand is < 4 GiB)
+    uint32_t xoff[MW][NI], woff[NW], soff[NW];
+#pragma unroll
+    for (int i = 0; i < MW; i++)
+#pragma unroll
+        for (int ii = 0; ii < NI; ii++)
+            xoff[i][ii] = (uint32_t)min(m_base + 16 * i + ii * RPI + trow, p.M - 1) * (uint32_t)p.K * ES;
 #pragma unroll
     for (int j = 0; j < NW; j++) {
+        woff[j] = (uint32_t)min(n_base + 16 * j + wrow, p.N - 1) * (uint32_t)p.nch * 16u;
         const uint32_t n = (uint32_t)min(n_base + 16 * j + ln, p.N - 1);
-        woff[j] = n * (uint32_t)p.nch * 16u;
         soff[j] = n * (uint32_t)(FMT == NQ_FMT_Q4_0 ? p.nch : p.groups);  // in elements
     }
 
@@ -200,28 +252,30 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
 
     // ---- loaders: unconditional, from clamped addresses; what lies past K is multiplied by a
-    // zero scale (4-bit formats) or replaced by zero activations (W8)
+    // zero scale (4-bit formats) and meets zero activations
     auto load_w = [&](int ks, u32x4 (&dst)[NW]) {
-        const uint32_t c = (uint32_t)min(ks * 4 + kb, p.nch - 1) * 16u;  // the 16-byte chunk this lane loads
+        const uint32_t c = (uint32_t)min(ks * 4 + wpc, p.nch - 1) * 16u;  // the 16-byte chunk this lane loads
 #pragma unroll
         for (int j = 0; j < NW; j++) dst[j] = ld16(p.codes, woff[j] + c);
     };
-    // scale records of a k-step: fp16 scale | zero point << 16
-    auto load_s = [&](int ks, uint32_t (&dst)[NW][NS]) {
+    // Scale records of a k-step.  The loads return raw registers and nothing is computed from them
+    // here: an instruction that uses a loaded value right away would make the wavefront wait out
+    // the whole memory latency at the point of the prefetch.  decode_s turns them into
+    // fp16 scale | zero point << 16 when the k-step is consumed.
+    constexpr int NR = FMT == NQ_FMT_Q4_0 ? 4 : FMT == NQ_FMT_W4_GROUP ? 2 * NS : 1;
+    auto load_s = [&](int ks, uint32_t (&dst)[NW][NR]) {
         if constexpr (FMT == NQ_FMT_Q4_0) {
             if (p.s_pairs) {  // rows are 4- or 8-byte aligned (the last load may run 4 bytes past a row)
                 const uint32_t c0 = (uint32_t)min(ks, nsteps - 1) * 8u;
 #pragma unroll
                 for (int j = 0; j < NW; j++) {
-                    uint32_t v0, v1;
                     if (p.s_pairs == 2) {
                         const u32x2 v = *reinterpret_cast<const u32x2*>(reinterpret_cast<const char*>(p.scales) +
                                                                         (soff[j] * 2u + c0));
-                        v0 = v[0], v1 = v[1];
+                        dst[j][0] = v[0], dst[j][1] = v[1];
                     } else {
-                        v0 = ld4(p.scales, soff[j] * 2u + c0), v1 = ld4(p.scales, soff[j] * 2u + c0 + 4u);
+                        dst[j][0] = ld4(p.scales, soff[j] * 2u + c0), dst[j][1] = ld4(p.scales, soff[j] * 2u + c0 + 4u);
                     }
-                    dst[j][0] = v0 & 0xFFFFu, dst[j][1] = v0 >> 16, dst[j][2] = v1 & 0xFFFFu, dst[j][3] = v1 >> 16;
                 }
             } else {
 #pragma unroll
@@ -237,18 +291,37 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
                 const int cc = min(ks * 4 + q, p.nch - 1);
                 const uint32_t g = (uint32_t)(((float)cc + 0.5f) * p.inv_cpg);  // cc / chunks per group
 #pragma unroll
-                for (int j = 0; j < NW; j++)
-                    dst[j][q] = ld2(p.scales, (soff[j] + g) * 2u) | (ld1(p.zps, soff[j] + g) << 16);
+                for (int j = 0; j < NW; j++) {
+                    dst[j][2 * q] = ld2(p.scales, (soff[j] + g) * 2u);
+                    dst[j][2 * q + 1] = ld1(p.zps, soff[j] + g);
+                }
             }
         }
     };
-    auto k_of = [&](int ks, int q) { return FOUR_BIT ? ks * 128 + q * 32 + kb * 8 : ks * 64 + kb * 16 + q * 8; };
-    auto load_x = [&](int ks, int q, int i, u32x4 (&dst)[NL]) {
-        int k0 = k_of(ks, q);
+    auto decode_s = [&](const uint32_t (&raw)[NW][NR], uint32_t (&sc)[NW][NS]) {
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            if constexpr (FMT == NQ_FMT_Q4_0) {
+                if (p.s_pairs) {
+                    sc[j][0] = raw[j][0] & 0xFFFFu, sc[j][1] = raw[j][0] >> 16;
+                    sc[j][2] = raw[j][1] & 0xFFFFu, sc[j][3] = raw[j][1] >> 16;
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) sc[j][q] = raw[j][q];
+                }
+            } else if constexpr (FMT == NQ_FMT_W4_GROUP) {
+#pragma unroll
+                for (int q = 0; q < NS; q++) sc[j][q] = raw[j][2 * q] | (raw[j][2 * q + 1] << 16);
+            }
+        }
+    };
+    // (a piece can lie past K only in a k-step that K cuts short: its address is clamped here
+    // and its value replaced by zero when the registers are staged)
+    auto load_x = [&](int ks, int i, int u, u32x4 (&dst)[NI]) {
+        int k0 = ks * KSTEP + u * KU + tpc * (16 / ES);
         if (k0 >= p.K) k0 = 0;
-        const uint32_t o = xoff[i] + (uint32_t)k0 * ES;
-        dst[0] = ld16(p.x, o);
-        if constexpr (XF32) dst[1] = ld16(p.x, o + 16u);
+#pragma unroll
+        for (int ii = 0; ii < NI; ii++) dst[ii] = ld16(p.x, xoff[i][ii] + (uint32_t)k0 * ES);
     };
     auto scale_of = [&](uint32_t rec, bool valid) {
         return valid ? __half2float(__ushort_as_half((uint16_t)(rec & 0xFFFFu))) : 0.0f;
@@ -256,29 +329,32 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     auto zero_of = [&](uint32_t rec) {  // 16 (the conversion offset) + the zero point
         return (FMT == NQ_FMT_Q4_0) ? 24.0f : 16.0f + (float)(rec >> 16);
     };
+    auto lds16 = [&](uint32_t off) -> u32x4& { return *reinterpret_cast<u32x4*>(scr + off); };
 
     u32x4 wv[NW];
-    uint32_t sv[NW][NS];
-    u32x4 xr[MW][NMF][NL];
+    uint32_t sv[NW][NR];
+    u32x4 xr[MW][NU][NI];
     load_w(wave, wv);
 #pragma unroll
-    for (int q = 0; q < NMF; q++)
+    for (int u = 0; u < NU; u++)
 #pragma unroll
-        for (int i = 0; i < MW; i++) load_x(wave, q, i, xr[i][q]);
+        for (int i = 0; i < MW; i++) load_x(wave, i, u, xr[i][u]);
     load_s(wave, sv);
 
     for (int ks = wave; ks < nsteps; ks += KW) {
-        const int kn = ks + KW;  // the k-step the registers are refilled for
+        const int kn = ks + KW;  // the k-step the registers are refilled for, if there is one
+        const bool more = kn < nsteps;
         u32x4 wc[NW];
         uint32_t sc[NW][NS];
 #pragma unroll
-        for (int j = 0; j < NW; j++) {
-            wc[j] = wv[j];
-#pragma unroll
-            for (int q = 0; q < NS; q++) sc[j][q] = sv[j][q];
+        for (int j = 0; j < NW; j++) lds16(w_st + j * 1024) = wv[j];
+        decode_s(sv, sc);
+        if (more) {
+            load_w(kn, wv);
+            load_s(kn, sv);
         }
-        load_w(kn, wv);
-        load_s(kn, sv);
+#pragma unroll
+        for (int j = 0; j < NW; j++) wc[j] = lds16(w_rd + j * 1024);
 
         if constexpr (FOUR_BIT) {
             // ---- transpose words among the four lanes (kb = 0..3) that share a row
@@ -291,62 +367,70 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
                 auto t23 = __builtin_amdgcn_permlane16_swap(wc[j][2], wc[j][3], false, false);
                 wc[j][0] = t01[0], wc[j][1] = t01[1], wc[j][2] = t23[0], wc[j][3] = t23[1];
             }
-            if constexpr (WHOLE) {
-                // one group for the whole k-step: sum the four chunks in the MFMA accumulator
-                f32x4 xs[MW], pp[MW][NW];
+        }
+
+        // WHOLE: one group for the whole k-step, the four chunks are summed in the MFMA accumulator
+        f32x4 xs_w[MW], pp_w[MW][NW];
+        if constexpr (FOUR_BIT && WHOLE) {
 #pragma unroll
-                for (int i = 0; i < MW; i++) {
-                    xs[i] = (f32x4){0, 0, 0, 0};
+            for (int i = 0; i < MW; i++) {
+                xs_w[i] = (f32x4){0, 0, 0, 0};
 #pragma unroll
-                    for (int j = 0; j < NW; j++) pp[i][j] = (f32x4){0, 0, 0, 0};
+                for (int j = 0; j < NW; j++) pp_w[i][j] = (f32x4){0, 0, 0, 0};
+            }
+        }
+
+#pragma unroll
+        for (int u = 0; u < NU; u++) {
+            // ---- the unit's activations: registers -> staging -> fragments; refill the registers
+            u32x4 fr[MW][QU][NL];
+#pragma unroll
+            for (int i = 0; i < MW; i++) {
+                if ((ks + 1) * KSTEP > p.K) {  // uniform over the wavefront
+                    const bool in = ks * KSTEP + u * KU + tpc * (16 / ES) < p.K;
+#pragma unroll
+                    for (int ii = 0; ii < NI; ii++) xr[i][u][ii] = in ? xr[i][u][ii] : (u32x4){0, 0, 0, 0};
                 }
 #pragma unroll
-                for (int q = 0; q < NMF; q++) {
-                    const bool kvalid = k_of(ks, q) < p.K;  // the last group may be cut short by K
-                    u32x4 bop[NW];
+                for (int ii = 0; ii < NI; ii++) lds16(x_st[ii]) = xr[i][u][ii];
+                if (more) load_x(kn, i, u, xr[i][u]);
 #pragma unroll
-                    for (int j = 0; j < NW; j++) bop[j] = nib_word_to_bf16(wc[j][q]);
+                for (int qq = 0; qq < QU; qq++)
 #pragma unroll
-                    for (int i = 0; i < MW; i++) {
-                        u32x4 raw[NL], at[NT];
+                    for (int h = 0; h < NL; h++) fr[i][qq][h] = lds16(x_rd[qq][h]);
+            }
 #pragma unroll
-                        for (int t = 0; t < NL; t++) raw[t] = kvalid ? xr[i][q][t] : (u32x4){0, 0, 0, 0};
-                        load_x(kn, q, i, xr[i][q]);  // refill
-                        make_terms<XF32>(raw, at);
+            for (int qq = 0; qq < QU; qq++) {
+                const int q = u * QU + qq;
+                u32x4 bop[NW];
+                if constexpr (FOUR_BIT) {
 #pragma unroll
-                        for (int t = 0; t < NT; t++) {
-                            xs[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xs[i],
-                                                                             0, 0, 0);
+                    for (int j = 0; j < NW; j++) bop[j] = nib_word_to_bf16(wc[j][q], magic);
+                } else {
 #pragma unroll
-                            for (int j = 0; j < NW; j++)
-                                pp[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]),
-                                                                                   pp[i][j], 0, 0, 0);
-                        }
+                    for (int j = 0; j < NW; j++) {
+                        uint32_t b0, b1, b2, b3;
+                        i8_word_to_bf16(wc[j][2 * q], b0, b1);
+                        i8_word_to_bf16(wc[j][2 * q + 1], b2, b3);
+                        bop[j] = (u32x4){b0, b1, b2, b3};
                     }
                 }
+                const bool cvalid = ks * 4 + q < p.nch;  // (activations past K arrive as zeros)
 #pragma unroll
-                for (int j = 0; j < NW; j++) {
-                    const float cs = scale_of(sc[j][0], true), cz = zero_of(sc[j][0]);
+                for (int i = 0; i < MW; i++) {
+                    u32x4 at[NT];
+                    make_terms<XF32>(fr[i][qq], at);
+                    if constexpr (FOUR_BIT && WHOLE) {
 #pragma unroll
-                    for (int i = 0; i < MW; i++)
+                        for (int t = 0; t < NT; t++) {
+                            xs_w[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones),
+                                                                               xs_w[i], 0, 0, 0);
 #pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            acc[i][j][r] = fmaf(cs, fmaf(-cz, xs[i][r], pp[i][j][r]), acc[i][j][r]);
-                }
-            } else {
-#pragma unroll
-                for (int q = 0; q < NMF; q++) {
-                    const bool cvalid = ks * 4 + q < p.nch;
-                    u32x4 bop[NW];
-#pragma unroll
-                    for (int j = 0; j < NW; j++) bop[j] = nib_word_to_bf16(wc[j][q]);
-#pragma unroll
-                    for (int i = 0; i < MW; i++) {
-                        u32x4 raw[NL], at[NT];
-#pragma unroll
-                        for (int t = 0; t < NL; t++) raw[t] = xr[i][q][t];
-                        load_x(kn, q, i, xr[i][q]);  // refill
-                        make_terms<XF32>(raw, at);
+                            for (int j = 0; j < NW; j++)
+                                pp_w[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                    as_bf16x8(at[t]), as_bf16x8(bop[j]), pp_w[i][j], 0, 0, 0);
+                        }
+                    } else if constexpr (FOUR_BIT) {
                         f32x4 xs = {0, 0, 0, 0};
 #pragma unroll
                         for (int t = 0; t < NT; t++)
@@ -367,38 +451,30 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 #pragma unroll
                             for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf(cs, pp[r], acc[i][j][r]);
                         }
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones),
+                                                                              xacc[i], 0, 0, 0);
+#pragma unroll
+                            for (int j = 0; j < NW; j++)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]),
+                                                                                    acc[i][j], 0, 0, 0);
+                        }
                     }
                 }
             }
-        } else {
+        }
+
+        if constexpr (FOUR_BIT && WHOLE) {
 #pragma unroll
-            for (int q = 0; q < NMF; q++) {
-                const bool kvalid = k_of(ks, q) < p.K;
-                u32x4 bop[NW];
+            for (int j = 0; j < NW; j++) {
+                const float cs = scale_of(sc[j][0], true), cz = zero_of(sc[j][0]);
 #pragma unroll
-                for (int j = 0; j < NW; j++) {
-                    uint32_t b0, b1, b2, b3;
-                    i8_word_to_bf16(wc[j][2 * q], b0, b1);
-                    i8_word_to_bf16(wc[j][2 * q + 1], b2, b3);
-                    bop[j] = (u32x4){b0, b1, b2, b3};
-                }
+                for (int i = 0; i < MW; i++)
 #pragma unroll
-                for (int i = 0; i < MW; i++) {
-                    u32x4 raw[NL], at[NT];
-#pragma unroll
-                    for (int t = 0; t < NL; t++) raw[t] = kvalid ? xr[i][q][t] : (u32x4){0, 0, 0, 0};
-                    load_x(kn, q, i, xr[i][q]);
-                    make_terms<XF32>(raw, at);
-#pragma unroll
-                    for (int t = 0; t < NT; t++) {
-                        xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xacc[i], 0,
-                                                                          0, 0);
-#pragma unroll
-                        for (int j = 0; j < NW; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]),
-                                                                                acc[i][j], 0, 0, 0);
-                    }
-                }
+                    for (int r = 0; r < 4; r++)
+                        acc[i][j][r] = fmaf(cs, fmaf(-cz, xs_w[i][r], pp_w[i][j][r]), acc[i][j][r]);
             }
         }
     }
@@ -415,6 +491,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     // ---- combine the K-slices: every wavefront posts its partial tile, then wavefront w sums
     // accumulators w, w + KW, ... over the slices in wave order (fixed, so results repeat bit
     // for bit) and stores them
+    __syncthreads();  // the reduction area overlays the staging areas
 #pragma unroll
     for (int i = 0; i < MW; i++)
 #pragma unroll
@@ -453,7 +530,9 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 
 template <int FMT, bool XF32, bool WHOLE>
 int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
-    const size_t lds = (size_t)kw * mw * nw * 4 * 64 * sizeof(float);
+    const bool four_bit = FMT != NQ_FMT_W8_CHANNEL;
+    const size_t staging = (size_t)kw * (16 * ((!four_bit && !XF32) ? 128 : 256) + nw * 1024);
+    const size_t lds = std::max(staging, (size_t)kw * mw * nw * 4 * 64 * sizeof(float));
     const dim3 block(64 * kw);
 #define NQ_A16_CASE(MW_, NW_, KW_)                                                                         \
     if (mw == MW_ && nw == NW_ && kw == KW_) {                                                             \
@@ -504,6 +583,8 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     // when that costs no extra padded rows
     // (measured at M = 100..256: the 2 x 4 tile only pays once there is work for several
     // rounds of workgroups, and below ~128 workgroups a narrower tile wins)
+    // (and that over a weight too large to stay in the caches a workgroup per CU is the least to ask for)
+    const bool big = (int64_t)L->in * L->out >= ((int64_t)4 << 20);
     static const int shapes[5][2] = {{2, 4}, {2, 2}, {1, 4}, {1, 2}, {1, 1}};
     int mw = 1, nw = 1;
     const int mt = (a.M + 15) / 16;
@@ -512,12 +593,21 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
         if (mw == 2 && (mt & 1) && mt < 16) continue;
         if (mw * nw == 8 && xf32) continue;  // would not fit the register budget
         const int64_t wgs = (int64_t)((mt + mw - 1) / mw) * ((L->out + 16 * nw - 1) / (16 * nw));
-        if (wgs >= (mw * nw == 8 ? 2048 : 128)) break;
+        if (wgs >= (mw * nw == 8 ? 2048 : big ? 160 : 128)) break;
     }
-    // K split: 8 wavefronts when there are more than 4 k-steps
     const int kstep = four_bit ? 128 : 64;
     const int nsteps = (L->in + kstep - 1) / kstep;
-    const int kw = nsteps > 4 ? 8 : 4;
+    auto wgs_of = [&](int mw_, int nw_) {
+        return (int64_t)((mt + mw_ - 1) / mw_) * ((L->out + 16 * nw_ - 1) / (16 * nw_));
+    };
+    // (measured with bf16 activations and short K, at most 8 k-steps: a few hundred workgroups of the
+    // wider tiles leave the chip waiting for the last round; the 16 x 32 tile in twice as many
+    // workgroups is faster)
+    if (!xf32 && nsteps <= 8 && (mw * nw == 4) && wgs_of(mw, nw) >= 300 && wgs_of(mw, nw) < 1000) mw = 1, nw = 2;
+    // K split: 8 wavefronts when there are more than 4 k-steps.  It follows K alone: the K split fixes
+    // the order in which an output's sum is formed, and a row must get the same bits whichever
+    // layer (its own, or a row-fused one) it is computed in.
+    int kw = nsteps > 4 ? 8 : 4;
     dim3 grid((L->out + 16 * nw - 1) / (16 * nw), (a.M + 16 * mw - 1) / (16 * mw));
     switch (L->format) {
         case NQ_FMT_Q4_0:
