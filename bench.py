@@ -152,8 +152,8 @@ def make_act_w8a16(M, copies, seed=2):
     return dict(step=step, bytes=nbytes, ops=ops, launches=2, keep=(sets, xs, bs, ys))
 
 
-def make_w8a16_one(K, N, copies, seed=9):
-    """One W8A16 linear at M = 1 (int8 weights, per-channel scales, bf16 activations, fp32 out)."""
+def make_w8a16_one(K, N, copies, seed=9, M=1):
+    """One W8A16 linear (int8 weights, per-channel scales, bf16 activations, fp32 out)."""
     import numpy as np
     import torch
 
@@ -167,13 +167,14 @@ def make_w8a16_one(K, N, copies, seed=9):
         lin = W8Linear(K, N)
         lin.set_weight(w, s)
         layers.append(lin)
-    x = bf16_t(rng.standard_normal((1, K))).cuda()
-    y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+    x = bf16_t(rng.standard_normal((M, K))).cuda()
+    y = torch.empty((M, N), dtype=torch.float32, device="cuda")
 
     def step(i):
         layers[i % copies].forward(x, out=y)
 
-    return dict(step=step, bytes=N * K + 4 * N + 2 * K + 4 * N, ops=2 * N * K, launches=1, keep=(layers, x, y))
+    return dict(step=step, bytes=N * K + 4 * N + 2 * K * M + 4 * N * M, ops=2 * M * N * K, launches=1,
+                keep=(layers, x, y))
 
 
 def make_q4_0(IN, OUT, M, copies, seed=3):
@@ -443,6 +444,10 @@ def sweep(skip_large=False):
         run("ref Q4_0 g32 4096->11008 M=1 fp32 (cold)", make_q4_0, "hbm", IN=4096, OUT=11008, M=1, copies=c, calls=c)
         run("W8A16 4096->11008 M=1 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, copies=max(1, c // 2),
             calls=max(1, c // 2))
+        run("W4A16 g128 4096->11008 M=16 (cold)", make_w4g, "hbm", K=4096, N=11008, M=16, copies=c, calls=c)
+        run("ref Q4_0 g32 4096->11008 M=16 fp32 (cold)", make_q4_0, "hbm", IN=4096, OUT=11008, M=16, copies=c, calls=c)
+        run("W8A16 4096->11008 M=16 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, M=16, copies=max(1, c // 2),
+            calls=max(1, c // 2))
     return out
 
 
@@ -486,6 +491,18 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_big, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "W4A16 g128, Q4_0 (fp32 x) and W8A16 at 4096->11008, M=1, cold rotation, one call each per step"
+    elif which == "smallm":
+        K, N, M = 4096, 11008, 16
+        c = max(1, COLD_BYTES // (N * K // 2))
+        wls = [make_w4g(K=K, N=N, M=M, copies=c), make_q4_0(IN=K, OUT=N, M=M, copies=c),
+               make_w8a16_one(K=K, N=N, M=M, copies=max(1, c // 2))]
+
+        def step_small(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_small, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "W4A16 g128, Q4_0 (fp32 x) and W8A16 at 4096->11008, M=16, cold rotation, one call each per step"
     elif which == "actor":
         wl = make_actor_fused()
         name = "cfg3 W8A8 actor 64->256->256->8 M=4096, fused"
@@ -546,11 +563,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
-                         "copy = a plain 256 MiB device copy (the counter calibration kernel)")
+                         "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
+                         "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16")
     ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -564,7 +582,7 @@ def main():
     ensure_built()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv"):
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 

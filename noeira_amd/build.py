@@ -33,12 +33,7 @@ FLAGS = [
 ]
 # GPTQ's codes depend on the last bit of every sum: its sums are written as separate multiplications and
 # additions, and must stay that way
-EXTRA_FLAGS = {
-    "nq_gptq.hip": ["-ffp-contract=off"],
-    # MFMA results of the medium-M kernel feed vector-ALU code at once: keep them out of the accumulator
-    # registers (one copy instruction per result register otherwise)
-    "nq_gemm_a16.hip": [],
-}
+EXTRA_FLAGS = {"nq_gptq.hip": ["-ffp-contract=off"]}
 
 
 def _deps():

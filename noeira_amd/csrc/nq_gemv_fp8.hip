@@ -56,69 +56,103 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
     return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
 }
 
-template <int SPW, int KW>
+// Loads are row-contiguous (a load instruction is priced by the pieces of cache line its lanes
+// touch: 8 rows x 128 bytes, eight adjacent lanes per row, is the cheapest way to bring in a
+// 16 x 128 tile) and reach the MFMA operand layout through a private 4 KiB of LDS per
+// wavefront: one 128-bit store and one 128-bit read per register quad, the 16-byte slot XORed
+// with row / 2 so that neither side has bank conflicts; no barrier is needed because LDS
+// executes one wavefront's accesses in order.
+// A workgroup computes MT tiles of 16 activation rows against one tile of 16 weight rows, so the
+// weights are read once for up to 64 rows of activations.
+template <int SPW, int KW, int MT>
 __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p) {
     __shared__ float red[KW][256];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) uint8_t stage[KW][4096];  // [weights 16 x 128 | activations 16 x 128]
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ln = lane & 15, kb = lane >> 4;
     const int n_base = blockIdx.x * 16;
-    const int m_base = blockIdx.y * 16;
+    const int m_base = blockIdx.y * (16 * MT);
 
-    const int64_t wrow = (int64_t)min(n_base + ln, p.N - 1) * p.K;
-    const int64_t xrow = (int64_t)min(m_base + ln, p.M - 1) * p.K;
+    // a load: lane -> row 8 t + lane / 8 of the tile, 16-byte piece lane % 8 of the step's 128 bytes
+    const int trow = lane >> 3, tpc = lane & 7;
+    int64_t wsrc[2], xsrc[MT][2];
+    uint32_t st[2], rd[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int row = 8 * t + trow;
+        wsrc[t] = (int64_t)min(n_base + row, p.N - 1) * p.K + tpc * 16;
+#pragma unroll
+        for (int i = 0; i < MT; i++) xsrc[i][t] = (int64_t)min(m_base + 16 * i + row, p.M - 1) * p.K + tpc * 16;
+        st[t] = row * 128 + ((tpc ^ (row >> 1)) & 7) * 16;
+        rd[t] = ln * 128 + (((2 * kb + t) ^ (ln >> 1)) & 7) * 16;  // the fragment: k = 32 kb .. 32 kb + 31
+    }
+    uint8_t* scr = stage[wave];
+    auto lds16 = [&](uint32_t off) -> u32x4& { return *reinterpret_cast<u32x4*>(scr + off); };
 
-    f32x4 acc = {0, 0, 0, 0};
+    f32x4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) acc[i] = (f32x4){0, 0, 0, 0};
     for (int s0 = wave * SPW; s0 < p.nsteps; s0 += KW * SPW) {
-        u32x4 wv[SPW][2], xv[SPW][2];
-        // unconditional loads from clamped step indices; a step past K is multiplied by zero
+        u32x4 wv[SPW][2], xv[MT][SPW][2];
+        // unconditional loads from clamped step indices; a step past K meets zero activations
 #pragma unroll
         for (int s = 0; s < SPW; s++) {
-            const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128 + kb * 32;
-            const u32x4* src = reinterpret_cast<const u32x4*>(p.w + wrow + k0);
-            wv[s][0] = __builtin_nontemporal_load(src);
-            wv[s][1] = __builtin_nontemporal_load(src + 1);
+            const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128;
+            wv[s][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[0] + k0));
+            wv[s][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[1] + k0));
         }
 #pragma unroll
-        for (int s = 0; s < SPW; s++) {
-            const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128 + kb * 32;
-            const u32x4* src = reinterpret_cast<const u32x4*>(p.x + xrow + k0);
-            const bool valid = s0 + s < p.nsteps;
-            const u32x4 t0 = src[0], t1 = src[1];
-            xv[s][0] = valid ? t0 : (u32x4){0, 0, 0, 0};
-            xv[s][1] = valid ? t1 : (u32x4){0, 0, 0, 0};
-        }
+        for (int i = 0; i < MT; i++)
+#pragma unroll
+            for (int s = 0; s < SPW; s++) {
+                const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128;
+                xv[i][s][0] = *reinterpret_cast<const u32x4*>(p.x + xsrc[i][0] + k0);
+                xv[i][s][1] = *reinterpret_cast<const u32x4*>(p.x + xsrc[i][1] + k0);
+            }
 #pragma unroll
         for (int s = 0; s < SPW; s++) {
-            const i32x8 a = {(int)xv[s][0][0], (int)xv[s][0][1], (int)xv[s][0][2], (int)xv[s][0][3],
-                             (int)xv[s][1][0], (int)xv[s][1][1], (int)xv[s][1][2], (int)xv[s][1][3]};
-            const i32x8 b = {(int)wv[s][0][0], (int)wv[s][0][1], (int)wv[s][0][2], (int)wv[s][0][3],
-                             (int)wv[s][1][0], (int)wv[s][1][1], (int)wv[s][1][2], (int)wv[s][1][3]};
-            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+            lds16(st[0]) = wv[s][0], lds16(st[1]) = wv[s][1];
+            const u32x4 b0 = lds16(rd[0]), b1 = lds16(rd[1]);
+            const i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                lds16(2048 + st[0]) = xv[i][s][0], lds16(2048 + st[1]) = xv[i][s][1];
+                u32x4 a0 = lds16(2048 + rd[0]), a1 = lds16(2048 + rd[1]);
+                if (s0 + s >= p.nsteps) a0 = a1 = (u32x4){0, 0, 0, 0};  // uniform over the wavefront
+                const i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],
+                                 (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+                acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], 0, 0, 0, 0, 0, 0);
+            }
         }
     }
 
-    // D layout: lane holds column n = lane % 16, rows m = 4 (lane / 16) + r
-#pragma unroll
-    for (int r = 0; r < 4; r++) red[wave][(4 * kb + r) * 16 + ln] = acc[r];
-    __syncthreads();
+    // D layout: lane holds column n = lane % 16, rows m = 4 (lane / 16) + r.  The K-slices of one
+    // activation tile at a time are summed in wave order (fixed, so results repeat bit for bit).
     const int t = threadIdx.x;
-    if (t < 256) {
-        const int m = m_base + (t >> 4), n = n_base + (t & 15);
-        if (m < p.M && n < p.N) {
-            float z = red[0][t];
 #pragma unroll
-            for (int w = 1; w < KW; w++) z += red[w][t];
-            z *= p.tscale * p.x_scale[0];
-            if (p.bias)
-                z += (p.bias_dtype == NQ_DT_F32)
-                         ? reinterpret_cast<const float*>(p.bias)[n]
-                         : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
-            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
-            const int64_t o = (int64_t)m * p.N + n;
-            if (p.y_dtype == NQ_DT_F32)
-                reinterpret_cast<float*>(p.y)[o] = z;
-            else
-                reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(z);
+    for (int i = 0; i < MT; i++) {
+        if (i) __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[wave][(4 * kb + r) * 16 + ln] = acc[i][r];
+        __syncthreads();
+        if (t < 256) {
+            const int m = m_base + 16 * i + (t >> 4), n = n_base + (t & 15);
+            if (m < p.M && n < p.N) {
+                float z = red[0][t];
+#pragma unroll
+                for (int w = 1; w < KW; w++) z += red[w][t];
+                z *= p.tscale * p.x_scale[0];
+                if (p.bias)
+                    z += (p.bias_dtype == NQ_DT_F32)
+                             ? reinterpret_cast<const float*>(p.bias)[n]
+                             : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+                if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                const int64_t o = (int64_t)m * p.N + n;
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(p.y)[o] = z;
+                else
+                    reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(z);
+            }
         }
     }
 }
@@ -218,14 +252,14 @@ int32_t launch_row(const Fp8GemvParams& p, int waves, hipStream_t s) {
 }
 
 
-template <int SPW>
+template <int SPW, int MT>
 int32_t launch_kw(const Fp8GemvParams& p, int kw, dim3 grid, hipStream_t s) {
     if (kw == 4)
-        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 4>), grid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 4, MT>), grid, dim3(256), 0, s, p);
     else if (kw == 8)
-        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 8>), grid, dim3(512), 0, s, p);
-    else if constexpr (SPW <= 4)
-        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 16>), grid, dim3(1024), 0, s, p);
+        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 8, MT>), grid, dim3(512), 0, s, p);
+    else if constexpr (SPW * MT <= 4)
+        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 16, MT>), grid, dim3(1024), 0, s, p);
     else
         return fail(NQ_ERR_INVALID, "nq_forward: no fp8 GEMV of that shape");
     NQ_HIP(hipGetLastError());
@@ -269,21 +303,29 @@ int32_t launch_gemv_fp8(const ForwardArgs& a) {
             default: return launch_row<8>(p, waves, a.stream);
         }
     }
-    // K split: up to 8 steps (16 KB) per wavefront, and enough wavefronts per workgroup that a
-    // small N still fills the chip
-    int kw = 4, spw = 8;
+    // Up to four tiles of activation rows per workgroup (the weights are then read once for all of
+    // M < 64).  K split: up to 8 steps (16 KB) of weights per wavefront and round, fewer with more
+    // activation tiles (registers), and enough wavefronts per workgroup that a small N still fills
+    // the chip.
+    const int mt = (a.M + 15) / 16;
+    int kw = 4, spw = mt == 1 ? 8 : mt == 2 ? 4 : 2;
     const int64_t wgs = ((int64_t)L->out + 15) / 16;
     if (wgs < 512) kw = 8;
     if (wgs < 128) kw = 16;
     while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
-    if (kw == 16 && spw > 4) spw = 4;
-    const dim3 grid((unsigned)wgs, (unsigned)((a.M + 15) / 16));
-    switch (spw) {
-        case 1: return launch_kw<1>(p, kw, grid, a.stream);
-        case 2: return launch_kw<2>(p, kw, grid, a.stream);
-        case 4: return launch_kw<4>(p, kw, grid, a.stream);
-        default: return launch_kw<8>(p, kw, grid, a.stream);
+    if (kw == 16 && spw * mt > 4) {
+        if (mt <= 2) spw = 4 / mt;
+        else kw = 8;
     }
+    const dim3 grid((unsigned)wgs, 1);
+#define NQ_FP8_CASE(SPW_, MT_) \
+    if (spw == SPW_ && mt == MT_) return launch_kw<SPW_, MT_>(p, kw, grid, a.stream);
+    NQ_FP8_CASE(1, 1) NQ_FP8_CASE(2, 1) NQ_FP8_CASE(4, 1) NQ_FP8_CASE(8, 1)
+    NQ_FP8_CASE(1, 2) NQ_FP8_CASE(2, 2) NQ_FP8_CASE(4, 2)
+    NQ_FP8_CASE(1, 3) NQ_FP8_CASE(2, 3)
+    NQ_FP8_CASE(1, 4) NQ_FP8_CASE(2, 4)
+#undef NQ_FP8_CASE
+    return fail(NQ_ERR_INVALID, "nq_forward: no fp8 GEMV of that shape");
 }
 
 }  // namespace nq
