@@ -258,12 +258,17 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 #pragma unroll
         for (int j = 0; j < NW; j++) dst[j] = ld16(p.codes, woff[j] + c);
     };
-    // Scale records of a k-step.  The loads return raw registers and nothing is computed from them
-    // here: an instruction that uses a loaded value right away would make the wavefront wait out
-    // the whole memory latency at the point of the prefetch.  decode_s turns them into
-    // fp16 scale | zero point << 16 when the k-step is consumed.
+    // Scale records.  A load instruction costs the same whether its lanes fetch 2 bytes or 16, and the
+    // four lanes (kb = 0..3) that share a weight row would all fetch the same record: instead lane
+    // (row, kb) fetches the record of the wavefront's k-step ks + kb KW, so one set of loads serves
+    // four consecutive k-steps of the wavefront ("a quad"), and each k-step picks its record out of
+    // the lane that holds it with a lane permute (ds_bpermute).  The loads return raw registers and
+    // nothing is computed from them here: an instruction that uses a loaded value right away would
+    // make the wavefront wait out the whole memory latency at the point of the prefetch.  decode_s
+    // turns them into fp16 scale | zero point << 16 when the k-step is consumed.
     constexpr int NR = FMT == NQ_FMT_Q4_0 ? 4 : FMT == NQ_FMT_W4_GROUP ? 2 * NS : 1;
-    auto load_s = [&](int ks, uint32_t (&dst)[NW][NR]) {
+    auto load_s = [&](int ks0, uint32_t (&dst)[NW][NR]) {
+        const int ks = ks0 + kb * KW;  // this lane's k-step of the quad
         if constexpr (FMT == NQ_FMT_Q4_0) {
             if (p.s_pairs) {  // rows are 4- or 8-byte aligned (the last load may run 4 bytes past a row)
                 const uint32_t c0 = (uint32_t)min(ks, nsteps - 1) * 8u;
@@ -298,20 +303,24 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
             }
         }
     };
-    auto decode_s = [&](const uint32_t (&raw)[NW][NR], uint32_t (&sc)[NW][NS]) {
+    // t: the k-step's place in its quad (0..3); its records sit in the lanes kb = t of each row
+    auto decode_s = [&](const uint32_t (&raw)[NW][NR], int t, uint32_t (&sc)[NW][NS]) {
+        const int src = (ln + 16 * t) * 4;
+        auto pick = [&](uint32_t v) { return (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)v); };
 #pragma unroll
         for (int j = 0; j < NW; j++) {
             if constexpr (FMT == NQ_FMT_Q4_0) {
                 if (p.s_pairs) {
-                    sc[j][0] = raw[j][0] & 0xFFFFu, sc[j][1] = raw[j][0] >> 16;
-                    sc[j][2] = raw[j][1] & 0xFFFFu, sc[j][3] = raw[j][1] >> 16;
+                    const uint32_t v0 = pick(raw[j][0]), v1 = pick(raw[j][1]);
+                    sc[j][0] = v0 & 0xFFFFu, sc[j][1] = v0 >> 16;
+                    sc[j][2] = v1 & 0xFFFFu, sc[j][3] = v1 >> 16;
                 } else {
 #pragma unroll
-                    for (int q = 0; q < 4; q++) sc[j][q] = raw[j][q];
+                    for (int q = 0; q < 4; q++) sc[j][q] = pick(raw[j][q]);
                 }
             } else if constexpr (FMT == NQ_FMT_W4_GROUP) {
 #pragma unroll
-                for (int q = 0; q < NS; q++) sc[j][q] = raw[j][2 * q] | (raw[j][2 * q + 1] << 16);
+                for (int q = 0; q < NS; q++) sc[j][q] = pick(raw[j][2 * q] | (raw[j][2 * q + 1] << 16));
             }
         }
     };
@@ -341,17 +350,18 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         for (int i = 0; i < MW; i++) load_x(wave, i, u, xr[i][u]);
     load_s(wave, sv);
 
-    for (int ks = wave; ks < nsteps; ks += KW) {
+    int t4 = 0;  // the k-step's place in its quad of scale records
+    for (int ks = wave; ks < nsteps; ks += KW, t4 = (t4 + 1) & 3) {
         const int kn = ks + KW;  // the k-step the registers are refilled for, if there is one
         const bool more = kn < nsteps;
         u32x4 wc[NW];
         uint32_t sc[NW][NS];
 #pragma unroll
         for (int j = 0; j < NW; j++) lds16(w_st + j * 1024) = wv[j];
-        decode_s(sv, sc);
+        decode_s(sv, t4, sc);
         if (more) {
             load_w(kn, wv);
-            load_s(kn, sv);
+            if (t4 == 3) load_s(kn, sv);  // the next quad (this one's last record has just been taken)
         }
 #pragma unroll
         for (int j = 0; j < NW; j++) wc[j] = lds16(w_rd + j * 1024);
