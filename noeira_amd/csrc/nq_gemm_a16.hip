@@ -236,17 +236,19 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 
     // the accumulators this wavefront finishes after the reduction are idx = wave + t KW; their
     // per-channel operands are requested now so that nothing is loaded after the reduction
-    float ep_scale[EPW], ep_bias[EPW];
+    // (raw: a bf16 bias is widened where it is used; a shift here would make the wavefront wait for
+    // the load before its operands are even requested)
+    float ep_scale[EPW];
+    uint32_t ep_bias[EPW];
 #pragma unroll
     for (int t = 0; t < EPW; t++) {
         const int idx = min(wave + t * KW, TA - 1);
         const int n = min(n_base + 16 * ((idx >> 2) % NW) + ln, p.N - 1);
         ep_scale[t] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[n] : 1.0f;
-        ep_bias[t] = 0.0f;
+        ep_bias[t] = 0;
         if (p.bias)
-            ep_bias[t] = (p.bias_dtype == NQ_DT_F32)
-                             ? reinterpret_cast<const float*>(p.bias)[n]
-                             : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+            ep_bias[t] = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                                     : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
     }
 
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
@@ -523,7 +525,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         const int n = n_base + 16 * j + ln;
         const int m = m_base + 16 * i + 4 * kb + r;  // D layout: row 4*(lane/16) + r, column lane%16
         if (FMT == NQ_FMT_W8_CHANNEL) z *= ep_scale[t];
-        z += ep_bias[t];
+        z += p.bias_dtype == NQ_DT_F32 ? __uint_as_float(ep_bias[t]) : __uint_as_float(ep_bias[t] << 16);
         if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
         if (n < p.N && m < p.M) {
             void* yp;

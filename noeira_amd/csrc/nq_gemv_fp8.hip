@@ -177,6 +177,14 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvP
     u32x4 wv[CPL], xv[CPL];
 #pragma unroll
     for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wr + min(j * 64 + lane, nch - 1));
+    // the epilogue's operands travel with the codes, raw: nothing is computed from them before the end
+    const float xsraw = p.x_scale[0];
+    uint32_t braw = 0;
+    if (p.bias) {
+        const int64_t n = min(row, (int64_t)p.N - 1);
+        braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                           : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
+    }
 #pragma unroll
     for (int i = 0; i < XPT; i++) {
         const int c = (int)threadIdx.x + i * 64 * WAVES;
@@ -185,15 +193,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvP
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < CPL; j++) xv[j] = xs[j * 64 + lane];
-    // the epilogue's operands travel with the codes
-    const float scale = p.tscale * p.x_scale[0];
-    float bias = 0.0f;
-    if (p.bias) {
-        const int64_t n = min(row, (int64_t)p.N - 1);
-        bias = (p.bias_dtype == NQ_DT_F32)
-                   ? reinterpret_cast<const float*>(p.bias)[n]
-                   : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
-    }
+    const float scale = p.tscale * xsraw;
+    const float bias = p.bias_dtype == NQ_DT_F32 ? __uint_as_float(braw) : __uint_as_float(braw << 16);
 
     f32x4 acc = {0, 0, 0, 0};
 #pragma unroll

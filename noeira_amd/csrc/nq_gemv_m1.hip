@@ -123,17 +123,18 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     // requested before x so that both arrive in one round trip; afterwards batch b+1 is in flight
     // while batch b is multiplied.
     auto fetch = [&](int64_t row0, u32x4 (&wv)[RPL][CPL], float (&cs)[RPL][CPL], float (&cz)[RPL][CPL],
-                     float (&rs)[RPL], float (&rbias)[RPL]) {
+                     float (&rs)[RPL], uint32_t (&rbias)[RPL]) {
 #pragma unroll
         for (int r = 0; r < RPL; r++) {
             const int64_t row = min(row0 + r, (int64_t)p.N - 1);
             // the epilogue's operands travel with the codes, so nothing is loaded after the reduction
             rs[r] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[row] : 1.0f;
-            rbias[r] = 0.0f;
+            // (the bias stays raw until the epilogue: widening a bf16 bias here would make the wavefront
+            // wait for it before the codes and x are requested)
+            rbias[r] = 0;
             if (p.bias)
-                rbias[r] = (p.bias_dtype == NQ_DT_F32)
-                               ? reinterpret_cast<const float*>(p.bias)[row]
-                               : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[row] << 16);
+                rbias[r] = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[row]
+                                                       : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[row];
 #pragma unroll
             for (int i = 0; i < CPL; i++) {
                 // Unconditional loads from clamped addresses: a lane whose chunk index runs past the
@@ -157,7 +158,8 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     };
     u32x4 wv[RPL][CPL], wn[RPL][CPL];
     float cs[RPL][CPL], cz[RPL][CPL], csn[RPL][CPL], czn[RPL][CPL];
-    float rs[RPL], rbias[RPL], rsn[RPL], rbiasn[RPL];
+    float rs[RPL], rsn[RPL];
+    uint32_t rbias[RPL], rbiasn[RPL];
     const float tscale = (FMT == NQ_FMT_FP8_E4M3) ? p.tscale * (p.x_scale ? p.x_scale[0] : 1.0f) : 1.0f;
     fetch(row_begin, wv, cs, cz, rs, rbias);
 
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
                 float z = acc[r];
                 if (FMT == NQ_FMT_W8_CHANNEL) z *= rs[r];
                 if (FMT == NQ_FMT_FP8_E4M3) z *= tscale;
-                z += rbias[r];
+                z += p.bias_dtype == NQ_DT_F32 ? __uint_as_float(rbias[r]) : __uint_as_float(rbias[r] << 16);
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
                 void* yp;
                 int width, col;
