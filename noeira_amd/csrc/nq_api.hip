@@ -353,6 +353,7 @@ void row_view(const nq_layer* L, int r0, int r1, nq_layer* v) {
 
 int32_t dispatch(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_I8) {
+        if (tile8_i8_applicable(a)) return launch_tile8_i8(a);
         if (gemm8_applicable(a)) return launch_gemm8(a);
         return launch_gemv_i8(a);
     }

@@ -119,9 +119,12 @@ int32_t launch_gemv_row4(const ForwardArgs& a);
 bool gemv_row8_applicable(const ForwardArgs& a);
 int32_t launch_gemv_row8(const ForwardArgs& a);
 
-// nq_gemv_fp8.hip: fp8 x fp8 GEMV for 1..16 activation rows on the matrix cores
+// nq_gemv_fp8.hip: fp8 x fp8 and int8 x int8 on the matrix cores for one row (fp8) and for as many
+// activation rows as the large-tile GEMM would leave most of the chip idle with
 bool gemv_fp8_applicable(const ForwardArgs& a);
 int32_t launch_gemv_fp8(const ForwardArgs& a);
+bool tile8_i8_applicable(const ForwardArgs& a);
+int32_t launch_tile8_i8(const ForwardArgs& a);
 
 // nq_gemm8.hip: LDS-tiled fp8 / int8 MFMA GEMM for large M
 bool gemm8_applicable(const ForwardArgs& a);

@@ -1,23 +1,29 @@
-// fp8 x fp8 GEMV for 1..63 activation rows on the matrix cores:
-//     y[M, N] = epi( (x[M, K] @ W[N, K]^T) * s_w * s_x + bias ),  x and W in e4m3.
+// 8-bit x 8-bit products for few activation rows on the matrix cores:
+//     fp8 e4m3 x fp8 e4m3:  y[M, N] = epi( (x[M, K] @ W[N, K]^T) * s_w * s_x + bias )
+//     int8 x int8:          y[M, N] = epi( (x . W^T)_int32 * s_x[m] * s_w[n] + bias ), or the raw int32 sums
 //
 // The call is bound by the weight stream (K = 4096, N = 11008 is 45 MB), and what a
-// streaming kernel can lose is issue slots: converting an fp8 code and multiplying it on the
+// streaming kernel can lose is issue slots: converting an 8-bit code and multiplying it on the
 // vector ALU costs about two instructions per weight per wavefront, which at one row per
 // wavefront is more instruction issue than the loads leave room for.  One
-// v_mfma_f32_16x16x128_f8f6f4 multiplies a 16-row x 128-k slab of weights (2 KB) by up to 16
-// activation rows in a single instruction, so the kernel is loads plus a handful of MFMAs:
-//   - a workgroup owns 16 weight rows; its KW wavefronts split K, SPW steps of 128 k each;
-//   - lane (n = lane % 16, kb = lane / 16) loads the 32 bytes of row n under k-block kb of a
-//     step (two 128-bit loads, 128 contiguous bytes per row across the four lanes) - this is
-//     exactly its share of the MFMA's B operand, so nothing is shuffled or converted;
-//   - the activations are the A operand: row m = lane % 16 of the workgroup's 16-row M tile
-//     (clamped to M - 1), same k-block; they stay in L1/L2, and more than 16 rows take one
-//     workgroup per M tile, re-reading the weights from L2;
-//   - all of a wavefront's loads are issued before its first MFMA (SPW x 32 bytes per lane,
-//     up to 16 KB per wavefront in flight);
+// v_mfma_f32_16x16x128_f8f6f4 (or two v_mfma_i32_16x16x64_i8) multiplies a 16-row x 128-k slab
+// of weights (2 KB) by 16 activation rows, so the kernel is loads plus a handful of MFMAs:
+//   - a workgroup owns 16 weight rows and up to 64 activation rows (MT tiles of 16; more rows
+//     take more workgroups along grid.y, re-reading the weights from L2); its KW wavefronts
+//     split K, SPW steps of 128 k each;
+//   - loads are row-contiguous: 8 rows x 128 bytes per instruction, eight adjacent lanes per row
+//     (a load instruction is priced by the pieces of cache line its lanes touch), and reach the
+//     MFMA operand layout through a private 4 KiB of LDS per wavefront: one 128-bit store and
+//     one 128-bit read per register quad, the 16-byte slot XORed with row / 2 so that neither
+//     side has bank conflicts; no barrier, LDS executes one wavefront's accesses in order;
+//   - all of a wavefront's loads of a round are issued before its first MFMA (up to 16 KB of
+//     weights per wavefront in flight);
 //   - the KW partial 16 x 16 tiles are summed through LDS in wave order (fixed, so a repeated
-//     call returns the same bits) and thread (m, n) applies scale, bias and epilogue.
+//     call returns the same bits; the int32 sums are exact in any order) and thread (m, n)
+//     applies scales, bias and epilogue.
+// The same kernel serves up to a few hundred rows where the 256 x 256-tile GEMM would leave most
+// of the chip idle (M = 64 .. 512 over a 4096 x 4096 weight is 16 .. 32 tiles on 256 CUs):
+// tile8_applicable holds the measured crossover.
 //
 // A single activation row (M = 1) takes a second kernel whose loads are fully coalesced: one
 // wavefront owns ONE weight row and reads it as 1 KB contiguous per load instruction (lane l
@@ -27,6 +33,9 @@
 // D[c][c] = <x segment c, W segment c> and the row's dot product is the trace of D.  15/16 of
 // the MFMA is wasted, which costs nothing here: the instruction replaces ~250 VALU
 // instructions per KB-row and the kernel issues little besides its loads.
+#include <algorithm>
+#include <type_traits>
+
 #include "nq_common.h"
 
 
@@ -35,13 +44,15 @@ namespace nq {
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 struct Fp8GemvParams {
     const uint8_t* w;
     const uint8_t* x;
-    const float* x_scale;
+    const float* x_scale;    // fp8: [1]; int8: per activation row [M] (null with raw int32 output)
+    const float* col_scale;  // int8: per output channel [N]
     void* y;
     const void* bias;
     int32_t M, N, K;
@@ -56,17 +67,10 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
     return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
 }
 
-// Loads are row-contiguous (a load instruction is priced by the pieces of cache line its lanes
-// touch: 8 rows x 128 bytes, eight adjacent lanes per row, is the cheapest way to bring in a
-// 16 x 128 tile) and reach the MFMA operand layout through a private 4 KiB of LDS per
-// wavefront: one 128-bit store and one 128-bit read per register quad, the 16-byte slot XORed
-// with row / 2 so that neither side has bank conflicts; no barrier is needed because LDS
-// executes one wavefront's accesses in order.
-// A workgroup computes MT tiles of 16 activation rows against one tile of 16 weight rows, so the
-// weights are read once for up to 64 rows of activations.
-template <int SPW, int KW, int MT>
-__global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p) {
-    __shared__ float red[KW][256];
+template <bool I8, int SPW, int KW, int MT>
+__global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
+    typedef typename std::conditional<I8, i32x4, f32x4>::type acc_t;
+    __shared__ uint32_t red[KW][256];
     __shared__ __attribute__((aligned(16))) uint8_t stage[KW][4096];  // [weights 16 x 128 | activations 16 x 128]
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ln = lane & 15, kb = lane >> 4;
@@ -84,14 +88,17 @@ __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p
 #pragma unroll
         for (int i = 0; i < MT; i++) xsrc[i][t] = (int64_t)min(m_base + 16 * i + row, p.M - 1) * p.K + tpc * 16;
         st[t] = row * 128 + ((tpc ^ (row >> 1)) & 7) * 16;
-        rd[t] = ln * 128 + (((2 * kb + t) ^ (ln >> 1)) & 7) * 16;  // the fragment: k = 32 kb .. 32 kb + 31
+        // the fragment of this lane.  fp8: one MFMA of 128 k, k = 32 kb .. 32 kb + 31 (pieces 2 kb, 2 kb + 1);
+        // int8: two MFMAs of 64 k, the t-th takes k = 64 t + 16 kb .. + 15 (piece 4 t + kb)
+        const int piece = I8 ? 4 * t + kb : 2 * kb + t;
+        rd[t] = ln * 128 + ((piece ^ (ln >> 1)) & 7) * 16;
     }
     uint8_t* scr = stage[wave];
     auto lds16 = [&](uint32_t off) -> u32x4& { return *reinterpret_cast<u32x4*>(scr + off); };
 
-    f32x4 acc[MT];
+    acc_t acc[MT];
 #pragma unroll
-    for (int i = 0; i < MT; i++) acc[i] = (f32x4){0, 0, 0, 0};
+    for (int i = 0; i < MT; i++) acc[i] = (acc_t){0, 0, 0, 0};
     for (int s0 = wave * SPW; s0 < p.nsteps; s0 += KW * SPW) {
         u32x4 wv[SPW][2], xv[MT][SPW][2];
         // unconditional loads from clamped step indices; a step past K meets zero activations
@@ -113,15 +120,23 @@ __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p
         for (int s = 0; s < SPW; s++) {
             lds16(st[0]) = wv[s][0], lds16(st[1]) = wv[s][1];
             const u32x4 b0 = lds16(rd[0]), b1 = lds16(rd[1]);
-            const i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
 #pragma unroll
             for (int i = 0; i < MT; i++) {
                 lds16(2048 + st[0]) = xv[i][s][0], lds16(2048 + st[1]) = xv[i][s][1];
                 u32x4 a0 = lds16(2048 + rd[0]), a1 = lds16(2048 + rd[1]);
                 if (s0 + s >= p.nsteps) a0 = a1 = (u32x4){0, 0, 0, 0};  // uniform over the wavefront
-                const i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],
-                                 (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
-                acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], 0, 0, 0, 0, 0, 0);
+                if constexpr (I8) {
+                    acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0),
+                                                                   __builtin_bit_cast(i32x4, b0), acc[i], 0, 0, 0);
+                    acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1),
+                                                                   __builtin_bit_cast(i32x4, b1), acc[i], 0, 0, 0);
+                } else {
+                    const i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],
+                                     (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+                    const i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3],
+                                     (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+                    acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], 0, 0, 0, 0, 0, 0);
+                }
             }
         }
     }
@@ -133,21 +148,34 @@ __global__ __launch_bounds__(64 * KW) void gemv_fp8_kernel(const Fp8GemvParams p
     for (int i = 0; i < MT; i++) {
         if (i) __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[wave][(4 * kb + r) * 16 + ln] = acc[i][r];
+        for (int r = 0; r < 4; r++)
+            red[wave][(4 * kb + r) * 16 + ln] = I8 ? (uint32_t)acc[i][r] : __float_as_uint((float)acc[i][r]);
         __syncthreads();
         if (t < 256) {
             const int m = m_base + 16 * i + (t >> 4), n = n_base + (t & 15);
             if (m < p.M && n < p.N) {
-                float z = red[0][t];
+                const int64_t o = (int64_t)m * p.N + n;
+                float z;
+                if constexpr (I8) {
+                    int32_t sum = (int32_t)red[0][t];
 #pragma unroll
-                for (int w = 1; w < KW; w++) z += red[w][t];
-                z *= p.tscale * p.x_scale[0];
+                    for (int w = 1; w < KW; w++) sum += (int32_t)red[w][t];
+                    if (p.y_dtype == NQ_DT_I32) {
+                        reinterpret_cast<int32_t*>(p.y)[o] = sum;
+                        continue;
+                    }
+                    z = (float)sum * (p.x_scale[m] * p.col_scale[n]);
+                } else {
+                    z = __uint_as_float(red[0][t]);
+#pragma unroll
+                    for (int w = 1; w < KW; w++) z += __uint_as_float(red[w][t]);
+                    z *= p.tscale * p.x_scale[0];
+                }
                 if (p.bias)
                     z += (p.bias_dtype == NQ_DT_F32)
                              ? reinterpret_cast<const float*>(p.bias)[n]
                              : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
-                const int64_t o = (int64_t)m * p.N + n;
                 if (p.y_dtype == NQ_DT_F32)
                     reinterpret_cast<float*>(p.y)[o] = z;
                 else
@@ -253,18 +281,46 @@ int32_t launch_row(const Fp8GemvParams& p, int waves, hipStream_t s) {
 }
 
 
-template <int SPW, int MT>
+template <bool I8, int SPW, int MT>
 int32_t launch_kw(const Fp8GemvParams& p, int kw, dim3 grid, hipStream_t s) {
     if (kw == 4)
-        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 4, MT>), grid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 4, MT>), grid, dim3(256), 0, s, p);
     else if (kw == 8)
-        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 8, MT>), grid, dim3(512), 0, s, p);
+        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 8, MT>), grid, dim3(512), 0, s, p);
     else if constexpr (SPW * MT <= 4)
-        hipLaunchKernelGGL((gemv_fp8_kernel<SPW, 16, MT>), grid, dim3(1024), 0, s, p);
+        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 16, MT>), grid, dim3(1024), 0, s, p);
     else
-        return fail(NQ_ERR_INVALID, "nq_forward: no fp8 GEMV of that shape");
+        return fail(NQ_ERR_INVALID, "nq_forward: no 8-bit tile kernel of that shape");
     NQ_HIP(hipGetLastError());
     return NQ_OK;
+}
+
+template <bool I8>
+int32_t launch_tile8(const Fp8GemvParams& p, int64_t out, hipStream_t stream) {
+    // Up to four tiles of activation rows per workgroup (the weights are then read once for up to 64
+    // rows; more rows go to grid.y).  K split: up to 8 steps (16 KB) of weights per wavefront and
+    // round, fewer with more activation tiles (registers), and enough wavefronts per workgroup that
+    // a small N still fills the chip.
+    const int mt_all = (p.M + 15) / 16;
+    const int mt = mt_all <= 4 ? mt_all : 4;
+    int kw = 4, spw = mt == 1 ? 8 : mt == 2 ? 4 : 2;
+    const int64_t wgs = (out + 15) / 16;
+    if (wgs < 512) kw = 8;
+    if (wgs < 128) kw = 16;
+    while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
+    if (kw == 16 && spw * mt > 4) {
+        if (mt <= 2) spw = 4 / mt;
+        else kw = 8;
+    }
+    const dim3 grid((unsigned)wgs, (unsigned)((mt_all + mt - 1) / mt));
+#define NQ_T8_CASE(SPW_, MT_) \
+    if (spw == SPW_ && mt == MT_) return launch_kw<I8, SPW_, MT_>(p, kw, grid, stream);
+    NQ_T8_CASE(1, 1) NQ_T8_CASE(2, 1) NQ_T8_CASE(4, 1) NQ_T8_CASE(8, 1)
+    NQ_T8_CASE(1, 2) NQ_T8_CASE(2, 2) NQ_T8_CASE(4, 2)
+    NQ_T8_CASE(1, 3) NQ_T8_CASE(2, 3)
+    NQ_T8_CASE(1, 4) NQ_T8_CASE(2, 4)
+#undef NQ_T8_CASE
+    return fail(NQ_ERR_INVALID, "nq_forward: no 8-bit tile kernel of that shape");
 }
 
 }  // namespace
@@ -275,20 +331,52 @@ static bool row_kernel_fits(const ForwardArgs& a) {
     return a.M == 1 && a.L->in % 16 == 0 && a.L->in >= 768 && a.L->in <= 8192;
 }
 
+// The tile kernel against the 256 x 256-tile GEMM (nq_gemm8.hip), both measured over K = 512 .. 8192,
+// N = 1024 .. 11008, M = 64 .. 2048: the tile kernel takes about 4 us + 5.6 us per 10^9 multiply-adds
+// (its weights are re-read per 64 activation rows), a round of GEMM tiles about 8 us + 1.15 us per
+// 128 k, at least 17 us.  Below 64 rows the GEMM does not apply.
+static bool tile8_wins(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (L->in % 128 != 0) return false;
+    if (a.M < 64) return true;
+    const double gmac = (double)a.M * (double)L->in * (double)L->out * 1e-9;
+    const int64_t tiles = (int64_t)((a.M + 255) / 256) * ((L->out + 255) / 256);
+    const double rounds = (double)((tiles + 255) / 256);
+    const double gemm_us = rounds * std::max(17.0, 8.0 + (double)L->in / 128.0 * 1.15);
+    return 4.0 + 5.6 * gmac < gemm_us;
+}
+
 bool gemv_fp8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (L->format != NQ_FMT_FP8_E4M3 || a.x_dtype != NQ_DT_FP8_E4M3 || a.x_scale == nullptr) return false;
-    return row_kernel_fits(a) || (a.M >= 1 && a.M < 64 && L->in % 128 == 0);
+    return row_kernel_fits(a) || tile8_wins(a);
 }
 
-int32_t launch_gemv_fp8(const ForwardArgs& a) {
+bool tile8_i8_applicable(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (L->format != NQ_FMT_W8_CHANNEL || a.x_dtype != NQ_DT_I8) return false;
+    // (one row over a large weight: the LDS kernel of nq_gemv.hip measures 4.1 us against 5.0 at 4096 x 4096)
+    if (a.M == 1 && (int64_t)L->in * L->out >= ((int64_t)8 << 20)) return false;
+    return tile8_wins(a);
+}
+
+static Fp8GemvParams tile8_params(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     Fp8GemvParams p{};
     p.w = L->d_codes, p.x = reinterpret_cast<const uint8_t*>(a.x), p.x_scale = a.x_scale;
+    p.col_scale = reinterpret_cast<const float*>(L->d_scales);
     p.y = a.y, p.bias = a.bias;
     p.M = a.M, p.N = L->out, p.K = L->in, p.nsteps = L->in / 128;
     p.tscale = L->scale;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    return p;
+}
+
+int32_t launch_tile8_i8(const ForwardArgs& a) { return launch_tile8<true>(tile8_params(a), a.L->out, a.stream); }
+
+int32_t launch_gemv_fp8(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    const Fp8GemvParams p = tile8_params(a);
     // one row: a wavefront per weight row once a row fills most of its 64 lanes (K >= 768)
     const int cpl = (L->in / 16 + 63) / 64;
     if (row_kernel_fits(a)) {
@@ -304,29 +392,7 @@ int32_t launch_gemv_fp8(const ForwardArgs& a) {
             default: return launch_row<8>(p, waves, a.stream);
         }
     }
-    // Up to four tiles of activation rows per workgroup (the weights are then read once for all of
-    // M < 64).  K split: up to 8 steps (16 KB) of weights per wavefront and round, fewer with more
-    // activation tiles (registers), and enough wavefronts per workgroup that a small N still fills
-    // the chip.
-    const int mt = (a.M + 15) / 16;
-    int kw = 4, spw = mt == 1 ? 8 : mt == 2 ? 4 : 2;
-    const int64_t wgs = ((int64_t)L->out + 15) / 16;
-    if (wgs < 512) kw = 8;
-    if (wgs < 128) kw = 16;
-    while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
-    if (kw == 16 && spw * mt > 4) {
-        if (mt <= 2) spw = 4 / mt;
-        else kw = 8;
-    }
-    const dim3 grid((unsigned)wgs, 1);
-#define NQ_FP8_CASE(SPW_, MT_) \
-    if (spw == SPW_ && mt == MT_) return launch_kw<SPW_, MT_>(p, kw, grid, a.stream);
-    NQ_FP8_CASE(1, 1) NQ_FP8_CASE(2, 1) NQ_FP8_CASE(4, 1) NQ_FP8_CASE(8, 1)
-    NQ_FP8_CASE(1, 2) NQ_FP8_CASE(2, 2) NQ_FP8_CASE(4, 2)
-    NQ_FP8_CASE(1, 3) NQ_FP8_CASE(2, 3)
-    NQ_FP8_CASE(1, 4) NQ_FP8_CASE(2, 4)
-#undef NQ_FP8_CASE
-    return fail(NQ_ERR_INVALID, "nq_forward: no fp8 GEMV of that shape");
+    return launch_tile8<false>(p, L->out, a.stream);
 }
 
 }  // namespace nq

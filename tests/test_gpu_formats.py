@@ -286,11 +286,15 @@ def test_config5_fp8_gemm_full_size_sampled(N):
     assert rel_rms(gemv, y64[5:6]) < 3e-4
 
 
-@pytest.mark.parametrize("M,K,N", [(4096, 256, 256), (300, 384, 520), (64, 128, 8), (1000, 1024, 264)])
+@pytest.mark.parametrize("M,K,N", [(4096, 256, 256), (300, 384, 520), (64, 128, 8), (1000, 1024, 264),
+                                   (5, 128, 24), (63, 4096, 100), (1, 512, 48),
+                                   (1100, 1024, 2296), (1100, 1024, 2300)])
 def test_int8_gemm_bit_exact(M, K, N):
-    """W8A8 through the int8 MFMA GEMM: int32 accumulators equal the oracle's
-    bit for bit, ragged M / N edges included; the fused epilogue matches the
-    oracle's fp32 expression."""
+    """W8A8 on the int8 matrix cores: int32 accumulators equal the oracle's bit for bit, ragged
+    M / N edges included; the fused epilogue matches the oracle's fp32 expression.  The first
+    seven shapes run on the 16-row tile kernel (few rows, or too few 256 x 256 tiles to fill the
+    chip), the last two on the large-tile GEMM (45 tiles, the last row and column of tiles cut
+    short, N a multiple of 8 and not)."""
     rng = np.random.default_rng(M + K + N)
     lin, w, s = w8_layer(rng, K, N)
     xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
@@ -307,6 +311,28 @@ def test_int8_gemm_bit_exact(M, K, N):
     yb = lin.forward_a8(xd, sd, bias=torch.from_numpy(bias).cuda(), out_dtype=torch.bfloat16)
     want_b = O.w8a8_epilogue(acc_o, sx, s, bias)
     assert np.abs(yb.float().cpu().numpy() - want_b).max() <= np.abs(want_b).max() * 2.0 ** -8
+
+
+@pytest.mark.parametrize("N", [2296, 2300])
+def test_fp8_gemm_ragged_tiles_vs_oracle(N):
+    """fp8 x fp8 through the large-tile GEMM at a size the oracle finishes in seconds: 5 x 9 tiles of
+    256 x 256 with the last row and column of tiles cut short; every element against the oracle."""
+    M, K = 1100, 1024
+    rng = np.random.default_rng(N)
+    a, b = fp8_operands(rng, M, N, K)
+    sa, sb = np.float32(0.5), np.float32(0.25)
+    bias = rng.standard_normal(N).astype(np.float32)
+    lin = FP8Linear(K, N)
+    lin.set_weight(b, float(sb))
+    xs = torch.tensor([sa], dtype=torch.float32, device="cuda")
+    yf = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    lin.forward(torch.from_numpy(a).cuda(), xs, bias=torch.from_numpy(bias).cuda(), out=yf, out_dtype=torch.float32)
+    y64, _ = O.fp8_forward_f64(a, b, sa, sb, want_bf16=False)
+    ref = y64 + bias.astype(np.float64)
+    rms = np.sqrt((ref ** 2).mean())
+    assert np.abs(yf.cpu().numpy() - ref).max() <= 3e-4 * rms
+    yb = lin.forward(torch.from_numpy(a).cuda(), xs, bias=torch.from_numpy(bias).cuda())
+    assert torch.equal(yb, yf.to(torch.bfloat16))
 
 
 def test_config4_w8a8_actor_fused_single_launch():
