@@ -305,8 +305,9 @@ int32_t launch_tile8(const Fp8GemvParams& p, int64_t out, hipStream_t stream) {
     const int mt = mt_all <= 4 ? mt_all : 4;
     int kw = 4, spw = mt == 1 ? 8 : mt == 2 ? 4 : 2;
     const int64_t wgs = (out + 15) / 16;
-    if (wgs < 512) kw = 8;
-    if (wgs < 128) kw = 16;
+    const int64_t all = wgs * ((mt_all + mt - 1) / mt);  // workgroups of the launch
+    if (all < 512 && p.nsteps > 4) kw = 8;
+    if (all < 128 && p.nsteps > 8) kw = 16;
     while (spw > 1 && kw * (spw / 2) >= p.nsteps) spw /= 2;
     if (kw == 16 && spw * mt > 4) {
         if (mt <= 2) spw = 4 / mt;
