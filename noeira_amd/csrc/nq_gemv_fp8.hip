@@ -56,7 +56,7 @@ struct Fp8GemvParams {
     void* y;
     const void* bias;
     int32_t M, N, K;
-    int32_t nsteps;  // K / 128
+    int32_t nsteps;  // steps of 128 k, the last one possibly cut short by K
     float tscale;
     int32_t y_dtype, bias_dtype, epilogue;
 };
@@ -99,12 +99,19 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
     acc_t acc[MT];
 #pragma unroll
     for (int i = 0; i < MT; i++) acc[i] = (acc_t){0, 0, 0, 0};
+    // K need not be a multiple of the step: a lane's 16-byte piece of the last step may lie past the row.
+    // Its address is then moved to the start of the step (inside the row) and, when the step is
+    // staged, both operands' pieces are replaced by zeros (an fp8 NaN times zero would not be zero).
+    const int klast = (p.K - 1) / 128 * 128;           // first k of the last step
+    const bool in_last = klast + tpc * 16 < p.K;       // this lane's piece of the last step lies inside K
+    const int64_t poff = in_last ? 0 : -(int64_t)tpc * 16;
     for (int s0 = wave * SPW; s0 < p.nsteps; s0 += KW * SPW) {
         u32x4 wv[SPW][2], xv[MT][SPW][2];
         // unconditional loads from clamped step indices; a step past K meets zero activations
 #pragma unroll
         for (int s = 0; s < SPW; s++) {
-            const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128;
+            const int ks = min(s0 + s, p.nsteps - 1);
+            const int64_t k0 = (int64_t)ks * 128 + (ks == p.nsteps - 1 ? poff : 0);
             wv[s][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[0] + k0));
             wv[s][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[1] + k0));
         }
@@ -112,12 +119,25 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
         for (int i = 0; i < MT; i++)
 #pragma unroll
             for (int s = 0; s < SPW; s++) {
-                const int64_t k0 = (int64_t)min(s0 + s, p.nsteps - 1) * 128;
+                const int ks = min(s0 + s, p.nsteps - 1);
+                const int64_t k0 = (int64_t)ks * 128 + (ks == p.nsteps - 1 ? poff : 0);
                 xv[i][s][0] = *reinterpret_cast<const u32x4*>(p.x + xsrc[i][0] + k0);
                 xv[i][s][1] = *reinterpret_cast<const u32x4*>(p.x + xsrc[i][1] + k0);
             }
 #pragma unroll
         for (int s = 0; s < SPW; s++) {
+            if (s0 + s == p.nsteps - 1 && (p.K & 127)) {  // uniform over the wavefront: the step K cuts short
+                const uint32_t keep = in_last ? ~0u : 0u;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) wv[s][t][e] &= keep;
+#pragma unroll
+                    for (int i = 0; i < MT; i++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) xv[i][s][t][e] &= keep;
+                }
+            }
             lds16(st[0]) = wv[s][0], lds16(st[1]) = wv[s][1];
             const u32x4 b0 = lds16(rd[0]), b1 = lds16(rd[1]);
 #pragma unroll
@@ -327,7 +347,7 @@ int32_t launch_tile8(const Fp8GemvParams& p, int64_t out, hipStream_t stream) {
 }  // namespace
 
 // a row of 768..8192 codes takes the one-row kernel (M = 1, K a multiple of 16); otherwise the
-// 16-row tile kernel (M < 64) needs whole MFMA steps (K a multiple of 128)
+// 16-row tile kernel (K a multiple of 16: a last step that K cuts short is padded with zeros)
 static bool row_kernel_fits(const ForwardArgs& a) {
     return a.M == 1 && a.L->in % 16 == 0 && a.L->in >= 768 && a.L->in <= 8192;
 }
@@ -338,8 +358,8 @@ static bool row_kernel_fits(const ForwardArgs& a) {
 // 128 k, at least 17 us.  Below 64 rows the GEMM does not apply.
 static bool tile8_wins(const ForwardArgs& a) {
     const nq_layer* L = a.L;
-    if (L->in % 128 != 0) return false;
-    if (a.M < 64) return true;
+    if (L->in % 16 != 0) return false;
+    if (a.M < 64 || L->in % 128 != 0) return true;  // (the GEMM needs 64 rows and whole 128-byte steps)
     const double gmac = (double)a.M * (double)L->in * (double)L->out * 1e-9;
     const int64_t tiles = (int64_t)((a.M + 255) / 256) * ((L->out + 255) / 256);
     const double rounds = (double)((tiles + 255) / 256);
@@ -367,7 +387,7 @@ static Fp8GemvParams tile8_params(const ForwardArgs& a) {
     p.w = L->d_codes, p.x = reinterpret_cast<const uint8_t*>(a.x), p.x_scale = a.x_scale;
     p.col_scale = reinterpret_cast<const float*>(L->d_scales);
     p.y = a.y, p.bias = a.bias;
-    p.M = a.M, p.N = L->out, p.K = L->in, p.nsteps = L->in / 128;
+    p.M = a.M, p.N = L->out, p.K = L->in, p.nsteps = (L->in + 127) / 128;
     p.tscale = L->scale;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     return p;

@@ -237,9 +237,10 @@ def test_config5_fp8_gemv_full_size_sampled():
 
 
 @pytest.mark.parametrize("M,K,N", [(1, 128, 16), (3, 384, 40), (16, 2560, 100), (2, 8192, 33),
-                                   (1, 784, 37), (1, 1024, 5), (1, 2576, 130), (1, 8192, 19), (1, 8208, 9)])
+                                   (1, 784, 37), (1, 1024, 5), (1, 2576, 130), (1, 8192, 19), (1, 8208, 9),
+                                   (3, 400, 40), (40, 1040, 100), (200, 16, 24), (1, 48, 7)])
 def test_fp8_small_m_bias_relu_and_shapes(M, K, N):
-    """fp8 x fp8 at 1..16 rows: ragged N, K from one MFMA step to several rounds of the K split,
+    """fp8 x fp8 at 1..200 rows: ragged N, K from a fraction of one MFMA step to several rounds of the K split,
     fp32 bias and ReLU fused; checked against the float64 oracle."""
     rng = np.random.default_rng(1000 + M + K)
     a, b = fp8_operands(rng, M, N, K)
@@ -288,13 +289,15 @@ def test_config5_fp8_gemm_full_size_sampled(N):
 
 @pytest.mark.parametrize("M,K,N", [(4096, 256, 256), (300, 384, 520), (64, 128, 8), (1000, 1024, 264),
                                    (5, 128, 24), (63, 4096, 100), (1, 512, 48),
+                                   (4096, 64, 256), (300, 960, 520), (5, 80, 24), (70, 16, 40),
                                    (1100, 1024, 2296), (1100, 1024, 2300)])
 def test_int8_gemm_bit_exact(M, K, N):
     """W8A8 on the int8 matrix cores: int32 accumulators equal the oracle's bit for bit, ragged
     M / N edges included; the fused epilogue matches the oracle's fp32 expression.  The first
     seven shapes run on the 16-row tile kernel (few rows, or too few 256 x 256 tiles to fill the
-    chip), the last two on the large-tile GEMM (45 tiles, the last row and column of tiles cut
-    short, N a multiple of 8 and not)."""
+    chip), the next four too, with K not a multiple of the kernel's 128-wide step (64 is the actor's
+    first layer), the last two on the large-tile GEMM (45 tiles, the last row and column of tiles
+    cut short, N a multiple of 8 and not)."""
     rng = np.random.default_rng(M + K + N)
     lin, w, s = w8_layer(rng, K, N)
     xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
