@@ -438,6 +438,10 @@ def sweep(skip_large=False):
     if not skip_large:
         run("W8A8 int8 GEMM M=8192 K=4096 N=4096 (scales + bias epilogue, bf16 out)", make_w8a8_gemm, "mfma", "int8",
             M=8192, N=4096, calls=10)
+        # a few rows to a few hundred: the 16-row tile kernel's range
+        for M in (16, 64, 256):
+            run(f"W8A8 int8 M={M} K=4096 N=4096 (warm)", make_w8a8_gemm, "mfma", "int8", M=M, N=4096, calls=20)
+            run(f"fp8 x fp8 M={M} K=4096 N=4096 (warm)", make_fp8, "mfma", "fp8", M=M, N=4096, copies=1, calls=20)
         # the dequant-GEMVs at a size where the HBM fraction means something (22 - 45 MB of codes)
         c = max(1, COLD_BYTES // (4096 * 11008 // 2))
         run("W4A16 g128 4096->11008 M=1 (cold)", make_w4g, "hbm", K=4096, N=11008, M=1, copies=c, calls=c)
@@ -503,6 +507,15 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_small, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "W4A16 g128, Q4_0 (fp32 x) and W8A16 at 4096->11008, M=16, cold rotation, one call each per step"
+    elif which == "tile8":
+        wls = [make_w8a8_gemm(M, 4096) for M in (16, 64, 256)] + [make_fp8(M, 4096) for M in (16, 64, 256)]
+
+        def step_t8(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_t8, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "W8A8 and fp8 x fp8 at 4096 x 4096, M = 16, 64, 256, one call each per step"
     elif which == "actor":
         wl = make_actor_fused()
         name = "cfg3 W8A8 actor 64->256->256->8 M=4096, fused"
@@ -563,12 +576,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
                          "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
-                         "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16")
+                         "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, tile8 = int8 and fp8 "
+                         "activations at M = 16, 64, 256 over 4096 x 4096")
     ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -582,7 +596,7 @@ def main():
     ensure_built()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm"):
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 
