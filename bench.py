@@ -385,6 +385,31 @@ def make_w8a8_gemm(M, N, K=4096, seed=8):
                 keep=(lin, xq, xs, bias, y))
 
 
+def make_w8a8_m1(K, N, copies, seed=10):
+    """int8 x int8 for one row of activations: the W8A8 layer of a single environment."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.qlinear import W8Linear
+
+    rng = np.random.default_rng(seed)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    layers = []
+    for _ in range(copies):
+        lin = W8Linear(K, N)
+        lin.set_weight(w, s)
+        layers.append(lin)
+    xq = torch.from_numpy(rng.integers(-127, 128, (1, K), dtype=np.int8)).cuda()
+    xs = torch.from_numpy(rng.uniform(1e-2, 2e-2, 1).astype(np.float32)).cuda()
+    y = torch.empty((1, N), dtype=torch.float32, device="cuda")
+
+    def step(i):
+        layers[i % copies].forward_a8(xq, xs, out=y, out_dtype=torch.float32)
+
+    return dict(step=step, bytes=N * K + K + 4 * N + 4 * N + 4, ops=2 * N * K, launches=1, keep=(layers, xq, xs, y))
+
+
 def report(name, wl, seconds, bound, peak_key=None):
     gbps = wl["bytes"] / seconds / 1e9
     tops = wl["ops"] / seconds / 1e12
@@ -438,6 +463,8 @@ def sweep(skip_large=False):
     if not skip_large:
         run("W8A8 int8 GEMM M=8192 K=4096 N=4096 (scales + bias epilogue, bf16 out)", make_w8a8_gemm, "mfma", "int8",
             M=8192, N=4096, calls=10)
+        c8 = max(1, COLD_BYTES // (4096 * 11008))
+        run("W8A8 int8 GEMV K=4096 N=11008 M=1 (cold)", make_w8a8_m1, "hbm", K=4096, N=11008, copies=c8, calls=c8)
         # a few rows to a few hundred: the 16-row tile kernel's range
         for M in (16, 64, 256):
             run(f"W8A8 int8 M={M} K=4096 N=4096 (warm)", make_w8a8_gemm, "mfma", "int8", M=M, N=4096, calls=20)
@@ -665,7 +692,7 @@ def main():
             best = max(gv, key=lambda r: r["GBps"])
             line["roofline_gemv"] = {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                      "frac": round(best["GBps"] / HBM_PEAK_GBPS, 5), "traffic": FP8_GEMV_TRAFFIC,
-                                     "kernel": "nq::gemv_fp8_row_kernel", "workload": best["workload"]}
+                                     "kernel": "nq::gemv8_row_kernel<fp8>", "workload": best["workload"]}
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

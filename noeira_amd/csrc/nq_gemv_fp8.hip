@@ -207,13 +207,14 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
 
 
 // ---- M = 1: one wavefront per weight row, coalesced loads, trace of the MFMA tile
-template <int CPL, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvParams p) {
+template <bool I8, int CPL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvParams p) {
     __shared__ u32x4 xs[CPL * 64];  // the activation row, shared by the workgroup's rows
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t row = (int64_t)blockIdx.x * WAVES + wave;
+    const int64_t rowc = min(row, (int64_t)p.N - 1);
     const int nch = p.K >> 4;  // 16-byte chunks per row
-    const u32x4* wr = reinterpret_cast<const u32x4*>(p.w + min(row, (int64_t)p.N - 1) * p.K);
+    const u32x4* wr = reinterpret_cast<const u32x4*>(p.w + rowc * p.K);
     const u32x4* xr = reinterpret_cast<const u32x4*>(p.x);
 
     // x goes first so that waiting for it leaves the weight loads in flight; every load is
@@ -226,13 +227,14 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvP
 #pragma unroll
     for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wr + min(j * 64 + lane, nch - 1));
     // the epilogue's operands travel with the codes, raw: nothing is computed from them before the end
-    const float xsraw = p.x_scale[0];
+    const bool raw_out = I8 && p.y_dtype == NQ_DT_I32;
+    float xsraw = 1.0f, csraw = 1.0f;
+    if (!raw_out) xsraw = p.x_scale[0];
+    if (I8 && !raw_out) csraw = p.col_scale[rowc];
     uint32_t braw = 0;
-    if (p.bias) {
-        const int64_t n = min(row, (int64_t)p.N - 1);
-        braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
-                                           : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
-    }
+    if (p.bias)
+        braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[rowc]
+                                           : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[rowc];
 #pragma unroll
     for (int i = 0; i < XPT; i++) {
         const int c = (int)threadIdx.x + i * 64 * WAVES;
@@ -241,45 +243,59 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvP
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < CPL; j++) xv[j] = xs[j * 64 + lane];
-    const float scale = p.tscale * xsraw;
-    const float bias = p.bias_dtype == NQ_DT_F32 ? __uint_as_float(braw) : __uint_as_float(braw << 16);
 
-    f32x4 acc = {0, 0, 0, 0};
-#pragma unroll
-    for (int j = 0; j < CPL; j += 2) {
-        const u32x4 x1 = (j + 1 < CPL) ? xv[j + 1] : (u32x4){0, 0, 0, 0};
-        const u32x4 w1 = (j + 1 < CPL) ? wv[j + 1] : (u32x4){0, 0, 0, 0};
-        const i32x8 a = {(int)xv[j][0], (int)xv[j][1], (int)xv[j][2], (int)xv[j][3],
-                         (int)x1[0],    (int)x1[1],    (int)x1[2],    (int)x1[3]};
-        const i32x8 b = {(int)wv[j][0], (int)wv[j][1], (int)wv[j][2], (int)wv[j][3],
-                         (int)w1[0],    (int)w1[1],    (int)w1[2],    (int)w1[3]};
-        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
-    }
     // lane holds D[4 (lane / 16) + r][lane % 16]: its diagonal entry, if any, is r = c % 4 where
     // c = lane % 16 and c / 4 == lane / 16
     const int c = lane & 15, r = c & 3;
-    float v = r == 0 ? acc[0] : r == 1 ? acc[1] : r == 2 ? acc[2] : acc[3];
-    v = ((c >> 2) == (lane >> 4)) ? v : 0.0f;
-    // fixed butterfly over the 64 lanes (so a repeated call returns the same bits)
-    int t;
-    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false);
-    v += __int_as_float(t);
-    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false);
-    v += __int_as_float(t);
-    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false);
-    v += __int_as_float(t);
-    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false);
-    v += __int_as_float(t);
+    const bool holder = (c >> 2) == (lane >> 4);
+    uint32_t vbits;  // the lane's share of the trace: fp32 bits, or an int32
+    if constexpr (I8) {
+        i32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < CPL; j++)
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xv[j]),
+                                                        __builtin_bit_cast(i32x4, wv[j]), acc, 0, 0, 0);
+        const int d = r == 0 ? acc[0] : r == 1 ? acc[1] : r == 2 ? acc[2] : acc[3];
+        vbits = holder ? (uint32_t)d : 0u;
+    } else {
+        f32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < CPL; j += 2) {
+            const u32x4 x1 = (j + 1 < CPL) ? xv[j + 1] : (u32x4){0, 0, 0, 0};
+            const u32x4 w1 = (j + 1 < CPL) ? wv[j + 1] : (u32x4){0, 0, 0, 0};
+            const i32x8 a = {(int)xv[j][0], (int)xv[j][1], (int)xv[j][2], (int)xv[j][3],
+                             (int)x1[0],    (int)x1[1],    (int)x1[2],    (int)x1[3]};
+            const i32x8 b = {(int)wv[j][0], (int)wv[j][1], (int)wv[j][2], (int)wv[j][3],
+                             (int)w1[0],    (int)w1[1],    (int)w1[2],    (int)w1[3]};
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+        }
+        const float d = r == 0 ? acc[0] : r == 1 ? acc[1] : r == 2 ? acc[2] : acc[3];
+        vbits = holder ? __float_as_uint(d) : 0u;
+    }
+    // fixed butterfly over the 64 lanes (so a repeated call returns the same bits; the int32 sum is exact)
+    auto add = [](uint32_t a, uint32_t b) -> uint32_t {
+        if constexpr (I8) return (uint32_t)((int32_t)a + (int32_t)b);
+        else return __float_as_uint(__uint_as_float(a) + __uint_as_float(b));
+    };
+    vbits = add(vbits, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)vbits, 0xB1, 0xF, 0xF, false));
+    vbits = add(vbits, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)vbits, 0x4E, 0xF, 0xF, false));
+    vbits = add(vbits, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)vbits, 0x141, 0xF, 0xF, false));
+    vbits = add(vbits, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)vbits, 0x140, 0xF, 0xF, false));
     {
-        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+        const auto sw = __builtin_amdgcn_permlane16_swap(vbits, vbits, false, false);
+        vbits = add(sw[0], sw[1]);
     }
     {
-        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+        const auto sw = __builtin_amdgcn_permlane32_swap(vbits, vbits, false, false);
+        vbits = add(sw[0], sw[1]);
     }
     if (lane == 0 && row < p.N) {
-        float z = v * scale + bias;
+        if (raw_out) {
+            reinterpret_cast<int32_t*>(p.y)[row] = (int32_t)vbits;
+            return;
+        }
+        const float bias = p.bias_dtype == NQ_DT_F32 ? __uint_as_float(braw) : __uint_as_float(braw << 16);
+        float z = I8 ? (float)(int32_t)vbits * (xsraw * csraw) + bias : __uint_as_float(vbits) * (p.tscale * xsraw) + bias;
         if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
         if (p.y_dtype == NQ_DT_F32)
             reinterpret_cast<float*>(p.y)[row] = z;
@@ -288,18 +304,27 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_fp8_row_kernel(const Fp8GemvP
     }
 }
 
-template <int CPL>
-int32_t launch_row(const Fp8GemvParams& p, int waves, hipStream_t s) {
-    if (waves == 4)
-        hipLaunchKernelGGL((gemv_fp8_row_kernel<CPL, 4>), dim3((unsigned)((p.N + 3) / 4)), dim3(256), 0, s, p);
-    else if (waves == 8)
-        hipLaunchKernelGGL((gemv_fp8_row_kernel<CPL, 8>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
-    else
-        hipLaunchKernelGGL((gemv_fp8_row_kernel<CPL, 16>), dim3((unsigned)((p.N + 15) / 16)), dim3(1024), 0, s, p);
+template <bool I8, int CPL>
+int32_t launch_row(const Fp8GemvParams& p, hipStream_t s) {
+    hipLaunchKernelGGL((gemv8_row_kernel<I8, CPL, 8>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
 
+template <bool I8>
+int32_t launch_row_cpl(const Fp8GemvParams& p, hipStream_t s) {
+    // a wavefront per weight row: CPL chunks of 16 bytes per lane
+    switch ((p.K / 16 + 63) / 64) {
+        case 1: return launch_row<I8, 1>(p, s);
+        case 2: return launch_row<I8, 2>(p, s);
+        case 3: return launch_row<I8, 3>(p, s);
+        case 4: return launch_row<I8, 4>(p, s);
+        case 5: return launch_row<I8, 5>(p, s);
+        case 6: return launch_row<I8, 6>(p, s);
+        case 7: return launch_row<I8, 7>(p, s);
+        default: return launch_row<I8, 8>(p, s);
+    }
+}
 
 template <bool I8, int SPW, int MT>
 int32_t launch_kw(const Fp8GemvParams& p, int kw, dim3 grid, hipStream_t s) {
@@ -376,9 +401,7 @@ bool gemv_fp8_applicable(const ForwardArgs& a) {
 bool tile8_i8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (L->format != NQ_FMT_W8_CHANNEL || a.x_dtype != NQ_DT_I8) return false;
-    // (one row over a large weight: the LDS kernel of nq_gemv.hip measures 4.1 us against 5.0 at 4096 x 4096)
-    if (a.M == 1 && (int64_t)L->in * L->out >= ((int64_t)8 << 20)) return false;
-    return tile8_wins(a);
+    return row_kernel_fits(a) || tile8_wins(a);
 }
 
 static Fp8GemvParams tile8_params(const ForwardArgs& a) {
@@ -393,27 +416,17 @@ static Fp8GemvParams tile8_params(const ForwardArgs& a) {
     return p;
 }
 
-int32_t launch_tile8_i8(const ForwardArgs& a) { return launch_tile8<true>(tile8_params(a), a.L->out, a.stream); }
+int32_t launch_tile8_i8(const ForwardArgs& a) {
+    const Fp8GemvParams p = tile8_params(a);
+    if (row_kernel_fits(a)) return launch_row_cpl<true>(p, a.stream);
+    return launch_tile8<true>(p, a.L->out, a.stream);
+}
 
 int32_t launch_gemv_fp8(const ForwardArgs& a) {
-    const nq_layer* L = a.L;
     const Fp8GemvParams p = tile8_params(a);
     // one row: a wavefront per weight row once a row fills most of its 64 lanes (K >= 768)
-    const int cpl = (L->in / 16 + 63) / 64;
-    if (row_kernel_fits(a)) {
-        const int waves = 8;
-        switch (cpl) {
-            case 1: return launch_row<1>(p, waves, a.stream);
-            case 2: return launch_row<2>(p, waves, a.stream);
-            case 3: return launch_row<3>(p, waves, a.stream);
-            case 4: return launch_row<4>(p, waves, a.stream);
-            case 5: return launch_row<5>(p, waves, a.stream);
-            case 6: return launch_row<6>(p, waves, a.stream);
-            case 7: return launch_row<7>(p, waves, a.stream);
-            default: return launch_row<8>(p, waves, a.stream);
-        }
-    }
-    return launch_tile8<false>(p, L->out, a.stream);
+    if (row_kernel_fits(a)) return launch_row_cpl<false>(p, a.stream);
+    return launch_tile8<false>(p, a.L->out, a.stream);
 }
 
 }  // namespace nq

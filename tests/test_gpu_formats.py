@@ -290,14 +290,16 @@ def test_config5_fp8_gemm_full_size_sampled(N):
 @pytest.mark.parametrize("M,K,N", [(4096, 256, 256), (300, 384, 520), (64, 128, 8), (1000, 1024, 264),
                                    (5, 128, 24), (63, 4096, 100), (1, 512, 48),
                                    (4096, 64, 256), (300, 960, 520), (5, 80, 24), (70, 16, 40),
+                                   (1, 784, 37), (1, 4096, 130), (1, 8192, 19), (1, 2576, 5),
                                    (1100, 1024, 2296), (1100, 1024, 2300)])
 def test_int8_gemm_bit_exact(M, K, N):
     """W8A8 on the int8 matrix cores: int32 accumulators equal the oracle's bit for bit, ragged
     M / N edges included; the fused epilogue matches the oracle's fp32 expression.  The first
     seven shapes run on the 16-row tile kernel (few rows, or too few 256 x 256 tiles to fill the
     chip), the next four too, with K not a multiple of the kernel's 128-wide step (64 is the actor's
-    first layer), the last two on the large-tile GEMM (45 tiles, the last row and column of tiles
-    cut short, N a multiple of 8 and not)."""
+    first layer), then four single rows of 768 .. 8192 codes on the one-row kernel, the last two on
+    the large-tile GEMM (45 tiles, the last row and column of tiles cut short, N a multiple of 8 and
+    not)."""
     rng = np.random.default_rng(M + K + N)
     lin, w, s = w8_layer(rng, K, N)
     xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
