@@ -126,3 +126,63 @@ def test_random_shapes(seed):
             y = lin.forward_a8(xq, sx, bias=bias, epilogue=epi, out_dtype=odt)
             _check(tag, y, fin(acc_exact * sx.double()[:, None] * sw[None, :]), odt == torch.bfloat16)
         del lin
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "w8", "w4g", "w4g64"])
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float32])
+def test_many_rows(fmt, xdt):
+    """From 2048 rows on, bf16 / fp32 activations take the kernel that stages a [64 or 128] x 128 tile per
+    workgroup: ragged M, N and K (K not a multiple of its k-step, N not a multiple of 128, M not a multiple
+    of the tile), bias, ReLU and bf16 output, against the fp64 product of the dequantised weights; and
+    the parts of a row-fused layer equal their own layers bit for bit."""
+    rng = np.random.default_rng(sum(map(ord, fmt + str(xdt))))
+    for (M, K, N) in ((2048, 960, 320), (2100, 992, 200), (2301, 4096, 130), (4096, 160, 1000)):
+        if fmt.startswith("w4g"):
+            group = 128 if fmt == "w4g" else 64
+            G = -(-K // group)
+            q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+            z = rng.integers(0, 16, (N, G), dtype=np.uint8)
+            codes, zps = F.pack_w4g(q, z)
+            lin = W4GroupLinear(K, N, group)
+            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+        elif fmt == "w8":
+            lin = W8Linear(K, N)
+            lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        else:
+            lin = QLinear(K, N)
+            blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0] = sc & 0xFF
+            blocks[:, :, 1] = sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+        deq = lin.dequantized_dev().double()
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
+        tag = "%s M=%d K=%d N=%d %s" % (fmt, M, K, N, str(xdt)[6:])
+        if fmt == "q4_0":
+            _check(tag, lin.forward(x), x.double() @ deq.T, False)
+        else:
+            bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+            y = lin.forward(x, bias=bias, epilogue="relu", out_dtype=torch.bfloat16)
+            _check(tag, y, (x.double() @ deq.T + bias.double()).clamp_min(0), True)
+            _check(tag, lin.forward(x), x.double() @ deq.T, False)
+        del lin
+
+
+def test_many_rows_fused_parts_equal_their_own_layers():
+    from noeira_amd.qlinear import FusedRows
+
+    rng = np.random.default_rng(77)
+    K, outs, M = 960, [320, 200, 130], 2100
+    layers = []
+    for n in outs:
+        ql = QLinear(K, n)
+        blocks = rng.integers(0, 256, (n, K // 32, 18), dtype=np.uint8)
+        sc = rng.uniform(1e-3, 1e-2, (n, K // 32)).astype(np.float16).view(np.uint16)
+        blocks[:, :, 0] = sc & 0xFF
+        blocks[:, :, 1] = sc >> 8
+        ql.set_blocks(blocks.reshape(-1))
+        layers.append(ql)
+    fused = FusedRows(layers)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda()
+    for l, y in zip(layers, fused.forward(x)):
+        assert torch.equal(y, l.forward(x))
