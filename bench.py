@@ -463,6 +463,10 @@ def sweep(skip_large=False):
     if not skip_large:
         run("W8A8 int8 GEMM M=8192 K=4096 N=4096 (scales + bias epilogue, bf16 out)", make_w8a8_gemm, "mfma", "int8",
             M=8192, N=4096, calls=10)
+        # thousands of rows with 16-bit activations (prefill over a 4-bit or 8-bit weight)
+        run("W4A16 g128 M=4096 K=4096 N=4096 (warm)", make_w4g, "mfma", "bf16", K=4096, N=4096, M=4096, copies=1, calls=10)
+        run("ref Q4_0 g32 960->2560 M=4096 fp32 (warm)", make_q4_0, "mfma", "bf16", IN=960, OUT=2560, M=4096, copies=1,
+            calls=10)
         c8 = max(1, COLD_BYTES // (4096 * 11008))
         run("W8A8 int8 GEMV K=4096 N=11008 M=1 (cold)", make_w8a8_m1, "hbm", K=4096, N=11008, copies=c8, calls=c8)
         # a few rows to a few hundred: the 16-row tile kernel's range
