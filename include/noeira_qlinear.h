@@ -160,9 +160,9 @@ int32_t nq_fused_parts(nq_handle h);
 
 /* nq_forward of a fused layer with one dense output per part:
  * ys[t] is [M, OUT_t], what nq_forward of part t alone would write: a row's
- * arithmetic does not depend on its neighbours (bit for bit at M >= 2; at
- * M = 1 the number of lanes that share a row, hence the order of its sum, may
- * follow the total row count).
+ * arithmetic does not depend on its neighbours (bit for bit at 2 <= M < 512;
+ * at M = 1 the number of lanes that share a row, and from 512 rows on the
+ * kernel, hence the order of a row's sum, may follow the total row count).
  * n_ys must equal nq_fused_parts(h).  bias, if any, is [sum OUT].  One launch
  * where the kernel for the shape can place rows by part (bf16/fp32
  * activations at any M), otherwise one launch per part. */

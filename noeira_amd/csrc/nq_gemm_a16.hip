@@ -552,8 +552,8 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 //   - scale records: one set of loads per four k-steps, as above;
 //   - the arithmetic per MFMA (exact codes, zero point through the C operand, scale in fp32 per
 //     chunk or per k-step, exact three-term split of fp32 activations) is the kernel above's.
-template <int FMT, bool XF32, int MT, bool WHOLE>
-__global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
+template <int FMT, bool XF32, int MT, int NW, bool WHOLE>
+__global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16Params p) {
     constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL);
     constexpr int NT = XF32 ? 3 : 1;
     constexpr int NL = XF32 ? 2 : 1;
@@ -561,17 +561,19 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
     constexpr int KSTEP = FOUR_BIT ? 128 : 64;
     constexpr int NMF = FOUR_BIT ? 4 : 2;
     constexpr int NS = WHOLE ? 1 : 4;
-    constexpr int NW = 4;                  // weight tiles (16 rows each) per wavefront
+    constexpr int WN = 8 / NW;             // wavefronts along N (NW weight tiles of 16 rows each): 2 x WN wavefronts
+    constexpr int NTHR = 128 * WN;
     constexpr int BM = 32 * MT, BN = 128;  // the workgroup's tile
     constexpr int XB = KSTEP * ES;         // bytes of an activation row per k-step (128, 256 or 512)
     constexpr int PPR = XB / 16;           // 16-byte pieces of it
     constexpr int XTILE = BM * XB, WTILE = BN * 64, STAGE = XTILE + WTILE;
-    constexpr int XI = BM * PPR / 256;     // activation pieces per thread and k-step
+    constexpr int XI = BM * PPR / NTHR;    // activation pieces per thread and k-step
+    constexpr int WI = 512 / NTHR;         // weight pieces per thread and k-step
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // [2][STAGE]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ln = lane & 15, kb = lane >> 4;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
 
     const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
@@ -579,20 +581,20 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
     asm volatile("" : "+v"(magic));
     auto swz = [](int row) { return XB >= 256 ? (row & 15) : ((row >> 1) & 7); };
 
-    // ---- staging: piece g = i 256 + tid of the tile -> row g / PPR, piece g % PPR
+    // ---- staging: piece g = i NTHR + tid of the tile -> row g / PPR, piece g % PPR
     uint32_t xsrc[XI], xdst[XI];
     int xpc[XI];
 #pragma unroll
     for (int i = 0; i < XI; i++) {
-        const int g = i * 256 + tid, row = g / PPR, pc = g % PPR;
+        const int g = i * NTHR + tid, row = g / PPR, pc = g % PPR;
         xsrc[i] = (uint32_t)min(m0 + row, p.M - 1) * (uint32_t)p.K * ES + pc * 16;
         xdst[i] = row * XB + ((pc ^ swz(row)) & (PPR - 1)) * 16;
         xpc[i] = pc;
     }
-    uint32_t wsrc[2], wdst[2];
+    uint32_t wsrc[WI], wdst[WI];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int g = i * 256 + tid, row = g >> 2, pc = g & 3;
+    for (int i = 0; i < WI; i++) {
+        const int g = i * NTHR + tid, row = g >> 2, pc = g & 3;
         wsrc[i] = (uint32_t)min(n0 + row, p.N - 1) * (uint32_t)p.nch * 16u;
         wdst[i] = XTILE + row * 64 + ((pc ^ (row >> 2)) & 3) * 16;
     }
@@ -609,17 +611,17 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
                 a_rd[i][q][h] = (wm * 16 * MT + 16 * i + ln) * XB + ((piece ^ swz(ln)) & (PPR - 1)) * 16;
             }
 #pragma unroll
-    for (int j = 0; j < NW; j++) b_rd[j] = XTILE + (wn * 64 + 16 * j + ln) * 64 + ((kb ^ (ln >> 2)) & 3) * 16;
+    for (int j = 0; j < NW; j++) b_rd[j] = XTILE + (wn * 16 * NW + 16 * j + ln) * 64 + ((kb ^ (ln >> 2)) & 3) * 16;
 
     uint32_t soff[NW];
 #pragma unroll
     for (int j = 0; j < NW; j++) {
-        const uint32_t n = (uint32_t)min(n0 + wn * 64 + 16 * j + ln, p.N - 1);
+        const uint32_t n = (uint32_t)min(n0 + wn * 16 * NW + 16 * j + ln, p.N - 1);
         soff[j] = n * (uint32_t)(FMT == NQ_FMT_Q4_0 ? p.nch : p.groups);
     }
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
 
-    u32x4 xv[XI], wv[2];
+    u32x4 xv[XI], wv[WI];
     auto load_tiles = [&](int ks) {
         const int k0 = ks * KSTEP;
 #pragma unroll
@@ -630,7 +632,7 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
         }
         const uint32_t c = (uint32_t)min(ks * 4 + wpc, p.nch - 1) * 16u;
 #pragma unroll
-        for (int i = 0; i < 2; i++) wv[i] = ld16(p.codes, wsrc[i] + c);
+        for (int i = 0; i < WI; i++) wv[i] = ld16(p.codes, wsrc[i] + c);
     };
     // scale records: lane (row, kb) fetches those of k-step ks0 + kb (one set of loads per four k-steps)
     constexpr int NR = FMT == NQ_FMT_Q4_0 ? 4 : FMT == NQ_FMT_W4_GROUP ? 2 * NS : 1;
@@ -717,7 +719,7 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
 #pragma unroll
         for (int i = 0; i < XI; i++) lds16(xdst[i]) = xv[i];
 #pragma unroll
-        for (int i = 0; i < 2; i++) lds16(wdst[i]) = wv[i];
+        for (int i = 0; i < WI; i++) lds16(wdst[i]) = wv[i];
         uint32_t sc[NW][NS];
         decode_s(ks & 3, sc);
         if (ks + 1 < nsteps) {
@@ -828,7 +830,7 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
     // ---- epilogue: lane holds column n = ln of tile j, rows 4 kb + r of tile i
 #pragma unroll
     for (int j = 0; j < NW; j++) {
-        const int n = n0 + wn * 64 + 16 * j + ln;
+        const int n = n0 + wn * 16 * NW + 16 * j + ln;
         const int nc = min(n, p.N - 1);
         const float cscale = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[nc] : 1.0f;
         float cbias = 0.0f;
@@ -860,26 +862,27 @@ __global__ __launch_bounds__(256) void gemm_a16_big_kernel(const A16Params p) {
 }
 
 template <int FMT, bool XF32, bool WHOLE>
-int32_t launch_big(const A16Params& p, int mt, hipStream_t s) {
+int32_t launch_big(const A16Params& p, int mt, int nw, hipStream_t s) {
     const bool four_bit = FMT != NQ_FMT_W8_CHANNEL;
     const int xb = (four_bit ? 128 : 64) * (XF32 ? 4 : 2);
     const size_t lds = 2 * ((size_t)32 * mt * xb + 128 * 64);
     const dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)((p.M + 32 * mt - 1) / (32 * mt)));
-#define NQ_BIG_CASE(MT_)                                                                          \
-    if (mt == MT_) {                                                                              \
-        auto kernel = gemm_a16_big_kernel<FMT, XF32, MT_, WHOLE>;                                 \
+#define NQ_BIG_CASE(MT_, NW_)                                                                     \
+    if (mt == MT_ && nw == NW_) {                                                                 \
+        auto kernel = gemm_a16_big_kernel<FMT, XF32, MT_, NW_, WHOLE>;                            \
         static bool attr = false;                                                                 \
         if (lds > 48 * 1024 && !attr) {                                                           \
             NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                     \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));    \
             attr = true;                                                                          \
         }                                                                                         \
-        hipLaunchKernelGGL(kernel, grid, dim3(256), lds, s, p);                                   \
+        hipLaunchKernelGGL(kernel, grid, dim3(128 * (8 / NW_)), lds, s, p);                       \
         NQ_HIP(hipGetLastError());                                                                \
         return NQ_OK;                                                                             \
     }
-    NQ_BIG_CASE(2)
-    if constexpr (!XF32) { NQ_BIG_CASE(4) }
+    NQ_BIG_CASE(2, 4)
+    NQ_BIG_CASE(2, 2)
+    if constexpr (!XF32) { NQ_BIG_CASE(4, 4) NQ_BIG_CASE(4, 2) }
 #undef NQ_BIG_CASE
     return fail(NQ_ERR_INVALID, "nq_forward: no large-M kernel of that tile shape");
 }
@@ -934,25 +937,28 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     p.s_pairs = L->format != NQ_FMT_Q4_0 ? 0 : (L->in / 32) % 4 == 0 ? 2 : (L->in / 32) % 2 == 0 ? 1 : 0;
     p.nch = L->in / (four_bit ? 32 : 16);
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
-    // From 2048 rows on, the kernel that unpacks a weight once per 64 or 128 rows (measured at M = 4096:
-    // 1.3 - 2 x faster over 960 .. 4096-wide layers; at M = 1120 it wins or loses with the number of
-    // workgroups, and the choice must not depend on N: a row gets the same bits in its own layer and in a
-    // row-fused one).  128 rows per workgroup for the formats and sizes where that measured better.
-    if (a.M >= 2048) {
-        const int big = (!xf32 && L->in >= 4096 && L->format != NQ_FMT_W4_GROUP) ? 4 : 2;
+    // Many rows: the kernel that unpacks a weight once per 64 or 128 rows, wherever its workgroups fill
+    // the chip (measured over 960 .. 4096-wide layers and M = 512 .. 4096: it wins from about 192
+    // workgroups of 64 rows on, 256 with fp32 activations, and is 2 x faster at M = 4096).  Its sums
+    // are formed in another order than the medium-M kernel's, and the choice follows N: from 512
+    // rows on, a row's bits in a row-fused layer may differ from those in its own layer.
+    const int64_t wgs64 = (int64_t)((L->out + 127) / 128) * ((a.M + 63) / 64);
+    if (a.M >= 512 && wgs64 >= (xf32 ? 256 : 192)) {
+        const int big = (!xf32 && L->in >= 4096 && wgs64 >= 384) ? 4 : 2;  // 128 rows per workgroup over a long K
+        const int bnw = xf32 ? 4 : 2;                                      // four or eight wavefronts
         switch (L->format) {
             case NQ_FMT_Q4_0:
-                return xf32 ? launch_big<NQ_FMT_Q4_0, true, false>(p, 2, a.stream)
-                            : launch_big<NQ_FMT_Q4_0, false, false>(p, big, a.stream);
+                return xf32 ? launch_big<NQ_FMT_Q4_0, true, false>(p, 2, bnw, a.stream)
+                            : launch_big<NQ_FMT_Q4_0, false, false>(p, big, bnw, a.stream);
             case NQ_FMT_W4_GROUP:
                 if (L->group % 128 == 0)
-                    return xf32 ? launch_big<NQ_FMT_W4_GROUP, true, true>(p, 2, a.stream)
-                                : launch_big<NQ_FMT_W4_GROUP, false, true>(p, big, a.stream);
-                return xf32 ? launch_big<NQ_FMT_W4_GROUP, true, false>(p, 2, a.stream)
-                            : launch_big<NQ_FMT_W4_GROUP, false, false>(p, big, a.stream);
+                    return xf32 ? launch_big<NQ_FMT_W4_GROUP, true, true>(p, 2, bnw, a.stream)
+                                : launch_big<NQ_FMT_W4_GROUP, false, true>(p, big, bnw, a.stream);
+                return xf32 ? launch_big<NQ_FMT_W4_GROUP, true, false>(p, 2, bnw, a.stream)
+                            : launch_big<NQ_FMT_W4_GROUP, false, false>(p, big, bnw, a.stream);
             case NQ_FMT_W8_CHANNEL:
-                return xf32 ? launch_big<NQ_FMT_W8_CHANNEL, true, false>(p, 2, a.stream)
-                            : launch_big<NQ_FMT_W8_CHANNEL, false, false>(p, big, a.stream);
+                return xf32 ? launch_big<NQ_FMT_W8_CHANNEL, true, false>(p, 2, bnw, a.stream)
+                            : launch_big<NQ_FMT_W8_CHANNEL, false, false>(p, big, bnw, a.stream);
         }
     }
     // Tile shape: as wide in N as still leaves enough workgroups to occupy the chip (the

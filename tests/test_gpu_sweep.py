@@ -131,12 +131,11 @@ def test_random_shapes(seed):
 @pytest.mark.parametrize("fmt", ["q4_0", "w8", "w4g", "w4g64"])
 @pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float32])
 def test_many_rows(fmt, xdt):
-    """From 2048 rows on, bf16 / fp32 activations take the kernel that stages a [64 or 128] x 128 tile per
+    """Many rows (512 and more, where its workgroups fill the chip): bf16 / fp32 activations take the kernel that stages a [64 or 128] x 128 tile per
     workgroup: ragged M, N and K (K not a multiple of its k-step, N not a multiple of 128, M not a multiple
-    of the tile), bias, ReLU and bf16 output, against the fp64 product of the dequantised weights; and
-    the parts of a row-fused layer equal their own layers bit for bit."""
+    of the tile), bias, ReLU and bf16 output, against the fp64 product of the dequantised weights."""
     rng = np.random.default_rng(sum(map(ord, fmt + str(xdt))))
-    for (M, K, N) in ((2048, 960, 320), (2100, 992, 200), (2301, 4096, 130), (4096, 160, 1000)):
+    for (M, K, N) in ((2048, 960, 1600), (2100, 992, 1200), (5000, 4096, 650), (4096, 160, 1000), (513, 960, 3000)):
         if fmt.startswith("w4g"):
             group = 128 if fmt == "w4g" else 64
             G = -(-K // group)
@@ -168,11 +167,13 @@ def test_many_rows(fmt, xdt):
         del lin
 
 
-def test_many_rows_fused_parts_equal_their_own_layers():
+def test_many_rows_fused_parts_match_their_own_layers():
+    """From 512 rows on the kernel, and with it the order of a row's sum, may follow the total row count:
+    a part of a row-fused layer then matches its own layer to the last bits' worth, not bit for bit."""
     from noeira_amd.qlinear import FusedRows
 
     rng = np.random.default_rng(77)
-    K, outs, M = 960, [320, 200, 130], 2100
+    K, outs, M = 960, [2560, 320, 130], 2100
     layers = []
     for n in outs:
         ql = QLinear(K, n)
@@ -185,4 +186,5 @@ def test_many_rows_fused_parts_equal_their_own_layers():
     fused = FusedRows(layers)
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda()
     for l, y in zip(layers, fused.forward(x)):
-        assert torch.equal(y, l.forward(x))
+        own = l.forward(x)
+        assert (y - own).abs().max().item() <= 2e-6 * own.abs().max().item()
