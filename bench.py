@@ -538,6 +538,17 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_small, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "W4A16 g128, Q4_0 (fp32 x) and W8A16 at 4096->11008, M=16, cold rotation, one call each per step"
+    elif which == "manyrows":
+        wls = [make_w4g(K=4096, N=4096, M=4096, copies=1), make_w8a16_one(K=4096, N=4096, M=4096, copies=1),
+               make_q4_0(IN=960, OUT=2560, M=4096, copies=1), make_q4_0(IN=960, OUT=2560, M=1120, copies=1)]
+
+        def step_mr(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_mr, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = ("W4A16 g128 and W8A16 at 4096 x 4096, M = 4096; Q4_0 (fp32 x) 960->2560 at M = 4096 and 1120; "
+                "one call each per step")
     elif which == "tile8":
         wls = [make_w8a8_gemm(M, 4096) for M in (16, 64, 256)] + [make_fp8(M, 4096) for M in (16, 64, 256)]
 
@@ -607,13 +618,14 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
                          "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
                          "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, tile8 = int8 and fp8 "
-                         "activations at M = 16, 64, 256 over 4096 x 4096")
+                         "activations at M = 16, 64, 256 over 4096 x 4096, manyrows = bf16 / fp32 activations at M = 1120 "
+                         "and 4096")
     ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -627,7 +639,7 @@ def main():
     ensure_built()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8"):
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 

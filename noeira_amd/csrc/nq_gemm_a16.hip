@@ -283,6 +283,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
                     } else {
                         dst[j][0] = ld4(p.scales, soff[j] * 2u + c0), dst[j][1] = ld4(p.scales, soff[j] * 2u + c0 + 4u);
                     }
+                    dst[j][2] = 0, dst[j][3] = 0;
                 }
             } else {
 #pragma unroll
