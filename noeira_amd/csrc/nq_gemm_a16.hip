@@ -185,40 +185,10 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     uint32_t magic = 0x41804180u;
     asm volatile("" : "+v"(magic));
 
-    f32x4 acc[MW][NW];
-    f32x4 xacc[MW];  // W8 only: sum_k x_k over the wave's k-steps
-#pragma unroll
-    for (int i = 0; i < MW; i++) {
-        xacc[i] = (f32x4){0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < NW; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
-    }
-
-    // ---- the lane's place in a load (row-contiguous) and in a fragment (MFMA layout)
-    // weights: lane -> row lane/4 of a 16-row tile, 16-byte piece lane%4 of the k-step's 64 bytes;
-    // staged at row * 64 + (piece ^ row/4) * 16 and read back as (row ln, piece kb)
+    // ---- the lane's place in a load: weights, row lane/4 of a 16-row tile and 16-byte piece lane%4 of the
+    // k-step's 64 bytes; activations, row lane/PPR of the instruction's RPI rows and piece lane%PPR
     const int wrow = lane >> 2, wpc = lane & 3;
-    const uint32_t w_st = XS + wrow * 64 + ((wpc ^ (wrow >> 2)) & 3) * 16;
-    const uint32_t w_rd = XS + ln * 64 + ((kb ^ (ln >> 2)) & 3) * 16;
-    // activations: lane -> row lane/PPR of the instruction's RPI rows, piece lane%PPR;
-    // staged at row * XB + (piece ^ f(row)) * 16 with f(row) = row (XB = 256) or row/2 (XB = 128)
     const int trow = lane / PPR, tpc = lane % PPR;
-    auto swz = [](int row) { return XB == 256 ? row : (row >> 1); };
-    uint32_t x_st[NI], x_rd[QU][NL];
-#pragma unroll
-    for (int ii = 0; ii < NI; ii++) {
-        const int row = ii * RPI + trow;
-        x_st[ii] = row * XB + ((tpc ^ swz(row)) & (PPR - 1)) * 16;
-    }
-#pragma unroll
-    for (int qq = 0; qq < QU; qq++)
-#pragma unroll
-        for (int h = 0; h < NL; h++) {
-            // the piece that holds the first 8 k of fragment q of this lane (second half: + 4) within its unit
-            const int piece = FOUR_BIT ? (XF32 ? 8 * qq + 2 * kb + h : 4 * qq + kb)
-                                       : (XF32 ? 4 * kb + 2 * qq + h : 2 * kb + qq);
-            x_rd[qq][h] = ln * XB + ((piece ^ swz(ln)) & (PPR - 1)) * 16;
-        }
 
     // byte offsets of the rows this lane loads (the host has checked that every operand is < 4 GiB)
     uint32_t xoff[MW][NI], woff[NW], soff[NW];
@@ -232,23 +202,6 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         woff[j] = (uint32_t)min(n_base + 16 * j + wrow, p.N - 1) * (uint32_t)p.nch * 16u;
         const uint32_t n = (uint32_t)min(n_base + 16 * j + ln, p.N - 1);
         soff[j] = n * (uint32_t)(FMT == NQ_FMT_Q4_0 ? p.nch : p.groups);  // in elements
-    }
-
-    // the accumulators this wavefront finishes after the reduction are idx = wave + t KW; their
-    // per-channel operands are requested now so that nothing is loaded after the reduction
-    // (raw: a bf16 bias is widened where it is used; a shift here would make the wavefront wait for
-    // the load before its operands are even requested)
-    float ep_scale[EPW];
-    uint32_t ep_bias[EPW];
-#pragma unroll
-    for (int t = 0; t < EPW; t++) {
-        const int idx = min(wave + t * KW, TA - 1);
-        const int n = min(n_base + 16 * ((idx >> 2) % NW) + ln, p.N - 1);
-        ep_scale[t] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[n] : 1.0f;
-        ep_bias[t] = 0;
-        if (p.bias)
-            ep_bias[t] = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
-                                                     : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
     }
 
     const int nsteps = (p.K + KSTEP - 1) / KSTEP;
@@ -352,6 +305,55 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 #pragma unroll
         for (int i = 0; i < MW; i++) load_x(wave, i, u, xr[i][u]);
     load_s(wave, sv);
+
+    // (everything from here to the loop is set up while the first loads are in flight)
+    f32x4 acc[MW][NW];
+    f32x4 xacc[MW];  // W8 only: sum_k x_k over the wave's k-steps
+#pragma unroll
+    for (int i = 0; i < MW; i++) {
+        xacc[i] = (f32x4){0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < NW; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
+    }
+
+    // ---- where a loaded register goes in the staging area and where a fragment (MFMA layout) comes from
+    // weights: staged at row * 64 + (piece ^ row/4) * 16 and read back as (row ln, piece kb)
+    const uint32_t w_st = XS + wrow * 64 + ((wpc ^ (wrow >> 2)) & 3) * 16;
+    const uint32_t w_rd = XS + ln * 64 + ((kb ^ (ln >> 2)) & 3) * 16;
+    // activations: staged at row * XB + (piece ^ f(row)) * 16 with f(row) = row (XB = 256) or row/2 (XB = 128)
+    auto swz = [](int row) { return XB == 256 ? row : (row >> 1); };
+    uint32_t x_st[NI], x_rd[QU][NL];
+#pragma unroll
+    for (int ii = 0; ii < NI; ii++) {
+        const int row = ii * RPI + trow;
+        x_st[ii] = row * XB + ((tpc ^ swz(row)) & (PPR - 1)) * 16;
+    }
+#pragma unroll
+    for (int qq = 0; qq < QU; qq++)
+#pragma unroll
+        for (int h = 0; h < NL; h++) {
+            // the piece that holds the first 8 k of fragment q of this lane (second half: + 4) within its unit
+            const int piece = FOUR_BIT ? (XF32 ? 8 * qq + 2 * kb + h : 4 * qq + kb)
+                                       : (XF32 ? 4 * kb + 2 * qq + h : 2 * kb + qq);
+            x_rd[qq][h] = ln * XB + ((piece ^ swz(ln)) & (PPR - 1)) * 16;
+        }
+
+    // the accumulators this wavefront finishes after the reduction are idx = wave + t KW; their
+    // per-channel operands are requested now so that nothing is loaded after the reduction
+    // (raw: a bf16 bias is widened where it is used; a shift here would make the wavefront wait for
+    // the load before its operands are even requested)
+    float ep_scale[EPW];
+    uint32_t ep_bias[EPW];
+#pragma unroll
+    for (int t = 0; t < EPW; t++) {
+        const int idx = min(wave + t * KW, TA - 1);
+        const int n = min(n_base + 16 * ((idx >> 2) % NW) + ln, p.N - 1);
+        ep_scale[t] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[n] : 1.0f;
+        ep_bias[t] = 0;
+        if (p.bias)
+            ep_bias[t] = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                                     : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
+    }
 
     int t4 = 0;  // the k-step's place in its quad of scale records
     for (int ks = wave; ks < nsteps; ks += KW, t4 = (t4 + 1) & 3) {
