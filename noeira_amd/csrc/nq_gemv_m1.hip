@@ -6,8 +6,9 @@
 // for the whole kernel: `lpr` lanes (a power of two) share a row, lane j owns
 // the 16-byte chunks j, j + lpr, ... (CPL of them), and the x values under
 // those chunks are loaded once, up front, together with the first weights -
-// one round trip to memory, no LDS, no barrier.  A lane group then walks its
-// rows RPL at a time (RPL x CPL independent loads in flight per lane); the
+// one round trip to memory, no LDS, no barrier (one exception: fp32 x under
+// 4-bit weights in a launch of a thousand wavefronts, STAGE_X below).  A lane
+// group then walks its rows RPL at a time (RPL x CPL independent loads in flight per lane); the
 // host picks one row per lane group and as many lanes per row as it takes to
 // launch ~1k wavefronts, which measured best from 68 KB to 45 MB of weights.
 // Every load is unconditional from a clamped address (a predicated load
@@ -101,12 +102,18 @@ __device__ __forceinline__ float group_sum(float v, int lpr) {
     return v;
 }
 
-template <int FMT, int XDT, bool DOT2, int CPL, int RPL>
+template <int FMT, int XDT, bool DOT2, int CPL, int RPL, bool STAGE_X>
 __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     constexpr bool FOUR_BIT = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP);
     constexpr int EPC = FOUR_BIT ? 32 : 16;
     constexpr int XR = DOT2 ? EPC / 2 : EPC;  // registers of x per chunk
     static_assert(!DOT2 || FOUR_BIT, "the bf16 dot path is for 4-bit weights");
+    // STAGE_X (4-bit weights with fp32 x, launches of a thousand wavefronts and more): a lane's chunk of x is
+    // 128 bytes, and eight loads whose lanes sit 128 bytes apart cost the L1 as much as eight times the cache
+    // lines they touch.  The workgroup fetches x once, adjacent lanes adjacent pieces, and hands it round
+    // through LDS instead.  (With fewer wavefronts the extra barrier costs more than the loads: measured.)
+    static_assert(!STAGE_X || (FOUR_BIT && !DOT2), "x is staged for 4-bit weights with fp32 x only");
+    extern __shared__ __attribute__((aligned(16))) uint8_t xstage[];  // STAGE_X: nch x 128 bytes
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lpr = p.lpr;
@@ -166,6 +173,17 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     // ---- this lane's slice of x, loaded once
     uint32_t xr[CPL][XR];  // fp32 bits, or bf16 pairs when DOT2
     float xsum[CPL];
+    // piece v (16 bytes) of chunk c sits at c * 128 + (v ^ (c / 2) % 8) * 16: 16 lanes reading the same piece
+    // of 16 consecutive chunks then touch every LDS bank once
+    auto xslot = [](int c, int v) { return c * 128 + ((v ^ ((c >> 1) & 7)) << 4); };
+    if constexpr (STAGE_X) {
+        const int npieces = p.nch * 8;
+        for (int e = threadIdx.x; e < npieces; e += 256) {
+            const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.x) + (size_t)e * 16);
+            *reinterpret_cast<u32x4*>(xstage + xslot(e >> 3, e & 7)) = t;
+        }
+        __syncthreads();
+    }
 #pragma unroll
     for (int i = 0; i < CPL; i++) {
         // clamped, unconditional loads; the product of a chunk past the end of the row is dropped below
@@ -183,7 +201,14 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
             }
         } else {
             float f[EPC];
-            if constexpr (XDT == NQ_DT_F32) {
+            if constexpr (STAGE_X) {
+                const int cc = min(lj + i * lpr, p.nch - 1);
+#pragma unroll
+                for (int v = 0; v < 8; v++) {
+                    const float4 t = *reinterpret_cast<const float4*>(xstage + xslot(cc, v));
+                    f[4 * v] = t.x, f[4 * v + 1] = t.y, f[4 * v + 2] = t.z, f[4 * v + 3] = t.w;
+                }
+            } else if constexpr (XDT == NQ_DT_F32) {
 #pragma unroll
                 for (int v = 0; v < EPC / 4; v++) {
                     const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.x) + k0 + 4 * v);
@@ -327,23 +352,24 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
 
 // Only the combinations the host picks are instantiated: at most 8 loads in flight per lane
 // (RPL x CPL), and at most 96 registers of x (CPL <= 3 when a chunk of x takes 32 registers).
-template <int FMT, int XDT, bool DOT2, int CPL>
+template <int FMT, int XDT, bool DOT2, int CPL, bool STAGE_X>
 int32_t launch_rpl(const M1Params& p, int rpl, dim3 grid, hipStream_t s) {
+    const size_t lds = STAGE_X ? (size_t)p.nch * 128 : 0;  // at most 3 x 64 chunks: 24 KiB
     if constexpr (CPL <= 2) {
         if (rpl >= 4) {
-            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 4>), grid, dim3(256), 0, s, p);
+            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 4, STAGE_X>), grid, dim3(256), lds, s, p);
             NQ_HIP(hipGetLastError());
             return NQ_OK;
         }
     }
     if constexpr (CPL <= 4) {
         if (rpl >= 2) {
-            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 2>), grid, dim3(256), 0, s, p);
+            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 2, STAGE_X>), grid, dim3(256), lds, s, p);
             NQ_HIP(hipGetLastError());
             return NQ_OK;
         }
     }
-    hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 1>), grid, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 1, STAGE_X>), grid, dim3(256), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
@@ -351,16 +377,25 @@ int32_t launch_rpl(const M1Params& p, int rpl, dim3 grid, hipStream_t s) {
 template <int FMT, int XDT, bool DOT2>
 int32_t launch_cpl(const M1Params& p, int cpl, int rpl, dim3 grid, hipStream_t s) {
     constexpr bool WIDE_X = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP) && !DOT2;
+    if constexpr (WIDE_X) {
+        if ((int64_t)grid.x * 4 >= 1024) {  // x through LDS
+            switch (cpl) {
+                case 1: return launch_rpl<FMT, XDT, DOT2, 1, true>(p, rpl, grid, s);
+                case 2: return launch_rpl<FMT, XDT, DOT2, 2, true>(p, rpl, grid, s);
+                case 3: return launch_rpl<FMT, XDT, DOT2, 3, true>(p, rpl, grid, s);
+            }
+        }
+    }
     switch (cpl) {
-        case 1: return launch_rpl<FMT, XDT, DOT2, 1>(p, rpl, grid, s);
-        case 2: return launch_rpl<FMT, XDT, DOT2, 2>(p, rpl, grid, s);
-        case 3: return launch_rpl<FMT, XDT, DOT2, 3>(p, rpl, grid, s);
+        case 1: return launch_rpl<FMT, XDT, DOT2, 1, false>(p, rpl, grid, s);
+        case 2: return launch_rpl<FMT, XDT, DOT2, 2, false>(p, rpl, grid, s);
+        case 3: return launch_rpl<FMT, XDT, DOT2, 3, false>(p, rpl, grid, s);
     }
     if constexpr (!WIDE_X) {
         switch (cpl) {
-            case 4: return launch_rpl<FMT, XDT, DOT2, 4>(p, rpl, grid, s);
-            case 5: return launch_rpl<FMT, XDT, DOT2, 5>(p, rpl, grid, s);
-            case 6: return launch_rpl<FMT, XDT, DOT2, 6>(p, rpl, grid, s);
+            case 4: return launch_rpl<FMT, XDT, DOT2, 4, false>(p, rpl, grid, s);
+            case 5: return launch_rpl<FMT, XDT, DOT2, 5, false>(p, rpl, grid, s);
+            case 6: return launch_rpl<FMT, XDT, DOT2, 6, false>(p, rpl, grid, s);
         }
     }
     return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no single-row GEMV variant for this IN");

@@ -188,3 +188,38 @@ def test_many_rows_fused_parts_match_their_own_layers():
     for l, y in zip(layers, fused.forward(x)):
         own = l.forward(x)
         assert (y - own).abs().max().item() <= 2e-6 * own.abs().max().item()
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "w4g", "w4g64"])
+def test_single_row_fp32_x_through_lds(fmt):
+    """One row of fp32 activations over a 4-bit weight with a thousand wavefronts and more: the workgroup
+    stages x in LDS and every lane takes its chunks from there.  A row of 30, 31 (odd) and 191 chunks (the
+    most the kernel holds; the last lane group's chunks run past the row), and a short launch that loads x
+    directly, for comparison."""
+    rng = np.random.default_rng(sum(map(ord, fmt)) + 5)
+    for (K, N) in ((960, 2560), (992, 3000), (6112, 1100), (960, 5120), (960, 700)):
+        if fmt.startswith("w4g"):
+            group = 128 if fmt == "w4g" else 64
+            G = -(-K // group)
+            q = rng.integers(0, 16, (N, K), dtype=np.uint8)
+            z = rng.integers(0, 16, (N, G), dtype=np.uint8)
+            codes, zps = F.pack_w4g(q, z)
+            lin = W4GroupLinear(K, N, group)
+            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+        else:
+            lin = QLinear(K, N)
+            blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0] = sc & 0xFF
+            blocks[:, :, 1] = sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+        deq = lin.dequantized_dev().double()
+        x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).cuda()
+        tag = "%s M=1 K=%d N=%d fp32" % (fmt, K, N)
+        exact = x.double() @ deq.T
+        y = lin.forward(x)
+        _check(tag, y, exact, False)
+        # the reference's band for its fp32 path: 1e-5 of the largest value
+        assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max()), tag
+        assert torch.equal(y, lin.forward(x)), tag + ": a repeated call differs"
+        del lin
