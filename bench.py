@@ -469,8 +469,8 @@ def sweep(skip_large=False):
             calls=10)
         c8 = max(1, COLD_BYTES // (4096 * 11008))
         run("W8A8 int8 GEMV K=4096 N=11008 M=1 (cold)", make_w8a8_m1, "hbm", K=4096, N=11008, copies=c8, calls=c8)
-        # a few rows to a few hundred: the 16-row tile kernel's range
-        for M in (16, 64, 256):
+        # a few rows to several hundred: the 16-row tile kernel's range
+        for M in (16, 64, 256, 512):
             run(f"W8A8 int8 M={M} K=4096 N=4096 (warm)", make_w8a8_gemm, "mfma", "int8", M=M, N=4096, calls=20)
             run(f"fp8 x fp8 M={M} K=4096 N=4096 (warm)", make_fp8, "mfma", "fp8", M=M, N=4096, copies=1, calls=20)
         # the dequant-GEMVs at a size where the HBM fraction means something (22 - 45 MB of codes)
@@ -550,14 +550,14 @@ def only_loop(which, steps, warmup):
         name = ("W4A16 g128 and W8A16 at 4096 x 4096, M = 4096; Q4_0 (fp32 x) 960->2560 at M = 4096 and 1120; "
                 "one call each per step")
     elif which == "tile8":
-        wls = [make_w8a8_gemm(M, 4096) for M in (16, 64, 256)] + [make_fp8(M, 4096) for M in (16, 64, 256)]
+        wls = [make_w8a8_gemm(M, 4096) for M in (16, 64, 128, 256, 512)] + [make_fp8(M, 4096) for M in (16, 64, 128, 256, 512)]
 
         def step_t8(i):
             for w in wls:
                 w["step"](i)
 
         wl = dict(step=step_t8, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
-        name = "W8A8 and fp8 x fp8 at 4096 x 4096, M = 16, 64, 256, one call each per step"
+        name = "W8A8 and fp8 x fp8 at 4096 x 4096, M = 16, 64, 128, 256, 512, one call each per step"
     elif which == "actor":
         wl = make_actor_fused()
         name = "cfg3 W8A8 actor 64->256->256->8 M=4096, fused"
@@ -624,7 +624,7 @@ def main():
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
                          "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
                          "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, tile8 = int8 and fp8 "
-                         "activations at M = 16, 64, 256 over 4096 x 4096, manyrows = bf16 / fp32 activations at M = 1120 "
+                         "activations at M = 16 .. 512 over 4096 x 4096, manyrows = bf16 / fp32 activations at M = 1120 "
                          "and 4096")
     ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--no-cpu", action="store_true")

@@ -421,7 +421,9 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     // int32) contiguous per row of y.
     const int wm0 = m0 + wm * 128, wn0 = n0 + wn * WN;
     const int lm = lane & 31, lh = lane >> 5;
-    const bool full_tile = (m0 + BM <= p.M) && (n0 + BN <= p.N) && (p.N % 8 == 0);
+    // whole 16-byte stores wherever the tile's columns all exist and rows of y stay 16-byte aligned
+    // (a tile that only M cuts short just skips the rows past M)
+    const bool full_cols = (n0 + BN <= p.N) && (p.N % 8 == 0);
 
     // channel scale and bias for the lane's channels of tile j, group g (needs n < N: clamped)
     auto chan = [&](int j, int g, float (&cs)[4], float (&cb)[4], bool need_scale) {
@@ -527,8 +529,9 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
                 const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * ROWB + c16 * 16);
                 const int m = wm0 + 32 * ip + row;
                 const int n = wn0 + c16 * (16 / ES);
-                if (full_tile) {
-                    *reinterpret_cast<i32x4*>(reinterpret_cast<uint8_t*>(p.y) + ((int64_t)m * p.N + n) * ES) = v;
+                if (full_cols) {
+                    if (m < p.M)
+                        *reinterpret_cast<i32x4*>(reinterpret_cast<uint8_t*>(p.y) + ((int64_t)m * p.N + n) * ES) = v;
                 } else if (m < p.M) {
                     // ragged edge: element by element
 #pragma unroll

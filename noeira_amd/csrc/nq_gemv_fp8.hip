@@ -10,7 +10,10 @@
 // of weights (2 KB) by 16 activation rows, so the kernel is loads plus a handful of MFMAs:
 //   - a workgroup owns 16 weight rows and up to 64 activation rows (MT tiles of 16; more rows
 //     take more workgroups along grid.y, re-reading the weights from L2); its KW wavefronts
-//     split K, SPW steps of 128 k each;
+//     split K, SPW steps of 128 k each.  With 64 rows and more, and enough weight rows that
+//     160 workgroups remain, a workgroup takes NT = 2 or 4 weight tiles: an activation
+//     fragment then serves NT MFMAs, and the activations (the larger operand at 64 rows
+//     against 16) are fetched once per 16 NT weight rows;
 //   - loads are row-contiguous: 8 rows x 128 bytes per instruction, eight adjacent lanes per row
 //     (a load instruction is priced by the pieces of cache line its lanes touch), and reach the
 //     MFMA operand layout through a private 4 KiB of LDS per wavefront: one 128-bit store and
@@ -21,9 +24,9 @@
 //   - the KW partial 16 x 16 tiles are summed through LDS in wave order (fixed, so a repeated
 //     call returns the same bits; the int32 sums are exact in any order) and thread (m, n)
 //     applies scales, bias and epilogue.
-// The same kernel serves up to a few hundred rows where the 256 x 256-tile GEMM would leave most
-// of the chip idle (M = 64 .. 512 over a 4096 x 4096 weight is 16 .. 32 tiles on 256 CUs):
-// tile8_applicable holds the measured crossover.
+// The same kernel serves up to several hundred rows where the 256 x 256-tile GEMM would leave most
+// of the chip idle (M = 64 .. 768 over a 4096 x 4096 weight is 16 .. 48 tiles on 256 CUs):
+// tile8_wins holds the measured crossover.
 //
 // A single activation row (M = 1) takes a second kernel whose loads are fully coalesced: one
 // wavefront owns ONE weight row and reads it as 1 KB contiguous per load instruction (lane l
@@ -67,24 +70,25 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
     return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
 }
 
-template <bool I8, int SPW, int KW, int MT>
+template <bool I8, int SPW, int KW, int MT, int NT>
 __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
     typedef typename std::conditional<I8, i32x4, f32x4>::type acc_t;
-    __shared__ uint32_t red[KW][256];
+    __shared__ uint32_t red[KW][NT * 256];
     __shared__ __attribute__((aligned(16))) uint8_t stage[KW][4096];  // [weights 16 x 128 | activations 16 x 128]
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ln = lane & 15, kb = lane >> 4;
-    const int n_base = blockIdx.x * 16;
+    const int n_base = blockIdx.x * (16 * NT);
     const int m_base = blockIdx.y * (16 * MT);
 
     // a load: lane -> row 8 t + lane / 8 of the tile, 16-byte piece lane % 8 of the step's 128 bytes
     const int trow = lane >> 3, tpc = lane & 7;
-    int64_t wsrc[2], xsrc[MT][2];
+    int64_t wsrc[NT][2], xsrc[MT][2];
     uint32_t st[2], rd[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const int row = 8 * t + trow;
-        wsrc[t] = (int64_t)min(n_base + row, p.N - 1) * p.K + tpc * 16;
+#pragma unroll
+        for (int j = 0; j < NT; j++) wsrc[j][t] = (int64_t)min(n_base + 16 * j + row, p.N - 1) * p.K + tpc * 16;
 #pragma unroll
         for (int i = 0; i < MT; i++) xsrc[i][t] = (int64_t)min(m_base + 16 * i + row, p.M - 1) * p.K + tpc * 16;
         st[t] = row * 128 + ((tpc ^ (row >> 1)) & 7) * 16;
@@ -96,9 +100,11 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
     uint8_t* scr = stage[wave];
     auto lds16 = [&](uint32_t off) -> u32x4& { return *reinterpret_cast<u32x4*>(scr + off); };
 
-    acc_t acc[MT];
+    acc_t acc[MT][NT];
 #pragma unroll
-    for (int i = 0; i < MT; i++) acc[i] = (acc_t){0, 0, 0, 0};
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[i][j] = (acc_t){0, 0, 0, 0};
     // K need not be a multiple of the step: a lane's 16-byte piece of the last step may lie past the row.
     // Its address is then moved to the start of the step (inside the row) and, when the step is
     // staged, both operands' pieces are replaced by zeros (an fp8 NaN times zero would not be zero).
@@ -106,14 +112,17 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
     const bool in_last = klast + tpc * 16 < p.K;       // this lane's piece of the last step lies inside K
     const int64_t poff = in_last ? 0 : -(int64_t)tpc * 16;
     for (int s0 = wave * SPW; s0 < p.nsteps; s0 += KW * SPW) {
-        u32x4 wv[SPW][2], xv[MT][SPW][2];
+        u32x4 wv[NT][SPW][2], xv[MT][SPW][2];
         // unconditional loads from clamped step indices; a step past K meets zero activations
 #pragma unroll
         for (int s = 0; s < SPW; s++) {
             const int ks = min(s0 + s, p.nsteps - 1);
             const int64_t k0 = (int64_t)ks * 128 + (ks == p.nsteps - 1 ? poff : 0);
-            wv[s][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[0] + k0));
-            wv[s][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[1] + k0));
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                wv[j][s][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[j][0] + k0));
+                wv[j][s][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.w + wsrc[j][1] + k0));
+            }
         }
 #pragma unroll
         for (int i = 0; i < MT; i++)
@@ -131,48 +140,61 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) wv[s][t][e] &= keep;
+                    for (int j = 0; j < NT; j++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) wv[j][s][t][e] &= keep;
 #pragma unroll
                     for (int i = 0; i < MT; i++)
 #pragma unroll
                         for (int e = 0; e < 4; e++) xv[i][s][t][e] &= keep;
                 }
             }
-            lds16(st[0]) = wv[s][0], lds16(st[1]) = wv[s][1];
-            const u32x4 b0 = lds16(rd[0]), b1 = lds16(rd[1]);
+            // (a wavefront's LDS accesses execute in order: tile j + 1 may overwrite tile j once its reads are issued)
+            u32x4 b0[NT], b1[NT];
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                lds16(st[0]) = wv[j][s][0], lds16(st[1]) = wv[j][s][1];
+                b0[j] = lds16(rd[0]), b1[j] = lds16(rd[1]);
+            }
 #pragma unroll
             for (int i = 0; i < MT; i++) {
                 lds16(2048 + st[0]) = xv[i][s][0], lds16(2048 + st[1]) = xv[i][s][1];
                 u32x4 a0 = lds16(2048 + rd[0]), a1 = lds16(2048 + rd[1]);
                 if (s0 + s >= p.nsteps) a0 = a1 = (u32x4){0, 0, 0, 0};  // uniform over the wavefront
-                if constexpr (I8) {
-                    acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0),
-                                                                   __builtin_bit_cast(i32x4, b0), acc[i], 0, 0, 0);
-                    acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1),
-                                                                   __builtin_bit_cast(i32x4, b1), acc[i], 0, 0, 0);
-                } else {
-                    const i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],
-                                     (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
-                    const i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3],
-                                     (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
-                    acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    if constexpr (I8) {
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a0),
+                                                                          __builtin_bit_cast(i32x4, b0[j]), acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a1),
+                                                                          __builtin_bit_cast(i32x4, b1[j]), acc[i][j], 0, 0, 0);
+                    } else {
+                        const i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3],
+                                         (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+                        const i32x8 b = {(int)b0[j][0], (int)b0[j][1], (int)b0[j][2], (int)b0[j][3],
+                                         (int)b1[j][0], (int)b1[j][1], (int)b1[j][2], (int)b1[j][3]};
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i][j], 0, 0, 0, 0, 0, 0);
+                    }
                 }
             }
         }
     }
 
     // D layout: lane holds column n = lane % 16, rows m = 4 (lane / 16) + r.  The K-slices of one
-    // activation tile at a time are summed in wave order (fixed, so results repeat bit for bit).
-    const int t = threadIdx.x;
+    // activation tile (all its NT weight tiles) at a time are summed in wave order (fixed, so results
+    // repeat bit for bit).
 #pragma unroll
     for (int i = 0; i < MT; i++) {
         if (i) __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-            red[wave][(4 * kb + r) * 16 + ln] = I8 ? (uint32_t)acc[i][r] : __float_as_uint((float)acc[i][r]);
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                red[wave][j * 256 + (4 * kb + r) * 16 + ln] =
+                    I8 ? (uint32_t)acc[i][j][r] : __float_as_uint((float)acc[i][j][r]);
         __syncthreads();
-        if (t < 256) {
-            const int m = m_base + 16 * i + (t >> 4), n = n_base + (t & 15);
+        for (int t = threadIdx.x; t < NT * 256; t += 64 * KW) {
+            const int m = m_base + 16 * i + ((t & 255) >> 4), n = n_base + 16 * (t >> 8) + (t & 15);
             if (m < p.M && n < p.N) {
                 const int64_t o = (int64_t)m * p.N + n;
                 float z;
@@ -326,18 +348,29 @@ int32_t launch_row_cpl(const Fp8GemvParams& p, hipStream_t s) {
     }
 }
 
-template <bool I8, int SPW, int MT>
+template <bool I8, int SPW, int MT, int NT>
 int32_t launch_kw(const Fp8GemvParams& p, int kw, dim3 grid, hipStream_t s) {
     if (kw == 4)
-        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 4, MT>), grid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 4, MT, NT>), grid, dim3(256), 0, s, p);
     else if (kw == 8)
-        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 8, MT>), grid, dim3(512), 0, s, p);
-    else if constexpr (SPW * MT <= 4)
-        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 16, MT>), grid, dim3(1024), 0, s, p);
+        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 8, MT, NT>), grid, dim3(512), 0, s, p);
+    else if constexpr (SPW * MT <= 4 && NT == 1)
+        hipLaunchKernelGGL((tile8_kernel<I8, SPW, 16, MT, 1>), grid, dim3(1024), 0, s, p);
     else
         return fail(NQ_ERR_INVALID, "nq_forward: no 8-bit tile kernel of that shape");
     NQ_HIP(hipGetLastError());
     return NQ_OK;
+}
+
+// weight tiles (of 16 rows) per workgroup: with 64 activation rows per workgroup, the most that still
+// leaves 160 workgroups (measured: 4096 x 4096 at 64 / 128 / 256 rows is best with 1 / 2 / 4); one for
+// K < 1024, where a wavefront has a single step and more, smaller workgroups hide its latency better
+int tile8_weight_tiles(int M, int64_t out, int K) {
+    const int mt_all = (M + 15) / 16;
+    if (mt_all < 4 || K < 1024) return 1;
+    for (int c = 4; c >= 2; c /= 2)
+        if (((out + 16 * c - 1) / (16 * c)) * ((mt_all + 3) / 4) >= 160) return c;
+    return 1;
 }
 
 template <bool I8>
@@ -358,9 +391,19 @@ int32_t launch_tile8(const Fp8GemvParams& p, int64_t out, hipStream_t stream) {
         if (mt <= 2) spw = 4 / mt;
         else kw = 8;
     }
+    // Several weight tiles per workgroup (an activation fragment then serves NT MFMAs and is fetched once
+    // per 16 NT weight rows) wherever that still leaves workgroups for every CU
+    const int nt = tile8_weight_tiles(p.M, out, p.K);
+    if (nt > 1) {
+        const int64_t wgn = (out + 16 * nt - 1) / (16 * nt);
+        const dim3 gridn((unsigned)wgn, (unsigned)((mt_all + 3) / 4));
+        const int kwn = p.nsteps > 4 ? 8 : 4;
+        if (nt == 4) return launch_kw<I8, 1, 4, 4>(p, kwn, gridn, stream);
+        return launch_kw<I8, 1, 4, 2>(p, kwn, gridn, stream);
+    }
     const dim3 grid((unsigned)wgs, (unsigned)((mt_all + mt - 1) / mt));
 #define NQ_T8_CASE(SPW_, MT_) \
-    if (spw == SPW_ && mt == MT_) return launch_kw<I8, SPW_, MT_>(p, kw, grid, stream);
+    if (spw == SPW_ && mt == MT_) return launch_kw<I8, SPW_, MT_, 1>(p, kw, grid, stream);
     NQ_T8_CASE(1, 1) NQ_T8_CASE(2, 1) NQ_T8_CASE(4, 1) NQ_T8_CASE(8, 1)
     NQ_T8_CASE(1, 2) NQ_T8_CASE(2, 2) NQ_T8_CASE(4, 2)
     NQ_T8_CASE(1, 3) NQ_T8_CASE(2, 3)
@@ -378,18 +421,30 @@ static bool row_kernel_fits(const ForwardArgs& a) {
 }
 
 // The tile kernel against the 256 x 256-tile GEMM (nq_gemm8.hip), both measured over K = 512 .. 8192,
-// N = 1024 .. 11008, M = 64 .. 2048: the tile kernel takes about 4 us + 5.6 us per 10^9 multiply-adds
-// (its weights are re-read per 64 activation rows), a round of GEMM tiles about 8 us + 1.15 us per
-// 128 k, at least 17 us.  Below 64 rows the GEMM does not apply.
+// N = 1024 .. 11008, M = 64 .. 2048.  A round of GEMM tiles (up to 256) takes about 14 us + 1.25 us per 128 k
+// (fp8: 10 + 1.1).
+// The tile kernel with 2 or 4 weight tiles per workgroup takes, per round of 256 workgroups, a fixed 5.5 us
+// (3.75 with four wavefronts) + 0.25 / 0.31 us per 128 k, half as much again when 64 rows at a time stream a
+// weight larger than the caches hold; with one weight tile (small launches, short K) about 4 us + 5.6 us per
+// 10^9 multiply-adds, more with few steps of K.  Below 64 rows the GEMM does not apply.
 static bool tile8_wins(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (L->in % 16 != 0) return false;
     if (a.M < 64 || L->in % 128 != 0) return true;  // (the GEMM needs 64 rows and whole 128-byte steps)
-    const double gmac = (double)a.M * (double)L->in * (double)L->out * 1e-9;
+    const double steps = (double)L->in / 128.0;
     const int64_t tiles = (int64_t)((a.M + 255) / 256) * ((L->out + 255) / 256);
-    const double rounds = (double)((tiles + 255) / 256);
-    const double gemm_us = rounds * std::max(17.0, 8.0 + (double)L->in / 128.0 * 1.15);
-    return 4.0 + 5.6 * gmac < gemm_us;
+    const bool i8 = a.x_dtype == NQ_DT_I8;
+    const double gemm_us = (double)((tiles + 255) / 256) * (i8 ? 14.0 + 1.25 * steps : 10.0 + 1.1 * steps);
+    const int nt = tile8_weight_tiles(a.M, L->out, L->in);
+    double tile_us;
+    if (nt == 1) {
+        tile_us = 4.0 + (5.6 + 9.6 / steps) * ((double)a.M * (double)L->in * (double)L->out * 1e-9);
+    } else {
+        const double wgs = (double)((L->out + 16 * nt - 1) / (16 * nt)) * (double)((a.M + 63) / 64);
+        tile_us = std::max(1.0, wgs / 256.0) * ((steps > 4 ? 5.5 : 3.75) + (nt == 4 ? 0.31 : 0.25) * steps);
+        if (a.M >= 128 && (int64_t)L->in * L->out > ((int64_t)32 << 20)) tile_us *= 1.5;
+    }
+    return tile_us < gemm_us;
 }
 
 bool gemv_fp8_applicable(const ForwardArgs& a) {

@@ -238,10 +238,12 @@ def test_config5_fp8_gemv_full_size_sampled():
 
 @pytest.mark.parametrize("M,K,N", [(1, 128, 16), (3, 384, 40), (16, 2560, 100), (2, 8192, 33),
                                    (1, 784, 37), (1, 1024, 5), (1, 2576, 130), (1, 8192, 19), (1, 8208, 9),
-                                   (3, 400, 40), (40, 1040, 100), (200, 16, 24), (1, 48, 7)])
+                                   (3, 400, 40), (40, 1040, 100), (200, 16, 24), (1, 48, 7),
+                                   (300, 960, 2600), (130, 1040, 2600), (520, 1024, 1288)])
 def test_fp8_small_m_bias_relu_and_shapes(M, K, N):
-    """fp8 x fp8 at 1..200 rows: ragged N, K from a fraction of one MFMA step to several rounds of the K split,
-    fp32 bias and ReLU fused; checked against the float64 oracle."""
+    """fp8 x fp8 at 1..520 rows: ragged N, K from a fraction of one MFMA step to several rounds of the K split,
+    fp32 bias and ReLU fused; checked against the float64 oracle.  The last three take the tile kernel with
+    four, two and four weight tiles per workgroup (K 64 short of a step, 16 past one, a multiple of it)."""
     rng = np.random.default_rng(1000 + M + K)
     a, b = fp8_operands(rng, M, N, K)
     sa, sb = np.float32(0.5), np.float32(0.25)
@@ -291,15 +293,17 @@ def test_config5_fp8_gemm_full_size_sampled(N):
                                    (5, 128, 24), (63, 4096, 100), (1, 512, 48),
                                    (4096, 64, 256), (300, 960, 520), (5, 80, 24), (70, 16, 40),
                                    (1, 784, 37), (1, 4096, 130), (1, 8192, 19), (1, 2576, 5),
-                                   (1100, 1024, 2296), (1100, 1024, 2300)])
+                                   (1100, 1024, 2296), (300, 960, 2600), (130, 1040, 2600),
+                                   (2100, 512, 2296), (2100, 512, 2300)])
 def test_int8_gemm_bit_exact(M, K, N):
     """W8A8 on the int8 matrix cores: int32 accumulators equal the oracle's bit for bit, ragged
     M / N edges included; the fused epilogue matches the oracle's fp32 expression.  The first
     seven shapes run on the 16-row tile kernel (few rows, or too few 256 x 256 tiles to fill the
     chip), the next four too, with K not a multiple of the kernel's 128-wide step (64 is the actor's
-    first layer), then four single rows of 768 .. 8192 codes on the one-row kernel, the last two on
-    the large-tile GEMM (45 tiles, the last row and column of tiles cut short, N a multiple of 8 and
-    not)."""
+    first layer), then four single rows of 768 .. 8192 codes on the one-row kernel, then three on the
+    tile kernel with four, four and two weight tiles per workgroup (ragged M and N, K a multiple of the
+    step, 64 short of it, 16 past it), the last two on the large-tile GEMM (81 tiles, the last row and
+    column of tiles cut short, N a multiple of 8 and not)."""
     rng = np.random.default_rng(M + K + N)
     lin, w, s = w8_layer(rng, K, N)
     xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
@@ -320,9 +324,9 @@ def test_int8_gemm_bit_exact(M, K, N):
 
 @pytest.mark.parametrize("N", [2296, 2300])
 def test_fp8_gemm_ragged_tiles_vs_oracle(N):
-    """fp8 x fp8 through the large-tile GEMM at a size the oracle finishes in seconds: 5 x 9 tiles of
+    """fp8 x fp8 through the large-tile GEMM at a size the oracle finishes in seconds: 9 x 9 tiles of
     256 x 256 with the last row and column of tiles cut short; every element against the oracle."""
-    M, K = 1100, 1024
+    M, K = 2100, 512
     rng = np.random.default_rng(N)
     a, b = fp8_operands(rng, M, N, K)
     sa, sb = np.float32(0.5), np.float32(0.25)
