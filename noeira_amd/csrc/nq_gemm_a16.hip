@@ -4,12 +4,13 @@
 // This is the regime of the reference's real caller, the SmolVLA prefill at
 // T = 135 tokens (noeira/deep_agents/smolvla/fused.mojo:255-384), and of
 // BASELINE's M = 100 / 256 configs: the weights are ~1 MB, so the call is
-// bound by instruction issue per wavefront and by L1 look-ups, not by MFMA or
-// bytes.  The kernel therefore has no LDS staging and no block-wide barrier in
-// its K loop: every wavefront pulls its own operand fragments straight from
-// global memory (x is L2-resident, W is read once per M tile) and the only
-// synchronisation is the final fixed-order reduction of the K-slices through
-// LDS.
+// bound by instruction issue per wavefront and by what its loads cost in the
+// L1, not by MFMA or bytes.  The medium-M kernel has no block-wide barrier in
+// its K loop: every wavefront fetches its own operands (row-contiguous loads,
+// x is L2-resident, W is read once per M tile), turns them into MFMA fragments
+// through a private piece of LDS, and the only synchronisation is the final
+// fixed-order reduction of the K-slices through LDS.  From 512 rows on a second
+// kernel stages tiles per workgroup (below).
 //
 // Exactness.  Weights enter the MFMA as the integer codes, converted to bf16
 // exactly: a 4-bit code q becomes 16 + q by OR-ing it into the mantissa of
@@ -28,11 +29,11 @@
 // (the reference's own AMD path is an fp32 GEMM over deq(W), gate 1e-5).
 //
 // 4-bit device layout (see nq_q4_0.hip): a 16-byte chunk holds 32 consecutive
-// k as four words of eight; lane (n, kb) loads the whole chunk c0 + kb of its
-// row with one 128-bit load, and two lane-swap stages (v_permlane32_swap,
-// v_permlane16_swap) transpose the 4 x 4 words among the four lanes of a row so
-// that lane kb ends up with word kb of chunks c0 .. c0+3: exactly its share of
-// the B operand of four MFMAs.
+// k as four words of eight; lane (n, kb) takes the whole chunk c0 + kb of its
+// row from the staging area with one 128-bit read, and two lane-swap stages
+// (v_permlane32_swap, v_permlane16_swap) transpose the 4 x 4 words among the
+// four lanes of a row so that lane kb ends up with word kb of chunks
+// c0 .. c0+3: exactly its share of the B operand of four MFMAs.
 #include <hip/hip_fp16.h>
 
 #include <algorithm>

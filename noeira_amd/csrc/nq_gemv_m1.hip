@@ -244,6 +244,9 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     }
 
 #define XF(i, e) __uint_as_float(xr[(i)][(e)])
+    // (p.rpw is RPL in every launch; with the trip count a compile-time 1 the compiler orders the
+    // prologue differently and most calls are 2 - 8 % slower: measured, with and without a scheduling
+    // barrier after the first loads)
     for (int rb = 0; rb < p.rpw; rb += RPL) {
         const int64_t row0 = row_begin + rb;
         if (row0 >= p.N) break;
@@ -350,52 +353,39 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
 
 #undef XF
 
-// Only the combinations the host picks are instantiated: at most 8 loads in flight per lane
-// (RPL x CPL), and at most 96 registers of x (CPL <= 3 when a chunk of x takes 32 registers).
+// Only the combinations the host picks are instantiated: one row per lane group (RPL = 1: more rows per
+// lane measured slower at every size, see launch_gemv_m1), and at most 96 registers of x (CPL <= 3 when a
+// chunk of x takes 32 registers).
 template <int FMT, int XDT, bool DOT2, int CPL, bool STAGE_X>
-int32_t launch_rpl(const M1Params& p, int rpl, dim3 grid, hipStream_t s) {
+int32_t launch_one(const M1Params& p, dim3 grid, hipStream_t s) {
     const size_t lds = STAGE_X ? (size_t)p.nch * 128 : 0;  // at most 3 x 64 chunks: 24 KiB
-    if constexpr (CPL <= 2) {
-        if (rpl >= 4) {
-            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 4, STAGE_X>), grid, dim3(256), lds, s, p);
-            NQ_HIP(hipGetLastError());
-            return NQ_OK;
-        }
-    }
-    if constexpr (CPL <= 4) {
-        if (rpl >= 2) {
-            hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 2, STAGE_X>), grid, dim3(256), lds, s, p);
-            NQ_HIP(hipGetLastError());
-            return NQ_OK;
-        }
-    }
     hipLaunchKernelGGL((gemv_m1_kernel<FMT, XDT, DOT2, CPL, 1, STAGE_X>), grid, dim3(256), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
 
 template <int FMT, int XDT, bool DOT2>
-int32_t launch_cpl(const M1Params& p, int cpl, int rpl, dim3 grid, hipStream_t s) {
+int32_t launch_cpl(const M1Params& p, int cpl, dim3 grid, hipStream_t s) {
     constexpr bool WIDE_X = (FMT == NQ_FMT_Q4_0 || FMT == NQ_FMT_W4_GROUP) && !DOT2;
     if constexpr (WIDE_X) {
         if ((int64_t)grid.x * 4 >= 1024) {  // x through LDS
             switch (cpl) {
-                case 1: return launch_rpl<FMT, XDT, DOT2, 1, true>(p, rpl, grid, s);
-                case 2: return launch_rpl<FMT, XDT, DOT2, 2, true>(p, rpl, grid, s);
-                case 3: return launch_rpl<FMT, XDT, DOT2, 3, true>(p, rpl, grid, s);
+                case 1: return launch_one<FMT, XDT, DOT2, 1, true>(p, grid, s);
+                case 2: return launch_one<FMT, XDT, DOT2, 2, true>(p, grid, s);
+                case 3: return launch_one<FMT, XDT, DOT2, 3, true>(p, grid, s);
             }
         }
     }
     switch (cpl) {
-        case 1: return launch_rpl<FMT, XDT, DOT2, 1, false>(p, rpl, grid, s);
-        case 2: return launch_rpl<FMT, XDT, DOT2, 2, false>(p, rpl, grid, s);
-        case 3: return launch_rpl<FMT, XDT, DOT2, 3, false>(p, rpl, grid, s);
+        case 1: return launch_one<FMT, XDT, DOT2, 1, false>(p, grid, s);
+        case 2: return launch_one<FMT, XDT, DOT2, 2, false>(p, grid, s);
+        case 3: return launch_one<FMT, XDT, DOT2, 3, false>(p, grid, s);
     }
     if constexpr (!WIDE_X) {
         switch (cpl) {
-            case 4: return launch_rpl<FMT, XDT, DOT2, 4, false>(p, rpl, grid, s);
-            case 5: return launch_rpl<FMT, XDT, DOT2, 5, false>(p, rpl, grid, s);
-            case 6: return launch_rpl<FMT, XDT, DOT2, 6, false>(p, rpl, grid, s);
+            case 4: return launch_one<FMT, XDT, DOT2, 4, false>(p, grid, s);
+            case 5: return launch_one<FMT, XDT, DOT2, 5, false>(p, grid, s);
+            case 6: return launch_one<FMT, XDT, DOT2, 6, false>(p, grid, s);
         }
     }
     return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no single-row GEMV variant for this IN");
@@ -448,33 +438,30 @@ int32_t launch_gemv_m1(const ForwardArgs& a) {
     // One row per lane group and one batch per wavefront: the most wavefronts, the shortest
     // dependency chain.  Measured best from 68 KB to 45 MB of weights (memory-level parallelism
     // comes from occupancy, not from rows per lane).
-    int rpl = 1;
-    const int mult = 1;
     cpl = (p.nch + lpr - 1) / lpr;
-    rpl = cpl <= 2 ? (rpl >= 4 ? 4 : (rpl >= 2 ? 2 : 1)) : (cpl <= 4 ? (rpl >= 2 ? 2 : 1) : 1);
     p.lpr = lpr;
     p.lpr_log2 = 0;
     while ((1 << p.lpr_log2) < lpr) p.lpr_log2++;
-    p.rpw = rpl * mult;
+    p.rpw = 1;
     const int64_t groups = ((int64_t)L->out + p.rpw - 1) / p.rpw;
     const int64_t groups_per_block = 4 * (64 / lpr);
     dim3 grid((unsigned)((groups + groups_per_block - 1) / groups_per_block));
     const int xd = a.x_dtype;
     switch (L->format) {
         case NQ_FMT_Q4_0:
-            if (dot2) return launch_cpl<NQ_FMT_Q4_0, NQ_DT_BF16, true>(p, cpl, rpl, grid, a.stream);
-            return launch_cpl<NQ_FMT_Q4_0, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
+            if (dot2) return launch_cpl<NQ_FMT_Q4_0, NQ_DT_BF16, true>(p, cpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_Q4_0, NQ_DT_F32, false>(p, cpl, grid, a.stream);
         case NQ_FMT_W4_GROUP:
-            if (dot2) return launch_cpl<NQ_FMT_W4_GROUP, NQ_DT_BF16, true>(p, cpl, rpl, grid, a.stream);
-            return launch_cpl<NQ_FMT_W4_GROUP, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
+            if (dot2) return launch_cpl<NQ_FMT_W4_GROUP, NQ_DT_BF16, true>(p, cpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_W4_GROUP, NQ_DT_F32, false>(p, cpl, grid, a.stream);
         case NQ_FMT_W8_CHANNEL:
-            if (xd == NQ_DT_BF16) return launch_cpl<NQ_FMT_W8_CHANNEL, NQ_DT_BF16, false>(p, cpl, rpl, grid, a.stream);
-            return launch_cpl<NQ_FMT_W8_CHANNEL, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
+            if (xd == NQ_DT_BF16) return launch_cpl<NQ_FMT_W8_CHANNEL, NQ_DT_BF16, false>(p, cpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_W8_CHANNEL, NQ_DT_F32, false>(p, cpl, grid, a.stream);
         case NQ_FMT_FP8_E4M3:
             if (xd == NQ_DT_FP8_E4M3)
-                return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_FP8_E4M3, false>(p, cpl, rpl, grid, a.stream);
-            if (xd == NQ_DT_BF16) return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_BF16, false>(p, cpl, rpl, grid, a.stream);
-            return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_F32, false>(p, cpl, rpl, grid, a.stream);
+                return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_FP8_E4M3, false>(p, cpl, grid, a.stream);
+            if (xd == NQ_DT_BF16) return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_BF16, false>(p, cpl, grid, a.stream);
+            return launch_cpl<NQ_FMT_FP8_E4M3, NQ_DT_F32, false>(p, cpl, grid, a.stream);
     }
     return fail(NQ_ERR_INVALID, "nq_forward: unknown format");
 }
