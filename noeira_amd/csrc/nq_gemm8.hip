@@ -85,6 +85,7 @@ struct Gemm8Params {
     int32_t M, N, K;
     int32_t tiles_m, tiles_n;
     int32_t y_dtype, bias_dtype, epilogue;
+    int32_t chan_vec;  // N % 4 == 0 and col_scale / bias aligned for one 16-byte (bf16 bias: 8-byte) load per 4 channels
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16(float v) {
@@ -426,10 +427,31 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     const bool full_cols = (n0 + BN <= p.N) && (p.N % 8 == 0);
 
     // channel scale and bias for the lane's channels of tile j, group g (needs n < N: clamped)
-    auto chan = [&](int j, int g, float (&cs)[4], float (&cb)[4], bool need_scale) {
+    auto chan = [&](int j, int g, float (&cs)[4], float (&cb)[4], bool need_scale, int zero) {
+        if (p.chan_vec) {  // uniform: the lane's four channels are adjacent, one load per operand
+            const int nb = min(wn0 + 32 * j + 8 * g + 4 * lh, p.N - 4) + zero;
+            if (need_scale) {
+                const float4 sv = *reinterpret_cast<const float4*>(p.col_scale + nb);
+                cs[0] = sv.x, cs[1] = sv.y, cs[2] = sv.z, cs[3] = sv.w;
+            } else {
+                cs[0] = cs[1] = cs[2] = cs[3] = 1.0f;
+            }
+            cb[0] = cb[1] = cb[2] = cb[3] = 0.0f;
+            if (p.bias) {
+                if (p.bias_dtype == NQ_DT_F32) {
+                    const float4 bv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + nb);
+                    cb[0] = bv.x, cb[1] = bv.y, cb[2] = bv.z, cb[3] = bv.w;
+                } else {
+                    const uint2 bv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.bias) + nb);
+                    cb[0] = __uint_as_float(bv.x << 16), cb[1] = __uint_as_float(bv.x & 0xFFFF0000u);
+                    cb[2] = __uint_as_float(bv.y << 16), cb[3] = __uint_as_float(bv.y & 0xFFFF0000u);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int n = min(wn0 + 32 * j + 8 * g + 4 * lh + r, p.N - 1);
+            const int n = min(wn0 + 32 * j + 8 * g + 4 * lh + r, p.N - 1) + zero;
             cs[r] = need_scale ? p.col_scale[n] : 1.0f;
             cb[r] = 0.0f;
             if (p.bias)
@@ -450,6 +472,11 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             // ---- registers -> LDS (this wavefront's region only).  Channel scales and biases are
             // fetched per channel tile j; the compiler barrier keeps it from hoisting all 16 (j, g)
             // sets above the loop, which would spill.
+            // (a zero the compiler cannot see through, new in every pass: the channel operands do not depend on
+            // the pass, and kept across all four passes of the fp32 epilogue they cost 129 spilled registers and
+            // 60 % of the call's time; they are re-read from L1 per pass instead)
+            int zero = 0;
+            asm volatile("" : "+v"(zero));
             float rscale[IP];
 #pragma unroll
             for (int ii = 0; ii < IP; ii++) {
@@ -461,7 +488,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
                 float cs[4][4], cb[4][4];
                 if constexpr (KIND != 2) {
 #pragma unroll
-                    for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8);
+                    for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8, zero);
                 }
                 if constexpr (KIND == 2) {
 #pragma unroll
@@ -595,6 +622,9 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + 255) / 256;
+    const bool i8 = a.x_dtype == NQ_DT_I8;
+    p.chan_vec = L->out % 4 == 0 && L->out >= 4 && (!i8 || a.y_dtype == NQ_DT_I32 || (uintptr_t)p.col_scale % 16 == 0) &&
+                 (!a.bias || (uintptr_t)a.bias % (a.bias_dtype == NQ_DT_F32 ? 16 : 8) == 0);
     static bool attr_set[5] = {false, false, false, false, false};
     const bool f32 = a.y_dtype == NQ_DT_F32;
     if (a.x_dtype == NQ_DT_FP8_E4M3)
