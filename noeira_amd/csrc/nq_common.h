@@ -119,6 +119,10 @@ int32_t launch_gemv_row4(const ForwardArgs& a);
 bool gemv_row8_applicable(const ForwardArgs& a);
 int32_t launch_gemv_row8(const ForwardArgs& a);
 
+// nq_gemv_split.hip: int8 weights under one bf16 / fp32 row, x split into int8 terms for the int8 matrix cores
+bool gemv_split8_applicable(const ForwardArgs& a);
+int32_t launch_gemv_split8(const ForwardArgs& a);
+
 // nq_gemv_fp8.hip: fp8 x fp8 and int8 x int8 on the matrix cores for one row (fp8) and for as many
 // activation rows as the large-tile GEMM would leave most of the chip idle with
 bool gemv_fp8_applicable(const ForwardArgs& a);

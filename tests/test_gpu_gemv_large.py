@@ -136,6 +136,71 @@ def test_w8_large_single_row(K, N, xdt):
     assert np.abs(yr - want).max() <= 1e-3 * rms + 2.0 ** -8 * np.abs(want).max()
 
 
+# the int8-matrix-core kernel that splits x into three int8 terms: rows of 4096 .. 8192 codes, 24 MB and more
+# (one, two and four rows per wavefront; N off every tile size)
+@pytest.mark.parametrize("K,N", [(4096, 6403), (4096, 8201), (5120, 8197), (8192, 3101), (4112, 8195)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_w8_split_single_row(K, N, xdt):
+    from noeira_amd.qlinear import W8Linear
+    rng = np.random.default_rng(K * 3 + N)
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    w[3, :] = -128
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    lin = W8Linear(K, N)
+    lin.set_weight(w, s)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    x[0, 5] = 300.0  # an outlier sets the scale of the split: the small elements still count
+    x = torch.from_numpy(x).to(xdt).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    wd = torch.from_numpy(w).cuda().double()
+    sd = torch.from_numpy(s).cuda().double()
+    exact = (x.double() @ wd.T) * sd + bias.double()
+    rms = float(exact.pow(2).mean().sqrt())
+    y = lin.forward(x, bias=bias)
+    # the split leaves up to 6e-8 of |x|max per element: under an outlier of 60 sigma that is 1e-5 of the output RMS,
+    # a hundredth of the band of 1e-3
+    assert float((y.double() - exact).abs().max()) < 1e-4 * rms
+    assert torch.equal(lin.forward(x, bias=bias), y)
+    yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16)
+    want = ((x.double() @ wd.T) * sd + bias.to(torch.bfloat16).double()).clamp_min(0)
+    assert float((yr.double() - want).abs().max()) <= 1e-3 * rms + 2.0 ** -8 * float(want.abs().max())
+
+
+def test_w8_split_special_rows():
+    from noeira_amd.qlinear import W8Linear
+    rng = np.random.default_rng(77)
+    K, N = 4096, 6400
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    lin = W8Linear(K, N)
+    lin.set_weight(w, s)
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    zero = torch.zeros((1, K), dtype=torch.float32, device="cuda")
+    assert torch.equal(lin.forward(zero, bias=bias)[0], bias)  # a zero row: the bias, bit for bit
+    tiny = torch.full((1, K), 1e-38, dtype=torch.float32, device="cuda")
+    assert float((lin.forward(tiny, bias=bias)[0] - bias).abs().max()) < 1e-30
+    for bad in (float("nan"), float("inf"), -float("inf")):  # a NaN or an infinity in x: every output is NaN
+        xb = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).cuda()
+        xb[0, 1234] = bad
+        assert bool(torch.isnan(lin.forward(xb, bias=bias)).all())
+
+
+def test_w8_split_fused_rows():
+    from noeira_amd.qlinear import W8Linear
+    rng = np.random.default_rng(22)
+    K = 4096
+    parts = []
+    for n in (6000, 2200, 260):
+        lin = W8Linear(K, n)
+        lin.set_weight(rng.integers(-127, 128, (n, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, n).astype(np.float32))
+        parts.append(lin)
+    fused = FusedRows(parts)
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    for lin, y in zip(parts, fused.forward(x)):
+        want = lin.forward(x)  # (the parts alone take other kernels: same products, another order of sums)
+        assert float((y - want).abs().max()) <= 2e-6 * float(want.abs().max())
+
+
 def test_w8_large_fused_rows_single_row():
     from noeira_amd.qlinear import W8Linear
     rng = np.random.default_rng(21)
