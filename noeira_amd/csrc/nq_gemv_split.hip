@@ -9,8 +9,8 @@
 // (each q the round-to-nearest-even of what the terms before it left over, so |q| <= 127), and the row's
 // dot product is three exact int32 sums combined in fp32.  The error of the split is 6e-8 of the row's
 // absmax per element, the size of an fp32 rounding of the products themselves.
-//   - one wavefront owns one to four adjacent weight rows and reads them as 1 KiB contiguous per load
-//     instruction, all loads requested before x is touched;
+//   - one wavefront owns one weight row and reads it as 1 KiB contiguous per load instruction, all loads
+//     requested before x is touched;
 //   - each thread converts one 16-element chunk of x (absmax: integer max over the bit patterns, so a NaN or
 //     an infinity in x is seen and turns every output into NaN) and leaves three 16-byte operands in LDS;
 //   - the MFMA is used "diagonally" as in the 8-bit x 8-bit row kernel (nq_gemv_fp8.hip): the 16 B columns
@@ -216,16 +216,9 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
 
 template <bool XF32, int CPL>
 int32_t launch_split8(const SplitParams& p, hipStream_t s) {
-    // Rows per wavefront (the split of x is paid once per workgroup): from 8192 rows on, four rows of up to
-    // 4 KiB or two longer ones.  Measured on 4096 -> 28672: 24.5 us with one row, 21.5 with four (68 % of HBM);
-    // 4096 -> 11008 takes 10.7 us either way.
-    const int rpw = p.N < 8192 ? 1 : CPL <= 4 ? 4 : 2;
-    const dim3 grid((unsigned)((p.N + 8 * rpw - 1) / (8 * rpw)));
-    if constexpr (CPL <= 4) {
-        if (rpw == 4) hipLaunchKernelGGL((gemv_split8_kernel<XF32, CPL, 8, 4>), grid, dim3(512), 0, s, p);
-    }
-    if (rpw == 2) hipLaunchKernelGGL((gemv_split8_kernel<XF32, CPL, 8, 2>), grid, dim3(512), 0, s, p);
-    if (rpw == 1) hipLaunchKernelGGL((gemv_split8_kernel<XF32, CPL, 8, 1>), grid, dim3(512), 0, s, p);
+    // one row per wavefront: two and four rows per wavefront (the split of x is then paid once per 16 or 32 rows)
+    // were measured and are slower, 4096 -> 11008 in 10.5 / 11.4 / 14.8 us, 8192 -> 8192 in 14.6 / 16.1 us
+    hipLaunchKernelGGL((gemv_split8_kernel<XF32, CPL, 8, 1>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
@@ -248,7 +241,7 @@ int32_t launch_split8_cpl(const SplitParams& p, hipStream_t s) {
 
 // One bf16 / fp32 row over int8 weights with rows of 4096 .. 8192 codes (a multiple of 16) and 24 MB and more.
 // Measured against the kernels that convert every code on the vector ALU (us, cold): 4096 -> 11008 10.7 / 11.5,
-// 4096 -> 14336 13.0 / 14.5, 4096 -> 28672 21.5 / 27.8, 5120 -> 5120 7.8 / 8.3, 8192 -> 8192 14.1 / 14.7; shorter
+// 4096 -> 14336 13.0 / 14.5, 4096 -> 28672 24.7 / 27.8, 5120 -> 5120 7.8 / 8.3, 8192 -> 8192 14.1 / 14.7; shorter
 // rows and smaller weights are launch- and latency-bound and lose 0.3 .. 1.6 us to the split and its two barriers.
 bool gemv_split8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
