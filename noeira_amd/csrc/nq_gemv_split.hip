@@ -11,8 +11,9 @@
 // absmax per element, the size of an fp32 rounding of the products themselves.
 //   - one wavefront owns one weight row and reads it as 1 KiB contiguous per load instruction, all loads
 //     requested before x is touched;
-//   - each thread converts one 16-element chunk of x (absmax: integer max over the bit patterns, so a NaN or
-//     an infinity in x is seen and turns every output into NaN) and leaves three 16-byte operands in LDS;
+//   - each thread converts 4, 8 or 16 elements of x, so that all 512 take part (absmax: integer max over the
+//     bit patterns, so a NaN or an infinity in x is seen and turns every output into NaN), and leaves one word
+//     per term and four elements in LDS;
 //   - the MFMA is used "diagonally" as in the 8-bit x 8-bit row kernel (nq_gemv_fp8.hip): the 16 B columns
 //     are 16 segments of the row, the 16 A rows the matching segments of the leading term of x, and the dot
 //     product is the trace of the tile: one v_mfma_i32_16x16x64_i8 per KiB of codes; the two small terms go
@@ -70,25 +71,35 @@ __device__ __forceinline__ float butterfly_sum(float v) {
     return v;
 }
 
-template <bool XF32, int CPL, int WAVES, int RPW>
+template <bool XF32, int CPL, int WAVES, int RPW, int EPT>
 __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitParams p) {
     constexpr int NTHR = 64 * WAVES;
-    constexpr int XPT = (CPL * 64 + NTHR - 1) / NTHR;  // 16-element chunks of x per thread
+    constexpr int NUNIT = CPL * 1024 / EPT;  // a thread splits one unit of EPT consecutive elements of x
+    static_assert(NUNIT <= NTHR && (EPT == 4 || EPT == 8 || EPT == 16), "one unit per thread");
+    constexpr int NW = XF32 ? EPT : EPT / 2;  // words of x per unit
     __shared__ u32x4 xs[3][CPL * 64];
     __shared__ uint32_t wmax[WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // a wavefront owns RPW adjacent rows (the split of x is paid once per workgroup: WAVES * RPW rows share it)
     const int64_t row0 = ((int64_t)blockIdx.x * WAVES + wave) * RPW;
     const int nch = p.K >> 4;
+    const int nunit = p.K / EPT;
 
-    // every load is unconditional from a clamped chunk index; a chunk past K meets x = 0
-    u32x4 xg[XPT][XF32 ? 4 : 2];
+    // every load is unconditional from a clamped index; a unit past K counts as x = 0
+    uint32_t xg[NW];
+    {
+        const int u = min(tid, nunit - 1);
+        if constexpr (NW == 2) {
+            const uint2 v = reinterpret_cast<const uint2*>(p.x)[u];
+            xg[0] = v.x, xg[1] = v.y;
+        } else {
+            const u32x4* xr = reinterpret_cast<const u32x4*>(p.x) + (int64_t)u * (NW / 4);
 #pragma unroll
-    for (int i = 0; i < XPT; i++) {
-        const int c = min(tid + i * NTHR, nch - 1);
-        const u32x4* xr = reinterpret_cast<const u32x4*>(p.x) + (int64_t)c * (XF32 ? 4 : 2);
-#pragma unroll
-        for (int q = 0; q < (XF32 ? 4 : 2); q++) xg[i][q] = xr[q];
+            for (int q = 0; q < NW / 4; q++) {
+                const u32x4 v = xr[q];
+                xg[4 * q] = v[0], xg[4 * q + 1] = v[1], xg[4 * q + 2] = v[2], xg[4 * q + 3] = v[3];
+            }
+        }
     }
     u32x4 wv[RPW][CPL];
     float csraw[RPW];
@@ -107,18 +118,17 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
     }
 
     // ---- x as fp32, and the largest magnitude of the row (as a bit pattern: NaN > inf > finite)
-    float xf[XPT][16];
+    float xf[EPT];
     uint32_t mbits = 0;
+    {
+        const bool live = tid < nunit;
 #pragma unroll
-    for (int i = 0; i < XPT; i++) {
-        const bool live = tid + i * NTHR < nch;
-#pragma unroll
-        for (int e = 0; e < 16; e++) {
+        for (int e = 0; e < EPT; e++) {
             uint32_t b;
-            if constexpr (XF32) b = xg[i][e >> 2][e & 3];
-            else b = (e & 1) ? (xg[i][e >> 3][(e >> 1) & 3] & 0xFFFF0000u) : (xg[i][e >> 3][(e >> 1) & 3] << 16);
+            if constexpr (XF32) b = xg[e];
+            else b = (e & 1) ? (xg[e >> 1] & 0xFFFF0000u) : (xg[e >> 1] << 16);
             if (!live) b = 0;
-            xf[i][e] = __uint_as_float(b);
+            xf[e] = __uint_as_float(b);
             mbits = max(mbits, b & 0x7FFFFFFFu);
         }
     }
@@ -134,22 +144,24 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
     const float inv_s = (finite && absmax > 1e-30f) ? 127.0f / absmax : 0.0f;
     const float s_x = inv_s != 0.0f ? absmax * (1.0f / 127.0f) : 0.0f;
 
+    if (tid < NUNIT) {
+        uint32_t* const x0 = reinterpret_cast<uint32_t*>(xs[0]) + tid * (EPT / 4);
+        uint32_t* const x1 = reinterpret_cast<uint32_t*>(xs[1]) + tid * (EPT / 4);
+        uint32_t* const x2 = reinterpret_cast<uint32_t*>(xs[2]) + tid * (EPT / 4);
+        if (tid - lane >= nunit) {  // uniform over the wavefront: nothing of x here, only the padding of the last load
 #pragma unroll
-    for (int i = 0; i < XPT; i++) {
-        const int c = tid + i * NTHR;
-        if (c - lane >= nch) {  // uniform over the wavefront: nothing of x here, only the padding of the last load
-            if (c < CPL * 64) xs[0][c] = xs[1][c] = xs[2][c] = (u32x4){0, 0, 0, 0};
-        } else if (c < CPL * 64) {
-            // four elements at a time, one word per term (few values live beside the rows in flight)
+            for (int q = 0; q < EPT / 4; q++) x0[q] = x1[q] = x2[q] = 0;
+        } else {
+            // four elements at a time, one word per term
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
+            for (int q = 0; q < EPT / 4; q++) {
                 uint32_t a1[4], a2[4], a3[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     // every byte comes from the very integer that is subtracted (a sum contracted into an fma
                     // would round a tie differently from the rounded product, and the next term would leave
                     // the int8 range)
-                    const float t = xf[i][4 * q + e] * inv_s;
+                    const float t = xf[4 * q + e] * inv_s;
                     const float q1 = __builtin_rintf(t);
                     a1[e] = __float_as_uint(q1 + MAGIC);
                     const float t2 = (t - q1) * 254.0f;
@@ -157,9 +169,9 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
                     a2[e] = __float_as_uint(q2 + MAGIC);
                     a3[e] = __float_as_uint(__builtin_rintf((t2 - q2) * 254.0f) + MAGIC);
                 }
-                reinterpret_cast<uint32_t*>(&xs[0][c])[q] = pack_low_bytes(a1[0], a1[1], a1[2], a1[3]);
-                reinterpret_cast<uint32_t*>(&xs[1][c])[q] = pack_low_bytes(a2[0], a2[1], a2[2], a2[3]);
-                reinterpret_cast<uint32_t*>(&xs[2][c])[q] = pack_low_bytes(a3[0], a3[1], a3[2], a3[3]);
+                x0[q] = pack_low_bytes(a1[0], a1[1], a1[2], a1[3]);
+                x1[q] = pack_low_bytes(a2[0], a2[1], a2[2], a2[3]);
+                x2[q] = pack_low_bytes(a3[0], a3[1], a3[2], a3[3]);
             }
         }
     }
@@ -218,7 +230,9 @@ template <bool XF32, int CPL>
 int32_t launch_split8(const SplitParams& p, hipStream_t s) {
     // one row per wavefront: two and four rows per wavefront (the split of x is then paid once per 16 or 32 rows)
     // were measured and are slower, 4096 -> 11008 in 10.5 / 11.4 / 14.8 us, 8192 -> 8192 in 14.6 / 16.1 us
-    hipLaunchKernelGGL((gemv_split8_kernel<XF32, CPL, 8, 1>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
+    // (likewise 16 wavefronts per workgroup: 12.6 / 27.2 us on 4096 -> 11008 / 28672 against 10.6 / 22 .. 24)
+    constexpr int EPT = CPL <= 2 ? 4 : CPL <= 4 ? 8 : 16;  // all 512 threads take part in the split of x
+    hipLaunchKernelGGL((gemv_split8_kernel<XF32, CPL, 8, 1, EPT>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
