@@ -485,6 +485,14 @@ def sweep(skip_large=False):
         run("ref Q4_0 g32 4096->11008 M=1 fp32 (cold)", make_q4_0, "hbm", IN=4096, OUT=11008, M=1, copies=c, calls=c)
         run("W8A16 4096->11008 M=1 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, copies=max(1, c // 2),
             calls=max(1, c // 2))
+        # the same kernels where the stream is long enough for the fixed part of a call (launch, first trip to
+        # memory, the last wavefronts) to vanish: 8192 -> 28672, 235 MB of 8-bit codes / 117 - 132 MB of 4-bit ones
+        KB, NB = 8192, 28672
+        run(f"fp8 x fp8 GEMV {KB}->{NB} M=1 (cold, 235 MB)", make_fp8, "hbm", M=1, N=NB, K=KB, copies=3)
+        run(f"W8A8 int8 GEMV {KB}->{NB} M=1 (cold, 235 MB)", make_w8a8_m1, "hbm", K=KB, N=NB, copies=3)
+        run(f"W8A16 {KB}->{NB} M=1 (cold, 235 MB)", make_w8a16_one, "hbm", K=KB, N=NB, copies=3)
+        run(f"W4A16 g128 {KB}->{NB} M=1 (cold, 122 MB)", make_w4g, "hbm", K=KB, N=NB, M=1, copies=5)
+        run(f"ref Q4_0 g32 {KB}->{NB} M=1 fp32 (cold, 132 MB)", make_q4_0, "hbm", IN=KB, OUT=NB, M=1, copies=4)
         run("W4A16 g128 4096->11008 M=16 (cold)", make_w4g, "hbm", K=4096, N=11008, M=16, copies=c, calls=c)
         run("ref Q4_0 g32 4096->11008 M=16 fp32 (cold)", make_q4_0, "hbm", IN=4096, OUT=11008, M=16, copies=c, calls=c)
         run("W8A16 4096->11008 M=16 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, M=16, copies=max(1, c // 2),
