@@ -177,8 +177,9 @@ def make_w8a16_one(K, N, copies, seed=9, M=1):
                 keep=(layers, x, y))
 
 
-def make_q4_0(IN, OUT, M, copies, seed=3):
-    """The reference's own layer: Q4_0 group 32, fp32 activations, fp32 out."""
+def make_q4_0(IN, OUT, M, copies, seed=3, bf16_x=False):
+    """The reference's own layer: Q4_0 group 32, fp32 activations (bf16 with `bf16_x`: the activations of the
+    reference's int4 tensor-core path, qlinear.mojo:430-463), fp32 out."""
     import numpy as np
     import torch
 
@@ -195,16 +196,18 @@ def make_q4_0(IN, OUT, M, copies, seed=3):
         ql.set_blocks(blocks)
         layers.append(ql)
     x = torch.from_numpy(rng.standard_normal((M, IN)).astype(np.float32)).cuda()
+    if bf16_x:
+        x = x.to(torch.bfloat16)
     y = torch.empty((M, OUT), dtype=torch.float32, device="cuda")
 
     def step(i):
         layers[i % copies].forward(x, out=y)
 
-    return dict(step=step, bytes=nb + 4 * IN * M + 4 * OUT * M, ops=2 * M * IN * OUT, launches=1,
+    return dict(step=step, bytes=nb + (2 if bf16_x else 4) * IN * M + 4 * OUT * M, ops=2 * M * IN * OUT, launches=1,
                 keep=(layers, x, y))
 
 
-def make_q4_0_fused(IN, OUTS, M, copies, seed=7):
+def make_q4_0_fused(IN, OUTS, M, copies, seed=7, bf16_x=False):
     """The reference caller's q|k|v or gate|up projections as one row-fused launch."""
     import numpy as np
     import torch
@@ -225,13 +228,15 @@ def make_q4_0_fused(IN, OUTS, M, copies, seed=7):
             parts.append(ql)
         fused.append(FusedRows(parts))  # the parts are copied; they are freed here
     x = torch.from_numpy(rng.standard_normal((M, IN)).astype(np.float32)).cuda()
+    if bf16_x:
+        x = x.to(torch.bfloat16)
     ys = [torch.empty((M, OUT), dtype=torch.float32, device="cuda") for OUT in OUTS]
     tot = sum(OUTS)
 
     def step(i):
         fused[i % copies].forward(x, outs=ys)
 
-    return dict(step=step, bytes=tot * (IN // 32) * 18 + 4 * IN * M + 4 * tot * M, ops=2 * M * IN * tot, launches=1,
+    return dict(step=step, bytes=tot * (IN // 32) * 18 + (2 if bf16_x else 4) * IN * M + 4 * tot * M, ops=2 * M * IN * tot, launches=1,
                 keep=(fused, x, ys))
 
 
@@ -453,12 +458,16 @@ def sweep(skip_large=False):
         run(f"ref Q4_0 g32 {IN}->{OUT} M=1 fp32 (cold)", make_q4_0, "hbm", IN=IN, OUT=OUT, M=1, copies=c, calls=c)
         run(f"ref Q4_0 g32 {IN}->{OUT} M=135 fp32 (warm)", make_q4_0, "mfma", "bf16", IN=IN, OUT=OUT, M=135,
             copies=1, calls=20)
+        run(f"ref Q4_0 g32 {IN}->{OUT} M=135 bf16 x (warm)", make_q4_0, "mfma", "bf16", IN=IN, OUT=OUT, M=135,
+            copies=1, calls=20, bf16_x=True)
     for (name, OUTS) in [("q|k|v 960->960|320|320", [960, 320, 320]), ("gate|up 960->2560|2560", [2560, 2560])]:
         c = max(1, COLD_BYTES // (sum(OUTS) * 960 * 9 // 16))
         run(f"ref Q4_0 {name} row-fused M=1 fp32 (cold)", make_q4_0_fused, "hbm", IN=960, OUTS=OUTS, M=1, copies=c,
             calls=c)
         run(f"ref Q4_0 {name} row-fused M=135 fp32 (warm)", make_q4_0_fused, "mfma", "bf16", IN=960, OUTS=OUTS,
             M=135, copies=1, calls=20)
+        run(f"ref Q4_0 {name} row-fused M=135 bf16 x (warm)", make_q4_0_fused, "mfma", "bf16", IN=960, OUTS=OUTS,
+            M=135, copies=1, calls=20, bf16_x=True)
     run("cfg3 W8A8 actor 64->256->256->8 M=4096 (fused, 1 launch)", make_actor_fused, "mfma", "int8", calls=20)
     run("cfg3 W8A8 actor 64->256->256->8 M=4096 (unfused, 6 launches)", make_actor_w8a8, "mfma", "int8", calls=20)
     for N in (4096, 11008):
