@@ -168,3 +168,49 @@ def test_lora_forward_add_against_numpy():
     ap = np.concatenate([a, np.zeros((IN, 11), np.float32)], axis=1)
     bp = np.concatenate([b, np.zeros((11, OUT), np.float32)], axis=0)
     assert np.array_equal(O.lora_forward_add(x, ap, bp, 0.4, y0.copy()), y)
+
+
+# ── the three-term int8 split of an activation row (nq_gemv_split.hip), restated in numpy fp32 ──
+def _split3(x, fused):
+    """x fp32 [K] -> (s, q1, q2, q3) with x ~ s (q1 + q2 / 254 + q3 / 254^2).  `fused` forms the second
+    leftover with one rounding (an fma), as a compiler may contract it; the kernel must hold either way."""
+    f32 = np.float32
+    absmax = f32(np.abs(x).max())
+    inv_s = f32(127.0) / absmax if absmax > 1e-30 else f32(0.0)
+    t = (x * inv_s).astype(f32)
+    q1 = np.rint(t).astype(f32)
+    r1 = (t - q1).astype(f32)                      # exact
+    t2 = (r1 * f32(254.0)).astype(f32)
+    q2 = np.rint(t2).astype(f32)
+    if fused:
+        r2 = (r1.astype(np.float64) * 254.0 - q2.astype(np.float64)).astype(f32)
+    else:
+        r2 = (t2 - q2).astype(f32)
+    q3 = np.rint((r2 * f32(254.0)).astype(f32)).astype(f32)
+    s = absmax * f32(1.0 / 127.0) if inv_s != 0 else f32(0.0)
+    return s, q1, q2, q3
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("kind", ["normal", "bf16", "outlier", "ties"])
+def test_three_term_int8_split_bounds(kind, fused):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(1 << 16).astype(np.float32)
+    if kind == "bf16":    # few significand bits: leftovers land on exact halves far more often
+        x = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    if kind == "outlier":
+        x[7] = 300.0
+    if kind == "ties":    # every multiple of 1 / 508 of the scale: all the .5 cases of the second term
+        x = (np.arange(-127 * 508, 127 * 508 + 1, dtype=np.float64) / 508.0).astype(np.float32)
+    s, q1, q2, q3 = _split3(x, fused)
+    for q in (q1, q2, q3):  # every term fits an int8, the range the byte packing keeps
+        assert np.abs(q).max() <= 127
+    rec = s.astype(np.float64) * (q1.astype(np.float64) + q2 / 254.0 + q3 / 254.0 ** 2)
+    bound = np.abs(x).max() / (127.0 * 254.0 ** 2 * 2.0)
+    assert np.abs(rec - x.astype(np.float64)).max() <= bound * 1.05 + np.abs(x).max() * 2.0 ** -23
+
+
+def test_three_term_int8_split_zero_and_tiny():
+    for x in (np.zeros(64, np.float32), np.full(64, 1e-38, np.float32)):
+        s, q1, q2, q3 = _split3(x, False)
+        assert s == 0 and not q1.any() and not q2.any() and not q3.any()
