@@ -158,16 +158,17 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
                 uint32_t a1[4], a2[4], a3[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    // every byte comes from the very integer that is subtracted (a sum contracted into an fma
-                    // would round a tie differently from the rounded product, and the next term would leave
-                    // the int8 range)
+                    // Round by adding 1.5 * 2^23 (the sum's low byte is the int8), and take every leftover against
+                    // the very integer that was packed: the second and third term round the exact product
+                    // (one fma each), so that no leftover exceeds a half and no term leaves the int8 range.
                     const float t = xf[4 * q + e] * inv_s;
-                    const float q1 = __builtin_rintf(t);
-                    a1[e] = __float_as_uint(q1 + MAGIC);
-                    const float t2 = (t - q1) * 254.0f;
-                    const float q2 = __builtin_rintf(t2);
-                    a2[e] = __float_as_uint(q2 + MAGIC);
-                    a3[e] = __float_as_uint(__builtin_rintf((t2 - q2) * 254.0f) + MAGIC);
+                    const float b1 = t + MAGIC;
+                    a1[e] = __float_as_uint(b1);
+                    const float r1 = t - (b1 - MAGIC);
+                    const float b2 = __builtin_fmaf(r1, 254.0f, MAGIC);
+                    a2[e] = __float_as_uint(b2);
+                    const float r2 = __builtin_fmaf(r1, 254.0f, MAGIC - b2);
+                    a3[e] = __float_as_uint(__builtin_fmaf(r2, 254.0f, MAGIC));
                 }
                 x0[q] = pack_low_bytes(a1[0], a1[1], a1[2], a1[3]);
                 x1[q] = pack_low_bytes(a2[0], a2[1], a2[2], a2[3]);

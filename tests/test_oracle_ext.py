@@ -172,21 +172,24 @@ def test_lora_forward_add_against_numpy():
 
 # ── the three-term int8 split of an activation row (nq_gemv_split.hip), restated in numpy fp32 ──
 def _split3(x, fused):
-    """x fp32 [K] -> (s, q1, q2, q3) with x ~ s (q1 + q2 / 254 + q3 / 254^2).  `fused` forms the second
-    leftover with one rounding (an fma), as a compiler may contract it; the kernel must hold either way."""
-    f32 = np.float32
+    """x fp32 [K] -> (s, q1, q2, q3) with x ~ s (q1 + q2 / 254 + q3 / 254^2).  `fused` rounds the exact
+    products r * 254 (one fma each, what the kernel does); without it the products are rounded to fp32 first.
+    The bounds must hold either way."""
+    f32, f64 = np.float32, np.float64
     absmax = f32(np.abs(x).max())
     inv_s = f32(127.0) / absmax if absmax > 1e-30 else f32(0.0)
     t = (x * inv_s).astype(f32)
     q1 = np.rint(t).astype(f32)
     r1 = (t - q1).astype(f32)                      # exact
-    t2 = (r1 * f32(254.0)).astype(f32)
-    q2 = np.rint(t2).astype(f32)
     if fused:
-        r2 = (r1.astype(np.float64) * 254.0 - q2.astype(np.float64)).astype(f32)
+        q2 = np.rint(r1.astype(f64) * 254.0).astype(f32)
+        r2 = (r1.astype(f64) * 254.0 - q2.astype(f64)).astype(f32)
+        q3 = np.rint(r2.astype(f64) * 254.0).astype(f32)
     else:
+        t2 = (r1 * f32(254.0)).astype(f32)
+        q2 = np.rint(t2).astype(f32)
         r2 = (t2 - q2).astype(f32)
-    q3 = np.rint((r2 * f32(254.0)).astype(f32)).astype(f32)
+        q3 = np.rint((r2 * f32(254.0)).astype(f32)).astype(f32)
     s = absmax * f32(1.0 / 127.0) if inv_s != 0 else f32(0.0)
     return s, q1, q2, q3
 
