@@ -54,10 +54,8 @@ struct MlpParams {
 };
 
 __device__ __forceinline__ int q8(float v, float s) {
-    float t = rintf(__fdiv_rn(v, s));
-    t = t > -127.0f ? t : -127.0f;
-    t = t < 127.0f ? t : 127.0f;
-    return (int)t;
+    // (v_med3_f32 clamps in one instruction; a NaN comes out as -127, as from the two compares it replaces)
+    return (int)__builtin_amdgcn_fmed3f(rintf(__fdiv_rn(v, s)), -127.0f, 127.0f);
 }
 
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {

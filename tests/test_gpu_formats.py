@@ -363,6 +363,28 @@ def test_config4_w8a8_actor_fused_single_launch():
         assert rel_rms(got, want) < 1e-5
 
 
+def test_config4_actor_fused_quantizer_on_ties():
+    """The fused kernel's quantizer must give the codes of the true division v / s.  Inputs that sit on and next
+    to the half-way points k + 0.5 of their token's scale: a quotient off by one ulp there flips a code, and a
+    flipped code shows as 1e-3."""
+    from noeira_amd.qlinear import mlp3_w8a8_forward
+    rng = np.random.default_rng(44)
+    layers = actor_layers(rng)
+    M = 512
+    s = rng.uniform(0.5, 2.0, M).astype(np.float32) * np.float32(2.0) ** rng.integers(-20, 20, M).astype(np.float32)
+    k = rng.integers(-127, 127, (M, 64)).astype(np.float32)
+    x = ((k + np.float32(0.5)) * s[:, None]).astype(np.float32)
+    step = rng.integers(-2, 3, (M, 64))
+    for d in (1, 2):  # one and two ulps to either side
+        x = np.where(step == d, np.nextafter(x, np.float32(np.inf)), x)
+        x = np.where(step == -d, np.nextafter(x, np.float32(-np.inf)), x)
+    x[:, 0] = np.float32(127.0) * s  # the token's absmax: its scale is s up to one rounding
+    want, _ = oracle_actor(layers, x)
+    bs = [torch.from_numpy(l[3]).cuda() for l in layers]
+    y = mlp3_w8a8_forward(layers[0][0], layers[1][0], layers[2][0], torch.from_numpy(x).cuda(), bs[0], bs[1], bs[2])
+    assert rel_rms(y.cpu().numpy(), want) < 1e-5
+
+
 def test_mlp3_other_shapes_and_errors():
     from noeira_amd import _lib as L
     from noeira_amd.qlinear import mlp3_w8a8_forward
