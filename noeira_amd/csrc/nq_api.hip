@@ -50,7 +50,8 @@ void free_device(nq_layer* L) {
     if (L->d_codes) (void)hipFree(L->d_codes);
     if (L->d_scales) (void)hipFree(L->d_scales);
     if (L->d_zps) (void)hipFree(L->d_zps);
-    L->d_codes = nullptr, L->d_scales = nullptr, L->d_zps = nullptr;
+    if (L->d_tiled) (void)hipFree(L->d_tiled);
+    L->d_codes = nullptr, L->d_scales = nullptr, L->d_zps = nullptr, L->d_tiled = nullptr;
 }
 
 int32_t check_handle(nq_handle h, const char* what) {
@@ -242,6 +243,22 @@ int32_t nq_set_weight_i8(nq_handle h, const int8_t* w_host, const float* scales_
     h->has_host_blocks = true;
     NQ_HIP(hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s));
     NQ_HIP(hipMemcpyAsync(h->d_scales, scales_host, (size_t)h->out * 4, hipMemcpyHostToDevice, s));
+    std::vector<uint8_t> tiled;
+    if (h->in <= 256 && h->out <= 256) {
+        // the fused MLP's copy: one contiguous KiB per (16-row tile, 64-k step), in the int8 MFMA's operand order
+        const int tiles = (h->out + 15) / 16, steps = (h->in + 63) / 64;
+        tiled.assign((size_t)tiles * steps * 1024, 0);
+        for (int j = 0; j < tiles; j++)
+            for (int st = 0; st < steps; st++)
+                for (int l = 0; l < 64; l++) {
+                    const int row = 16 * j + (l & 15), k0 = 64 * st + 16 * (l >> 4);
+                    if (row >= h->out) continue;
+                    for (int b = 0; b < 16 && k0 + b < h->in; b++)
+                        tiled[((size_t)j * steps + st) * 1024 + 16 * l + b] = (uint8_t)w_host[(size_t)row * h->in + k0 + b];
+                }
+        NQ_HIP(hipMalloc((void**)&h->d_tiled, tiled.size()));
+        NQ_HIP(hipMemcpyAsync(h->d_tiled, tiled.data(), tiled.size(), hipMemcpyHostToDevice, s));
+    }
     NQ_HIP(hipStreamSynchronize(s));
     h->row_bytes = h->in;
     h->loaded = true;
@@ -796,6 +813,9 @@ int32_t nq_mlp3_w8a8_forward(nq_handle l1, nq_handle l2, nq_handle l3, const flo
         if ((rc = need_loaded(ls[i], "forward"))) return rc;
         if (ls[i]->format != NQ_FMT_W8_CHANNEL)
             return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: every layer must be W8_CHANNEL");
+        if (ls[i]->in <= 256 && ls[i]->out <= 256 && !ls[i]->d_tiled)
+            return fail(NQ_ERR_INVALID, "nq_mlp3_w8a8_forward: layer " + std::to_string(i + 1) +
+                                            " was not loaded with nq_set_weight_i8 (a row-fused layer cannot be used here)");
         if (ls[i]->in > 256 || ls[i]->out > 256)
             return fail(NQ_ERR_UNSUPPORTED, "nq_mlp3_w8a8_forward: layer " + std::to_string(i + 1) + " is [" +
                                                 std::to_string(ls[i]->in) + " -> " + std::to_string(ls[i]->out) +

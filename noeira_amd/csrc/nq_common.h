@@ -49,6 +49,9 @@ struct nq_layer {
     uint8_t* d_codes = nullptr;
     void* d_scales = nullptr;
     uint8_t* d_zps = nullptr;
+    // W8_CHANNEL layers of at most 256 x 256: a second copy of the codes as MFMA operand tiles for the fused MLP
+    // (tile (j, s) = rows 16 j .., k = 64 s .. is 1 KiB, lane l's 16 bytes at 16 l; zeros beyond OUT and IN)
+    uint8_t* d_tiled = nullptr;
     float scale = 1.0f;
     int64_t row_bytes = 0;     // bytes of one row of d_codes
     std::vector<int32_t> seg_end;  // a row-fused layer: the end row of each fused part (else empty)

@@ -385,6 +385,27 @@ def test_config4_actor_fused_quantizer_on_ties():
     assert rel_rms(y.cpu().numpy(), want) < 1e-5
 
 
+@pytest.mark.parametrize("dims", [[(48, 112), (112, 80), (80, 7)], [(256, 256), (256, 240), (240, 255)]])
+def test_mlp3_widths_off_every_multiple(dims):
+    """A last layer whose width is no multiple of 4 (channel scales and biases fetched one by one) or of 16 (a last
+    tile cut short), inner widths that are no multiple of 64 (a last k-step cut short), against the layer-by-layer
+    oracle."""
+    from noeira_amd.qlinear import mlp3_w8a8_forward
+    rng = np.random.default_rng(43)
+    layers = []
+    for K, N in dims:
+        lin, w, s = w8_layer(rng, K, N)
+        layers.append((lin, w, s, (rng.standard_normal(N) * 0.02).astype(np.float32)))
+    x = rng.standard_normal((77, dims[0][0])).astype(np.float32)
+    h = x
+    for i, (_, w, s, b) in enumerate(layers):
+        hq, sx = O.quantize_rows_i8(h)
+        h = O.w8a8_epilogue(O.w8a8_acc_i32(hq, w), sx, s, b, relu=(i < 2))
+    bs = [torch.from_numpy(l[3]).cuda() for l in layers]
+    y = mlp3_w8a8_forward(layers[0][0], layers[1][0], layers[2][0], torch.from_numpy(x).cuda(), bs[0], bs[1], bs[2])
+    assert rel_rms(y.cpu().numpy(), h) < TOL_RMS
+
+
 def test_mlp3_other_shapes_and_errors():
     from noeira_amd import _lib as L
     from noeira_amd.qlinear import mlp3_w8a8_forward
