@@ -172,16 +172,39 @@ __global__ __launch_bounds__(64 * WAVES) void mlp3_w8a8_kernel(const MlpParams p
     constexpr int TPW = MAXT / WAVES;  // 16-channel tiles per wavefront and layer
     __shared__ __attribute__((aligned(16))) uint8_t hq[2][16 * HROW];
     __shared__ float amax_part[2][16 * WAVES];
+    __shared__ __attribute__((aligned(16))) float xsh[16][256 + 4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kb = lane >> 4;
     const int m = blockIdx.x * 16 + ln;          // this lane's token
-    const int mc = min(m, p.M - 1);
     LayerRegs<TPW> R0, R1, R2;
 
-    // ---- layer 1 input: fp32 x, 16 consecutive k per lane per k-step, quantised in registers
-    // (every wavefront does this for the same 16 tokens: cheaper than a hand-over)
+    // ---- layer 1 input: the workgroup's 16 tokens of fp32 x are one contiguous piece of memory; it is fetched
+    // once, a KiB per load instruction, into LDS (rows padded by 16 bytes against bank conflicts).  Each lane then
+    // takes its token's 16 consecutive k per k-step from there and quantises them in registers (every wavefront
+    // for the same 16 tokens: cheaper than a hand-over of the codes).  Read straight from memory in that shape,
+    // a load instruction touched 64 separate 16-byte pieces, in each of the eight wavefronts.
     const int K0 = p.l[0].K;
     const int steps0 = (K0 + 63) >> 6;
+    constexpr int XU = (4 * 256 + 64 * WAVES - 1) / (64 * WAVES);  // float4 units of the 16 x K0 tile per thread
+    const int units = 4 * K0;                                      // (K0 is a multiple of 16)
+    float4 xr[XU];
+#pragma unroll
+    for (int n = 0; n < XU; n++) {
+        const int i = min((int)threadIdx.x + n * 64 * WAVES, units - 1);
+        const int row = (4 * i) / K0, col = (4 * i) % K0;
+        const int64_t mrow = min((int64_t)blockIdx.x * 16 + row, (int64_t)p.M - 1);
+        xr[n] = *reinterpret_cast<const float4*>(p.x + mrow * K0 + col);
+    }
+    // (x is requested first and the weights right behind it: the store to LDS below waits for x alone)
+    layer_load<TPW>(p.l[0], wave, ln, kb, R0);
+    layer_load<TPW>(p.l[1], wave, ln, kb, R1);
+    layer_load<TPW>(p.l[2], wave, ln, kb, R2);
+#pragma unroll
+    for (int n = 0; n < XU; n++) {
+        const int i = (int)threadIdx.x + n * 64 * WAVES;
+        if (i < units) *reinterpret_cast<float4*>(&xsh[(4 * i) / K0][(4 * i) % K0]) = xr[n];
+    }
+    __syncthreads();
     float xv[MAXS][16];
     float amax = 0.0f;
 #pragma unroll
@@ -191,14 +214,11 @@ __global__ __launch_bounds__(64 * WAVES) void mlp3_w8a8_kernel(const MlpParams p
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (k0 + 4 * q < K0) v = *reinterpret_cast<const float4*>(p.x + (int64_t)mc * K0 + k0 + 4 * q);
+            if (k0 + 4 * q < K0) v = *reinterpret_cast<const float4*>(&xsh[ln][k0 + 4 * q]);
             xv[s][4 * q] = v.x, xv[s][4 * q + 1] = v.y, xv[s][4 * q + 2] = v.z, xv[s][4 * q + 3] = v.w;
             amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         }
     }
-    layer_load<TPW>(p.l[0], wave, ln, kb, R0);
-    layer_load<TPW>(p.l[1], wave, ln, kb, R1);
-    layer_load<TPW>(p.l[2], wave, ln, kb, R2);
     amax = fmaxf(amax, __shfl_xor(amax, 16));
     amax = fmaxf(amax, __shfl_xor(amax, 32));
     float sx = amax / 127.0f;
@@ -214,9 +234,8 @@ __global__ __launch_bounds__(64 * WAVES) void mlp3_w8a8_kernel(const MlpParams p
                                    q8(xv[s][4 * q + 3], sx));
     }
 
-    // zero the hand-over rows once: channels a layer does not produce must read as 0
-    for (int i = threadIdx.x; i < 2 * 16 * HROW / 4; i += 64 * WAVES) reinterpret_cast<uint32_t*>(&hq[0][0])[i] = 0u;
-    __syncthreads();
+    // (the hand-over rows need no clearing: every requantisation writes all 256 bytes of a token's row, zeros for the
+    // channels its layer does not produce, because z is 0 there)
 
     float z[TPW][4];
     layer_forward<TPW>(p.l[0], R0, bop, sx, true, wave, ln, kb, z);
