@@ -726,9 +726,11 @@ def main():
                                      "unit": "TFLOP/s", "frac": round(best["TOPS"] / MFMA_PEAK_TOPS["fp8"], 5),
                                      "traffic": FP8_GEMM_TRAFFIC, "kernel": "nq::gemm8_kernel<fp8>",
                                      "workload": best["workload"]}
-        gv = [r for r in line["results"] if "fp8 GEMV" in r["workload"]]
+        gv = [r for r in line["results"] if "cfg4 fp8 GEMV" in r["workload"]]
         if gv:
-            best = max(gv, key=lambda r: r["GBps"])
+            # config 5's own GEMV (N = 11008: the shape the traffic figure was counted on); the 235 MB rows of
+            # `results` show the same kernel where a call's fixed part no longer counts
+            best = next((r for r in gv if "N=11008" in r["workload"]), gv[0])
             line["roofline_gemv"] = {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                                      "frac": round(best["GBps"] / HBM_PEAK_GBPS, 5), "traffic": FP8_GEMV_TRAFFIC,
                                      "kernel": "nq::gemv8_row_kernel<fp8>", "workload": best["workload"]}
