@@ -138,7 +138,12 @@ int32_t nq_keep_only_repacked(nq_handle h);
  * (x_scale = fp32 [1]).  x_scale is NULL otherwise.
  * y_dtype: F32 or BF16; I32 with x_dtype I8 returns the raw accumulators
  * (no scale, bias or epilogue).  bias may be NULL; bias_dtype F32 or BF16.
- * The dequantised weight is never materialised. */
+ * The dequantised weight is never materialised.
+ * Non-finite activations: products and sums follow IEEE, with one exception.
+ * A single F32 / BF16 row (M = 1) over W8_CHANNEL weights of 24 MB and more
+ * (IN 4096..8192) is split into int8 terms under the row's largest magnitude
+ * (error <= 6e-8 of that magnitude per element); if the row holds a NaN or
+ * an infinity, every output of the call is NaN. */
 int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
                    int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype,
                    int32_t epilogue, void* stream);
