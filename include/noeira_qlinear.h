@@ -140,7 +140,7 @@ int32_t nq_keep_only_repacked(nq_handle h);
  * (no scale, bias or epilogue).  bias may be NULL; bias_dtype F32 or BF16.
  * The dequantised weight is never materialised.
  * Non-finite activations: products and sums follow IEEE, with one exception.
- * A single F32 / BF16 row (M = 1) over W8_CHANNEL weights of 24 MB and more
+ * A single F32 / BF16 row (M = 1) over W8_CHANNEL weights of 16 MB and more
  * (IN 4096..8192) is split into int8 terms under the row's largest magnitude
  * (error <= 6e-8 of that magnitude per element); if the row holds a NaN or
  * an infinity, every output of the call is NaN. */

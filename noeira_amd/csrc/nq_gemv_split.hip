@@ -254,17 +254,18 @@ int32_t launch_split8_cpl(const SplitParams& p, hipStream_t s) {
 
 }  // namespace
 
-// One bf16 / fp32 row over int8 weights with rows of 4096 .. 8192 codes (a multiple of 16) and 24 MB and more.
-// Measured against the kernels that convert every code on the vector ALU (us, cold): 4096 -> 11008 10.7 / 11.5,
-// 4096 -> 14336 13.0 / 14.5, 4096 -> 28672 24.7 / 27.8, 5120 -> 5120 7.8 / 8.3, 8192 -> 8192 14.1 / 14.7; shorter
-// rows and smaller weights are launch- and latency-bound and lose 0.3 .. 1.6 us to the split and its two barriers.
+// One bf16 / fp32 row over int8 weights with rows of 4096 .. 8192 codes (a multiple of 16) and 16 MB and more.
+// Measured against the kernels that convert every code on the vector ALU (us, cold): 4096 -> 4096 5.3 / 5.4,
+// 4096 -> 6144 6.6 / 7.7, 4096 -> 11008 10.3 / 11.5, 4096 -> 28672 21 .. 23 / 27.8, 5120 -> 5120 7.2 / 8.3,
+// 8192 -> 8192 14.1 / 14.7.  Shorter rows lose (3072 -> 9216 8.2 / 7.8, 2048 -> 16384 9.7 / 8.4, 1024 -> 16384
+// 7.5 / 6.5): the split and its two barriers are paid per 8 rows whatever their length.
 bool gemv_split8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (a.M != 1 || L->format != NQ_FMT_W8_CHANNEL || ((uintptr_t)a.x & 15)) return false;
     if (a.x_dtype != NQ_DT_BF16 && a.x_dtype != NQ_DT_F32) return false;
     if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
     if (L->in % 16 != 0 || L->in < 4096 || L->in > 8192) return false;
-    return (int64_t)L->in * L->out >= ((int64_t)24 << 20);
+    return (int64_t)L->in * L->out >= ((int64_t)16 << 20);
 }
 
 int32_t launch_gemv_split8(const ForwardArgs& a) {

@@ -136,7 +136,7 @@ def test_w8_large_single_row(K, N, xdt):
     assert np.abs(yr - want).max() <= 1e-3 * rms + 2.0 ** -8 * np.abs(want).max()
 
 
-# the int8-matrix-core kernel that splits x into three int8 terms: rows of 4096 .. 8192 codes, 24 MB and more
+# the int8-matrix-core kernel that splits x into three int8 terms: rows of 4096 .. 8192 codes, 16 MB and more
 # (one, two and four rows per wavefront; N off every tile size)
 @pytest.mark.parametrize("K,N", [(4096, 6403), (4096, 8201), (5120, 8197), (8192, 3101), (4112, 8195)])
 @pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
