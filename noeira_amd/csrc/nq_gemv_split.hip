@@ -240,10 +240,8 @@ int32_t launch_split8(const SplitParams& p, hipStream_t s) {
 
 template <bool XF32>
 int32_t launch_split8_cpl(const SplitParams& p, hipStream_t s) {
+    // (rows of 4096 codes and more: four to eight loads per lane)
     switch ((p.K / 16 + 63) / 64) {
-        case 1: return launch_split8<XF32, 1>(p, s);
-        case 2: return launch_split8<XF32, 2>(p, s);
-        case 3: return launch_split8<XF32, 3>(p, s);
         case 4: return launch_split8<XF32, 4>(p, s);
         case 5: return launch_split8<XF32, 5>(p, s);
         case 6: return launch_split8<XF32, 6>(p, s);
