@@ -695,11 +695,12 @@ def main():
         "metric": "qlinear GB/s at M=1 and TOPS at M=4096, as % of MI355X roofline",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 weights x bf16 activations, fp32 accumulate", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic",
         "config": {"workload": "BASELINE configs[1], ACT-style policy MLP W8A16 at M=1: linears 512->3200 and "
                                "3200->512, int8 weights + per-channel fp32 scales, bf16 x, bf16 bias, fp32 y; "
                                f"cold: rotating over {copies} distinct weight copies ({copies * per_pair >> 20} MiB); "
                                f"launched as HIP-graph replays of {g_steps} steps",
+                   "arithmetic": "int8 codes and bf16 activations widened to fp32, fp32 products and sums",
                    "algorithmic_bytes_per_step": wl["bytes"], "launches_per_step": wl["launches"]},
         "pct_of_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 3),
         "eager": {"GBps": round(wl["bytes"] * a.steps / eager_sec / 1e9, 2),
