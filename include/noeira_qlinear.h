@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define NQ_ABI_VERSION 3
+#define NQ_ABI_VERSION 4
 
 /* status codes */
 #define NQ_OK 0
@@ -65,6 +65,13 @@ extern "C" {
 #define NQ_DT_FP8_E4M3 3  /* x only: e4m3fn codes with one fp32 scale */
 #define NQ_DT_I32 4       /* y only: raw int32 accumulators (W8 x I8) */
 
+/* nq_create flags */
+#define NQ_FLAG_NO_TILE_COPY 1 /* a layer of 4 M weights and more (Q4_0, W4_GROUP with groups of 128,
+                                  W8_CHANNEL) normally keeps a second copy of its codes on the device, ordered
+                                  for the matrix cores 16 rows at a time, which its single-row calls with
+                                  bf16 / fp32 activations stream 1.2 .. 1.5 times faster than the row-ordered
+                                  codes; this flag saves that memory (0.5 or 1 byte per weight) */
+
 /* epilogues (LinearAct's, noeira/nn/primitives/linear_act.mojo:81-115) */
 #define NQ_EPI_NONE 0
 #define NQ_EPI_RELU 1     /* z > 0 ? z : 0  (ops/relu_op.mojo:29-31) */
@@ -86,7 +93,7 @@ int64_t nq_last_error(char* buf, int64_t n);
 
 /* `QLinear[IN, OUT].make` (qlinear.mojo:253-260): an empty layer.  `group` is
  * 32 for NQ_FMT_Q4_0 (IN % 32 == 0 is required, qlinear.mojo:243-245), the
- * group width for NQ_FMT_W4_GROUP, ignored otherwise.  flags = 0. */
+ * group width for NQ_FMT_W4_GROUP, ignored otherwise.  flags: 0 or NQ_FLAG_NO_TILE_COPY. */
 int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t out_features,
                   int32_t group, int32_t flags);
 
@@ -140,10 +147,12 @@ int32_t nq_keep_only_repacked(nq_handle h);
  * (no scale, bias or epilogue).  bias may be NULL; bias_dtype F32 or BF16.
  * The dequantised weight is never materialised.
  * Non-finite activations: products and sums follow IEEE, with one exception.
- * A single F32 / BF16 row (M = 1) over W8_CHANNEL weights of 16 MB and more
- * (IN 4096..8192) is split into int8 terms under the row's largest magnitude
- * (error <= 6e-8 of that magnitude per element); if the row holds a NaN or
- * an infinity, every output of the call is NaN. */
+ * A single F32 / BF16 row (M = 1) over W8_CHANNEL weights of 4 M codes and
+ * more is split into int8 terms under the largest magnitude of the row (or of
+ * a slice of it; error <= 6e-8 of that magnitude per element); if the row
+ * holds a NaN or an infinity, every output of the call is NaN before the
+ * epilogue.  The epilogue NQ_EPI_RELU is z > 0 ? z : 0 in every kernel: a NaN
+ * pre-activation becomes 0 and -0.0 becomes +0.0 (ops/relu_op.mojo:29-31). */
 int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
                    int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype,
                    int32_t epilogue, void* stream);

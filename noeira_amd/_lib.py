@@ -18,7 +18,8 @@ NQ_OK, NQ_ERR_INVALID, NQ_ERR_NOT_LOADED, NQ_ERR_NO_BLOCKS, NQ_ERR_SIZE, NQ_ERR_
 FMT_Q4_0, FMT_W8_CHANNEL, FMT_W4_GROUP, FMT_FP8_E4M3 = range(4)
 DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
 EPI_NONE, EPI_RELU = 0, 1
-ABI_VERSION = 3
+ABI_VERSION = 4
+FLAG_NO_TILE_COPY = 1
 
 EXPORTS = [
     "nq_abi_version", "nq_last_error", "nq_create", "nq_destroy", "nq_set_blocks", "nq_set_weight_f32",

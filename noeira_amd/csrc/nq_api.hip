@@ -51,7 +51,10 @@ void free_device(nq_layer* L) {
     if (L->d_scales) (void)hipFree(L->d_scales);
     if (L->d_zps) (void)hipFree(L->d_zps);
     if (L->d_tiled) (void)hipFree(L->d_tiled);
+    if (L->d_tile16) (void)hipFree(L->d_tile16);
+    if (L->d_tile16_scales) (void)hipFree(L->d_tile16_scales);
     L->d_codes = nullptr, L->d_scales = nullptr, L->d_zps = nullptr, L->d_tiled = nullptr;
+    L->d_tile16 = nullptr, L->d_tile16_scales = nullptr, L->tile_nj = 0;
 }
 
 int32_t check_handle(nq_handle h, const char* what) {
@@ -95,7 +98,7 @@ int32_t adopt_q4_0_blocks(nq_layer* L, const uint8_t* raw_dev, hipStream_t s) {
     int32_t rc = launch_q4_0_repack(raw_dev, L->d_codes, reinterpret_cast<uint16_t*>(L->d_scales), nblocks, s);
     if (rc) return rc;
     L->row_bytes = (int64_t)(L->in / Q4_GROUP) * 16;
-    return NQ_OK;
+    return build_tile_copy(L, s);
 }
 
 }  // namespace
@@ -125,7 +128,7 @@ int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t o
         return fail(NQ_ERR_INVALID, "nq_create: unknown format " + std::to_string(format));
     if (in_features <= 0 || out_features <= 0)
         return fail(NQ_ERR_INVALID, "nq_create: IN and OUT must be positive");
-    if (flags != 0) return fail(NQ_ERR_INVALID, "nq_create: flags must be 0");
+    if (flags & ~NQ_FLAG_NO_TILE_COPY) return fail(NQ_ERR_INVALID, "nq_create: unknown flags");
     if (format == NQ_FMT_Q4_0) {
         // qlinear.mojo:243-245
         if (in_features % Q4_GROUP != 0)
@@ -148,6 +151,7 @@ int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t o
     if (!L) return fail(NQ_ERR_INVALID, "nq_create: out of host memory");
     L->format = format, L->in = in_features, L->out = out_features, L->group = group;
     L->groups = group ? (in_features + group - 1) / group : 0;
+    L->no_tile_copy = (flags & NQ_FLAG_NO_TILE_COPY) != 0;
     *out = L;
     return NQ_OK;
 }
@@ -237,12 +241,6 @@ int32_t nq_set_weight_i8(nq_handle h, const int8_t* w_host, const float* scales_
     if ((rc = bind_device(h))) return rc;
     free_device(h);
     const size_t n = (size_t)h->in * h->out;
-    NQ_HIP(hipMalloc((void**)&h->d_codes, n + 16));
-    NQ_HIP(hipMalloc(&h->d_scales, (size_t)h->out * 4 + 16));
-    h->host_blocks.assign(reinterpret_cast<const uint8_t*>(w_host), reinterpret_cast<const uint8_t*>(w_host) + n);
-    h->has_host_blocks = true;
-    NQ_HIP(hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s));
-    NQ_HIP(hipMemcpyAsync(h->d_scales, scales_host, (size_t)h->out * 4, hipMemcpyHostToDevice, s));
     std::vector<uint8_t> tiled;
     if (h->in <= 256 && h->out <= 256) {
         // the fused MLP's copy: one contiguous KiB per (16-row tile, 64-k step), in the int8 MFMA's operand order
@@ -256,11 +254,23 @@ int32_t nq_set_weight_i8(nq_handle h, const int8_t* w_host, const float* scales_
                     for (int b = 0; b < 16 && k0 + b < h->in; b++)
                         tiled[((size_t)j * steps + st) * 1024 + 16 * l + b] = (uint8_t)w_host[(size_t)row * h->in + k0 + b];
                 }
-        NQ_HIP(hipMalloc((void**)&h->d_tiled, tiled.size()));
-        NQ_HIP(hipMemcpyAsync(h->d_tiled, tiled.data(), tiled.size(), hipMemcpyHostToDevice, s));
     }
-    NQ_HIP(hipStreamSynchronize(s));
+    h->host_blocks.assign(reinterpret_cast<const uint8_t*>(w_host), reinterpret_cast<const uint8_t*>(w_host) + n);
+    h->has_host_blocks = true;
     h->row_bytes = h->in;
+    hipError_t e = hipMalloc((void**)&h->d_codes, n + 16);
+    if (e == hipSuccess) e = hipMalloc(&h->d_scales, (size_t)h->out * 4 + 16);
+    if (e == hipSuccess && !tiled.empty()) e = hipMalloc((void**)&h->d_tiled, tiled.size());
+    if (e == hipSuccess) e = hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipMemcpyAsync(h->d_scales, scales_host, (size_t)h->out * 4, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess && !tiled.empty())
+        e = hipMemcpyAsync(h->d_tiled, tiled.data(), tiled.size(), hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) rc = build_tile_copy(h, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);  // (tiled is read by the copy until here)
+    if (e != hipSuccess || rc) {
+        free_device(h);
+        return e != hipSuccess ? fail_hip(e, "nq_set_weight_i8 upload") : rc;
+    }
     h->loaded = true;
     return NQ_OK;
 }
@@ -281,22 +291,25 @@ int32_t nq_set_weight_w4g(nq_handle h, const uint8_t* codes_host, const uint16_t
     const size_t ng = (size_t)h->out * h->groups;
     const size_t nz = (size_t)h->out * ((h->groups + 1) / 2);
     uint8_t* zp_packed = nullptr;
-    NQ_HIP(hipMalloc((void**)&h->d_codes, n + 16));
-    NQ_HIP(hipMalloc(&h->d_scales, ng * 2 + 16));
-    NQ_HIP(hipMalloc((void**)&h->d_zps, ng + 16));
-    NQ_HIP(hipMalloc((void**)&zp_packed, nz + 16));
     h->host_blocks.assign(codes_host, codes_host + n);
     h->has_host_blocks = true;
-    hipError_t e = hipMemcpyAsync(h->d_codes, codes_host, n, hipMemcpyHostToDevice, s);
+    h->row_bytes = h->in / 2;
+    hipError_t e = hipMalloc((void**)&h->d_codes, n + 16);
+    if (e == hipSuccess) e = hipMalloc(&h->d_scales, ng * 2 + 16);
+    if (e == hipSuccess) e = hipMalloc((void**)&h->d_zps, ng + 16);
+    if (e == hipSuccess) e = hipMalloc((void**)&zp_packed, nz + 16);
+    if (e == hipSuccess) e = hipMemcpyAsync(h->d_codes, codes_host, n, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = hipMemcpyAsync(h->d_scales, scales_f16_host, ng * 2, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = hipMemcpyAsync(zp_packed, zps_host, nz, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) rc = launch_w4g_unpack_zps(zp_packed, h->d_zps, h->out, h->groups, s);
     if (e == hipSuccess && rc == NQ_OK) rc = launch_w4g_repack(h->d_codes, (int64_t)h->out * (h->in / 32), s);
+    if (e == hipSuccess && rc == NQ_OK) rc = build_tile_copy(h, s);
     if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
     (void)hipFree(zp_packed);
-    if (e != hipSuccess) return fail_hip(e, "nq_set_weight_w4g upload");
-    if (rc) return rc;
-    h->row_bytes = h->in / 2;
+    if (e != hipSuccess || rc) {
+        free_device(h);
+        return e != hipSuccess ? fail_hip(e, "nq_set_weight_w4g upload") : rc;
+    }
     h->loaded = true;
     return NQ_OK;
 }
@@ -312,11 +325,15 @@ int32_t nq_set_weight_fp8(nq_handle h, const uint8_t* w_host, float scale, void*
     if ((rc = bind_device(h))) return rc;
     free_device(h);
     const size_t n = (size_t)h->in * h->out;
-    NQ_HIP(hipMalloc((void**)&h->d_codes, n + 16));
     h->host_blocks.assign(w_host, w_host + n);
     h->has_host_blocks = true;
-    NQ_HIP(hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s));
-    NQ_HIP(hipStreamSynchronize(s));
+    hipError_t e = hipMalloc((void**)&h->d_codes, n + 16);
+    if (e == hipSuccess) e = hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) {
+        free_device(h);
+        return fail_hip(e, "nq_set_weight_fp8 upload");
+    }
     h->scale = scale;
     h->row_bytes = h->in;
     h->loaded = true;
@@ -377,6 +394,7 @@ int32_t dispatch(const ForwardArgs& a) {
     if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
+    if (gemv_tile_applicable(a)) return launch_gemv_tile(a);
     if (gemv_split8_applicable(a)) return launch_gemv_split8(a);
     if (gemv_row4_applicable(a)) return launch_gemv_row4(a);
     if (gemv_row8_applicable(a)) return launch_gemv_row8(a);
@@ -388,7 +406,7 @@ int32_t dispatch(const ForwardArgs& a) {
 bool places_parts(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_I8) return false;
     if (gemv_fp8_applicable(a) || gemm8_applicable(a)) return false;
-    return gemm_a16_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
+    return gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
 }
 
 // argument checks shared by nq_forward and nq_forward_fused, then the launch(es)
@@ -483,6 +501,7 @@ int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* s
     if (!F) return fail(NQ_ERR_INVALID, "nq_fuse_rows: out of host memory");
     F->format = a->format, F->in = a->in, F->out = (int32_t)rows, F->group = a->group, F->groups = a->groups;
     F->scale = a->scale, F->row_bytes = a->row_bytes, F->device = a->device;
+    F->no_tile_copy = a->no_tile_copy;
     int32_t rc = bind_device(F);
     if (rc) {
         delete F;
@@ -515,11 +534,12 @@ int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* s
         F->seg_end.push_back((int32_t)r0);
         all_blocks = all_blocks && b->has_host_blocks;
     }
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
-    if (e != hipSuccess) {
+    if (e == hipSuccess) rc = build_tile_copy(F, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
+    if (e != hipSuccess || rc) {
         free_device(F);
         delete F;
-        return fail_hip(e, "nq_fuse_rows");
+        return e != hipSuccess ? fail_hip(e, "nq_fuse_rows") : rc;
     }
     // the logical bytes are row-major over OUT in every format, so the fused layer's are the
     // concatenation (W4_GROUP's logical form is three arrays: not kept)

@@ -52,6 +52,12 @@ struct nq_layer {
     // W8_CHANNEL layers of at most 256 x 256: a second copy of the codes as MFMA operand tiles for the fused MLP
     // (tile (j, s) = rows 16 j .., k = 64 s .. is 1 KiB, lane l's 16 bytes at 16 l; zeros beyond OUT and IN)
     uint8_t* d_tiled = nullptr;
+    // large layers (nq_gemv_tile.hip): a second copy of the codes in the matrix core's operand order for 16 rows
+    // at a time, and (4-bit) of the group records in the same order; tile_nj = steps of K per row tile
+    uint8_t* d_tile16 = nullptr;
+    void* d_tile16_scales = nullptr;
+    int32_t tile_nj = 0;
+    bool no_tile_copy = false;  // NQ_FLAG_NO_TILE_COPY
     float scale = 1.0f;
     int64_t row_bytes = 0;     // bytes of one row of d_codes
     std::vector<int32_t> seg_end;  // a row-fused layer: the end row of each fused part (else empty)
@@ -125,6 +131,12 @@ int32_t launch_gemv_row8(const ForwardArgs& a);
 // nq_gemv_split.hip: int8 weights under one bf16 / fp32 row, x split into int8 terms for the int8 matrix cores
 bool gemv_split8_applicable(const ForwardArgs& a);
 int32_t launch_gemv_split8(const ForwardArgs& a);
+
+// nq_gemv_tile.hip: one bf16 / fp32 row over a large 4-bit or int8 weight, from the tile-ordered copy of the codes
+bool tile_copy_wanted(const nq_layer* L);
+int32_t build_tile_copy(nq_layer* L, hipStream_t s);
+bool gemv_tile_applicable(const ForwardArgs& a);
+int32_t launch_gemv_tile(const ForwardArgs& a);
 
 // nq_gemv_fp8.hip: fp8 x fp8 and int8 x int8 on the matrix cores for one row (fp8) and for as many
 // activation rows as the large-tile GEMM would leave most of the chip idle with

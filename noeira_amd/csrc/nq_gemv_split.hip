@@ -215,7 +215,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
             const float bias = p.bias_dtype == NQ_DT_F32 ? __uint_as_float(braw[rr]) : __uint_as_float(braw[rr] << 16);
             float z = v * (s_x * csraw[rr]) + bias;
             if (!finite) z = __uint_as_float(0x7FC00000u);
-            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : (finite ? 0.0f : z);
+            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
             void* y;
             int width, col;
             seg_lookup(p.seg, (int)row, y, width, col);

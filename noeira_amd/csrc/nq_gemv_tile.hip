@@ -1,0 +1,519 @@
+// Dequant-GEMV for ONE activation row (M = 1) over a LARGE weight, from a second, tile-ordered copy of the codes:
+//     y[N] = epi( deq(W)[N, K] x + bias ),   x bf16 or fp32,
+//     W: Q4_0 (group 32), W4_GROUP with groups of 128 k, or W8_CHANNEL (int8 + per-channel scale).
+//
+// What holds a streaming kernel for 4-bit codes below the weight stream is instruction issue, and most of
+// what the row-ordered kernels issue is not arithmetic: with one weight row per wavefront the matrix core
+// can only be used "diagonally" (16 columns = 16 segments of the row, one useful entry per column, picked
+// out per group), every wavefront stages x again, and the codes must be transposed between lanes.  Here
+// the codes are laid out at load time the way the matrix core wants them for 16 weight rows at once:
+//
+//   4-bit   tile[R][J][lane l = c + 16 q][word m]  (16 bytes per lane, 1 KiB per (R, J))
+//             = word q (codes 8 q .. 8 q + 7, device nibble order of nq_nib.h) of the 32-code chunk
+//               4 J + m of row 16 R + c:  MFMA m of step J (v_mfma_f32_16x16x32_bf16) takes word m as
+//               its B operand, so column c is one chunk of row 16 R + c, i.e. one Q4_0 group, and the
+//               four MFMAs of a step are one group of 128;
+//           scales[R][J][c][m] fp16 (Q4_0) or [R][J][c] = fp16 scale | zero point << 16 (groups of 128)
+//   int8    tile[R][J][lane][16 B] = codes 64 J + 16 q .. + 15 of row 16 R + c: the B operand of
+//           v_mfma_i32_16x16x64_i8 as it lies in memory
+//
+// so a load instruction is 1 KiB contiguous, nothing is transposed or picked, and the 16 results of a
+// step sit in the same register of lanes 0 .. 15.  A workgroup owns one tile of 16 rows; its KW
+// wavefronts split K (JPW steps each; all of a wavefront's loads are requested before anything else)
+// and meet in LDS in wave order (fixed: a repeated call returns the same bits).
+//
+// The A operand is x, and its 16 rows are free: a lane's A row is lane % 16, and only the rows that hold
+// something are read back.  bf16 x is row 0.  fp32 x is the exact three-term bf16 split hi + mid + lo in
+// rows 0, 1, 2 of the SAME MFMA (so fp32 activations cost the one MFMA bf16 activations cost; the three
+// partial dot products are added in fp32).  For int8 weights x is split, per wavefront and slice of K, into
+// three int8 terms under the slice's largest magnitude,
+//     x[k] = (absmax / 127) (q1[k] + q2[k] / 254 + q3[k] / 254^2) + e,  |e| <= 6e-8 absmax,
+// again rows 0, 1, 2 of one MFMA: three exact int32 sums per slice, combined in fp32.  A wavefront stages
+// its own slice of x in its own piece of LDS (LDS runs one wavefront's accesses in order: no barrier).
+// 4-bit codes become the exact bf16 values 16 + q (bits 0x4180 | q << 3); the zero point leaves the
+// inner loop through the slice's group sums of x, which stay in registers and are read with v_readlane.
+//
+// Steps past K (K is a multiple of the step; the last round of a wavefront may be short) load from a
+// clamped address, meet x = 0 and get scale 0.
+#include <hip/hip_fp16.h>
+
+#include <algorithm>
+
+#include "nq_common.h"
+
+namespace nq {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+struct TileParams {
+    const u32x4* tile;
+    const void* tscales;      // 4-bit: the tile-ordered group records
+    const float* col_scale;   // int8: per output channel [N]
+    const void* x;
+    const void* bias;
+    int32_t N, K, NJ;         // NJ steps per row tile (128 k for 4-bit, 64 k for int8)
+    int32_t y_dtype, bias_dtype, epilogue;
+    SegTable seg;
+};
+
+__device__ __forceinline__ bf16x8 as_bf16x8(const u32x4& v) { return __builtin_bit_cast(bf16x8, v); }
+
+// eight nibbles of a word -> four packed bf16 pairs holding 16 + code, in k order (nq_nib.h); `magic` is
+// 0x41804180 in a vector register the compiler cannot see through (one v_and_or_b32 per pair)
+__device__ __forceinline__ u32x4 nib_word_to_bf16(uint32_t w, uint32_t magic) {
+    u32x4 r;
+    r[0] = ((w << 3) & 0x00780078u) | magic;
+    r[1] = ((w >> 1) & 0x00780078u) | magic;
+    r[2] = ((w >> 5) & 0x00780078u) | magic;
+    r[3] = ((w >> 9) & 0x00780078u) | magic;
+    return r;
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
+    uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
+#define NQ_DPP(v, ctrl) __builtin_amdgcn_update_dpp(0, (int)(v), ctrl, 0xF, 0xF, false)
+#define NQ_DPP_F32(v, ctrl) __int_as_float(NQ_DPP(__float_as_int(v), ctrl))
+
+// the workgroup's 16 rows: the wavefronts' shares summed in wave order, bias, epilogue, placement by part
+template <int KW>
+__device__ __forceinline__ void finish_rows(const TileParams& p, const float (&red)[KW][16], int64_t R) {
+    if (threadIdx.x < 16) {
+        float z = red[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < KW; w++) z += red[w][threadIdx.x];
+        const int64_t n = R * 16 + threadIdx.x;
+        if (n < p.N) {
+            if (p.col_scale) z *= p.col_scale[n];
+            if (p.bias)
+                z += (p.bias_dtype == NQ_DT_F32)
+                         ? reinterpret_cast<const float*>(p.bias)[n]
+                         : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+            void* yp;
+            int width, col;
+            seg_lookup(p.seg, (int)n, yp, width, col);  // M = 1: the part's row is its only row
+            if (p.y_dtype == NQ_DT_F32)
+                reinterpret_cast<float*>(yp)[col] = z;
+            else
+                reinterpret_cast<uint16_t*>(yp)[col] = f32_to_bf16_rne(z);
+        }
+    }
+}
+
+// ---- 4-bit codes ----------------------------------------------------------------------------------
+template <int FMT, bool XF32, int KW, int JPW>
+__global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p) {
+    constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
+    constexpr int NT = XF32 ? 3 : 1;
+    constexpr int NP = JPW * 16;         // 16-byte pieces (8 values) of x per wavefront and term
+    constexpr int PPL = (NP + 63) / 64;  // pieces per lane
+    __shared__ __attribute__((aligned(16))) uint8_t xs[KW][NT][NP * 16];
+    __shared__ float red[KW][16];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const int64_t R = blockIdx.x;
+    uint32_t magic = 0x41804180u;
+    asm volatile("" : "+v"(magic));
+    // A row = lane % 16: rows 0 .. NT - 1 are the terms of x, the others repeat the last (their results are unused)
+    const uint8_t* const arow = &xs[wave][XF32 ? min(c, 2) : 0][q * 16];
+    float acc = 0.0f;
+
+    for (int J0 = wave * JPW; J0 < p.NJ; J0 += KW * JPW) {
+        u32x4 wv[JPW];
+        uint2 sc[JPW];
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const int64_t at = R * p.NJ + min(J0 + j, p.NJ - 1);
+            wv[j] = __builtin_nontemporal_load(p.tile + at * 64 + lane);
+            const uint32_t keep = J0 + j < p.NJ ? ~0u : 0u;
+            if constexpr (!G128) {
+                sc[j] = reinterpret_cast<const uint2*>(p.tscales)[at * 16 + c];
+                sc[j].x &= keep, sc[j].y &= keep;
+            } else {
+                sc[j].x = reinterpret_cast<const uint32_t*>(p.tscales)[at * 16 + c] & keep;
+            }
+        }
+        // the slice of x under this round: lane l holds pieces l, l + 64; a piece past K is zero
+        float part[PPL];
+#pragma unroll
+        for (int h = 0; h < PPL; h++) {
+            const int pc = lane + 64 * h;               // piece of the slice
+            const int k0 = J0 * 128 + pc * 8;           // its first k
+            const int kc = min(k0, p.K - 8);
+            const uint32_t keep = k0 < p.K ? ~0u : 0u;
+            const bool mine = pc < NP;
+            if constexpr (XF32) {
+                const float* xf = reinterpret_cast<const float*>(p.x) + kc;
+                const u32x4 r0 = *reinterpret_cast<const u32x4*>(xf), r1 = *reinterpret_cast<const u32x4*>(xf + 4);
+                uint32_t v[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = r0[i] & keep, v[4 + i] = r1[i] & keep;
+                // hi + mid + lo = the fp32 value: each split truncates, so each residual is exact in fp32
+                u32x4 t0, t1, t2;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t a = v[2 * i], b = v[2 * i + 1];
+                    const float ra = __uint_as_float(a) - __uint_as_float(a & 0xFFFF0000u);
+                    const float rb = __uint_as_float(b) - __uint_as_float(b & 0xFFFF0000u);
+                    const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                    const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                    t0[i] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+                    t1[i] = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+                    t2[i] = __builtin_amdgcn_perm(__float_as_uint(sb), __float_as_uint(sa), 0x07060302u);
+                }
+                if (mine) {
+                    *reinterpret_cast<u32x4*>(&xs[wave][0][pc * 16]) = t0;
+                    *reinterpret_cast<u32x4*>(&xs[wave][1][pc * 16]) = t1;
+                    *reinterpret_cast<u32x4*>(&xs[wave][2][pc * 16]) = t2;
+                }
+                part[h] = ((__uint_as_float(v[0]) + __uint_as_float(v[1])) + (__uint_as_float(v[2]) + __uint_as_float(v[3]))) +
+                          ((__uint_as_float(v[4]) + __uint_as_float(v[5])) + (__uint_as_float(v[6]) + __uint_as_float(v[7])));
+            } else {
+                u32x4 r0 = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+#pragma unroll
+                for (int i = 0; i < 4; i++) r0[i] &= keep;
+                if (mine) *reinterpret_cast<u32x4*>(&xs[wave][0][pc * 16]) = r0;
+                float s = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) s += __uint_as_float(r0[i] << 16) + __uint_as_float(r0[i] & 0xFFFF0000u);
+                part[h] = s;
+            }
+            // the sum of x under a chunk (four lanes), under a group of 128 (sixteen): fixed butterflies
+            part[h] += NQ_DPP_F32(part[h], 0xB1);
+            part[h] += NQ_DPP_F32(part[h], 0x4E);
+            if constexpr (G128) {
+                part[h] += NQ_DPP_F32(part[h], 0x141);
+                part[h] += NQ_DPP_F32(part[h], 0x140);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            f32x4 dd[G128 ? 1 : 4];
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const u32x4 bop = nib_word_to_bf16(wv[j][m], magic);
+                const u32x4 aop = *reinterpret_cast<const u32x4*>(arow + (16 * j + 4 * m) * 16);
+                if (!G128 || m == 0) dd[G128 ? 0 : m] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+                dd[G128 ? 0 : m] =
+                    __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop), as_bf16x8(bop), dd[G128 ? 0 : m], 0, 0, 0);
+            }
+            auto rowsum = [](const f32x4& d) -> float { return XF32 ? (d[0] + d[1]) + d[2] : d[0]; };
+            if constexpr (!G128) {
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    const uint32_t sbits = (m < 2 ? sc[j].x : sc[j].y) >> (16 * (m & 1));
+                    const float d = __half2float(__ushort_as_half((uint16_t)(sbits & 0xFFFFu)));
+                    const int g4 = 4 * (4 * j + m);  // the chunk's sum sits in lanes g4 .. g4 + 3 of part[g4 / 64]
+                    const float xsg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part[g4 / 64]), g4 % 64));
+                    acc = fmaf(d, fmaf(-24.0f, xsg, rowsum(dd[m])), acc);
+                }
+            } else {
+                const float d = __half2float(__ushort_as_half((uint16_t)(sc[j].x & 0xFFFFu)));
+                const float zoff = 16.0f + (float)(sc[j].x >> 16);
+                const int g16 = 16 * j;
+                const float xsg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part[g16 / 64]), g16 % 64));
+                acc = fmaf(d, fmaf(-zoff, xsg, rowsum(dd[0])), acc);
+            }
+        }
+    }
+    if (q == 0) red[wave][c] = acc;
+    __syncthreads();
+    finish_rows<KW>(p, red, R);
+}
+
+// ---- int8 codes -----------------------------------------------------------------------------------
+constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: the low byte of (t + MAGIC)'s bits is rne(t) as an int8
+
+__device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3) {
+    return __builtin_amdgcn_perm(a1, a0, 0x0c0c0400u) | __builtin_amdgcn_perm(a3, a2, 0x04000c0cu);
+}
+
+template <bool XF32, int KW, int JPW>
+__global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p) {
+    constexpr int SL = JPW * 64;  // k per wavefront and round
+    constexpr int VPL = SL > 256 ? 8 : 4;  // values of x per lane (one or two words of int8 per term)
+    constexpr int NL = SL / VPL;           // lanes that hold a piece of the slice (16 .. 64)
+    __shared__ __attribute__((aligned(16))) uint8_t xq[KW][3][SL];
+    __shared__ float red[KW][16];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const int64_t R = blockIdx.x;
+    const uint8_t* const arow = &xq[wave][min(c, 2)][q * 16];
+    float accf = 0.0f;
+
+    for (int J0 = wave * JPW; J0 < p.NJ; J0 += KW * JPW) {
+        u32x4 wv[JPW];
+#pragma unroll
+        for (int j = 0; j < JPW; j++)
+            wv[j] = __builtin_nontemporal_load(p.tile + (R * p.NJ + min(J0 + j, p.NJ - 1)) * 64 + lane);
+        // the slice of x under this round: lane l < NL holds values VPL l .. ; past K they are zero
+        const int k0 = J0 * 64 + min(lane, NL - 1) * VPL;
+        const int kc = min(k0, p.K - VPL);
+        const bool live = k0 < p.K;
+        float xf[VPL];
+        if constexpr (XF32) {
+            const float* xr = reinterpret_cast<const float*>(p.x) + kc;
+#pragma unroll
+            for (int i = 0; i < VPL; i += 4) {
+                const f32x4 t = *reinterpret_cast<const f32x4*>(xr + i);
+                xf[i] = t[0], xf[i + 1] = t[1], xf[i + 2] = t[2], xf[i + 3] = t[3];
+            }
+        } else {
+            const uint32_t* xr = reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+            uint32_t t[VPL / 2];
+            if constexpr (VPL == 8) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(xr);
+                t[0] = v[0], t[1] = v[1], t[2] = v[2], t[3] = v[3];
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>(xr);
+                t[0] = v.x, t[1] = v.y;
+            }
+#pragma unroll
+            for (int i = 0; i < VPL; i += 2)
+                xf[i] = __uint_as_float(t[i / 2] << 16), xf[i + 1] = __uint_as_float(t[i / 2] & 0xFFFF0000u);
+        }
+        // the slice's largest magnitude as a bit pattern (NaN > inf > finite), over the wavefront
+        uint32_t mbits = 0;
+#pragma unroll
+        for (int i = 0; i < VPL; i++) {
+            if (!live) xf[i] = 0.0f;
+            mbits = max(mbits, __float_as_uint(xf[i]) & 0x7FFFFFFFu);
+        }
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0xB1));
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0x4E));
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0x141));
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0x140));
+        {
+            const auto sw = __builtin_amdgcn_permlane16_swap(mbits, mbits, false, false);
+            mbits = max(sw[0], sw[1]);
+        }
+        {
+            const auto sw = __builtin_amdgcn_permlane32_swap(mbits, mbits, false, false);
+            mbits = max(sw[0], sw[1]);
+        }
+        const bool finite = mbits < 0x7F800000u;
+        const float absmax = __uint_as_float(mbits);
+        // (below 1e-30 the reciprocal would overflow: such a slice counts as zero, an error below 1e-30 * sum |w|)
+        const float inv_s = (finite && absmax > 1e-30f) ? 127.0f / absmax : 0.0f;
+        // a NaN or an infinity in the slice makes the slice's share, hence every output, NaN
+        const float s_x = finite ? (inv_s != 0.0f ? absmax * (1.0f / 127.0f) : 0.0f) : __uint_as_float(0x7FC00000u);
+        uint32_t pk[3][VPL / 4];
+#pragma unroll
+        for (int i = 0; i < VPL; i += 4) {
+            uint32_t a1[4], a2[4], a3[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                // round by adding 1.5 * 2^23 (the sum's low byte is the int8) and take every leftover against the
+                // very integer that was packed: no leftover exceeds a half, no term leaves the int8 range
+                const float t = xf[i + e] * inv_s;
+                const float b1 = t + MAGIC;
+                a1[e] = __float_as_uint(b1);
+                const float r1 = t - (b1 - MAGIC);
+                const float b2 = __builtin_fmaf(r1, 254.0f, MAGIC);
+                a2[e] = __float_as_uint(b2);
+                const float r2 = __builtin_fmaf(r1, 254.0f, MAGIC - b2);
+                a3[e] = __float_as_uint(__builtin_fmaf(r2, 254.0f, MAGIC));
+            }
+            pk[0][i / 4] = pack_low_bytes(a1[0], a1[1], a1[2], a1[3]);
+            pk[1][i / 4] = pack_low_bytes(a2[0], a2[1], a2[2], a2[3]);
+            pk[2][i / 4] = pack_low_bytes(a3[0], a3[1], a3[2], a3[3]);
+        }
+        if (lane < NL) {
+#pragma unroll
+            for (int t = 0; t < 3; t++) {
+                if constexpr (VPL == 8)
+                    *reinterpret_cast<uint2*>(&xq[wave][t][lane * 8]) = make_uint2(pk[t][0], pk[t][1]);
+                else
+                    *reinterpret_cast<uint32_t*>(&xq[wave][t][lane * 4]) = pk[t][0];
+            }
+        }
+        i32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const i32x4 aop = *reinterpret_cast<const i32x4*>(arow + 64 * j);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, __builtin_bit_cast(i32x4, wv[j]), acc, 0, 0, 0);
+        }
+        // |sum| <= 128 * 127 * 512 < 2^24: exact as fp32
+        accf += s_x * fmaf((float)acc[2], 1.0f / 64516.0f, fmaf((float)acc[1], 1.0f / 254.0f, (float)acc[0]));
+    }
+    if (q == 0) red[wave][c] = accf;
+    __syncthreads();
+    finish_rows<KW>(p, red, R);
+}
+
+// ---- load time: the tile-ordered copies -------------------------------------------------------------
+// codes [N][nch][4 words] (row order) -> tile[R][J][lane][4 words]; one thread per lane slot
+__global__ __launch_bounds__(256) void tile4_repack_kernel(const uint32_t* __restrict__ codes, u32x4* __restrict__ tile,
+                                                           int64_t N, int64_t NJ, int64_t slots) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= slots) return;
+    const int l = (int)(t & 63), c = l & 15, q = l >> 4;
+    const int64_t J = (t >> 6) % NJ, R = (t >> 6) / NJ, row = R * 16 + c;
+    u32x4 v = {0, 0, 0, 0};
+    if (row < N) {
+        const uint32_t* src = codes + (row * NJ * 4 + J * 4) * 4 + q;  // chunk 4 J of the row, word q
+#pragma unroll
+        for (int m = 0; m < 4; m++) v[m] = src[m * 4];
+    }
+    tile[t] = v;
+}
+
+// Q4_0 scales [N][nch] fp16 -> [R][J][c][4]; groups of 128: scales [N][G] fp16, zps [N][G] -> [R][J][c] u32
+__global__ __launch_bounds__(256) void tile4_scales_kernel(const uint16_t* __restrict__ scales, const uint8_t* __restrict__ zps,
+                                                           uint32_t* __restrict__ out, int64_t N, int64_t NJ, int64_t count,
+                                                           int g128) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= count) return;
+    const int c = (int)(t & 15);
+    const int64_t J = (t >> 4) % NJ, R = (t >> 4) / NJ, row = R * 16 + c;
+    if (g128) {
+        out[t] = row < N ? ((uint32_t)scales[row * NJ + J] | ((uint32_t)zps[row * NJ + J] << 16)) : 0u;
+    } else {
+        uint32_t lo = 0, hi = 0;
+        if (row < N) {
+            const uint16_t* s = scales + row * NJ * 4 + J * 4;
+            lo = (uint32_t)s[0] | ((uint32_t)s[1] << 16), hi = (uint32_t)s[2] | ((uint32_t)s[3] << 16);
+        }
+        out[2 * t] = lo, out[2 * t + 1] = hi;
+    }
+}
+
+// int8 codes [N][K] -> tile[R][J][lane][16 B]
+__global__ __launch_bounds__(256) void tile8_repack_kernel(const uint8_t* __restrict__ codes, u32x4* __restrict__ tile,
+                                                           int64_t N, int64_t K, int64_t NJ, int64_t slots) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= slots) return;
+    const int l = (int)(t & 63), c = l & 15, q = l >> 4;
+    const int64_t J = (t >> 6) % NJ, R = (t >> 6) / NJ, row = R * 16 + c;
+    u32x4 v = {0, 0, 0, 0};
+    if (row < N) v = *reinterpret_cast<const u32x4*>(codes + row * K + J * 64 + q * 16);
+    tile[t] = v;
+}
+
+template <int FMT, bool XF32, int KW>
+int32_t launch4_jpw(const TileParams& p, int jpw, dim3 grid, hipStream_t s) {
+#define NQ_T4(J_)                                                                                       \
+    case J_:                                                                                            \
+        hipLaunchKernelGGL((gemv_tile4_kernel<FMT, XF32, KW, J_>), grid, dim3(64 * KW), 0, s, p);       \
+        break;
+    switch (jpw) {
+        NQ_T4(1) NQ_T4(2) NQ_T4(3) NQ_T4(4) NQ_T4(5) NQ_T4(6) NQ_T4(7) NQ_T4(8)
+        default: return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no tile GEMV for this IN");
+    }
+#undef NQ_T4
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+template <int FMT, bool XF32>
+int32_t launch4(const TileParams& p, hipStream_t s) {
+    // about four steps (4 KiB of codes) per wavefront measured best: 8 wavefronts up to K = 4096, 16 beyond
+    const int kw = p.NJ <= 32 ? 8 : 16;
+    const int jpw = std::min(8, (p.NJ + kw - 1) / kw);
+    const dim3 grid((unsigned)((p.N + 15) / 16));
+    return kw == 8 ? launch4_jpw<FMT, XF32, 8>(p, jpw, grid, s) : launch4_jpw<FMT, XF32, 16>(p, jpw, grid, s);
+}
+
+template <bool XF32, int KW>
+int32_t launch8_jpw(const TileParams& p, int jpw, dim3 grid, hipStream_t s) {
+#define NQ_T8(J_)                                                                                  \
+    case J_:                                                                                       \
+        hipLaunchKernelGGL((gemv_tile8_kernel<XF32, KW, J_>), grid, dim3(64 * KW), 0, s, p);       \
+        break;
+    switch (jpw) {
+        NQ_T8(1) NQ_T8(2) NQ_T8(3) NQ_T8(4) NQ_T8(5) NQ_T8(6) NQ_T8(7) NQ_T8(8)
+        default: return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no tile GEMV for this IN");
+    }
+#undef NQ_T8
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+template <bool XF32>
+int32_t launch8(const TileParams& p, hipStream_t s) {
+    // eight steps (8 KiB of codes) per wavefront: 8 wavefronts up to K = 4096, 16 beyond; longer rows take rounds
+    const int kw = p.NJ <= 64 ? 8 : 16;
+    const int jpw = std::min(8, (p.NJ + kw - 1) / kw);
+    const dim3 grid((unsigned)((p.N + 15) / 16));
+    return kw == 8 ? launch8_jpw<XF32, 8>(p, jpw, grid, s) : launch8_jpw<XF32, 16>(p, jpw, grid, s);
+}
+
+}  // namespace
+
+// Which layers get the tile-ordered copy (a second copy of the codes: 0.5 or 1 byte per weight on top):
+// weights of 4 M codes and more, whose single-row calls are bound by the weight stream.  4-bit: Q4_0 or
+// groups of exactly 128, IN a multiple of 128 in 2048 .. 16384; int8: IN a multiple of 64, at least 1024.
+bool tile_copy_wanted(const nq_layer* L) {
+    if (L->no_tile_copy) return false;
+    if ((int64_t)L->in * L->out < ((int64_t)4 << 20)) return false;
+    if (L->format == NQ_FMT_Q4_0 || (L->format == NQ_FMT_W4_GROUP && L->group == 128))
+        return L->in % 128 == 0 && L->in >= 2048 && L->in <= 16384;
+    if (L->format == NQ_FMT_W8_CHANNEL) return L->in % 64 == 0 && L->in >= 1024;
+    return false;
+}
+
+// builds (or drops) the tile-ordered copy from the row-ordered device arrays of a loaded layer
+int32_t build_tile_copy(nq_layer* L, hipStream_t s) {
+    if (L->d_tile16) (void)hipFree(L->d_tile16);
+    if (L->d_tile16_scales) (void)hipFree(L->d_tile16_scales);
+    L->d_tile16 = nullptr, L->d_tile16_scales = nullptr, L->tile_nj = 0;
+    if (!tile_copy_wanted(L)) return NQ_OK;
+    const int64_t N = L->out, R = (N + 15) / 16;
+    const bool w8 = L->format == NQ_FMT_W8_CHANNEL;
+    const int64_t NJ = w8 ? L->in / 64 : L->in / 128;
+    const int64_t slots = R * NJ * 64;
+    NQ_HIP(hipMalloc((void**)&L->d_tile16, (size_t)slots * 16));
+    if (w8) {
+        hipLaunchKernelGGL(tile8_repack_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, s, L->d_codes,
+                           reinterpret_cast<u32x4*>(L->d_tile16), N, (int64_t)L->in, NJ, slots);
+    } else {
+        const bool g128 = L->format == NQ_FMT_W4_GROUP;
+        const int64_t count = R * NJ * 16;
+        NQ_HIP(hipMalloc(&L->d_tile16_scales, (size_t)count * (g128 ? 4 : 8)));
+        hipLaunchKernelGGL(tile4_repack_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, s,
+                           reinterpret_cast<const uint32_t*>(L->d_codes), reinterpret_cast<u32x4*>(L->d_tile16), N, NJ, slots);
+        hipLaunchKernelGGL(tile4_scales_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s,
+                           reinterpret_cast<const uint16_t*>(L->d_scales), L->d_zps,
+                           reinterpret_cast<uint32_t*>(L->d_tile16_scales), N, NJ, count, (int)g128);
+    }
+    NQ_HIP(hipGetLastError());
+    L->tile_nj = (int32_t)NJ;
+    return NQ_OK;
+}
+
+bool gemv_tile_applicable(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (a.M != 1 || !L->d_tile16) return false;
+    if (a.x_dtype != NQ_DT_BF16 && a.x_dtype != NQ_DT_F32) return false;
+    return a.y_dtype == NQ_DT_F32 || a.y_dtype == NQ_DT_BF16;
+}
+
+int32_t launch_gemv_tile(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    TileParams p{};
+    p.tile = reinterpret_cast<const u32x4*>(L->d_tile16), p.tscales = L->d_tile16_scales;
+    p.col_scale = L->format == NQ_FMT_W8_CHANNEL ? reinterpret_cast<const float*>(L->d_scales) : nullptr;
+    p.x = a.x, p.bias = a.bias, p.seg = a.seg;
+    p.N = L->out, p.K = L->in, p.NJ = L->tile_nj;
+    p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
+    switch (L->format) {
+        case NQ_FMT_Q4_0:
+            return xf32 ? launch4<NQ_FMT_Q4_0, true>(p, a.stream) : launch4<NQ_FMT_Q4_0, false>(p, a.stream);
+        case NQ_FMT_W4_GROUP:
+            return xf32 ? launch4<NQ_FMT_W4_GROUP, true>(p, a.stream) : launch4<NQ_FMT_W4_GROUP, false>(p, a.stream);
+        case NQ_FMT_W8_CHANNEL: return xf32 ? launch8<true>(p, a.stream) : launch8<false>(p, a.stream);
+    }
+    return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no tile GEMV for this format");
+}
+
+}  // namespace nq

@@ -59,10 +59,13 @@ class _Layer:
 
     FORMAT = -1
 
-    def __init__(self, IN: int, OUT: int, group: int = 0):
+    def __init__(self, IN: int, OUT: int, group: int = 0, tile_copy: bool = True):
+        """tile_copy=False (NQ_FLAG_NO_TILE_COPY): a large layer does not keep the second,
+        matrix-core-ordered copy of its codes that its single-row calls stream faster."""
         self.IN, self.OUT, self.group = int(IN), int(OUT), int(group)
         h = C.c_void_p()
-        L.check(L.lib().nq_create(C.byref(h), self.FORMAT, self.IN, self.OUT, self.group, 0))
+        flags = 0 if tile_copy else L.FLAG_NO_TILE_COPY
+        L.check(L.lib().nq_create(C.byref(h), self.FORMAT, self.IN, self.OUT, self.group, flags))
         self._h = h
         self._loaded = False
 
@@ -93,9 +96,15 @@ class _Layer:
         return out
 
     def dequantized_dev(self, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """deq(W) [OUT, IN] fp32 on the device (`dequant_q4_0_kernel`, q4_0.mojo:242-266)."""
+        """deq(W) [OUT, IN] fp32 on the device (`dequant_q4_0_kernel`, q4_0.mojo:242-266).  Without `out` it is
+        written into the buffer handed to `share_scratch`, if any (its first OUT*IN values, returned as a
+        [OUT, IN] view), else into a new tensor."""
         if out is None:
-            out = torch.empty((self.OUT, self.IN), dtype=torch.float32, device="cuda")
+            shared = getattr(self, "deq", None)
+            if shared is not None:
+                out = shared.view(-1)[: self.OUT * self.IN].view(self.OUT, self.IN)
+            else:
+                out = torch.empty((self.OUT, self.IN), dtype=torch.float32, device="cuda")
         L.check(L.lib().nq_dequantize(self._h, _dev_ptr(out), out.numel(), _stream_ptr()))
         return out
 
@@ -107,10 +116,10 @@ class QLinear(_Layer):
     FORMAT = L.FMT_Q4_0
     ARITY = 1
 
-    def __init__(self, IN: int, OUT: int):
+    def __init__(self, IN: int, OUT: int, tile_copy: bool = True):
         if IN % Q4_GROUP != 0:  # the comptime assert of qlinear.mojo:243-245
             raise L.NQError(L.NQ_ERR_INVALID, "QLinear: IN must be a multiple of 32 (one Q4_0 group)")
-        super().__init__(IN, OUT, Q4_GROUP)
+        super().__init__(IN, OUT, Q4_GROUP, tile_copy)
         self.W_SIZE = IN * OUT
         self.ROW_BYTES = (IN // Q4_GROUP) * Q4_BLOCK
         self.BYTES = OUT * self.ROW_BYTES
@@ -155,13 +164,14 @@ class QLinear(_Layer):
         return self.dequantized_dev().cpu().numpy()
 
     def share_scratch(self, buf: torch.Tensor, n: int):
-        """Use `buf` (n fp32 values, at least OUT*IN) as the dequantize scratch
-        (qlinear.mojo:330-340).  This build's forward never materialises
-        deq(W); the buffer is what `dequantized_dev` without an argument
-        writes."""
-        if n < self.W_SIZE:
+        """Use `buf` (n fp32 values on the device, at least OUT*IN) as the dequantize scratch
+        (qlinear.mojo:330-340).  This build's forward never materialises deq(W), so the forward does not
+        touch it; it is where `dequantized_dev()` and `dequantized()` write deq(W) from now on."""
+        if n < self.W_SIZE or buf.numel() < n:
             raise L.NQError(L.NQ_ERR_SIZE,
-                            f"QLinear.share_scratch: {n} values for a [{self.OUT}, {self.IN}] weight")
+                            f"QLinear.share_scratch: {min(n, buf.numel())} values for a [{self.OUT}, {self.IN}] weight")
+        if buf.dtype != torch.float32 or not buf.is_cuda or not buf.is_contiguous():
+            raise L.NQError(L.NQ_ERR_INVALID, "QLinear.share_scratch: the scratch must be a contiguous fp32 device tensor")
         self.deq = buf
 
     def keep_only_repacked(self):
@@ -171,13 +181,18 @@ class QLinear(_Layer):
 
     # ── Module ─────────────────────────────────────────────────────────────
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None, target: str = "gpu",
-                ctx=None) -> torch.Tensor:
+                ctx=None, bias: Optional[torch.Tensor] = None, epilogue: str = "none",
+                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
         """y[B, OUT] = x[B, IN] @ deq(W)^T (qlinear.mojo:407-477).  x fp32 (the
-        reference's boundary) or bf16; y fp32."""
+        reference's boundary) or bf16; y fp32.  Beyond the reference's surface: `bias` / `epilogue`
+        (`LinearAct`'s, linear_act.mojo:81-115) and `out_dtype=torch.bfloat16` (a bf16-flow tower takes
+        bf16 in and hands bf16 on, without the boundary casts of qlinear.mojo:430-463)."""
         _need_gpu(target)
         if x.dtype not in _TORCH_DT:
             raise L.NQError(L.NQ_ERR_INVALID, "QLinear.forward: x must be fp32 or bf16")
-        return self._forward(x, _TORCH_DT[x.dtype], None, out, torch.float32, None, "none", "QLinear.forward")
+        if out_dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "QLinear.forward: y must be fp32 or bf16")
+        return self._forward(x, _TORCH_DT[x.dtype], None, out, out_dtype, bias, epilogue, "QLinear.forward")
 
     def vjp(self, forward_input: torch.Tensor, grad_output: torch.Tensor,
             grad_input: Optional[torch.Tensor] = None, target: str = "gpu", ctx=None) -> torch.Tensor:
@@ -232,8 +247,8 @@ class W4GroupLinear(_Layer):
 
     FORMAT = L.FMT_W4_GROUP
 
-    def __init__(self, IN, OUT, group=128):
-        super().__init__(IN, OUT, group)
+    def __init__(self, IN, OUT, group=128, tile_copy: bool = True):
+        super().__init__(IN, OUT, group, tile_copy)
         self.G = -(-IN // group)
 
     def set_weight(self, codes, scales_f16, zps):
