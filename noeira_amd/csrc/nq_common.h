@@ -73,13 +73,16 @@ struct SegTable {
     void* y[4];
 };
 
-// row n -> (part's y, its width, the column in it)
+// row n -> (part's y, its width, the column in it).  Every table entry is read with a constant index, so the
+// table stays in scalar registers (a run-time index would turn into a load from the argument buffer, a round
+// trip to memory at the end of the kernel).
 __device__ __forceinline__ void seg_lookup(const SegTable& sg, int n, void*& y, int& width, int& col) {
-    int s = 0, base = 0;
+    int base = 0, end = sg.end[0];
+    void* yy = sg.y[0];
 #pragma unroll
     for (int t = 0; t < 3; t++)
-        if (t + 1 < sg.nseg && n >= sg.end[t]) s = t + 1, base = sg.end[t];
-    y = sg.y[s], width = sg.end[s] - base, col = n - base;
+        if (t + 1 < sg.nseg && n >= sg.end[t]) base = sg.end[t], end = sg.end[t + 1], yy = sg.y[t + 1];
+    y = yy, width = end - base, col = n - base;
 }
 
 struct ForwardArgs {

@@ -83,20 +83,35 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float v) {
 #define NQ_DPP(v, ctrl) __builtin_amdgcn_update_dpp(0, (int)(v), ctrl, 0xF, 0xF, false)
 #define NQ_DPP_F32(v, ctrl) __int_as_float(NQ_DPP(__float_as_int(v), ctrl))
 
+// The epilogue's operands of row 16 R + lane % 16, requested at kernel start (raw: nothing is computed from them
+// before the end, so their latency hides under the weight stream instead of following the barrier).
+struct RowTail {
+    float cs;
+    uint32_t braw;
+};
+
+__device__ __forceinline__ RowTail fetch_tail(const TileParams& p, int64_t R, int lane) {
+    RowTail t;
+    const int64_t n = min(R * 16 + (lane & 15), (int64_t)p.N - 1);
+    t.cs = p.col_scale ? p.col_scale[n] : 1.0f;
+    t.braw = 0;
+    if (p.bias)
+        t.braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                             : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
+    return t;
+}
+
 // the workgroup's 16 rows: the wavefronts' shares summed in wave order, bias, epilogue, placement by part
 template <int KW>
-__device__ __forceinline__ void finish_rows(const TileParams& p, const float (&red)[KW][16], int64_t R) {
+__device__ __forceinline__ void finish_rows(const TileParams& p, const float (&red)[KW][16], int64_t R, const RowTail& t) {
     if (threadIdx.x < 16) {
         float z = red[0][threadIdx.x];
 #pragma unroll
         for (int w = 1; w < KW; w++) z += red[w][threadIdx.x];
         const int64_t n = R * 16 + threadIdx.x;
         if (n < p.N) {
-            if (p.col_scale) z *= p.col_scale[n];
-            if (p.bias)
-                z += (p.bias_dtype == NQ_DT_F32)
-                         ? reinterpret_cast<const float*>(p.bias)[n]
-                         : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+            if (p.col_scale) z *= t.cs;
+            if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? t.braw : t.braw << 16);
             if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
             void* yp;
             int width, col;
@@ -110,7 +125,8 @@ __device__ __forceinline__ void finish_rows(const TileParams& p, const float (&r
 }
 
 // ---- 4-bit codes ----------------------------------------------------------------------------------
-template <int FMT, bool XF32, int KW, int JPW>
+// EXACT: K is exactly KW * JPW steps (one round, no step past K): the clamps and masks below fall away
+template <int FMT, bool XF32, int KW, int JPW, bool EXACT>
 __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p) {
     constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
     constexpr int NT = XF32 ? 3 : 1;
@@ -127,36 +143,50 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
     const uint8_t* const arow = &xs[wave][XF32 ? min(c, 2) : 0][q * 16];
     float acc = 0.0f;
 
-    for (int J0 = wave * JPW; J0 < p.NJ; J0 += KW * JPW) {
-        u32x4 wv[JPW];
-        uint2 sc[JPW];
+    RowTail tail{};
+    if (wave == 0) tail = fetch_tail(p, R, lane);
+
+    for (int J0 = wave * JPW; J0 < p.NJ; J0 += EXACT ? p.NJ : KW * JPW) {
+        // Every load of the round is requested here, x first (it is needed first, and waiting for it leaves the
+        // codes in flight), from clamped addresses, and nothing loaded is touched before it is needed: an
+        // instruction on a loaded value makes the wavefront wait for that load and every load before it.
+        // The slice of x under this round: lane l holds the 8-value pieces l, l + 64.
+        u32x4 xr[PPL][XF32 ? 2 : 1];
 #pragma unroll
-        for (int j = 0; j < JPW; j++) {
-            const int64_t at = R * p.NJ + min(J0 + j, p.NJ - 1);
-            wv[j] = __builtin_nontemporal_load(p.tile + at * 64 + lane);
-            const uint32_t keep = J0 + j < p.NJ ? ~0u : 0u;
-            if constexpr (!G128) {
-                sc[j] = reinterpret_cast<const uint2*>(p.tscales)[at * 16 + c];
-                sc[j].x &= keep, sc[j].y &= keep;
+        for (int h = 0; h < PPL; h++) {
+            const int kx = J0 * 128 + (lane + 64 * h) * 8;
+            const int kc = (EXACT && NP % 64 == 0) ? kx : min(kx, p.K - 8);
+            if constexpr (XF32) {
+                const float* xf = reinterpret_cast<const float*>(p.x) + kc;
+                xr[h][0] = *reinterpret_cast<const u32x4*>(xf), xr[h][1] = *reinterpret_cast<const u32x4*>(xf + 4);
             } else {
-                sc[j].x = reinterpret_cast<const uint32_t*>(p.tscales)[at * 16 + c] & keep;
+                xr[h][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
             }
         }
-        // the slice of x under this round: lane l holds pieces l, l + 64; a piece past K is zero
+        u32x4 wv[JPW];
+        uint2 sc[JPW];
+        // (32-bit offsets from the tile's base: a layer's tile copy is below 4 GB)
+        const u32x4* const wbase = p.tile + R * p.NJ * 64;
+        const uint32_t* const sbase = reinterpret_cast<const uint32_t*>(p.tscales) + R * p.NJ * (G128 ? 16 : 32);
+#pragma unroll
+        for (int j = 0; j < JPW; j++) wv[j] = __builtin_nontemporal_load(wbase + ((EXACT ? J0 + j : min(J0 + j, p.NJ - 1)) * 64 + lane));
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const int at = (EXACT ? J0 + j : min(J0 + j, p.NJ - 1)) * 16 + c;
+            if constexpr (!G128) sc[j] = reinterpret_cast<const uint2*>(sbase)[at];
+            else sc[j].x = sbase[at], sc[j].y = 0;
+        }
+        // x -> this wavefront's piece of LDS, and the sums of x under every chunk / group; a piece past K is zero
         float part[PPL];
 #pragma unroll
         for (int h = 0; h < PPL; h++) {
             const int pc = lane + 64 * h;               // piece of the slice
-            const int k0 = J0 * 128 + pc * 8;           // its first k
-            const int kc = min(k0, p.K - 8);
-            const uint32_t keep = k0 < p.K ? ~0u : 0u;
+            const uint32_t keep = (EXACT || J0 * 128 + pc * 8 < p.K) ? ~0u : 0u;
             const bool mine = pc < NP;
             if constexpr (XF32) {
-                const float* xf = reinterpret_cast<const float*>(p.x) + kc;
-                const u32x4 r0 = *reinterpret_cast<const u32x4*>(xf), r1 = *reinterpret_cast<const u32x4*>(xf + 4);
                 uint32_t v[8];
 #pragma unroll
-                for (int i = 0; i < 4; i++) v[i] = r0[i] & keep, v[4 + i] = r1[i] & keep;
+                for (int i = 0; i < 4; i++) v[i] = xr[h][0][i] & keep, v[4 + i] = xr[h][1][i] & keep;
                 // hi + mid + lo = the fp32 value: each split truncates, so each residual is exact in fp32
                 u32x4 t0, t1, t2;
 #pragma unroll
@@ -178,14 +208,14 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
                 part[h] = ((__uint_as_float(v[0]) + __uint_as_float(v[1])) + (__uint_as_float(v[2]) + __uint_as_float(v[3]))) +
                           ((__uint_as_float(v[4]) + __uint_as_float(v[5])) + (__uint_as_float(v[6]) + __uint_as_float(v[7])));
             } else {
-                u32x4 r0 = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+                u32x4 r0 = xr[h][0];
 #pragma unroll
                 for (int i = 0; i < 4; i++) r0[i] &= keep;
                 if (mine) *reinterpret_cast<u32x4*>(&xs[wave][0][pc * 16]) = r0;
-                float s = 0.0f;
+                float sum = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 4; i++) s += __uint_as_float(r0[i] << 16) + __uint_as_float(r0[i] & 0xFFFF0000u);
-                part[h] = s;
+                for (int i = 0; i < 4; i++) sum += __uint_as_float(r0[i] << 16) + __uint_as_float(r0[i] & 0xFFFF0000u);
+                part[h] = sum;
             }
             // the sum of x under a chunk (four lanes), under a group of 128 (sixteen): fixed butterflies
             part[h] += NQ_DPP_F32(part[h], 0xB1);
@@ -197,6 +227,9 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
         }
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
+            // a step past K (its loads were clamped, its x is zero) gets scale 0; the choice is uniform over the
+            // wavefront and made here, not where the record was loaded
+            const bool live = EXACT || J0 + j < p.NJ;
             f32x4 dd[G128 ? 1 : 4];
 #pragma unroll
             for (int m = 0; m < 4; m++) {
@@ -211,13 +244,13 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
 #pragma unroll
                 for (int m = 0; m < 4; m++) {
                     const uint32_t sbits = (m < 2 ? sc[j].x : sc[j].y) >> (16 * (m & 1));
-                    const float d = __half2float(__ushort_as_half((uint16_t)(sbits & 0xFFFFu)));
+                    const float d = live ? __half2float(__ushort_as_half((uint16_t)(sbits & 0xFFFFu))) : 0.0f;
                     const int g4 = 4 * (4 * j + m);  // the chunk's sum sits in lanes g4 .. g4 + 3 of part[g4 / 64]
                     const float xsg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part[g4 / 64]), g4 % 64));
                     acc = fmaf(d, fmaf(-24.0f, xsg, rowsum(dd[m])), acc);
                 }
             } else {
-                const float d = __half2float(__ushort_as_half((uint16_t)(sc[j].x & 0xFFFFu)));
+                const float d = live ? __half2float(__ushort_as_half((uint16_t)(sc[j].x & 0xFFFFu))) : 0.0f;
                 const float zoff = 16.0f + (float)(sc[j].x >> 16);
                 const int g16 = 16 * j;
                 const float xsg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(part[g16 / 64]), g16 % 64));
@@ -227,7 +260,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
     }
     if (q == 0) red[wave][c] = acc;
     __syncthreads();
-    finish_rows<KW>(p, red, R);
+    finish_rows<KW>(p, red, R, tail);
 }
 
 // ---- int8 codes -----------------------------------------------------------------------------------
@@ -237,7 +270,7 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a0, uint32_t a1, uin
     return __builtin_amdgcn_perm(a1, a0, 0x0c0c0400u) | __builtin_amdgcn_perm(a3, a2, 0x04000c0cu);
 }
 
-template <bool XF32, int KW, int JPW>
+template <bool XF32, int KW, int JPW, bool EXACT>
 __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p) {
     constexpr int SL = JPW * 64;  // k per wavefront and round
     constexpr int VPL = SL > 256 ? 8 : 4;  // values of x per lane (one or two words of int8 per term)
@@ -250,36 +283,42 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p)
     const uint8_t* const arow = &xq[wave][min(c, 2)][q * 16];
     float accf = 0.0f;
 
-    for (int J0 = wave * JPW; J0 < p.NJ; J0 += KW * JPW) {
-        u32x4 wv[JPW];
-#pragma unroll
-        for (int j = 0; j < JPW; j++)
-            wv[j] = __builtin_nontemporal_load(p.tile + (R * p.NJ + min(J0 + j, p.NJ - 1)) * 64 + lane);
-        // the slice of x under this round: lane l < NL holds values VPL l .. ; past K they are zero
+    RowTail tail{};
+    if (wave == 0) tail = fetch_tail(p, R, lane);
+
+    for (int J0 = wave * JPW; J0 < p.NJ; J0 += EXACT ? p.NJ : KW * JPW) {
+        // x first (it is needed first, and waiting for it leaves the codes in flight), every load from a clamped
+        // address.  The slice of x under this round: lane l < NL holds values VPL l .. ; past K they are zero.
         const int k0 = J0 * 64 + min(lane, NL - 1) * VPL;
-        const int kc = min(k0, p.K - VPL);
-        const bool live = k0 < p.K;
-        float xf[VPL];
+        const int kc = EXACT ? k0 : min(k0, p.K - VPL);
+        const bool live = EXACT || k0 < p.K;
+        uint32_t xraw[XF32 ? VPL : VPL / 2];
         if constexpr (XF32) {
             const float* xr = reinterpret_cast<const float*>(p.x) + kc;
 #pragma unroll
             for (int i = 0; i < VPL; i += 4) {
-                const f32x4 t = *reinterpret_cast<const f32x4*>(xr + i);
-                xf[i] = t[0], xf[i + 1] = t[1], xf[i + 2] = t[2], xf[i + 3] = t[3];
+                const u32x4 t = *reinterpret_cast<const u32x4*>(xr + i);
+                xraw[i] = t[0], xraw[i + 1] = t[1], xraw[i + 2] = t[2], xraw[i + 3] = t[3];
             }
         } else {
             const uint32_t* xr = reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
-            uint32_t t[VPL / 2];
             if constexpr (VPL == 8) {
                 const u32x4 v = *reinterpret_cast<const u32x4*>(xr);
-                t[0] = v[0], t[1] = v[1], t[2] = v[2], t[3] = v[3];
+                xraw[0] = v[0], xraw[1] = v[1], xraw[2] = v[2], xraw[3] = v[3];
             } else {
                 const uint2 v = *reinterpret_cast<const uint2*>(xr);
-                t[0] = v.x, t[1] = v.y;
+                xraw[0] = v.x, xraw[1] = v.y;
             }
+        }
+        u32x4 wv[JPW];
+        const u32x4* const wbase = p.tile + R * p.NJ * 64;  // (32-bit offsets from the tile's base)
 #pragma unroll
-            for (int i = 0; i < VPL; i += 2)
-                xf[i] = __uint_as_float(t[i / 2] << 16), xf[i + 1] = __uint_as_float(t[i / 2] & 0xFFFF0000u);
+        for (int j = 0; j < JPW; j++) wv[j] = __builtin_nontemporal_load(wbase + ((EXACT ? J0 + j : min(J0 + j, p.NJ - 1)) * 64 + lane));
+        float xf[VPL];
+#pragma unroll
+        for (int i = 0; i < VPL; i++) {
+            if constexpr (XF32) xf[i] = __uint_as_float(xraw[i]);
+            else xf[i] = (i & 1) ? __uint_as_float(xraw[i / 2] & 0xFFFF0000u) : __uint_as_float(xraw[i / 2] << 16);
         }
         // the slice's largest magnitude as a bit pattern (NaN > inf > finite), over the wavefront
         uint32_t mbits = 0;
@@ -347,7 +386,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p)
     }
     if (q == 0) red[wave][c] = accf;
     __syncthreads();
-    finish_rows<KW>(p, red, R);
+    finish_rows<KW>(p, red, R, tail);
 }
 
 // ---- load time: the tile-ordered copies -------------------------------------------------------------
@@ -401,9 +440,11 @@ __global__ __launch_bounds__(256) void tile8_repack_kernel(const uint8_t* __rest
 
 template <int FMT, bool XF32, int KW>
 int32_t launch4_jpw(const TileParams& p, int jpw, dim3 grid, hipStream_t s) {
-#define NQ_T4(J_)                                                                                       \
-    case J_:                                                                                            \
-        hipLaunchKernelGGL((gemv_tile4_kernel<FMT, XF32, KW, J_>), grid, dim3(64 * KW), 0, s, p);       \
+    const bool exact = p.NJ == KW * jpw;
+#define NQ_T4(J_)                                                                                                 \
+    case J_:                                                                                                      \
+        if (exact) hipLaunchKernelGGL((gemv_tile4_kernel<FMT, XF32, KW, J_, true>), grid, dim3(64 * KW), 0, s, p); \
+        else hipLaunchKernelGGL((gemv_tile4_kernel<FMT, XF32, KW, J_, false>), grid, dim3(64 * KW), 0, s, p);      \
         break;
     switch (jpw) {
         NQ_T4(1) NQ_T4(2) NQ_T4(3) NQ_T4(4) NQ_T4(5) NQ_T4(6) NQ_T4(7) NQ_T4(8)
@@ -425,9 +466,11 @@ int32_t launch4(const TileParams& p, hipStream_t s) {
 
 template <bool XF32, int KW>
 int32_t launch8_jpw(const TileParams& p, int jpw, dim3 grid, hipStream_t s) {
-#define NQ_T8(J_)                                                                                  \
-    case J_:                                                                                       \
-        hipLaunchKernelGGL((gemv_tile8_kernel<XF32, KW, J_>), grid, dim3(64 * KW), 0, s, p);       \
+    const bool exact = p.NJ == KW * jpw;
+#define NQ_T8(J_)                                                                                            \
+    case J_:                                                                                                 \
+        if (exact) hipLaunchKernelGGL((gemv_tile8_kernel<XF32, KW, J_, true>), grid, dim3(64 * KW), 0, s, p); \
+        else hipLaunchKernelGGL((gemv_tile8_kernel<XF32, KW, J_, false>), grid, dim3(64 * KW), 0, s, p);      \
         break;
     switch (jpw) {
         NQ_T8(1) NQ_T8(2) NQ_T8(3) NQ_T8(4) NQ_T8(5) NQ_T8(6) NQ_T8(7) NQ_T8(8)
@@ -454,6 +497,7 @@ int32_t launch8(const TileParams& p, hipStream_t s) {
 // groups of exactly 128, IN a multiple of 128 in 2048 .. 16384; int8: IN a multiple of 64, at least 1024.
 bool tile_copy_wanted(const nq_layer* L) {
     if (L->no_tile_copy) return false;
+    if ((int64_t)L->in * ((L->out + 15) / 16 * 16) >= ((int64_t)1 << 32)) return false;  // (32-bit offsets in a tile copy)
     if ((int64_t)L->in * L->out < ((int64_t)4 << 20)) return false;
     if (L->format == NQ_FMT_Q4_0 || (L->format == NQ_FMT_W4_GROUP && L->group == 128))
         return L->in % 128 == 0 && L->in >= 2048 && L->in <= 16384;
