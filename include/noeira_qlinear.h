@@ -259,6 +259,15 @@ int32_t nq_hessian_set(nq_hessian h, const double* h_host, int64_t count, int64_
  * (dense.mojo:229-236). */
 int32_t nq_hinv_upper_f64(const double* h_host, int32_t n, double* u_host, void* stream);
 
+/* nq_hinv_upper_f64 for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  h_dev and u_dev are [n, n] fp64
+ * on the device (h_dev is not modified), pivot_dev a device int32 that is set to INT32_MAX, or to the index of
+ * the first non-positive pivot (of the index-reversed matrix) when h is not positive definite, in which case
+ * u_dev holds no result.  The call only enqueues on `stream`: it allocates nothing, frees nothing and does not
+ * synchronise; its working copy of h lives in a fixed device array of the library, which limits n to 1024
+ * (NQ_ERR_SIZE beyond) and is shared by every call on the same GPU: calls that overlap on one GPU race. */
+int32_t nq_hinv_upper_f64_dev(const double* h_dev, int32_t n, double* u_dev, int32_t* pivot_dev, void* stream);
+
 /* `gptq_q4_0` (noeira/nn/quant/gptq.mojo:62-150) followed by `pack_q4_0` and the upload: quantizes
  * the host fp32 weight w [OUT, IN] of a Q4_0 layer column by column against the Hessian of the
  * layer's inputs (not modified), and loads the layer with the result, as nq_set_weight_f32 does

@@ -27,7 +27,7 @@ EXPORTS = [
     "nq_keep_only_repacked", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
     "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward", "nq_fuse_rows", "nq_fused_parts",
     "nq_forward_fused", "nq_hessian_create", "nq_hessian_destroy", "nq_hessian_add", "nq_hessian_rows",
-    "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_set_weight_gptq", "nq_q4_0_objective", "nq_lora_forward_add",
+    "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_hinv_upper_f64_dev", "nq_set_weight_gptq", "nq_q4_0_objective", "nq_lora_forward_add",
 ]
 
 
@@ -136,6 +136,8 @@ def lib() -> C.CDLL:
     L.nq_hessian_set.argtypes = [p, p, i64, i64]
     L.nq_hinv_upper_f64.restype = i32
     L.nq_hinv_upper_f64.argtypes = [p, i32, p, p]
+    L.nq_hinv_upper_f64_dev.restype = i32
+    L.nq_hinv_upper_f64_dev.argtypes = [p, i32, p, p, p]
     L.nq_set_weight_gptq.restype = i32
     L.nq_set_weight_gptq.argtypes = [p, p, i64, p, f64, C.POINTER(i64), C.POINTER(f64), p]
     L.nq_q4_0_objective.restype = i32

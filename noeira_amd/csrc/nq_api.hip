@@ -727,6 +727,18 @@ int32_t nq_hinv_upper_f64(const double* h_host, int32_t n, double* u_host, void*
     return NQ_OK;
 }
 
+int32_t nq_hinv_upper_f64_dev(const double* h_dev, int32_t n, double* u_dev, int32_t* pivot_dev, void* stream) {
+    if (!h_dev || !u_dev || !pivot_dev || n <= 0)
+        return fail(NQ_ERR_INVALID, "hinv_upper_f64_dev: null matrix, null pivot or n <= 0");
+    if (n > hinv_dev_max_n())
+        return fail(NQ_ERR_SIZE, "hinv_upper_f64_dev: n = " + std::to_string(n) + " exceeds the " +
+                                     std::to_string(hinv_dev_max_n()) + " the library's fixed scratch holds "
+                                     "(nq_hinv_upper_f64 takes any n)");
+    if (((uintptr_t)h_dev & 7) || ((uintptr_t)u_dev & 7) || ((uintptr_t)pivot_dev & 3))
+        return fail(NQ_ERR_INVALID, "hinv_upper_f64_dev: misaligned pointer");
+    return run_hinv_upper_f64_dev(h_dev, n, u_dev, pivot_dev, (hipStream_t)stream);
+}
+
 int32_t nq_set_weight_gptq(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess, double damp_frac,
                            int64_t* dead_out, double* damp_out, void* stream) {
     int32_t rc = check_handle(h, "nq_set_weight_gptq");

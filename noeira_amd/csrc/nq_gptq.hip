@@ -23,6 +23,8 @@
 // A CPU restatement that follows the same orders reproduces the codes bit for bit.
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "nq_common.h"
 
 namespace nq {
@@ -319,6 +321,51 @@ int32_t launch_hinv_upper_f64(double* h, int n, double* u, int* status_dev, hipS
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
+
+// ---------------------------------------------------------------------------
+// The same factorization for callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid it): device in, device out, the working copy of h in a file-scope device array
+// instead of a hipMalloc'd one.  Every call on a GPU shares that GPU's array: calls that overlap on one
+// GPU race.  Nothing of the array needs to start at zero (the copy of h overwrites all n * n values used).
+// ---------------------------------------------------------------------------
+constexpr int HINV_DEV_MAX_N = 1024;                                               // 8 MiB of fp64
+static __device__ __align__(256) double scratch[HINV_DEV_MAX_N * HINV_DEV_MAX_N];  // (host code: a stand-in, not an address)
+constexpr int MAX_DEVICES = 64;
+static double* g_scratch_ptr[MAX_DEVICES];  // the array's address on each device, looked up once per device
+static std::mutex g_scratch_mutex;
+
+// the device address of `scratch` on the current device
+static int32_t scratch_address(double** out) {
+    int dev = -1;
+    NQ_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(NQ_ERR_UNSUPPORTED, "hinv_upper_f64_dev: device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        double* ptr = nullptr;
+        NQ_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return NQ_OK;
+}
+
+__global__ __launch_bounds__(256) void copy_f64_kernel(const double* __restrict__ src, double* __restrict__ dst, int64_t count,
+                                                       int* __restrict__ pivot) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e == 0) *pivot = 0x7FFFFFFF;  // (a fill kernel, not a memset: a caller may capture this)
+    if (e < count) dst[e] = src[e];
+}
+
+int32_t run_hinv_upper_f64_dev(const double* h_dev, int n, double* u_dev, int* pivot_dev, hipStream_t s) {
+    double* work = nullptr;
+    int32_t rc = scratch_address(&work);
+    if (rc) return rc;
+    const int64_t nn = (int64_t)n * n;
+    hipLaunchKernelGGL(copy_f64_kernel, dim3(blocks_for(nn)), dim3(256), 0, s, h_dev, work, nn, pivot_dev);
+    return launch_hinv_upper_f64(work, n, u_dev, pivot_dev, s);
+}
+
+int32_t hinv_dev_max_n() { return HINV_DEV_MAX_N; }
 
 int32_t launch_hessian_add(double* H, int n, const void* x, int32_t x_dtype, int rows, hipStream_t s) {
     if (rows <= 0) return NQ_OK;

@@ -81,6 +81,21 @@ def hinv_upper_f64(h) -> np.ndarray:
     return u
 
 
+def hinv_upper_f64_dev(h: torch.Tensor, u: Optional[torch.Tensor] = None, pivot: Optional[torch.Tensor] = None):
+    """`hinv_upper_f64` without any allocation inside the library (nq_hinv_upper_f64_dev): `h`, `u` are [n, n] fp64
+    device tensors, `pivot` a device int32.  Only enqueues; returns (u, pivot).  n <= 1024; calls that overlap
+    on one GPU race (they share the library's fixed scratch)."""
+    if h.dtype != torch.float64 or not h.is_cuda or not h.is_contiguous() or h.dim() != 2 or h.shape[0] != h.shape[1]:
+        raise L.NQError(L.NQ_ERR_INVALID, "hinv_upper_f64_dev: h must be a contiguous [n, n] fp64 device tensor")
+    n = h.shape[0]
+    if u is None:
+        u = torch.empty_like(h)
+    if pivot is None:
+        pivot = torch.empty((1,), dtype=torch.int32, device=h.device)
+    L.check(L.lib().nq_hinv_upper_f64_dev(_dev_ptr(h), n, _dev_ptr(u), _dev_ptr(pivot), _stream_ptr()))
+    return u, pivot
+
+
 def set_weight_gptq(layer: QLinear, w, hess: HessianAccumulator, damp_frac: float = 0.01) -> GPTQStats:
     """Quantize the fp32 [OUT, IN] weight with GPTQ against `hess` and load the layer with it."""
     w = np.ascontiguousarray(w, dtype=np.float32)
