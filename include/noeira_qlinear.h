@@ -281,6 +281,18 @@ int32_t nq_set_weight_gptq(nq_handle h, const float* w_host, int64_t n_values, n
 int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess,
                           double* out, void* stream);
 
+/* ---- diagnostics ---------------------------------------------------------------------------- */
+
+/* What the matrix cores alone sustain on this GPU (no counterpart in the reference; bench.py reports it
+ * beside the 8-bit GEMM so that the GEMM's fraction of the published peak can be read against what the chip's
+ * power limit leaves): `workgroups` workgroups of four wavefronts issue 16 * iters MFMAs of 32 x 32 each, back
+ * to back, on register operands taken from `operands` (device, operand_bytes >= 4096; what the bytes are,
+ * constant or random codes, is the caller's choice).  kind 0: v_mfma_f32_32x32x64_f8f6f4 on e4m3 codes
+ * (131072 operations each), kind 1: v_mfma_i32_32x32x32_i8 (65536 each).  stamps: device int64
+ * [workgroups][2] = the loop's duration in shader clocks and in ticks of the constant 100 MHz clock. */
+int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_bytes, int32_t iters, int32_t workgroups,
+                          int64_t* stamps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

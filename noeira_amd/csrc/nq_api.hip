@@ -2,6 +2,7 @@
 // checking, the layer's storage, and dispatch to the kernels.  No C++
 // exception crosses the boundary and nothing here aborts; every failure is a
 // status code plus a sentence for nq_last_error().
+#include <algorithm>
 #include <cstring>
 #include <new>
 #include <string>
@@ -804,6 +805,18 @@ int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq
     (void)hipFree(wd), (void)hipFree(deq);
     if (e != hipSuccess) return fail_hip(e, "nq_q4_0_objective");
     return rc;
+}
+
+int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_bytes, int32_t iters, int32_t workgroups,
+                          int64_t* stamps, void* stream) {
+    if (kind != 0 && kind != 1) return fail(NQ_ERR_INVALID, "nq_diag_mfma_rate: kind must be 0 (fp8) or 1 (int8)");
+    if (!operands || operand_bytes < 4096 || ((uintptr_t)operands & 3))
+        return fail(NQ_ERR_INVALID, "nq_diag_mfma_rate: at least 4096 bytes of 4-byte aligned operands are needed");
+    if (iters <= 0 || workgroups <= 0 || !stamps)
+        return fail(NQ_ERR_INVALID, "nq_diag_mfma_rate: iters and workgroups must be positive, stamps not null");
+    // (the kernel's sink is never written: its condition cannot hold; stamps doubles as its address)
+    return launch_mfma_rate(kind, reinterpret_cast<const int*>(operands), (int)std::min<int64_t>(operand_bytes / 4, 1 << 24),
+                            iters, workgroups, stamps, reinterpret_cast<float*>(stamps), (hipStream_t)stream);
 }
 
 int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M, int32_t K,

@@ -26,6 +26,10 @@ int32_t fail_hip(hipError_t e, const char* what);
         if (_e != hipSuccess) return nq::fail_hip(_e, #expr); \
     } while (0)
 
+// nq_diag.hip: the matrix cores' own rate (a diagnostic)
+int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
+                         hipStream_t s);
+
 }  // namespace nq
 
 // One quantized linear layer.  Device layouts (all row-major over OUT):
@@ -178,5 +182,9 @@ int32_t run_gptq_q4_0(float* w_dev, int64_t n, int k, double* h_dev, double damp
                       double* stats_host, hipStream_t s);
 int32_t run_q4_0_objective(const float* w_dev, const float* deq_dev, int64_t n, int k, const double* h_dev,
                            double* out_host, hipStream_t s);
+
+// nq_diag.hip: the matrix cores' own rate (a diagnostic)
+int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
+                         hipStream_t s);
 
 }  // namespace nq

@@ -1,0 +1,72 @@
+// A diagnostic, not part of the forward path: what the matrix cores alone sustain on this GPU.
+// Every wavefront issues v_mfma back to back on register operands (no memory, no LDS in the loop), 16
+// independent accumulators of 32 x 32 as in the 8-bit GEMM's inner loop, one wavefront per SIMD and one
+// workgroup per CU.  The operands come from a caller's buffer, so the caller chooses what the multipliers
+// see (constant bytes, random e4m3 codes ...): on data that toggles them the chip runs at its power limit and
+// the clock, hence the rate, drops.  The kernel stamps the shader clock and the constant 100 MHz clock
+// around its loop, from which the effective shader clock follows.
+#include <type_traits>
+
+#include "nq_common.h"
+
+namespace nq {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(16))) int i32x16;
+
+// KIND 0: v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3), 1: v_mfma_i32_32x32x32_i8
+template <int KIND>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void mfma_rate_kernel(const int* __restrict__ seed, int seed_words, int iters, int64_t* __restrict__ stamps, float* sink) {
+    // four A fragments and four B fragments per wavefront, as one k-step of the GEMM's 4 x 4 register tile
+    i32x8 a[4], b[4];
+#pragma unroll
+    for (int o = 0; o < 4; o++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            a[o][i] = seed[(threadIdx.x * 8 + i + 2048 * o) % seed_words];
+            b[o][i] = seed[(threadIdx.x * 8 + i + 2048 * o + 1024) % seed_words];
+        }
+    typedef typename std::conditional<KIND == 0, f32x16, i32x16>::type acc_t;
+    acc_t acc[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0;
+    const int64_t c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            if constexpr (KIND == 0)
+                acc[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b[j % 4], a[j / 4], acc[j], 0, 0, 0, 0, 0, 0);
+            else
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8((i32x4){b[j % 4][0], b[j % 4][1], b[j % 4][2], b[j % 4][3]},
+                                                               (i32x4){a[j / 4][0], a[j / 4][1], a[j / 4][2], a[j / 4][3]},
+                                                               acc[j], 0, 0, 0);
+        }
+    }
+    const int64_t c1 = clock64(), w1 = wall_clock64();
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; j++) s += (float)acc[j][0];
+    if (s == 12345.678f) sink[0] = s;  // (keeps the accumulators alive)
+    if (threadIdx.x == 0) stamps[2 * blockIdx.x] = c1 - c0, stamps[2 * blockIdx.x + 1] = w1 - w0;
+}
+
+}  // namespace
+
+int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
+                         hipStream_t s) {
+    if (kind == 0)
+        hipLaunchKernelGGL(mfma_rate_kernel<0>, dim3(blocks), dim3(256), 0, s, seed, seed_words, iters, stamps, sink);
+    else
+        hipLaunchKernelGGL(mfma_rate_kernel<1>, dim3(blocks), dim3(256), 0, s, seed, seed_words, iters, stamps, sink);
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+}  // namespace nq
