@@ -68,6 +68,7 @@ class _Layer:
         L.check(L.lib().nq_create(C.byref(h), self.FORMAT, self.IN, self.OUT, self.group, flags))
         self._h = h
         self._loaded = False
+        self.bias: Optional[torch.Tensor] = None  # `Linear`'s fp32 [OUT] bias, set by from_linear
 
     def __del__(self):
         h = getattr(self, "_h", None)
@@ -78,10 +79,29 @@ class _Layer:
                 pass
             self._h = None
 
+    @staticmethod
+    def _linear_params(w_in_out, bias, IN: int, OUT: int, what: str):
+        """`Linear[IN, OUT]` keeps W as [IN, OUT] row-major fp32 and an fp32 [OUT] bias
+        (noeira/nn/primitives/linear.mojo:970-971): the opposite orientation from the [OUT, IN] this library (and
+        `QLinear`) holds, so a drop-in transposes at load, as the reference's own gates do
+        (tests/nn/quant/qlinear_common.mojo:86-91).  Returns (W^T [OUT, IN] contiguous fp32, device bias or None)."""
+        w = np.asarray(w_in_out, dtype=np.float32)
+        if w.shape != (IN, OUT):
+            raise L.NQError(L.NQ_ERR_SIZE, f"{what}: the weight is {list(w.shape)}, expected Linear's [IN, OUT] = [{IN}, {OUT}]")
+        b = None
+        if bias is not None:
+            bh = np.ascontiguousarray(bias, dtype=np.float32)
+            if bh.shape != (OUT,):
+                raise L.NQError(L.NQ_ERR_SIZE, f"{what}: the bias has {bh.size} values, expected OUT = {OUT}")
+            b = torch.from_numpy(bh).cuda()
+        return np.ascontiguousarray(w.T), b
+
     # shared by every format ------------------------------------------------
     def _forward(self, x: torch.Tensor, x_dtype: int, x_scale: Optional[torch.Tensor], out: Optional[torch.Tensor],
                  out_dtype: torch.dtype, bias: Optional[torch.Tensor], epilogue: str, what: str) -> torch.Tensor:
         M = _check_x(x, self.IN, what)
+        if bias is None:
+            bias = self.bias
         if out is None or out.numel() < M * self.OUT or out.dtype != out_dtype:
             out = torch.empty((M, self.OUT), dtype=out_dtype, device=x.device)
         y_dt = {torch.float32: L.DT_F32, torch.bfloat16: L.DT_BF16, torch.int32: L.DT_I32}[out_dtype]
@@ -135,6 +155,16 @@ class QLinear(_Layer):
         from an initializer (qlinear.mojo:253-260)."""
         _need_gpu(target)
         return cls(IN, OUT)
+
+    @classmethod
+    def from_linear(cls, w_in_out, bias=None, tile_copy: bool = True) -> "QLinear":
+        """A Q4_0 layer from `Linear[IN, OUT]`'s parameters: W [IN, OUT] is transposed to [OUT, IN] and quantized
+        by RTN (set_weight); the fp32 bias, if any, is kept on the device and added by forward."""
+        IN, OUT = np.asarray(w_in_out).shape
+        lin = cls(IN, OUT, tile_copy=tile_copy)
+        wt, lin.bias = cls._linear_params(w_in_out, bias, IN, OUT, "QLinear.from_linear")
+        lin.set_weight(wt)
+        return lin
 
     # ── weights ────────────────────────────────────────────────────────────
     def set_weight(self, w, target: str = "gpu", ctx=None):
@@ -217,6 +247,20 @@ class W8Linear(_Layer):
 
     FORMAT = L.FMT_W8_CHANNEL
 
+    @classmethod
+    def from_linear(cls, w_in_out, bias=None, tile_copy: bool = True) -> "W8Linear":
+        """A drop-in for `Linear[IN, OUT]` / `LinearAct`: W [IN, OUT] fp32 is transposed to [OUT, IN] and quantized
+        per output channel (symmetric int8, s = absmax / 127); the fp32 bias, if any, is kept on the device and
+        added by forward (pass epilogue="relu" for `LinearAct[..., ReLU]`)."""
+        from . import formats as F
+
+        IN, OUT = np.asarray(w_in_out).shape
+        lin = cls(IN, OUT, tile_copy=tile_copy)
+        wt, lin.bias = cls._linear_params(w_in_out, bias, IN, OUT, "W8Linear.from_linear")
+        q, s = F.quantize_w8_channel(wt)
+        lin.set_weight(q, s)
+        return lin
+
     def set_weight(self, w_i8, scales):
         w = np.ascontiguousarray(w_i8, dtype=np.int8)
         s = np.ascontiguousarray(scales, dtype=np.float32)
@@ -251,6 +295,20 @@ class W4GroupLinear(_Layer):
         super().__init__(IN, OUT, group, tile_copy)
         self.G = -(-IN // group)
 
+    @classmethod
+    def from_linear(cls, w_in_out, bias=None, group: int = 128, tile_copy: bool = True) -> "W4GroupLinear":
+        """`Linear[IN, OUT]`'s W [IN, OUT] transposed and quantized to asymmetric uint4, group-wise along IN
+        (min / max per group); the fp32 bias, if any, is kept on the device and added by forward."""
+        from . import formats as F
+
+        IN, OUT = np.asarray(w_in_out).shape
+        lin = cls(IN, OUT, group, tile_copy=tile_copy)
+        wt, lin.bias = cls._linear_params(w_in_out, bias, IN, OUT, "W4GroupLinear.from_linear")
+        q, s, z = F.quantize_w4g_asym(wt, group)
+        codes, zps = F.pack_w4g(q, z)
+        lin.set_weight(codes, s, zps)
+        return lin
+
     def set_weight(self, codes, scales_f16, zps):
         c = np.ascontiguousarray(codes, dtype=np.uint8)
         s = np.ascontiguousarray(scales_f16)
@@ -275,6 +333,20 @@ class FP8Linear(_Layer):
     one fp32 scale (or fp32/bf16); fp32 accumulation; bf16 or fp32 output."""
 
     FORMAT = L.FMT_FP8_E4M3
+
+    @classmethod
+    def from_linear(cls, w_in_out, bias=None) -> "FP8Linear":
+        """`Linear[IN, OUT]`'s W [IN, OUT] transposed and encoded as e4m3fn under one scale (absmax / 448); the
+        fp32 bias, if any, is kept on the device and added by forward."""
+        from . import formats as F
+
+        IN, OUT = np.asarray(w_in_out).shape
+        lin = cls(IN, OUT)
+        wt, lin.bias = cls._linear_params(w_in_out, bias, IN, OUT, "FP8Linear.from_linear")
+        amax = float(np.abs(wt).max())
+        scale = amax / 448.0 if amax > 0 else 1.0
+        lin.set_weight(F.encode_e4m3(wt / np.float32(scale)), scale)
+        return lin
 
     def set_weight(self, w_codes, scale: float):
         w = np.ascontiguousarray(w_codes, dtype=np.uint8)

@@ -69,7 +69,6 @@ def test_random_shapes(seed):
             blocks[:, :, 0] = sc & 0xFF
             blocks[:, :, 1] = sc >> 8
             lin.set_blocks(blocks.reshape(-1))
-            use_bias, epi, odt = 0, "none", torch.float32
         elif fmt in ("w8", "w8a8"):
             K = _pick_k(rng, 128 if (fmt == "w8a8" and rng.integers(0, 2)) else 16)
             lin = W8Linear(K, N)
@@ -103,9 +102,7 @@ def test_random_shapes(seed):
                 e = e + bias.double()
             return e.clamp_min(0) if epi == "relu" else e
 
-        if fmt == "q4_0":
-            _check(tag, lin.forward(x), x.double() @ deq.T, False)
-        elif fmt in ("w8", "w4g"):
+        if fmt in ("q4_0", "w8", "w4g"):
             y = lin.forward(x, bias=bias, epilogue=epi, out_dtype=odt)
             _check(tag, y, fin(x.double() @ deq.T), odt == torch.bfloat16)
         elif fmt == "fp8":
@@ -157,13 +154,10 @@ def test_many_rows(fmt, xdt):
         deq = lin.dequantized_dev().double()
         x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
         tag = "%s M=%d K=%d N=%d %s" % (fmt, M, K, N, str(xdt)[6:])
-        if fmt == "q4_0":
-            _check(tag, lin.forward(x), x.double() @ deq.T, False)
-        else:
-            bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
-            y = lin.forward(x, bias=bias, epilogue="relu", out_dtype=torch.bfloat16)
-            _check(tag, y, (x.double() @ deq.T + bias.double()).clamp_min(0), True)
-            _check(tag, lin.forward(x), x.double() @ deq.T, False)
+        bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+        y = lin.forward(x, bias=bias, epilogue="relu", out_dtype=torch.bfloat16)
+        _check(tag, y, (x.double() @ deq.T + bias.double()).clamp_min(0), True)
+        _check(tag, lin.forward(x), x.double() @ deq.T, False)
         del lin
 
 

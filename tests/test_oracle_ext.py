@@ -217,3 +217,28 @@ def test_three_term_int8_split_zero_and_tiny():
     for x in (np.zeros(64, np.float32), np.full(64, 1e-38, np.float32)):
         s, q1, q2, q3 = _split3(x, False)
         assert s == 0 and not q1.any() and not q2.any() and not q3.any()
+
+
+def test_w8_qlinear_forward_cpu_is_dequantize_then_the_serial_loop():
+    """The function bench.py times as the CPU baseline: a fresh dequantise (float(code) * scale) into an fp32
+    [OUT, IN] scratch, then the reference's serial triple loop (cpu_gemm.mojo:88-98), then the bias."""
+    rng = np.random.default_rng(12)
+    N, K, M = 37, 96, 3
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    y = O.w8_qlinear_forward_cpu(w, s, x, b)
+    deq = w.astype(np.float32) * s[:, None]
+    want = np.empty((M, N), np.float32)
+    for m in range(M):
+        for n in range(N):
+            acc = np.float32(0)
+            for k in range(K):  # k ascending, one fp32 accumulator, multiply and add rounded separately or fused
+                acc = np.float32(acc + np.float32(x[m, k] * deq[n, k]))
+            want[m, n] = np.float32(acc + b[n])
+    exact = x.astype(np.float64) @ deq.astype(np.float64).T + b
+    assert np.abs(y - exact).max() <= 1e-5 * np.abs(exact).max()
+    # the serial order itself: equal to the loop above unless the C compiler fused multiply and add (then within an ulp or two)
+    assert np.abs(y - want).max() <= 4e-7 * np.abs(exact).max()
+    assert np.array_equal(O.w8_qlinear_forward_cpu(w, s, x), O.w8_qlinear_forward_cpu(w, s, x, np.zeros(N, np.float32)))

@@ -96,6 +96,10 @@ def test_gptq_parity_with_reference_fixture(fix, case):
     assert rel < 0.01, rel
     assert rows_same.sum() * 10 >= n * 9, (int(rows_same.sum()), n)
     assert scale_bad == 0
+    # this restatement follows the reference's order of operations, so it does better than that gate: every
+    # code and every scale of the fixture, bit for bit
+    assert np.array_equal(q, c["q"]), int((q != c["q"]).sum())
+    assert np.array_equal(d.view(np.uint32), c["d"].view(np.uint32))
 
 
 # ── [2] a diagonal Hessian propagates nothing: GPTQ is RTN, bit for bit (test_gptq.mojo:90-113)
