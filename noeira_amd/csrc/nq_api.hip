@@ -18,6 +18,17 @@ int32_t fail(int32_t code, const std::string& msg) {
     return code;
 }
 
+hipError_t set_max_lds_once(LdsAttrOnce& st, const void* kernel, size_t bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (tracked && st.done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess && tracked) st.done[dev] = true;
+    return e;
+}
+
 int32_t fail_hip(hipError_t e, const char* what) {
     g_last_error = std::string("HIP error ") + hipGetErrorName(e) + " (" + hipGetErrorString(e) + ") in " + what;
     return NQ_ERR_HIP;
@@ -614,6 +625,9 @@ int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features,
     if (T < 0) return fail(NQ_ERR_INVALID, "LoRAAdapter.forward_add: T must be >= 0");
     if (T == 0) return NQ_OK;
     if (!a || !b || !x || !y) return fail(NQ_ERR_INVALID, "LoRAAdapter.forward_add: null pointer");
+    if ((int64_t)T * in_features >= ((int64_t)1 << 32) || (int64_t)T * out_features >= ((int64_t)1 << 32))
+        return fail(NQ_ERR_UNSUPPORTED, "LoRAAdapter.forward_add: T * IN and T * OUT must stay below 2^32 (the kernel "
+                                        "addresses x and y with 32-bit element offsets)");
     return launch_lora_add(x, x_dtype, a, b, y, T, in_features, out_features, r_pad, scale, (hipStream_t)stream);
 }
 
@@ -624,7 +638,17 @@ struct nq_hessian_s {
     int64_t rows = 0;
     int device = -1;
     double* d_h = nullptr;
+    hipStream_t last_stream = nullptr;  // the stream of the last nq_hessian_add: a reader on another stream waits for it
+    bool pending = false;
 };
+
+// a call that reads H on `s` after nq_hessian_add enqueued on another stream waits for that stream first
+static hipError_t hessian_order(nq_hessian h, hipStream_t s) {
+    if (!h->pending || h->last_stream == s) return hipSuccess;
+    const hipError_t e = hipStreamSynchronize(h->last_stream);
+    if (e == hipSuccess) h->pending = false;
+    return e;
+}
 
 static int32_t check_hessian(nq_hessian h, const char* what) {
     if (!h || h->magic != 0x4E514853u) return fail(NQ_ERR_INVALID, std::string(what) + ": not a Hessian handle");
@@ -672,8 +696,9 @@ int32_t nq_hessian_add(nq_hessian h, const void* x, int32_t x_dtype, int32_t row
     if (rows < 0) return fail(NQ_ERR_INVALID, "HessianAccumulator.add: rows must be >= 0");
     if (rows == 0) return NQ_OK;
     if (!x) return fail(NQ_ERR_INVALID, "HessianAccumulator.add: null slab");
+    NQ_HIP(hessian_order(h, (hipStream_t)stream));  // (adds on two streams: the second waits for the first)
     rc = launch_hessian_add(h->d_h, h->n, x, x_dtype, rows, (hipStream_t)stream);
-    if (rc == NQ_OK) h->rows += rows;
+    if (rc == NQ_OK) h->rows += rows, h->last_stream = (hipStream_t)stream, h->pending = true;
     return rc;
 }
 
@@ -686,6 +711,7 @@ int32_t nq_hessian_get(nq_hessian h, double* out_host, int64_t count) {
         return fail(NQ_ERR_SIZE, "nq_hessian_get: the buffer must hold n * n = " +
                                      std::to_string((int64_t)h->n * h->n) + " values");
     NQ_HIP(hipDeviceSynchronize());
+    h->pending = false;
     NQ_HIP(hipMemcpy(out_host, h->d_h, (size_t)count * 8, hipMemcpyDeviceToHost));
     return NQ_OK;
 }
@@ -697,6 +723,7 @@ int32_t nq_hessian_set(nq_hessian h, const double* h_host, int64_t count, int64_
         return fail(NQ_ERR_SIZE, "nq_hessian_set: expected n * n = " + std::to_string((int64_t)h->n * h->n) +
                                      " values");
     NQ_HIP(hipDeviceSynchronize());
+    h->pending = false;
     NQ_HIP(hipMemcpy(h->d_h, h_host, (size_t)count * 8, hipMemcpyHostToDevice));
     h->rows = rows;
     return NQ_OK;
@@ -762,7 +789,8 @@ int32_t nq_set_weight_gptq(nq_handle h, const float* w_host, int64_t n_values, n
     float* wd = nullptr;
     uint8_t* raw = nullptr;
     double* hd = nullptr;
-    hipError_t e = hipMalloc((void**)&wd, (size_t)want * 4);
+    hipError_t e = hessian_order(hess, s);
+    if (e == hipSuccess) e = hipMalloc((void**)&wd, (size_t)want * 4);
     if (e == hipSuccess) e = hipMalloc((void**)&raw, (size_t)nbytes + 16);
     if (e == hipSuccess) e = hipMalloc((void**)&hd, hbytes);
     double stats[2] = {0, 0};
@@ -797,7 +825,8 @@ int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq
         return fail(NQ_ERR_SIZE, "q4_0_objective: w must hold [OUT, IN] values and h be [IN, IN]");
     hipStream_t s = (hipStream_t)stream;
     float *wd = nullptr, *deq = nullptr;
-    hipError_t e = hipMalloc((void**)&wd, (size_t)want * 4);
+    hipError_t e = hessian_order(hess, s);
+    if (e == hipSuccess) e = hipMalloc((void**)&wd, (size_t)want * 4);
     if (e == hipSuccess) e = hipMalloc((void**)&deq, (size_t)want * 4);
     if (e == hipSuccess) e = hipMemcpyAsync(wd, w_host, (size_t)want * 4, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) rc = launch_dequantize(h, deq, s);

@@ -30,6 +30,12 @@ int32_t fail_hip(hipError_t e, const char* what);
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
                          hipStream_t s);
 
+// hipFuncAttributeMaxDynamicSharedMemorySize is a per-device setting of a kernel: set once per (kernel, device)
+struct LdsAttrOnce {
+    bool done[64] = {};
+};
+hipError_t set_max_lds_once(LdsAttrOnce& st, const void* kernel, size_t bytes);
+
 }  // namespace nq
 
 // One quantized linear layer.  Device layouts (all row-major over OUT):

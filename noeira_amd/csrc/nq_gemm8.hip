@@ -424,7 +424,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     const int lm = lane & 31, lh = lane >> 5;
     // whole 16-byte stores wherever the tile's columns all exist and rows of y stay 16-byte aligned
     // (a tile that only M cuts short just skips the rows past M)
-    const bool full_cols = (n0 + BN <= p.N) && (p.N % 8 == 0);
+    const bool full_cols = (n0 + BN <= p.N) && (p.N % 8 == 0) && (((uintptr_t)p.y & 15) == 0);
 
     // channel scale and bias for the lane's channels of tile j, group g (needs n < N: clamped)
     auto chan = [&](int j, int g, float (&cs)[4], float (&cb)[4], bool need_scale, int zero) {
@@ -588,13 +588,9 @@ void gemm8_kernel(const Gemm8Params p) {
 }
 
 template <typename K>
-int32_t launch_cfg(K kernel, bool* attr_set, const Gemm8Params& p, int bn, int bk, hipStream_t s) {
+int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int bn, int bk, hipStream_t s) {
     const size_t lds = (size_t)2 * (BM + bn) * bk;
-    if (!*attr_set) {
-        NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)lds));
-        *attr_set = true;
-    }
+    NQ_HIP(set_max_lds_once(*attr, reinterpret_cast<const void*>(kernel), lds));
     hipLaunchKernelGGL(kernel, dim3(p.tiles_m * p.tiles_n), dim3(256), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
@@ -625,7 +621,7 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     const bool i8 = a.x_dtype == NQ_DT_I8;
     p.chan_vec = L->out % 4 == 0 && L->out >= 4 && (!i8 || a.y_dtype == NQ_DT_I32 || (uintptr_t)p.col_scale % 16 == 0) &&
                  (!a.bias || (uintptr_t)a.bias % (a.bias_dtype == NQ_DT_F32 ? 16 : 8) == 0);
-    static bool attr_set[5] = {false, false, false, false, false};
+    static LdsAttrOnce attr_set[5];
     const bool f32 = a.y_dtype == NQ_DT_F32;
     if (a.x_dtype == NQ_DT_FP8_E4M3)
         return f32 ? launch_cfg(gemm8_kernel<true, 0>, &attr_set[0], p, 256, 128, a.stream)

@@ -894,12 +894,8 @@ int32_t launch_big(const A16Params& p, int mt, int nw, hipStream_t s) {
 #define NQ_BIG_CASE(MT_, NW_)                                                                     \
     if (mt == MT_ && nw == NW_) {                                                                 \
         auto kernel = gemm_a16_big_kernel<FMT, XF32, MT_, NW_, WHOLE>;                            \
-        static bool attr = false;                                                                 \
-        if (lds > 48 * 1024 && !attr) {                                                           \
-            NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                     \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));    \
-            attr = true;                                                                          \
-        }                                                                                         \
+        static LdsAttrOnce attr;                                                                  \
+        if (lds > 48 * 1024) NQ_HIP(set_max_lds_once(attr, reinterpret_cast<const void*>(kernel), lds)); \
         hipLaunchKernelGGL(kernel, grid, dim3(128 * (8 / NW_)), lds, s, p);                       \
         NQ_HIP(hipGetLastError());                                                                \
         return NQ_OK;                                                                             \

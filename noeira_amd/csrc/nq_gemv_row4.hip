@@ -279,12 +279,8 @@ int32_t launch_one(const Row4Params& p, hipStream_t s) {
     constexpr int NT = XF32 ? 3 : 1;
     constexpr size_t lds = (size_t)NT * CPL * 2048 * 2 + (size_t)CPL * 64 * 4;
     auto kernel = gemv_row4_kernel<FMT, XF32, CPL, WAVES, RPW>;
-    static bool attr_set = false;
-    if (lds > 48 * 1024 && !attr_set) {
-        NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)lds));
-        attr_set = true;
-    }
+    static LdsAttrOnce attr;
+    if (lds > 48 * 1024) NQ_HIP(set_max_lds_once(attr, reinterpret_cast<const void*>(kernel), lds));
     const int rows_per_wg = WAVES * RPW;
     hipLaunchKernelGGL(kernel, dim3((unsigned)((p.N + rows_per_wg - 1) / rows_per_wg)), dim3(64 * WAVES), lds, s, p);
     NQ_HIP(hipGetLastError());

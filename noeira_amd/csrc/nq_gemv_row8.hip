@@ -142,12 +142,8 @@ int32_t launch_one(const Row8Params& p, hipStream_t s) {
     constexpr int WAVES = 16;  // 10.6 us against 11.4 with 8 and 12.7 with 4 (4096 -> 11008): x is staged once for 16 rows
     constexpr size_t lds = (size_t)CPL * 1024 * 4;
     auto kernel = gemv_row8_kernel<FMT, XF32, CPL, WAVES>;
-    static bool attr_set = false;
-    if (lds > 48 * 1024 && !attr_set) {
-        NQ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)lds));
-        attr_set = true;
-    }
+    static LdsAttrOnce attr;
+    if (lds > 48 * 1024) NQ_HIP(set_max_lds_once(attr, reinterpret_cast<const void*>(kernel), lds));
     hipLaunchKernelGGL(kernel, dim3((unsigned)((p.N + WAVES - 1) / WAVES)), dim3(64 * WAVES), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;

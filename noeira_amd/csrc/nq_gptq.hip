@@ -603,12 +603,8 @@ int32_t run_gptq_q4_0(float* w_dev, int64_t n, int k, double* h_dev, double damp
                                       " of the reversed matrix)");
     if (e == hipSuccess && rc == NQ_OK) {
         const size_t lds = (size_t)(GPTQ_BLOCK * GPTQ_BLOCK + ROWS_PER_WG * GPTQ_BLOCK) * 4;
-        static bool attr_set = false;
-        if (!attr_set) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(gptq_rows_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            attr_set = e == hipSuccess;
-        }
+        static LdsAttrOnce attr;
+        e = set_max_lds_once(attr, reinterpret_cast<const void*>(gptq_rows_kernel), lds);
         if (e == hipSuccess) {
             hipLaunchKernelGGL(gptq_rows_kernel, dim3(blocks_for(n, ROWS_PER_WG)), dim3(64 * ROWS_PER_WG), lds, s,
                                w_dev, (int)n, k, u, q, d);
