@@ -462,6 +462,26 @@ def mfma_only(iters=4096, reps=5):
     return out
 
 
+def make_read(nbytes, copies):
+    """The floor of a weight-streaming call: nq_diag_stream_read over `nbytes` (a kernel that only reads, with
+    1 KiB loads), rotating over `copies` distinct regions so that every call streams from HBM."""
+    import ctypes as C
+
+    import torch
+
+    from noeira_amd import _lib as L
+
+    stride = (nbytes + 4095) // 4096 * 4096
+    buf = torch.full((stride * copies,), 0x5A, dtype=torch.uint8, device="cuda")
+    lib = L.lib()
+
+    def step(i):
+        L.check(lib.nq_diag_stream_read(C.c_void_p(buf.data_ptr() + (i % copies) * stride), nbytes,
+                                        C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+    return dict(step=step, bytes=nbytes, ops=0, launches=1, keep=(buf,))
+
+
 def report(name, wl, seconds, bound, peak_key=None):
     gbps = wl["bytes"] / seconds / 1e9
     tops = wl["ops"] / seconds / 1e12
@@ -541,6 +561,11 @@ def sweep(skip_large=False):
         run("ref Q4_0 g32 4096->11008 M=1 fp32 (cold)", make_q4_0, "hbm", IN=4096, OUT=11008, M=1, copies=c, calls=c)
         run("W8A16 4096->11008 M=1 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, copies=max(1, c // 2),
             calls=max(1, c // 2))
+        # what a kernel that only reads those weights takes (launch + stream): the floor of the rows above
+        for mb, nb in (("16.8 MB", 4096 * 4096), ("23.2 MB", 4096 * 11008 // 2 + 2 * 32 * 11008 + 16 * 11008),
+                       ("45.1 MB", 4096 * 11008)):
+            cr = max(1, COLD_BYTES // nb)
+            run(f"floor: plain read of {mb}, no arithmetic (cold)", make_read, "hbm", nbytes=nb, copies=cr, calls=cr)
         # the same kernels where the stream is long enough for the fixed part of a call (launch, first trip to
         # memory, the last wavefronts) to vanish: 8192 -> 28672, 235 MB of 8-bit codes / 117 - 132 MB of 4-bit ones
         KB, NB = 8192, 28672

@@ -293,6 +293,12 @@ int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq
 int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_bytes, int32_t iters, int32_t workgroups,
                           int64_t* stamps, void* stream);
 
+/* The floor of a weight-streaming call (no counterpart in the reference): a kernel that only reads the first
+ * nbytes / 1024 KiB of `src` (device, 16-byte aligned) with 1 KiB load instructions and computes nothing.
+ * bench.py times it on the bytes of each large GEMV's weight: launch + stream, what no GEMV over those bytes
+ * can beat on this GPU. */
+int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

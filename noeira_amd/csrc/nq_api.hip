@@ -848,6 +848,12 @@ int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_by
                             iters, workgroups, stamps, reinterpret_cast<float*>(stamps), (hipStream_t)stream);
 }
 
+int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream) {
+    if (!src || nbytes < 1024 || ((uintptr_t)src & 15))
+        return fail(NQ_ERR_INVALID, "nq_diag_stream_read: at least 1 KiB at a 16-byte aligned device address is needed");
+    return launch_stream_read(src, nbytes / 1024, (hipStream_t)stream);
+}
+
 int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M, int32_t K,
                             void* stream) {
     if (M < 0 || K <= 0 || K % 4 != 0)

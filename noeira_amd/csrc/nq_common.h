@@ -27,6 +27,7 @@ int32_t fail_hip(hipError_t e, const char* what);
     } while (0)
 
 // nq_diag.hip: the matrix cores' own rate (a diagnostic)
+int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s);
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
                          hipStream_t s);
 
@@ -190,6 +191,7 @@ int32_t run_q4_0_objective(const float* w_dev, const float* deq_dev, int64_t n, 
                            double* out_host, hipStream_t s);
 
 // nq_diag.hip: the matrix cores' own rate (a diagnostic)
+int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s);
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
                          hipStream_t s);
 

@@ -57,7 +57,30 @@ void mfma_rate_kernel(const int* __restrict__ seed, int seed_words, int iters, i
     if (threadIdx.x == 0) stamps[2 * blockIdx.x] = c1 - c0, stamps[2 * blockIdx.x + 1] = w1 - w0;
 }
 
+// A second yardstick: a kernel that only READS `kib` KiB (one 1 KiB load instruction per wavefront and KiB, four
+// in flight per wavefront, eight wavefronts per workgroup) and computes nothing.  What it takes for the bytes
+// of a GEMV's weight is the floor of that GEMV on this GPU: launch + the stream.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+__global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restrict__ src, int64_t kib, uint32_t* sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t b0 = ((int64_t)blockIdx.x * 8 + wave) * 4;
+    u32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = __builtin_nontemporal_load(src + min(b0 + j, kib - 1) * 64 + lane);
+    uint32_t x = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) x ^= v[j][0] ^ v[j][1] ^ v[j][2] ^ v[j][3];
+    if (x == 0x9E3779B9u && lane == 77) sink[0] = x;  // (never true: lane < 64)
+}
+
 }  // namespace
+
+int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s) {
+    hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)((kib + 31) / 32)), dim3(512), 0, s,
+                       reinterpret_cast<const u32x4*>(src), kib, (uint32_t*)nullptr);
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
 
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
                          hipStream_t s) {
