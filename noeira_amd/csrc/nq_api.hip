@@ -405,6 +405,7 @@ int32_t dispatch(const ForwardArgs& a) {
     }
     if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
+    if (gemv_tile_rows_applicable(a)) return launch_gemv_tile_rows(a);
     if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
     if (gemv_tile_applicable(a)) return launch_gemv_tile(a);
     if (gemv_split8_applicable(a)) return launch_gemv_split8(a);
@@ -418,7 +419,7 @@ int32_t dispatch(const ForwardArgs& a) {
 bool places_parts(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_I8) return false;
     if (gemv_fp8_applicable(a) || gemm8_applicable(a)) return false;
-    return gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
+    return gemv_tile_rows_applicable(a) || gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
 }
 
 // argument checks shared by nq_forward and nq_forward_fused, then the launch(es)

@@ -150,6 +150,8 @@ int32_t launch_gemv_split8(const ForwardArgs& a);
 bool tile_copy_wanted(const nq_layer* L);
 int32_t build_tile_copy(nq_layer* L, hipStream_t s);
 bool gemv_tile_applicable(const ForwardArgs& a);
+bool gemv_tile_rows_applicable(const ForwardArgs& a);
+int32_t launch_gemv_tile_rows(const ForwardArgs& a);
 int32_t launch_gemv_tile(const ForwardArgs& a);
 
 // nq_gemv_fp8.hip: fp8 x fp8 and int8 x int8 on the matrix cores for one row (fp8) and for as many

@@ -263,6 +263,191 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
     finish_rows<KW>(p, red, R, tail);
 }
 
+
+// ---- a few activation rows (2 <= M <= 16) over 4-bit codes ---------------------------------------------
+// The tile of 16 weight rows is the same; the A operand now holds real rows: bf16 x row i is A row i
+// (M <= 16), fp32 x row i is A rows 3 i, 3 i + 1, 3 i + 2 (its three bf16 terms; M <= 5).  One workgroup of 16
+// wavefronts per CU visits tiles blockIdx.x, blockIdx.x + gridDim.x, ...; wavefront w takes the same steps
+// 16-byte pieces of K in every tile, so its A operands are fetched from memory once, straight into registers (a
+// lane's 16 bytes of row lane % 16), and stay there, and so do the zero-point terms: the sum of x under a
+// chunk, per row, comes out of the matrix core in the product's own register layout when the B operand is all
+// ones (Q4_0: times -24 and used as the product MFMA's C operand; groups of 128: times -(16 + z) first).  The
+// next tile's codes are requested before the current tile is multiplied.  The 16 wavefronts' [16 x 16] shares
+// meet in LDS in wave order (two buffers, one barrier per tile); thread (row, column) adds bias and epilogue.
+struct TileMrParams {
+    TileParams t;
+    int32_t M;
+};
+
+template <int FMT, bool XF32, int JPW>
+__global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParams pm) {
+    const TileParams& p = pm.t;
+    constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
+    constexpr int KW = 16;
+    constexpr int NT = XF32 ? 3 : 1;
+    constexpr bool XS_REGS = G128 || JPW <= 2;  // Q4_0 keeps 4 JPW row-sum tiles: beyond 2 steps they no longer fit
+    __shared__ __attribute__((aligned(16))) float red[2][KW][256];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const int ntiles = (p.N + 15) / 16;
+    const int J0 = wave * JPW;
+    const int vrow = c / NT, vterm = c % NT;   // this lane's A row: activation row and term
+    const int xrow = min(vrow, pm.M - 1);
+    uint32_t magic = 0x41804180u;
+    asm volatile("" : "+v"(magic));
+
+    auto fetch = [&](int tile, u32x4 (&wv)[JPW], uint2 (&sc)[JPW]) {
+        const int64_t R = min(tile, ntiles - 1);
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const int64_t at = R * p.NJ + min(J0 + j, p.NJ - 1);
+            wv[j] = __builtin_nontemporal_load(p.tile + at * 64 + lane);
+            if constexpr (!G128) sc[j] = reinterpret_cast<const uint2*>(p.tscales)[at * 16 + c];
+            else sc[j].x = reinterpret_cast<const uint32_t*>(p.tscales)[at * 16 + c], sc[j].y = 0;
+        }
+    };
+    u32x4 wv[JPW], wn[JPW];
+    uint2 sc[JPW], sn[JPW];
+    fetch(blockIdx.x, wv, sc);
+
+    // ---- A operands, once: 16 bytes of bf16 per (step, MFMA); rows past M and steps past K are zero
+    u32x4 aop[JPW][4];
+#pragma unroll
+    for (int j = 0; j < JPW; j++)
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int k = min((J0 + j) * 128 + 32 * m + 8 * q, p.K - 8);
+            u32x4 t;
+            if constexpr (XF32) {
+                const float* xf = reinterpret_cast<const float*>(p.x) + (int64_t)xrow * p.K + k;
+                const u32x4 r0 = *reinterpret_cast<const u32x4*>(xf), r1 = *reinterpret_cast<const u32x4*>(xf + 4);
+                uint32_t v[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = r0[i], v[4 + i] = r1[i];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    // hi + mid + lo = the fp32 value (each split truncates: every residual is exact); this lane keeps one
+                    const uint32_t a = v[2 * i], b = v[2 * i + 1];
+                    const float ra = __uint_as_float(a) - __uint_as_float(a & 0xFFFF0000u);
+                    const float rb = __uint_as_float(b) - __uint_as_float(b & 0xFFFF0000u);
+                    const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                    const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                    const uint32_t ta = vterm == 0 ? a : vterm == 1 ? __float_as_uint(ra) : __float_as_uint(sa);
+                    const uint32_t tb = vterm == 0 ? b : vterm == 1 ? __float_as_uint(rb) : __float_as_uint(sb);
+                    t[i] = __builtin_amdgcn_perm(tb, ta, 0x07060302u);
+                }
+            } else {
+                t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + (int64_t)xrow * p.K + k);
+            }
+            const uint32_t keep = (vrow < pm.M && J0 + j < p.NJ) ? ~0u : 0u;
+#pragma unroll
+            for (int i = 0; i < 4; i++) t[i] &= keep;
+            aop[j][m] = t;
+        }
+    // ---- the rows' sums of x under every chunk (Q4_0, times -24) or group of 128, in the product's layout
+    const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4 xs[XS_REGS ? JPW : 1][G128 ? 1 : 4];
+    if constexpr (XS_REGS) {
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            if constexpr (G128) {
+                xs[j][0] = zero4;
+#pragma unroll
+                for (int m = 0; m < 4; m++)
+                    xs[j][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[j][m]), as_bf16x8(ones), xs[j][0], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    xs[j][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[j][m]), as_bf16x8(ones), zero4, 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) xs[j][m][t] *= -24.0f;
+                }
+            }
+        }
+    }
+    // the epilogue's operands of this thread's column (threads 0 .. 255 finish a tile: row = thread / 16)
+    const int fr = threadIdx.x >> 4, fc = threadIdx.x & 15;
+
+    int buf = 0;
+    for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x, buf ^= 1) {
+        fetch(tile + gridDim.x, wn, sn);  // the next tile's codes are on their way while this one is multiplied
+        uint32_t braw = 0;
+        const int64_t fn = min((int64_t)tile * 16 + fc, (int64_t)p.N - 1);
+        if (p.bias && threadIdx.x < 256)
+            braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[fn]
+                                               : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[fn];
+        f32x4 acc = zero4;
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const bool live = J0 + j < p.NJ;  // (a step past K: its A operand is zero; its scale is set to zero too)
+            if constexpr (!G128) {
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    const u32x4 bop = nib_word_to_bf16(wv[j][m], magic);
+                    f32x4 cin;
+                    if constexpr (XS_REGS) {
+                        cin = xs[j][m];
+                    } else {
+                        cin = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[j][m]), as_bf16x8(ones), zero4, 0, 0, 0);
+#pragma unroll
+                        for (int t = 0; t < 4; t++) cin[t] *= -24.0f;
+                    }
+                    const f32x4 dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[j][m]), as_bf16x8(bop), cin, 0, 0, 0);
+                    const uint32_t sbits = (m < 2 ? sc[j].x : sc[j].y) >> (16 * (m & 1));
+                    const float d = live ? __half2float(__ushort_as_half((uint16_t)(sbits & 0xFFFFu))) : 0.0f;
+#pragma unroll
+                    for (int t = 0; t < 4; t++) acc[t] = fmaf(d, dd[t], acc[t]);
+                }
+            } else {
+                const float d = live ? __half2float(__ushort_as_half((uint16_t)(sc[j].x & 0xFFFFu))) : 0.0f;
+                const float zoff = -(16.0f + (float)(sc[j].x >> 16));
+                f32x4 dd;
+#pragma unroll
+                for (int t = 0; t < 4; t++) dd[t] = zoff * xs[j][0][t];
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    const u32x4 bop = nib_word_to_bf16(wv[j][m], magic);
+                    dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[j][m]), as_bf16x8(bop), dd, 0, 0, 0);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; t++) acc[t] = fmaf(d, dd[t], acc[t]);
+            }
+        }
+        *reinterpret_cast<f32x4*>(&red[buf][wave][lane * 4]) = acc;
+        __syncthreads();
+        // D[v][cc] sits in lane cc + 16 (v / 4), register v % 4.  Thread (row fr, column fc) sums its row's terms'
+        // shares, each over the wavefronts in wave order.
+        if (threadIdx.x < 256 && fr < pm.M && (!XF32 || fr < 5)) {
+            float z = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int v = NT * fr + t;
+                const int at = (fc + 16 * (v >> 2)) * 4 + (v & 3);
+                float zt = red[buf][0][at];
+#pragma unroll
+                for (int w = 1; w < KW; w++) zt += red[buf][w][at];
+                z = t == 0 ? zt : z + zt;
+            }
+            const int64_t n = (int64_t)tile * 16 + fc;
+            if (n < p.N) {
+                if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
+                if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                void* yp;
+                int width, col;
+                seg_lookup(p.seg, (int)n, yp, width, col);
+                const int64_t o = (int64_t)fr * width + col;
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(yp)[o] = z;
+                else
+                    reinterpret_cast<uint16_t*>(yp)[o] = f32_to_bf16_rne(z);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < JPW; j++) wv[j] = wn[j], sc[j] = sn[j];
+    }
+}
+
 // ---- int8 codes -----------------------------------------------------------------------------------
 constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: the low byte of (t + MAGIC)'s bits is rne(t) as an int8
 
@@ -490,6 +675,24 @@ int32_t launch8(const TileParams& p, hipStream_t s) {
     return kw == 8 ? launch8_jpw<XF32, 8>(p, jpw, grid, s) : launch8_jpw<XF32, 16>(p, jpw, grid, s);
 }
 
+template <int FMT, bool XF32>
+int32_t launch4_rows(const TileMrParams& pm, hipStream_t s) {
+    const int jpw = (pm.t.NJ + 15) / 16;
+    int dev = 0, cus = 0;
+    NQ_HIP(hipGetDevice(&dev));
+    NQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int ntiles = (pm.t.N + 15) / 16;
+    const dim3 grid((unsigned)std::min(ntiles, std::max(cus, 1)));
+    switch (jpw) {
+        case 1: hipLaunchKernelGGL((gemv_tile4_rows_kernel<FMT, XF32, 1>), grid, dim3(1024), 0, s, pm); break;
+        case 2: hipLaunchKernelGGL((gemv_tile4_rows_kernel<FMT, XF32, 2>), grid, dim3(1024), 0, s, pm); break;
+        case 3: hipLaunchKernelGGL((gemv_tile4_rows_kernel<FMT, XF32, 3>), grid, dim3(1024), 0, s, pm); break;
+        default: return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no tile kernel for this IN");
+    }
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
 }  // namespace
 
 // Which layers get the tile-ordered copy (a second copy of the codes: 0.5 or 1 byte per weight on top):
@@ -539,6 +742,33 @@ bool gemv_tile_applicable(const ForwardArgs& a) {
     if (a.M != 1 || !L->d_tile16) return false;
     if (a.x_dtype != NQ_DT_BF16 && a.x_dtype != NQ_DT_F32) return false;
     return a.y_dtype == NQ_DT_F32 || a.y_dtype == NQ_DT_BF16;
+}
+
+// 2 .. 16 rows of bf16 activations, 2 .. 5 of fp32, over a 4-bit layer that keeps its tile copy, K <= 6144 (a
+// wavefront's A operands for up to three steps of K fit its registers beside the codes of two tiles; with four
+// the kernel spills)
+bool gemv_tile_rows_applicable(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (!L->d_tile16 || L->format == NQ_FMT_W8_CHANNEL || L->tile_nj > 48) return false;
+    if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
+    if (a.x_dtype == NQ_DT_BF16) return a.M >= 2 && a.M <= 16;
+    if (a.x_dtype == NQ_DT_F32) return a.M >= 2 && a.M <= 5;
+    return false;
+}
+
+int32_t launch_gemv_tile_rows(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    TileMrParams pm{};
+    TileParams& p = pm.t;
+    p.tile = reinterpret_cast<const u32x4*>(L->d_tile16), p.tscales = L->d_tile16_scales, p.col_scale = nullptr;
+    p.x = a.x, p.bias = a.bias, p.seg = a.seg;
+    p.N = L->out, p.K = L->in, p.NJ = L->tile_nj;
+    p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    pm.M = a.M;
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
+    if (L->format == NQ_FMT_Q4_0)
+        return xf32 ? launch4_rows<NQ_FMT_Q4_0, true>(pm, a.stream) : launch4_rows<NQ_FMT_Q4_0, false>(pm, a.stream);
+    return xf32 ? launch4_rows<NQ_FMT_W4_GROUP, true>(pm, a.stream) : launch4_rows<NQ_FMT_W4_GROUP, false>(pm, a.stream);
 }
 
 int32_t launch_gemv_tile(const ForwardArgs& a) {

@@ -1,0 +1,102 @@
+"""A few activation rows (2 .. 16) over a large 4-bit weight: the persistent tile kernel of nq_gemv_tile.hip
+(bf16 rows as the matrix core's A rows, fp32 rows as three A rows each), through the C ABI, against fp64 products of
+the layer's dequantised weights (pinned bit for bit against the oracle elsewhere) and against the oracle's own
+forward at a size it finishes in seconds.  Bars: 1e-5 of the largest reference value (the reference's fp32 band,
+tests/nn/quant/qlinear_common.mojo:39-45); repeated calls return the same bits."""
+import numpy as np
+import pytest
+import torch
+
+from noeira_amd import formats as F
+from noeira_amd.qlinear import FusedRows, QLinear, W4GroupLinear
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def q4_layer(rng, K, N, tile_copy=True):
+    lin = QLinear(K, N, tile_copy=tile_copy)
+    blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+    sc = (rng.uniform(1e-3, 1e-2, (N, K // 32)) * rng.choice([-1.0, 1.0], (N, K // 32))).astype(np.float16).view(np.uint16)
+    blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+    lin.set_blocks(blocks.reshape(-1))
+    return lin
+
+
+def w4g_layer(rng, K, N, tile_copy=True):
+    G = K // 128
+    codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
+    lin = W4GroupLinear(K, N, 128, tile_copy=tile_copy)
+    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+    return lin
+
+
+# K = 2048 (one step per wavefront), 2176 (17 steps: a ragged second step), 4096 (two), 5504 (43 steps: three, ragged),
+# 6144 (the most the kernel holds); N off the tile size; fewer tiles than CUs and several tiles per workgroup
+SHAPES = [(2048, 2051), (2176, 1999), (4096, 1100), (4096, 11008), (5504, 800), (6144, 700)]
+
+
+@pytest.mark.parametrize("K,N", SHAPES)
+@pytest.mark.parametrize("fmt", ["q4_0", "w4g"])
+@pytest.mark.parametrize("xdt,M", [(torch.bfloat16, 2), (torch.bfloat16, 7), (torch.bfloat16, 16), (torch.float32, 2),
+                                   (torch.float32, 5)])
+def test_few_rows_over_tile_copy(K, N, fmt, xdt, M):
+    rng = np.random.default_rng(K + N + M + len(fmt))
+    lin = q4_layer(rng, K, N) if fmt == "q4_0" else w4g_layer(rng, K, N)
+    deq = lin.dequantized_dev().double()
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    y = lin.forward(x, bias=bias)
+    exact = x.double() @ deq.T + bias.double()
+    assert y.shape == (M, N)
+    assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
+    assert torch.equal(lin.forward(x, bias=bias), y)
+    yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16)
+    want = (x.double() @ deq.T + bias.to(torch.bfloat16).double()).clamp_min(0)
+    rms = float(exact.pow(2).mean().sqrt())
+    assert float((yr.double() - want).abs().max()) <= 1e-3 * rms + 2.0 ** -8 * float(want.abs().max())
+
+
+def test_few_rows_against_oracle_forward():
+    rng = np.random.default_rng(17)
+    K, N, M = 4096, 1024, 5
+    lin = q4_layer(rng, K, N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    y = lin.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    assert O.rel_max(y, O.qlinear_forward_cpu(lin.blocks(), K, N, x)) < 1e-5
+
+
+def test_few_rows_agree_with_the_row_ordered_kernels_and_with_one_row():
+    rng = np.random.default_rng(19)
+    K, N, M = 4096, 2048, 4
+    a, b = q4_layer(np.random.default_rng(3), K, N), q4_layer(np.random.default_rng(3), K, N, tile_copy=False)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    ya, yb = a.forward(x), b.forward(x)
+    assert float((ya - yb).abs().max()) <= 2e-6 * float(yb.abs().max())
+    for m in range(M):  # a row of the batch against the same row alone (another kernel: same products, another order)
+        y1 = a.forward(x[m:m + 1].contiguous())
+        assert float((ya[m] - y1[0]).abs().max()) <= 2e-6 * float(y1.abs().max())
+
+
+def test_few_rows_fused_parts():
+    rng = np.random.default_rng(23)
+    K = 4096
+    parts = [q4_layer(rng, K, n) for n in (1024, 256, 260)]
+    fused = FusedRows(parts)
+    x = torch.from_numpy(rng.standard_normal((3, K)).astype(np.float32)).cuda()
+    for lin, y in zip(parts, fused.forward(x)):
+        want = lin.forward(x)
+        assert y.shape == want.shape
+        assert float((y - want).abs().max()) <= 2e-6 * float(want.abs().max())
+
+
+def test_few_rows_nonfinite_stay_in_their_row():
+    rng = np.random.default_rng(29)
+    K, N, M = 4096, 1040, 6
+    lin = w4g_layer(rng, K, N)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    x[2, 100] = float("nan")
+    x[4, 7] = float("inf")
+    y = lin.forward(x)
+    assert bool(torch.isnan(y[2]).all()) and not bool(torch.isnan(y[[0, 1, 3, 5]]).any())
+    assert not bool(torch.isfinite(y[4]).any())
