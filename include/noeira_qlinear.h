@@ -75,6 +75,7 @@ extern "C" {
 /* epilogues (LinearAct's, noeira/nn/primitives/linear_act.mojo:81-115) */
 #define NQ_EPI_NONE 0
 #define NQ_EPI_RELU 1     /* z > 0 ? z : 0  (ops/relu_op.mojo:29-31) */
+#define NQ_EPI_SWIGLU 2   /* layers made by nq_fuse_glu only: up * silu(gate)  (primitives/swiglu.mojo:41-60) */
 
 typedef struct nq_layer* nq_handle;
 
@@ -168,6 +169,15 @@ int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_s
  * is an ordinary layer (nq_forward writes one [M, sum OUT] y) that also
  * remembers its parts for nq_forward_fused. */
 int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* stream);
+
+/* gate | up of a decoder MLP and the SwiGLU between them and `down`, as ONE layer: the reference's caller runs
+ * two projections, a concatenation and `SwiGLU.forward` (noeira/deep_agents/smolvla/fused.mojo:337-353:
+ * `proj_fwd[LORA_GATE]`, `proj_fwd[LORA_UP]`, `glu_cat`, `glu`; out = up * silu(gate), silu(v) = v / (1 + exp(-v)),
+ * noeira/nn/primitives/swiglu.mojo:41-60).  The two loaded layers (same format, IN, OUT, group width; Q4_0,
+ * W4_GROUP or W8_CHANNEL) are copied on the device with their rows interleaved, so the sources may be destroyed.
+ * The result runs with nq_forward(..., epilogue = NQ_EPI_SWIGLU) only and writes y[M, OUT]: x fp32 or bf16,
+ * y fp32 or bf16, no bias; one launch for M = 1 and for M >= 2.  nq_get_blocks and nq_fuse_rows refuse it. */
+int32_t nq_fuse_glu(nq_handle* out, nq_handle gate, nq_handle up, void* stream);
 
 /* Number of parts of a layer made by nq_fuse_rows (1 for any other layer). */
 int32_t nq_fused_parts(nq_handle h);

@@ -17,7 +17,7 @@ LIB_NAME = "libnoeira_qlinear.so"
 NQ_OK, NQ_ERR_INVALID, NQ_ERR_NOT_LOADED, NQ_ERR_NO_BLOCKS, NQ_ERR_SIZE, NQ_ERR_HIP, NQ_ERR_UNSUPPORTED = range(7)
 FMT_Q4_0, FMT_W8_CHANNEL, FMT_W4_GROUP, FMT_FP8_E4M3 = range(4)
 DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
-EPI_NONE, EPI_RELU = 0, 1
+EPI_NONE, EPI_RELU, EPI_SWIGLU = 0, 1, 2
 ABI_VERSION = 4
 FLAG_NO_TILE_COPY = 1
 
@@ -26,7 +26,7 @@ EXPORTS = [
     "nq_set_weight_i8", "nq_set_weight_w4g", "nq_set_weight_fp8", "nq_blocks_bytes", "nq_get_blocks",
     "nq_keep_only_repacked", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
     "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward", "nq_fuse_rows", "nq_fused_parts",
-    "nq_forward_fused", "nq_hessian_create", "nq_hessian_destroy", "nq_hessian_add", "nq_hessian_rows",
+    "nq_forward_fused", "nq_fuse_glu", "nq_hessian_create", "nq_hessian_destroy", "nq_hessian_add", "nq_hessian_rows",
     "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_hinv_upper_f64_dev", "nq_set_weight_gptq", "nq_q4_0_objective", "nq_lora_forward_add", "nq_diag_mfma_rate", "nq_diag_stream_read",
 ]
 
@@ -117,6 +117,8 @@ def lib() -> C.CDLL:
     L.nq_mlp3_w8a8_forward.argtypes = [p, p, p, p, p, i32, p, p, p, i32, p]
     L.nq_fuse_rows.restype = i32
     L.nq_fuse_rows.argtypes = [C.POINTER(p), C.POINTER(p), i32, p]
+    L.nq_fuse_glu.restype = i32
+    L.nq_fuse_glu.argtypes = [C.POINTER(p), p, p, p]
     L.nq_fused_parts.restype = i32
     L.nq_fused_parts.argtypes = [p]
     L.nq_forward_fused.restype = i32

@@ -398,6 +398,14 @@ void row_view(const nq_layer* L, int r0, int r1, nq_layer* v) {
 }
 
 int32_t dispatch(const ForwardArgs& a) {
+    if (a.L->glu) {
+        // gate | up pairs meet in the epilogue of the kernels whose result layout keeps a pair in one wavefront
+        if (a.M == 1 && gemv_m1_applicable(a)) return launch_gemv_m1(a);
+        if (a.M >= 2 && gemm_a16_applicable(a)) return launch_gemm_a16(a);
+        return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no SwiGLU kernel for this shape (IN = " + std::to_string(a.L->in) +
+                                            ", M = " + std::to_string(a.M) + "): run gate | up with nq_forward_fused "
+                                            "and apply SwiGLU separately");
+    }
     if (a.x_dtype == NQ_DT_I8) {
         if (tile8_i8_applicable(a)) return launch_tile8_i8(a);
         if (gemm8_applicable(a)) return launch_gemm8(a);
@@ -430,8 +438,13 @@ int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x
     for (int t = 0; t < seg.nseg; t++)
         if (!seg.y[t] || ((uintptr_t)seg.y[t] & 3))
             return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
-    if (epilogue != NQ_EPI_NONE && epilogue != NQ_EPI_RELU)
+    if (epilogue != NQ_EPI_NONE && epilogue != NQ_EPI_RELU && epilogue != NQ_EPI_SWIGLU)
         return fail(NQ_ERR_INVALID, "nq_forward: unknown epilogue " + std::to_string(epilogue));
+    if (h->glu != (epilogue == NQ_EPI_SWIGLU))
+        return fail(NQ_ERR_INVALID, h->glu ? "nq_forward: a layer made by nq_fuse_glu runs with NQ_EPI_SWIGLU only"
+                                           : "nq_forward: NQ_EPI_SWIGLU needs a layer made by nq_fuse_glu");
+    if (h->glu && (bias || (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16) || seg.nseg != 1))
+        return fail(NQ_ERR_INVALID, "nq_forward: a SwiGLU layer takes fp32 or bf16 activations, no bias, one output");
     if (bias && bias_dtype != NQ_DT_F32 && bias_dtype != NQ_DT_BF16)
         return fail(NQ_ERR_INVALID, "nq_forward: bias must be fp32 or bf16");
     if (x_dtype == NQ_DT_I8) {
@@ -505,7 +518,7 @@ int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* s
             return fail(NQ_ERR_INVALID, "nq_fuse_rows: the layers must share format, IN, group width and device");
         if (a->format == NQ_FMT_FP8_E4M3 && b->scale != a->scale)
             return fail(NQ_ERR_INVALID, "nq_fuse_rows: FP8_E4M3 layers must share their per-tensor scale");
-        if (!b->seg_end.empty()) return fail(NQ_ERR_INVALID, "nq_fuse_rows: a fused layer cannot be fused again");
+        if (!b->seg_end.empty() || b->glu) return fail(NQ_ERR_INVALID, "nq_fuse_rows: a fused layer cannot be fused again");
         rows += b->out;
     }
     if (rows > INT32_MAX) return fail(NQ_ERR_INVALID, "nq_fuse_rows: too many rows");
@@ -560,6 +573,68 @@ int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* s
         for (int i = 0; i < n; i++)
             F->host_blocks.insert(F->host_blocks.end(), layers[i]->host_blocks.begin(), layers[i]->host_blocks.end());
         F->has_host_blocks = true;
+    }
+    F->loaded = true;
+    *out = F;
+    return NQ_OK;
+}
+
+int32_t nq_fuse_glu(nq_handle* out, nq_handle gate, nq_handle up, void* stream) {
+    if (!out) return fail(NQ_ERR_INVALID, "nq_fuse_glu: null output handle");
+    *out = nullptr;
+    nq_handle both[2] = {gate, up};
+    for (int i = 0; i < 2; i++) {
+        int32_t rc = check_handle(both[i], "nq_fuse_glu");
+        if (rc) return rc;
+        if ((rc = need_loaded(both[i], "fuse_glu"))) return rc;
+        if (!both[i]->seg_end.empty() || both[i]->glu)
+            return fail(NQ_ERR_INVALID, "nq_fuse_glu: a fused layer cannot be fused again");
+    }
+    const nq_layer* a = gate;
+    const nq_layer* b = up;
+    if (a->format == NQ_FMT_FP8_E4M3)
+        return fail(NQ_ERR_UNSUPPORTED, "nq_fuse_glu: Q4_0, W4_GROUP and W8_CHANNEL layers only");
+    if (b->format != a->format || b->in != a->in || b->out != a->out || b->group != a->group || b->device != a->device)
+        return fail(NQ_ERR_INVALID, "nq_fuse_glu: gate and up must share format, IN, OUT, group width and device");
+    if ((int64_t)a->out * 2 > INT32_MAX) return fail(NQ_ERR_INVALID, "nq_fuse_glu: too many rows");
+    nq_layer* F = new (std::nothrow) nq_layer();
+    if (!F) return fail(NQ_ERR_INVALID, "nq_fuse_glu: out of host memory");
+    F->format = a->format, F->in = a->in, F->out = 2 * a->out, F->group = a->group, F->groups = a->groups;
+    F->scale = a->scale, F->row_bytes = a->row_bytes, F->device = a->device;
+    F->glu = true, F->no_tile_copy = true;  // (the tile kernels keep a pair in two workgroups)
+    int32_t rc = bind_device(F);
+    if (rc) {
+        delete F;
+        return rc;
+    }
+    int64_t scale_row = 0;
+    switch (a->format) {
+        case NQ_FMT_Q4_0: scale_row = (int64_t)(a->in / Q4_GROUP) * 2; break;
+        case NQ_FMT_W4_GROUP: scale_row = (int64_t)a->groups * 2; break;
+        default: scale_row = 4;  // W8_CHANNEL
+    }
+    const int64_t rows = F->out, H = a->out;
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e = hipMalloc((void**)&F->d_codes, (size_t)(rows * F->row_bytes) + 128);
+    if (e == hipSuccess) e = hipMalloc(&F->d_scales, (size_t)(rows * scale_row) + 128);
+    if (e == hipSuccess && a->d_zps) e = hipMalloc((void**)&F->d_zps, (size_t)(rows * F->groups) + 128);
+    // row 2 n <- gate row n, row 2 n + 1 <- up row n: strided device copies, one per array and source
+    for (int i = 0; i < 2 && e == hipSuccess; i++) {
+        const nq_layer* src = both[i];
+        e = hipMemcpy2DAsync(F->d_codes + i * F->row_bytes, (size_t)(2 * F->row_bytes), src->d_codes, (size_t)F->row_bytes,
+                             (size_t)F->row_bytes, (size_t)H, hipMemcpyDeviceToDevice, s);
+        if (e == hipSuccess)
+            e = hipMemcpy2DAsync(reinterpret_cast<uint8_t*>(F->d_scales) + i * scale_row, (size_t)(2 * scale_row),
+                                 src->d_scales, (size_t)scale_row, (size_t)scale_row, (size_t)H, hipMemcpyDeviceToDevice, s);
+        if (e == hipSuccess && a->d_zps)
+            e = hipMemcpy2DAsync(F->d_zps + i * F->groups, (size_t)(2 * F->groups), src->d_zps, (size_t)F->groups,
+                                 (size_t)F->groups, (size_t)H, hipMemcpyDeviceToDevice, s);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e != hipSuccess) {
+        free_device(F);
+        delete F;
+        return fail_hip(e, "nq_fuse_glu");
     }
     F->loaded = true;
     *out = F;

@@ -72,6 +72,9 @@ struct nq_layer {
     float scale = 1.0f;
     int64_t row_bytes = 0;     // bytes of one row of d_codes
     std::vector<int32_t> seg_end;  // a row-fused layer: the end row of each fused part (else empty)
+    // nq_fuse_glu: rows 2 n and 2 n + 1 are row n of the gate and of the up projection; the forward writes
+    // [M, OUT / 2] = up * silu(gate) (epilogue NQ_EPI_SWIGLU) and nothing else
+    bool glu = false;
 };
 
 namespace nq {
@@ -83,6 +86,19 @@ struct SegTable {
     int32_t end[4];
     void* y[4];
 };
+
+// `SwiGLU`'s forward as the reference writes it (noeira/nn/primitives/swiglu.mojo:41-60): s = 1 / (1 + exp(-v)),
+// out = u * (v * s), with u the up projection and v the gate, in fp32.
+__device__ __forceinline__ float swiglu_f32(float up, float gate) {
+    const float sg = 1.0f / (1.0f + expf(-gate));
+    return up * (gate * sg);
+}
+
+// the value the neighbouring lane (lane ^ 1) holds: in the matrix core's result layout adjacent lanes are adjacent
+// output columns, i.e. the gate and the up row of one pair
+__device__ __forceinline__ float lane_xor1(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false));
+}
 
 // row n -> (part's y, its width, the column in it).  Every table entry is read with a constant index, so the
 // table stays in scalar registers (a run-time index would turn into a load from the argument buffer, a round

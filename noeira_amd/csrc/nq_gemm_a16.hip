@@ -548,6 +548,19 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         if (FMT == NQ_FMT_W8_CHANNEL) z *= ep_scale[t];
         z += p.bias_dtype == NQ_DT_F32 ? __uint_as_float(ep_bias[t]) : __uint_as_float(ep_bias[t] << 16);
         if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+        if (p.epilogue == NQ_EPI_SWIGLU) {
+            // (uniform) even columns are gate rows, the odd column next to each its up row, one lane over
+            const float other = lane_xor1(z);
+            if ((n & 1) == 0 && n + 1 < p.N && m < p.M) {
+                const float g = swiglu_f32(other, z);
+                const int64_t o = (int64_t)m * (p.N >> 1) + (n >> 1);
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(p.y)[o] = g;
+                else
+                    reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(g);
+            }
+            continue;
+        }
         if (n < p.N && m < p.M) {
             void* yp;
             int width, col;
@@ -874,6 +887,18 @@ __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16P
                 if constexpr (!FOUR_BIT) z = fmaf(-128.0f, xacc[i][r], z) * cscale;
                 z += cbias;
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                if (p.epilogue == NQ_EPI_SWIGLU) {  // (uniform) gate in the even column, up one lane over
+                    const float other = lane_xor1(z);
+                    if ((n & 1) == 0 && n + 1 < p.N && m < p.M) {
+                        const float g = swiglu_f32(other, z);
+                        const int64_t o = (int64_t)m * (p.N >> 1) + (n >> 1);
+                        if (p.y_dtype == NQ_DT_F32)
+                            reinterpret_cast<float*>(p.y)[o] = g;
+                        else
+                            reinterpret_cast<uint16_t*>(p.y)[o] = f32_to_bf16_rne(g);
+                    }
+                    continue;
+                }
                 if (n < p.N && m < p.M) {
                     const int64_t o = (int64_t)m * width + col;
                     if (p.y_dtype == NQ_DT_F32)

@@ -321,6 +321,31 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
 #pragma unroll
         for (int r = 0; r < RPL; r++) acc[r] = group_sum(acc[r], lpr);
 
+        if (p.epilogue == NQ_EPI_SWIGLU) {
+            // (uniform) rows 2 n and 2 n + 1 are the gate and the up row of output n: adjacent lane groups
+            // (every lane of a group holds its row's sum), or adjacent wavefronts when a row takes all 64 lanes
+            float z = acc[0];
+            if (FMT == NQ_FMT_W8_CHANNEL) z *= rs[0];
+            if (FMT == NQ_FMT_FP8_E4M3) z *= tscale;
+            float other;
+            if (lpr < 64) {
+                other = __shfl_xor(z, lpr);
+            } else {
+                __shared__ float pair[4];
+                if (lane == 0) pair[wave] = z;
+                __syncthreads();
+                other = pair[wave ^ 1];
+            }
+            const int64_t n = row0;
+            if (lj == 0 && (n & 1) == 0 && n + 1 < p.N) {
+                const float g = swiglu_f32(other, z);
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(p.y)[n >> 1] = g;
+                else
+                    reinterpret_cast<uint16_t*>(p.y)[n >> 1] = to_bf16(g);
+            }
+            continue;  // (one row per lane group in every launch: the loop runs once)
+        }
         if (lj == 0) {
 #pragma unroll
             for (int r = 0; r < RPL; r++) {

@@ -423,6 +423,40 @@ class FusedRows:
         return outs
 
 
+class FusedGLU:
+    """gate | up of a decoder MLP with the SwiGLU between them and `down` in ONE launch (nq_fuse_glu): the
+    reference's caller runs two projections, a concatenation and `SwiGLU.forward`
+    (noeira/deep_agents/smolvla/fused.mojo:337-353).  `forward` returns up(x) * silu(gate(x)) as [M, OUT];
+    with bf16 in and `out_dtype=torch.bfloat16` nothing of the MLP's first half leaves the GPU's registers in
+    fp32 (the bf16 flow the reference lists as unbuilt, peft-quant.mdx:215-216)."""
+
+    def __init__(self, gate, up):
+        h = C.c_void_p()
+        L.check(L.lib().nq_fuse_glu(C.byref(h), gate._h, up._h, _stream_ptr()))
+        self._h = h
+        self.IN, self.OUT = gate.IN, gate.OUT
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h is not None and h.value:
+            try:
+                L.lib().nq_destroy(h)
+            except Exception:
+                pass
+            self._h = None
+
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        if x.dtype not in _TORCH_DT or out_dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "FusedGLU.forward: x and y must be fp32 or bf16")
+        M = _check_x(x, self.IN, "FusedGLU.forward")
+        if out is None or out.numel() < M * self.OUT or out.dtype != out_dtype:
+            out = torch.empty((M, self.OUT), dtype=out_dtype, device=x.device)
+        L.check(L.lib().nq_forward(self._h, _dev_ptr(x), _TORCH_DT[x.dtype], C.c_void_p(0), _dev_ptr(out),
+                                   _TORCH_DT[out_dtype], M, C.c_void_p(0), L.DT_F32, L.EPI_SWIGLU, _stream_ptr()))
+        return out
+
+
 def quantize_rows_i8(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None):
     """Per-token absmax int8 quantisation on the device: (q int8 [M, K], s fp32 [M])."""
     if x.dtype not in _TORCH_DT or x.dim() != 2 or not x.is_contiguous():

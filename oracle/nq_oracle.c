@@ -13,6 +13,7 @@
  *     noeira/nn/core/cpu_gemm.mojo:88  the Linux CPU GEMM (a triple loop)
  *     noeira/nn/quant/qlinear.mojo:416 QLinear.forward["cpu"] and vjp["cpu"]
  *     noeira/nn/peft/lora.mojo:292     LoRAAdapter.forward_add["cpu"]
+ *     noeira/nn/primitives/swiglu.mojo SwiGLU.forward["cpu"] (the caller's step between gate | up and down)
  *     noeira/nn/quant/gptq.mojo,       GPTQ onto the Q4_0 grid, the factor of H^-1 it
  *       dense.mojo, hessian.mojo       reads, the calibration Hessian (load time)
  * and is pinned by the reference's own golden vectors
@@ -353,6 +354,16 @@ int nqo_lora_forward_add(const float* x, const float* a, const float* b, int64_t
     nqo_gemm_cpu(0, 0, T, out, r, s, h, r, b, out, 1.0f, y, out);
     free(h);
     return NQO_OK;
+}
+
+/* swiglu.mojo:120-141 (`SwiGLU.forward["cpu"]`; the GPU kernel :41-60 is the same expression): the input row is
+ * [u | v] (2 * hidden wide), s = 1 / (1 + exp(-v)), out = u * (v * s), all in fp32.  The SmolVLA caller feeds it
+ * (up, gate) (fused.mojo:343-350), so out = up * silu(gate).  Here u and v come as two [rows, hidden] arrays. */
+void nqo_swiglu(const float* u, const float* v, int64_t count, float* out) {
+    for (int64_t i = 0; i < count; i++) {
+        float s = 1.0f / (1.0f + expf(-v[i]));
+        out[i] = u[i] * (v[i] * s);
+    }
 }
 
 /* ------------------------------------------------------------------------ */

@@ -107,6 +107,8 @@ def lib() -> C.CDLL:
             getattr(L, name).argtypes = [p, i64, p]
         L.nqo_lora_forward_add.restype = C.c_int
         L.nqo_lora_forward_add.argtypes = [p, p, p, i64, i64, i64, i64, f32, p]
+        L.nqo_swiglu.restype = None
+        L.nqo_swiglu.argtypes = [p, p, i64, p]
         L.nqo_cholesky_f64.restype = i64
         L.nqo_cholesky_f64.argtypes = [p, i64]
         L.nqo_tri_inv_lower_f64.restype = None
@@ -230,6 +232,14 @@ def lora_forward_add(x, a, b, s, y):
 
 
 # ── GPTQ (gptq.mojo, dense.mojo, hessian.mojo) ─────────────────────────────
+def swiglu(u, v):
+    """`SwiGLU.forward` on (u, v) of equal shape: u * (v / (1 + exp(-v))) in fp32 (swiglu.mojo:120-141)."""
+    u, v = _c(u, np.float32), _c(v, np.float32)
+    out = np.empty_like(u)
+    lib().nqo_swiglu(_ptr(u), _ptr(v), u.size, _ptr(out))
+    return out
+
+
 def cholesky_f64(a):
     """L (lower, L L^T = a); raises at a non-positive pivot like dense.mojo:229-236."""
     a = np.array(a, dtype=np.float64, order="C")

@@ -242,3 +242,22 @@ def test_w8_qlinear_forward_cpu_is_dequantize_then_the_serial_loop():
     # the serial order itself: equal to the loop above unless the C compiler fused multiply and add (then within an ulp or two)
     assert np.abs(y - want).max() <= 4e-7 * np.abs(exact).max()
     assert np.array_equal(O.w8_qlinear_forward_cpu(w, s, x), O.w8_qlinear_forward_cpu(w, s, x, np.zeros(N, np.float32)))
+
+
+def test_swiglu_is_u_times_v_sigmoid_v():
+    """Pinned by the closed form in fp64 and by the values that tell a wrong variant apart: silu(0) = 0,
+    silu(v) -> v for large v, -> 0 for very negative v, (u, v) not interchangeable."""
+    rng = np.random.default_rng(4)
+    u = rng.standard_normal(4000).astype(np.float32) * 3
+    v = rng.standard_normal(4000).astype(np.float32) * 4
+    got = O.swiglu(u, v)
+    want = u.astype(np.float64) * v.astype(np.float64) / (1.0 + np.exp(-v.astype(np.float64)))
+    assert np.abs(got - want).max() <= 4e-7 * np.abs(want).max()
+    assert np.abs(got - want).max() > 0  # fp32 arithmetic, not the fp64 formula retyped
+    assert np.array_equal(O.swiglu(np.float32([2, 2, 2, -3]), np.float32([0, 100, -100, 1])),
+                          np.float32([0, 200, -0.0, -3 * 0.7310585786]).astype(np.float32))
+    assert not np.allclose(O.swiglu(u, v), O.swiglu(v, u))
+    # the reference's grouping: u * (v * s), not (u * v) * s (they differ in the last bit now and then)
+    s32 = np.float32(1) / (np.float32(1) + np.exp(-v).astype(np.float32))
+    regroup = (u * v) * s32
+    assert np.abs(got - regroup).max() <= 2e-7 * np.abs(want).max()
