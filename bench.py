@@ -213,12 +213,13 @@ def make_q4_0(IN, OUT, M, copies, seed=3, bf16_x=False):
                 keep=(layers, x, y))
 
 
-def make_q4_0_fused(IN, OUTS, M, copies, seed=7, bf16_x=False):
-    """The reference caller's q|k|v or gate|up projections as one row-fused launch."""
+def make_q4_0_fused(IN, OUTS, M, copies, seed=7, bf16_x=False, glu=False, bf16_y=False):
+    """The reference caller's q|k|v or gate|up projections as one row-fused launch; with `glu` the SwiGLU between
+    gate | up and `down` (fused.mojo:337-353) runs in that launch's epilogue and one [M, H] tensor comes out."""
     import numpy as np
     import torch
 
-    from noeira_amd.qlinear import FusedRows, QLinear
+    from noeira_amd.qlinear import FusedGLU, FusedRows, QLinear
 
     rng = np.random.default_rng(seed)
     fused = []
@@ -232,18 +233,30 @@ def make_q4_0_fused(IN, OUTS, M, copies, seed=7, bf16_x=False):
             ql = QLinear.make(IN, OUT, "gpu")
             ql.set_blocks(blocks)
             parts.append(ql)
-        fused.append(FusedRows(parts))  # the parts are copied; they are freed here
+        fused.append(FusedGLU(*parts) if glu else FusedRows(parts))  # the parts are copied; they are freed here
     x = torch.from_numpy(rng.standard_normal((M, IN)).astype(np.float32)).cuda()
     if bf16_x:
         x = x.to(torch.bfloat16)
-    ys = [torch.empty((M, OUT), dtype=torch.float32, device="cuda") for OUT in OUTS]
     tot = sum(OUTS)
+    ydt = torch.bfloat16 if bf16_y else torch.float32
+    if glu:
+        yg = torch.empty((M, OUTS[0]), dtype=ydt, device="cuda")
+        ybytes = yg.element_size() * OUTS[0] * M
 
-    def step(i):
-        fused[i % copies].forward(x, outs=ys)
+        def step(i):
+            fused[i % copies].forward(x, out=yg)
 
-    return dict(step=step, bytes=tot * (IN // 32) * 18 + (2 if bf16_x else 4) * IN * M + 4 * tot * M, ops=2 * M * IN * tot, launches=1,
-                keep=(fused, x, ys))
+        keep = (fused, x, yg)
+    else:
+        ys = [torch.empty((M, OUT), dtype=torch.float32, device="cuda") for OUT in OUTS]
+        ybytes = 4 * tot * M
+
+        def step(i):
+            fused[i % copies].forward(x, outs=ys)
+
+        keep = (fused, x, ys)
+    return dict(step=step, bytes=tot * (IN // 32) * 18 + (2 if bf16_x else 4) * IN * M + ybytes, ops=2 * M * IN * tot,
+                launches=1, keep=keep)
 
 
 def make_w4g(K, N, M, copies, seed=4):
@@ -535,6 +548,13 @@ def sweep(skip_large=False):
             M=135, copies=1, calls=20)
         run(f"ref Q4_0 {name} row-fused M=135 bf16 x (warm)", make_q4_0_fused, "mfma", "bf16", IN=960, OUTS=OUTS,
             M=135, copies=1, calls=20, bf16_x=True)
+    cg = max(1, COLD_BYTES // (5120 * 960 * 9 // 16))
+    run("ref Q4_0 gate|up + SwiGLU 960->2560 one launch M=1 fp32 (cold)", make_q4_0_fused, "hbm", IN=960,
+        OUTS=[2560, 2560], M=1, copies=cg, calls=cg, glu=True)
+    run("ref Q4_0 gate|up + SwiGLU 960->2560 one launch M=135 fp32 (warm)", make_q4_0_fused, "mfma", "bf16", IN=960,
+        OUTS=[2560, 2560], M=135, copies=1, calls=20, glu=True)
+    run("ref Q4_0 gate|up + SwiGLU 960->2560 one launch M=135 bf16 in / bf16 out (warm)", make_q4_0_fused, "mfma",
+        "bf16", IN=960, OUTS=[2560, 2560], M=135, copies=1, calls=20, glu=True, bf16_x=True, bf16_y=True)
     run("cfg4 W8A8 actor 64->256->256->8 M=4096 (fused, 1 launch)", make_actor_fused, "mfma", "int8", calls=20)
     run("cfg4 W8A8 actor 64->256->256->8 M=4096 (unfused, 6 launches)", make_actor_w8a8, "mfma", "int8", calls=20)
     for N in (4096, 11008):

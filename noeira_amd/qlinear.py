@@ -447,10 +447,12 @@ class FusedGLU:
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        if out is not None:
+            out_dtype = out.dtype
         if x.dtype not in _TORCH_DT or out_dtype not in _TORCH_DT:
             raise L.NQError(L.NQ_ERR_INVALID, "FusedGLU.forward: x and y must be fp32 or bf16")
         M = _check_x(x, self.IN, "FusedGLU.forward")
-        if out is None or out.numel() < M * self.OUT or out.dtype != out_dtype:
+        if out is None or out.numel() < M * self.OUT:
             out = torch.empty((M, self.OUT), dtype=out_dtype, device=x.device)
         L.check(L.lib().nq_forward(self._h, _dev_ptr(x), _TORCH_DT[x.dtype], C.c_void_p(0), _dev_ptr(out),
                                    _TORCH_DT[out_dtype], M, C.c_void_p(0), L.DT_F32, L.EPI_SWIGLU, _stream_ptr()))
