@@ -361,8 +361,9 @@ def make_actor_fused(M=4096, seed=5):
     return dict(step=step, bytes=nbytes, ops=ops, launches=1, keep=(lins, biases, x, y))
 
 
-def make_fp8(M, N, K=4096, copies=1, seed=6):
-    """config 5 (configs[4]): e4m3 x e4m3, per-tensor scales, fp32 accumulate, bf16 out."""
+def make_fp8(M, N, K=4096, copies=1, seed=6, a16=False):
+    """config 5 (configs[4]): e4m3 x e4m3, per-tensor scales, fp32 accumulate, bf16 out.  With `a16` the same
+    weight under bf16 activations (the codes decoded to bf16 on their way into the bf16 matrix cores)."""
     import numpy as np
     import torch
 
@@ -379,6 +380,14 @@ def make_fp8(M, N, K=4096, copies=1, seed=6):
     a = torch.randn((M, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).cuda()
     sa = torch.tensor([1.0 / 16], dtype=torch.float32, device="cuda")
     y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    if a16:
+        xb = torch.randn((M, K), generator=g).to(torch.bfloat16).cuda()
+
+        def step16(i):
+            layers[i % copies].forward_a16(xb, out=y, out_dtype=torch.bfloat16)
+
+        return dict(step=step16, bytes=N * K + 2 * M * K + 2 * M * N, ops=2 * M * N * K, launches=1,
+                    keep=(layers, xb, y))
 
     def step(i):
         layers[i % copies].forward(a, sa, out=y)
@@ -575,6 +584,10 @@ def sweep(skip_large=False):
         for M in (16, 64, 256, 512):
             run(f"W8A8 int8 M={M} K=4096 N=4096 (warm)", make_w8a8_gemm, "mfma", "int8", M=M, N=4096, calls=20)
             run(f"fp8 x fp8 M={M} K=4096 N=4096 (warm)", make_fp8, "mfma", "fp8", M=M, N=4096, copies=1, calls=20)
+        # e4m3 weights under bf16 activations: the bf16 matrix-core kernels
+        for M in (16, 256, 4096):
+            run(f"fp8 W x bf16 A M={M} K=4096 N=4096 (warm)", make_fp8, "mfma", "bf16", M=M, N=4096, copies=1, calls=20,
+                a16=True)
         # the dequant-GEMVs at a size where the HBM fraction means something (22 - 45 MB of codes)
         c = max(1, COLD_BYTES // (4096 * 11008 // 2))
         run("W4A16 g128 4096->11008 M=1 (cold)", make_w4g, "hbm", K=4096, N=11008, M=1, copies=c, calls=c)

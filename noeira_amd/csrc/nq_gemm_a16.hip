@@ -60,6 +60,7 @@ struct A16Params {
     int32_t M, N, K;
     int32_t groups;
     float inv_cpg;    // W4_GROUP: 1 / (16-byte chunks per group)
+    float tscale;     // FP8_E4M3: the weight's per-tensor scale
     int32_t s_pairs;  // Q4_0: scale rows are 4-byte (1) or 8-byte (2) aligned, else 0
     int32_t nch;      // 16-byte chunks per weight row
     int32_t y_dtype, bias_dtype, epilogue;
@@ -122,6 +123,24 @@ __device__ __forceinline__ void i8_word_to_bf16(uint32_t w, uint32_t& p0, uint32
     p1 = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
 }
 
+// four fp8 e4m3 codes of one word -> two bf16 pairs holding the decoded values (exact: 4 significant bits;
+// the hardware converter decodes OCP e4m3fn, NaN codes included)
+__device__ __forceinline__ void fp8_word_to_bf16(uint32_t w, uint32_t& p0, uint32_t& p1) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2;
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    p0 = __builtin_amdgcn_perm(__float_as_uint(a[1]), __float_as_uint(a[0]), 0x07060302u);
+    p1 = __builtin_amdgcn_perm(__float_as_uint(b[1]), __float_as_uint(b[0]), 0x07060302u);
+}
+
+template <int FMT>
+__device__ __forceinline__ void byte_word_to_bf16(uint32_t w, uint32_t& p0, uint32_t& p1) {
+    if constexpr (FMT == NQ_FMT_FP8_E4M3)
+        fp8_word_to_bf16(w, p0, p1);
+    else
+        i8_word_to_bf16(w, p0, p1);
+}
+
 // A-operand terms of 8 consecutive activations held raw in registers: one term for bf16
 // input, three for fp32 (hi + mid + lo = the fp32 value exactly: each split truncates, so
 // each residual is exact in fp32 and the third has at most 8 significant bits).  A term pair
@@ -165,7 +184,7 @@ __device__ __forceinline__ void make_terms(const u32x4 (&raw)[XF32 ? 2 : 1], u32
 //     one group (WHOLE) the scale is applied once per k-step instead of once per chunk.
 template <int FMT, bool XF32, int MW, int NW, int KW, bool WHOLE>
 __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
-    constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL);
+    constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL && FMT != NQ_FMT_FP8_E4M3);
     constexpr int NT = XF32 ? 3 : 1;            // bf16 terms per activation
     constexpr int NL = XF32 ? 2 : 1;            // 16-byte pieces per activation fragment
     constexpr int ES = XF32 ? 4 : 2;            // bytes per activation
@@ -366,7 +385,9 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
     for (int t = 0; t < EPW; t++) {
         const int idx = min(wave + t * KW, TA - 1);
         const int n = min(n_base + 16 * ((idx >> 2) % NW) + ln, p.N - 1);
-        ep_scale[t] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[n] : 1.0f;
+        ep_scale[t] = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[n]
+                      : (FMT == NQ_FMT_FP8_E4M3)  ? p.tscale
+                                                   : 1.0f;
         ep_bias[t] = 0;
         if (p.bias)
             ep_bias[t] = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
@@ -443,8 +464,8 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 #pragma unroll
                     for (int j = 0; j < NW; j++) {
                         uint32_t b0, b1, b2, b3;
-                        i8_word_to_bf16(wc[j][2 * q], b0, b1);
-                        i8_word_to_bf16(wc[j][2 * q + 1], b2, b3);
+                        byte_word_to_bf16<FMT>(wc[j][2 * q], b0, b1);
+                        byte_word_to_bf16<FMT>(wc[j][2 * q + 1], b2, b3);
                         bop[j] = (u32x4){b0, b1, b2, b3};
                     }
                 }
@@ -487,8 +508,9 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
                     } else {
 #pragma unroll
                         for (int t = 0; t < NT; t++) {
-                            xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones),
-                                                                              xacc[i], 0, 0, 0);
+                            if constexpr (FMT == NQ_FMT_W8_CHANNEL)
+                                xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones),
+                                                                                  xacc[i], 0, 0, 0);
 #pragma unroll
                             for (int j = 0; j < NW; j++)
                                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]),
@@ -512,7 +534,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         }
     }
 
-    if constexpr (!FOUR_BIT) {
+    if constexpr (FMT == NQ_FMT_W8_CHANNEL) {
 #pragma unroll
         for (int i = 0; i < MW; i++)
 #pragma unroll
@@ -545,7 +567,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
         const int r = idx & 3, j = (idx >> 2) % NW, i = (idx >> 2) / NW;
         const int n = n_base + 16 * j + ln;
         const int m = m_base + 16 * i + 4 * kb + r;  // D layout: row 4*(lane/16) + r, column lane%16
-        if (FMT == NQ_FMT_W8_CHANNEL) z *= ep_scale[t];
+        if (!FOUR_BIT) z *= ep_scale[t];
         z += p.bias_dtype == NQ_DT_F32 ? __uint_as_float(ep_bias[t]) : __uint_as_float(ep_bias[t] << 16);
         if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
         if (p.epilogue == NQ_EPI_SWIGLU) {
@@ -588,7 +610,7 @@ __global__ __launch_bounds__(64 * KW) void gemm_a16_kernel(const A16Params p) {
 //     chunk or per k-step, exact three-term split of fp32 activations) is the kernel above's.
 template <int FMT, bool XF32, int MT, int NW, bool WHOLE>
 __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16Params p) {
-    constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL);
+    constexpr bool FOUR_BIT = (FMT != NQ_FMT_W8_CHANNEL && FMT != NQ_FMT_FP8_E4M3);
     constexpr int NT = XF32 ? 3 : 1;
     constexpr int NL = XF32 ? 2 : 1;
     constexpr int ES = XF32 ? 4 : 2;
@@ -798,8 +820,8 @@ __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16P
 #pragma unroll
                 for (int j = 0; j < NW; j++) {
                     uint32_t b0, b1, b2, b3;
-                    i8_word_to_bf16(wc[j][2 * q], b0, b1);
-                    i8_word_to_bf16(wc[j][2 * q + 1], b2, b3);
+                    byte_word_to_bf16<FMT>(wc[j][2 * q], b0, b1);
+                    byte_word_to_bf16<FMT>(wc[j][2 * q + 1], b2, b3);
                     bop[j] = (u32x4){b0, b1, b2, b3};
                 }
             }
@@ -841,8 +863,9 @@ __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16P
                 } else {
 #pragma unroll
                     for (int t = 0; t < NT; t++) {
-                        xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xacc[i], 0,
-                                                                          0, 0);
+                        if constexpr (FMT == NQ_FMT_W8_CHANNEL)
+                            xacc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(ones), xacc[i],
+                                                                              0, 0, 0);
 #pragma unroll
                         for (int j = 0; j < NW; j++)
                             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(at[t]), as_bf16x8(bop[j]),
@@ -869,7 +892,9 @@ __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16P
     for (int j = 0; j < NW; j++) {
         const int n = n0 + wn * 16 * NW + 16 * j + ln;
         const int nc = min(n, p.N - 1);
-        const float cscale = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[nc] : 1.0f;
+        const float cscale = (FMT == NQ_FMT_W8_CHANNEL) ? reinterpret_cast<const float*>(p.scales)[nc]
+                             : (FMT == NQ_FMT_FP8_E4M3)  ? p.tscale
+                                                          : 1.0f;
         float cbias = 0.0f;
         if (p.bias)
             cbias = (p.bias_dtype == NQ_DT_F32)
@@ -884,7 +909,8 @@ __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16P
             for (int r = 0; r < 4; r++) {
                 const int m = m0 + wm * 16 * MT + 16 * i + 4 * kb + r;
                 float z = acc[i][j][r];
-                if constexpr (!FOUR_BIT) z = fmaf(-128.0f, xacc[i][r], z) * cscale;
+                if constexpr (FMT == NQ_FMT_W8_CHANNEL) z = fmaf(-128.0f, xacc[i][r], z);
+                if constexpr (!FOUR_BIT) z *= cscale;
                 z += cbias;
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
                 if (p.epilogue == NQ_EPI_SWIGLU) {  // (uniform) gate in the even column, up one lane over
@@ -912,7 +938,7 @@ __global__ __launch_bounds__(128 * (8 / NW)) void gemm_a16_big_kernel(const A16P
 
 template <int FMT, bool XF32, bool WHOLE>
 int32_t launch_big(const A16Params& p, int mt, int nw, hipStream_t s) {
-    const bool four_bit = FMT != NQ_FMT_W8_CHANNEL;
+    const bool four_bit = FMT != NQ_FMT_W8_CHANNEL && FMT != NQ_FMT_FP8_E4M3;
     const int xb = (four_bit ? 128 : 64) * (XF32 ? 4 : 2);
     const size_t lds = 2 * ((size_t)32 * mt * xb + 128 * 64);
     const dim3 grid((unsigned)((p.N + 127) / 128), (unsigned)((p.M + 32 * mt - 1) / (32 * mt)));
@@ -934,7 +960,7 @@ int32_t launch_big(const A16Params& p, int mt, int nw, hipStream_t s) {
 
 template <int FMT, bool XF32, bool WHOLE>
 int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipStream_t s) {
-    const bool four_bit = FMT != NQ_FMT_W8_CHANNEL;
+    const bool four_bit = FMT != NQ_FMT_W8_CHANNEL && FMT != NQ_FMT_FP8_E4M3;
     const size_t staging = (size_t)kw * (16 * ((!four_bit && !XF32) ? 128 : 256) + nw * 1024);
     const size_t lds = std::max(staging, (size_t)kw * mw * nw * 4 * 64 * sizeof(float));
     const dim3 block(64 * kw);
@@ -960,9 +986,8 @@ int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipSt
 bool gemm_a16_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (a.x_dtype != NQ_DT_F32 && a.x_dtype != NQ_DT_BF16) return false;
-    if (L->format == NQ_FMT_FP8_E4M3) return false;
-    if (L->format != NQ_FMT_W8_CHANNEL && L->in % 32 != 0) return false;
-    if (L->format == NQ_FMT_W8_CHANNEL && L->in % 16 != 0) return false;
+    const bool bytes = L->format == NQ_FMT_W8_CHANNEL || L->format == NQ_FMT_FP8_E4M3;
+    if (L->in % (bytes ? 16 : 32) != 0) return false;
     // the kernel addresses each operand with 32-bit byte offsets
     const int64_t lim = (int64_t)1 << 32;
     if ((int64_t)a.M * L->in * 4 >= lim || (int64_t)L->out * L->in >= lim) return false;
@@ -971,7 +996,7 @@ bool gemm_a16_applicable(const ForwardArgs& a) {
 
 int32_t launch_gemm_a16(const ForwardArgs& a) {
     const nq_layer* L = a.L;
-    const bool four_bit = L->format != NQ_FMT_W8_CHANNEL;
+    const bool four_bit = L->format != NQ_FMT_W8_CHANNEL && L->format != NQ_FMT_FP8_E4M3;
     const bool xf32 = a.x_dtype == NQ_DT_F32;
     A16Params p{};
     p.codes = L->d_codes, p.scales = L->d_scales, p.zps = L->d_zps;
@@ -979,6 +1004,7 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.groups = L->groups;
     p.inv_cpg = L->group ? 32.0f / (float)L->group : 1.0f;
+    p.tscale = L->scale;
     p.s_pairs = L->format != NQ_FMT_Q4_0 ? 0 : (L->in / 32) % 4 == 0 ? 2 : (L->in / 32) % 2 == 0 ? 1 : 0;
     p.nch = L->in / (four_bit ? 32 : 16);
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
@@ -1004,6 +1030,9 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
             case NQ_FMT_W8_CHANNEL:
                 return xf32 ? launch_big<NQ_FMT_W8_CHANNEL, true, false>(p, 2, bnw, a.stream)
                             : launch_big<NQ_FMT_W8_CHANNEL, false, false>(p, big, bnw, a.stream);
+            case NQ_FMT_FP8_E4M3:
+                return xf32 ? launch_big<NQ_FMT_FP8_E4M3, true, false>(p, 2, bnw, a.stream)
+                            : launch_big<NQ_FMT_FP8_E4M3, false, false>(p, big, bnw, a.stream);
         }
     }
     // Tile shape: as wide in N as still leaves enough workgroups to occupy the chip (the
@@ -1051,6 +1080,9 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
         case NQ_FMT_W8_CHANNEL:
             return xf32 ? launch_tile<NQ_FMT_W8_CHANNEL, true, false>(p, mw, nw, kw, grid, a.stream)
                         : launch_tile<NQ_FMT_W8_CHANNEL, false, false>(p, mw, nw, kw, grid, a.stream);
+        case NQ_FMT_FP8_E4M3:
+            return xf32 ? launch_tile<NQ_FMT_FP8_E4M3, true, false>(p, mw, nw, kw, grid, a.stream)
+                        : launch_tile<NQ_FMT_FP8_E4M3, false, false>(p, mw, nw, kw, grid, a.stream);
     }
     return fail(NQ_ERR_INVALID, "nq_forward: unknown format");
 }

@@ -363,6 +363,13 @@ class FP8Linear(_Layer):
             raise L.NQError(L.NQ_ERR_INVALID, "FP8Linear.forward: x must be e4m3fn codes")
         return self._forward(x_codes, L.DT_FP8_E4M3, x_scale, out, out_dtype, bias, epilogue, "FP8Linear.forward")
 
+    def forward_a16(self, x: torch.Tensor, bias=None, epilogue="none", out=None, out_dtype=torch.float32):
+        """fp32 or bf16 activations over the e4m3fn weight: y = x @ (decode(W) * scale)^T.  The codes enter the
+        bf16 matrix cores as their exact decoded values, fp32 activations as three bf16 terms."""
+        if x.dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "FP8Linear.forward_a16: x must be fp32 or bf16")
+        return self._forward(x, _TORCH_DT[x.dtype], None, out, out_dtype, bias, epilogue, "FP8Linear.forward_a16")
+
 
 class FusedRows:
     """Up to four loaded layers that read the same activations (q|k|v, gate|up

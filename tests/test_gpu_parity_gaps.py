@@ -276,3 +276,40 @@ def test_share_scratch_receives_the_dequantised_weight():
     assert np.array_equal(got_b.cpu().numpy(), O.dequantize_q4_0(b.blocks().reshape(960, -1), 960, 320))
     with pytest.raises(L.NQError, match="share_scratch"):
         a.share_scratch(shared, 960 * 320 - 1)
+
+
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,K,N", [(1, 512, 3200), (2, 512, 3200), (7, 784, 40), (100, 3200, 512), (256, 4096, 1000),
+                                   (600, 512, 3200), (2050, 1040, 650)])
+def test_fp8_weights_under_16bit_activations(M, K, N, xdt):
+    """e4m3fn weights with fp32 / bf16 activations at every M: one row on the GEMV, from two rows on the bf16
+    matrix-core kernels (the codes decode to bf16 exactly, fp32 activations enter as three exact bf16 terms), so
+    the result is the fp64 product over the dequantised weights - which `nq_dequantize` pins to the oracle's
+    decode table bit for bit - to fp32 accumulation accuracy.  With bias, ReLU and bf16 out; a NaN code poisons
+    its own output channel and no other."""
+    rng = np.random.default_rng(M + K + N)
+    lin = FP8Linear(K, N)
+    wt = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).to(torch.float8_e4m3fn)
+    codes = wt.view(torch.uint8).numpy().copy()
+    lin.set_weight(codes, 1.0 / 16)
+    deq = lin.dequantized_dev().double()
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.5).astype(np.float32)).cuda()
+    want = x.double() @ deq.T
+    y = lin.forward_a16(x)
+    assert y.dtype == torch.float32 and y.shape == (M, N)
+    assert float((y.double() - want).abs().max()) <= 1e-5 * float(want.abs().max())
+    assert torch.equal(lin.forward_a16(x), y)
+    yr = lin.forward_a16(x, bias=bias, epilogue="relu")
+    want_r = (want + bias.double()).clamp_min(0)
+    assert float((yr.double() - want_r).abs().max()) <= 1e-5 * float(want_r.abs().max())
+    yb = lin.forward_a16(x, bias=bias, out_dtype=torch.bfloat16)
+    want_b = want + bias.double()
+    assert float((yb.double() - want_b).abs().max()) <= 2.0 ** -8 * float(want_b.abs().max())
+    codes[N // 2, K // 3] = 0x7F  # NaN
+    lin.set_weight(codes, 1.0 / 16)
+    yn = lin.forward_a16(x)
+    assert bool(torch.isnan(yn[:, N // 2]).all())
+    keep = torch.ones(N, dtype=torch.bool, device="cuda")
+    keep[N // 2] = False
+    assert torch.equal(yn[:, keep], y[:, keep])
