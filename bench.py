@@ -484,6 +484,54 @@ def mfma_only(iters=4096, reps=5):
     return out
 
 
+def gemm_timeline(N=4096, K=4096, M=8192):
+    """Where a config-5 GEMM call's time goes: every workgroup of the 256 x 256 tile kernel stamps the GPU's
+    constant 100 MHz clock at entry, when its first K stage has landed, after its K loop and after its stores
+    are acknowledged (nq_diag_gemm8_timeline).  Reported per round of workgroups (the hardware hands out the
+    next tile as a CU frees up): medians in microseconds."""
+    import ctypes as C
+
+    import numpy as np
+    import torch
+
+    from noeira_amd import _lib as L
+
+    wl = make_fp8(M, N, K=K)
+    layers, a, sa, y = wl["keep"]
+    for i in range(5):
+        wl["step"](i)
+    torch.cuda.synchronize()
+    tiles = (M // 256) * ((N + 255) // 256)
+    buf = torch.zeros((tiles, 4), dtype=torch.int64, device="cuda")
+    null = C.c_void_p(0)
+    t = None
+    for _ in range(7):  # single launches differ by a few percent with the clock the chip happens to be at: the fastest
+        for i in range(3):
+            wl["step"](i)
+        L.check(L.lib().nq_diag_gemm8_timeline(layers[0]._h, C.c_void_p(a.data_ptr()), L.DT_FP8_E4M3,
+                                                C.c_void_p(sa.data_ptr()), C.c_void_p(y.data_ptr()), L.DT_BF16, M,
+                                                C.c_void_p(buf.data_ptr()), tiles, null))
+        ti = buf.cpu().numpy().astype(np.float64) * 0.01  # ticks of 10 ns -> us
+        ti -= ti[:, 0].min()
+        if t is None or ti[:, 3].max() < t[:, 3].max():
+            t = ti
+    order = np.argsort(t[:, 0])
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rounds = []
+    for r in range(0, tiles, cus):
+        idx = order[r:r + cus]
+        rounds.append({"workgroups": int(len(idx)),
+                       "entry_us": [round(float(t[idx, 0].min()), 2), round(float(t[idx, 0].max()), 2)],
+                       "first_stage_us": round(float(np.median(t[idx, 1] - t[idx, 0])), 2),
+                       "k_loop_us": round(float(np.median(t[idx, 2] - t[idx, 1])), 2),
+                       "epilogue_us": round(float(np.median(t[idx, 3] - t[idx, 2])), 2),
+                       "end_us": [round(float(t[idx, 3].min()), 2), round(float(t[idx, 3].max()), 2)]})
+    stages = K // 128
+    return {"workload": f"fp8 GEMM M={M} K={K} N={N}, bf16 out", "tiles": tiles, "kernel_us": round(float(t[:, 3].max()), 2),
+            "stage_us": round(float(np.median(t[:, 2] - t[:, 1])) / stages, 4), "stages_per_tile": stages,
+            "epilogue_bytes_per_round": min(tiles, cus) * 256 * 256 * 2, "rounds": rounds}
+
+
 def make_read(nbytes, copies):
     """The floor of a weight-streaming call: nq_diag_stream_read over `nbytes` (a kernel that only reads, with
     1 KiB loads), rotating over `copies` distinct regions so that every call streams from HBM."""
@@ -686,6 +734,8 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_t8, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "W8A8 and fp8 x fp8 at 4096 x 4096, M = 16, 64, 128, 256, 512, one call each per step"
+    elif which == "gemm_timeline":
+        return {"only": which, "timelines": [gemm_timeline(4096, 4096), gemm_timeline(4096, 8192), gemm_timeline(11008, 4096)]}
     elif which == "mfma_peak":
         return {"only": which, "mfma_only": mfma_only()}
     elif which == "actor":
@@ -748,14 +798,15 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "mfma_peak"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "mfma_peak", "gemm_timeline"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
                          "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
                          "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, tile8 = int8 and fp8 "
                          "activations at M = 16 .. 512 over 4096 x 4096, manyrows = bf16 / fp32 activations at M = 1120 "
-                         "and 4096, mfma_peak = the matrix cores alone (nq_diag_mfma_rate) on constant and random operands")
+                         "and 4096, mfma_peak = the matrix cores alone (nq_diag_mfma_rate) on constant and random operands, gemm_timeline = the "
+                         "config-5 GEMM's workgroups stamping entry / first stage / K loop / stores (nq_diag_gemm8_timeline)")
     ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--rows-layout", action="store_true",
                     help="large layers keep only their row-ordered codes (NQ_FLAG_NO_TILE_COPY): the single-row kernels "
@@ -775,7 +826,7 @@ def main():
     if a.rows_layout:
         global TILE_COPY
         TILE_COPY = False
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "mfma_peak"):
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "mfma_peak", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 

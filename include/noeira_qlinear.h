@@ -309,6 +309,16 @@ int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_by
  * can beat on this GPU. */
 int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream);
 
+/* Where the time of a large-tile 8-bit GEMM goes (no counterpart in the reference): nq_forward with 8-bit
+ * activations and M >= 64 rows, with every workgroup of the 256 x 256 tile kernel reporting four readings of
+ * the GPU's constant 100 MHz clock - entry, first K stage landed, K loop done, stores acknowledged - into
+ * stamps (device uint64 [tiles][4], tiles = ceil(M / 256) * ceil(OUT / 256) <= max_tiles, else NQ_ERR_INVALID).
+ * The arguments are nq_forward's for that case (x: int8 with per-row x_scale, or e4m3 codes with one scale; no
+ * bias).  Synchronises the stream before it returns; calls of nq_forward from other threads meanwhile would
+ * write stamps too. */
+int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
+                               int32_t y_dtype, int32_t M, uint64_t* stamps, int64_t max_tiles, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

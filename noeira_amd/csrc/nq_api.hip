@@ -930,6 +930,22 @@ int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream) {
     return launch_stream_read(src, nbytes / 1024, (hipStream_t)stream);
 }
 
+int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
+                               int32_t y_dtype, int32_t M, uint64_t* stamps, int64_t max_tiles, void* stream) {
+    int32_t rc = check_handle(h, "nq_diag_gemm8_timeline");
+    if (rc) return rc;
+    if (!stamps || M < 64 || (x_dtype != NQ_DT_I8 && x_dtype != NQ_DT_FP8_E4M3))
+        return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: 8-bit activations, M >= 64 and a stamp buffer are needed");
+    const int64_t tiles = (int64_t)((M + 255) / 256) * ((h->out + 255) / 256);
+    if (tiles > max_tiles) return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: the stamp buffer is smaller than the tile count");
+    gemm8_set_stamps(reinterpret_cast<unsigned long long*>(stamps));
+    rc = nq_forward(h, x, x_dtype, x_scale, y, y_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_NONE, stream);
+    gemm8_set_stamps(nullptr);
+    if (rc) return rc;
+    NQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return NQ_OK;
+}
+
 int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M, int32_t K,
                             void* stream) {
     if (M < 0 || K <= 0 || K % 4 != 0)

@@ -26,6 +26,9 @@ int32_t fail_hip(hipError_t e, const char* what);
         if (_e != hipSuccess) return nq::fail_hip(_e, #expr); \
     } while (0)
 
+// nq_gemm8.hip: per-workgroup clock readings of the next large-tile GEMM launches (a diagnostic; null = off)
+void gemm8_set_stamps(unsigned long long* buf);
+
 // nq_diag.hip: the matrix cores' own rate (a diagnostic)
 int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s);
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,

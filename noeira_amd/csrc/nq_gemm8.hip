@@ -85,6 +85,7 @@ struct Gemm8Params {
     int32_t M, N, K;
     int32_t tiles_m, tiles_n;
     int32_t y_dtype, bias_dtype, epilogue;
+    unsigned long long* stamps;  // a diagnostic: per workgroup, four readings of the constant 100 MHz clock, or null
     int32_t chan_vec;  // N % 4 == 0 and col_scale / bias aligned for one 16-byte (bf16 bias: 8-byte) load per 4 channels
 };
 
@@ -107,6 +108,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int WN = BN / 2;         // channels per wavefront
     constexpr int TJ = WN / 32;        // weight fragments (MFMA tiles along N) per wavefront
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const unsigned long long t_entry = wall_clock64();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -395,6 +397,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
         }
 #undef NQ_DMA_ALL
     }
+    const unsigned long long t_first = wall_clock64();  // stage 0 has landed
     // what groups G-2 and G-1 of a previous stage (in buffer 1) would have requested
     requests(std::integral_constant<int, G - 2>{}, std::integral_constant<int, 1>{});
     requests(std::integral_constant<int, G - 1>{}, std::integral_constant<int, 1>{});
@@ -406,6 +409,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     }
     if (st < KT) NQ_STAGE(0)  // an odd number of stages: the last one, in buffer 0 again
     NQ_LDS_WAIT(0);  // requests past the last stage still target registers: let them land
+    const unsigned long long t_loop = wall_clock64();
 #undef NQ_STAGE
 #undef NQ_GROUP
 #undef NQ_DMA_SLOT
@@ -579,6 +583,13 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
         }
     };
     emit(std::integral_constant<int, KIND_>{});
+    if (p.stamps) {  // (uniform) entry, first stage landed, loop done, stores acknowledged
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (tid == 0) {
+            unsigned long long* o = p.stamps + 4 * (size_t)blockIdx.x;
+            o[0] = t_entry, o[1] = t_first, o[2] = t_loop, o[3] = wall_clock64();
+        }
+    }
 }
 
 template <bool FP8, int KIND>
@@ -597,6 +608,12 @@ int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int bn, in
 }
 
 }  // namespace
+
+namespace {
+unsigned long long* g_stamps = nullptr;  // set by the timeline diagnostic around one call, null otherwise
+}
+
+void gemm8_set_stamps(unsigned long long* buf) { g_stamps = buf; }
 
 bool gemm8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
@@ -618,6 +635,7 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + 255) / 256;
+    p.stamps = g_stamps;
     const bool i8 = a.x_dtype == NQ_DT_I8;
     p.chan_vec = L->out % 4 == 0 && L->out >= 4 && (!i8 || a.y_dtype == NQ_DT_I32 || (uintptr_t)p.col_scale % 16 == 0) &&
                  (!a.bias || (uintptr_t)a.bias % (a.bias_dtype == NQ_DT_F32 ? 16 : 8) == 0);

@@ -313,3 +313,36 @@ def test_fp8_weights_under_16bit_activations(M, K, N, xdt):
     keep = torch.ones(N, dtype=torch.bool, device="cuda")
     keep[N // 2] = False
     assert torch.equal(yn[:, keep], y[:, keep])
+
+
+def test_gemm8_timeline_diagnostic_reports_ordered_stamps_and_the_same_output():
+    """nq_diag_gemm8_timeline: the call nq_forward would make, with every workgroup of the large-tile kernel
+    reporting its four clock readings: ordered, all written, and y as without them."""
+    import ctypes as C
+
+    from noeira_amd import _lib as L
+
+    M, K, N = 2048, 512, 2304   # 8 x 9 tiles
+    rng = np.random.default_rng(3)
+    lin = FP8Linear(K, N)
+    wt = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).to(torch.float8_e4m3fn)
+    lin.set_weight(wt.view(torch.uint8).numpy(), 0.25)
+    xc = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.float8_e4m3fn).view(torch.uint8).cuda()
+    sa = torch.tensor([0.5], dtype=torch.float32, device="cuda")
+    want = lin.forward(xc, sa)
+    y = torch.zeros_like(want)
+    tiles = 8 * 9
+    stamps = torch.zeros((tiles, 4), dtype=torch.int64, device="cuda")
+    args = (lin._h, C.c_void_p(xc.data_ptr()), L.DT_FP8_E4M3, C.c_void_p(sa.data_ptr()), C.c_void_p(y.data_ptr()),
+            L.DT_BF16, M, C.c_void_p(stamps.data_ptr()))
+    assert L.lib().nq_diag_gemm8_timeline(*args, tiles - 1, C.c_void_p(0)) == L.NQ_ERR_INVALID
+    L.check(L.lib().nq_diag_gemm8_timeline(*args, tiles, C.c_void_p(0)))
+    assert torch.equal(y, want)
+    t = stamps.cpu().numpy()
+    assert (t > 0).all() and (np.diff(t, axis=1) >= 0).all()
+    assert (t[:, 3] - t[:, 0]).max() < 100000   # under a millisecond of 10 ns ticks
+    # and the next ordinary call writes no stamps
+    stamps.zero_()
+    lin.forward(xc, sa)
+    torch.cuda.synchronize()
+    assert int(stamps.abs().sum()) == 0
