@@ -643,8 +643,9 @@ def sweep(skip_large=False):
         run("W8A16 4096->11008 M=1 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, copies=max(1, c // 2),
             calls=max(1, c // 2))
         # what a kernel that only reads those weights takes (launch + stream): the floor of the rows above
-        for mb, nb in (("16.8 MB", 4096 * 4096), ("23.2 MB", 4096 * 11008 // 2 + 2 * 32 * 11008 + 16 * 11008),
-                       ("45.1 MB", 4096 * 11008)):
+        for mb, nb in (("1.66 MB", 512 * 3200 + 4 * 3200), ("16.8 MB", 4096 * 4096),
+                       ("23.2 MB", 4096 * 11008 // 2 + 2 * 32 * 11008 + 16 * 11008), ("45.1 MB", 4096 * 11008),
+                       ("235 MB", 8192 * 28672)):
             cr = max(1, COLD_BYTES // nb)
             run(f"floor: plain read of {mb}, no arithmetic (cold)", make_read, "hbm", nbytes=nb, copies=cr, calls=cr)
         # the same kernels where the stream is long enough for the fixed part of a call (launch, first trip to

@@ -61,7 +61,10 @@ void mfma_rate_kernel(const int* __restrict__ seed, int seed_words, int iters, i
 // in flight per wavefront, eight wavefronts per workgroup) and computes nothing.  What it takes for the bytes
 // of a GEMV's weight is the floor of that GEMV on this GPU: launch + the stream.
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-__global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restrict__ src, int64_t kib, uint32_t* sink) {
+// (written only: `used` and a volatile store keep the compiler from deleting it, and with it the loads)
+__device__ __attribute__((used)) uint32_t g_read_sink;
+// `never`: a value the XOR of the data is not expected to take, from the host, so that the compiler must keep the loads
+__global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restrict__ src, int64_t kib, uint32_t never) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t b0 = ((int64_t)blockIdx.x * 8 + wave) * 4;
     u32x4 v[4];
@@ -70,14 +73,14 @@ __global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restric
     uint32_t x = 0;
 #pragma unroll
     for (int j = 0; j < 4; j++) x ^= v[j][0] ^ v[j][1] ^ v[j][2] ^ v[j][3];
-    if (x == 0x9E3779B9u && lane == 77) sink[0] = x;  // (never true: lane < 64)
+    if (x == never) *(volatile uint32_t*)&g_read_sink = x;
 }
 
 }  // namespace
 
 int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s) {
     hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)((kib + 31) / 32)), dim3(512), 0, s,
-                       reinterpret_cast<const u32x4*>(src), kib, (uint32_t*)nullptr);
+                       reinterpret_cast<const u32x4*>(src), kib, 0x9E3779B9u);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }

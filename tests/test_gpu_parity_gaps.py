@@ -346,3 +346,29 @@ def test_gemm8_timeline_diagnostic_reports_ordered_stamps_and_the_same_output():
     lin.forward(xc, sa)
     torch.cuda.synchronize()
     assert int(stamps.abs().sum()) == 0
+
+
+def test_stream_read_diagnostic_really_reads():
+    """nq_diag_stream_read is the floor bench.py prints beside the large GEMVs: it must move the bytes.  256 MiB
+    cannot come out of HBM in less than 256 MiB / 8 TB/s = 33.5 us (the published peak), whatever the clocks."""
+    import ctypes as C
+
+    from noeira_amd import _lib as L
+
+    nbytes = 256 << 20
+    bufs = [torch.full((nbytes,), 0x5A, dtype=torch.uint8, device="cuda") for _ in range(3)]   # > the 256 MB cache
+    lib = L.lib()
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for b in bufs:
+        L.check(lib.nq_diag_stream_read(C.c_void_p(b.data_ptr()), nbytes, s))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(4):
+        for b in bufs:
+            L.check(lib.nq_diag_stream_read(C.c_void_p(b.data_ptr()), nbytes, s))
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / 12
+    assert us > 33.5, f"a plain read of 256 MiB took {us:.1f} us: the loads were not issued"
+    assert us < 200
