@@ -46,9 +46,9 @@ MFMA_PEAK_TOPS = {"fp8": 5000.0, "int8": 5000.0, "bf16": 2500.0}
 SAMPLES, COLD_BYTES = 7, 512 << 20
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (fetched + written), scaled by
 # what the same counters read for a plain copy of known size; None until measured
-HEADLINE_TRAFFIC = 1791744      # mean of the two linears' launches (1.66 MB algorithmic)
-FP8_GEMV_TRAFFIC = 45199360     # K=4096, N=11008 (45.09 MB algorithmic)
-FP8_GEMM_TRAFFIC = 270030438    # M=8192, K=4096, N=4096 (117.4 MB algorithmic; the re-reads hit the Infinity Cache)
+HEADLINE_TRAFFIC = 1804544      # mean of the two linears' launches (1.66 MB algorithmic)
+FP8_GEMV_TRAFFIC = 45185024     # K=4096, N=11008 (45.09 MB algorithmic)
+FP8_GEMM_TRAFFIC = 269343334    # M=8192, K=4096, N=4096 (117.4 MB algorithmic; the re-reads hit the Infinity Cache)
 
 
 def ensure_built():
@@ -643,6 +643,7 @@ def sweep(skip_large=False):
         run("W8A16 4096->11008 M=1 (cold)", make_w8a16_one, "hbm", K=4096, N=11008, copies=max(1, c // 2),
             calls=max(1, c // 2))
         # what a kernel that only reads those weights takes (launch + stream): the floor of the rows above
+        run("floor: a launch alone (plain read of 1 KiB as a graph node)", make_read, "hbm", nbytes=1024, copies=1, calls=200)
         for mb, nb in (("1.66 MB", 512 * 3200 + 4 * 3200), ("16.8 MB", 4096 * 4096),
                        ("23.2 MB", 4096 * 11008 // 2 + 2 * 32 * 11008 + 16 * 11008), ("45.1 MB", 4096 * 11008),
                        ("235 MB", 8192 * 28672)):
