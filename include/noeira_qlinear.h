@@ -70,7 +70,12 @@ extern "C" {
                                   W8_CHANNEL) normally keeps a second copy of its codes on the device, ordered
                                   for the matrix cores 16 rows at a time, which its single-row calls with
                                   bf16 / fp32 activations stream 1.2 .. 1.5 times faster than the row-ordered
-                                  codes; this flag saves that memory (0.5 or 1 byte per weight) */
+                                  codes; 4-bit layers with 512 <= IN <= 6144 keep it too, for calls with a
+                                  hundred activation rows and more over wide layers; this flag saves that memory
+                                  (0.5 or 1 byte per weight) */
+#define NQ_FLAG_PREFER_TILE 2  /* take the kernels that read the tile-ordered copy wherever they apply (2 .. 512
+                                  activation rows, any width), not only where they were measured to win: for
+                                  tuning on other shapes, and for tests that walk every instantiation */
 
 /* epilogues (LinearAct's, noeira/nn/primitives/linear_act.mojo:81-115) */
 #define NQ_EPI_NONE 0
@@ -94,7 +99,7 @@ int64_t nq_last_error(char* buf, int64_t n);
 
 /* `QLinear[IN, OUT].make` (qlinear.mojo:253-260): an empty layer.  `group` is
  * 32 for NQ_FMT_Q4_0 (IN % 32 == 0 is required, qlinear.mojo:243-245), the
- * group width for NQ_FMT_W4_GROUP, ignored otherwise.  flags: 0 or NQ_FLAG_NO_TILE_COPY. */
+ * group width for NQ_FMT_W4_GROUP, ignored otherwise.  flags: 0 or an OR of NQ_FLAG_*. */
 int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t out_features,
                   int32_t group, int32_t flags);
 

@@ -20,6 +20,7 @@ DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
 EPI_NONE, EPI_RELU, EPI_SWIGLU = 0, 1, 2
 ABI_VERSION = 4
 FLAG_NO_TILE_COPY = 1
+FLAG_PREFER_TILE = 2
 
 EXPORTS = [
     "nq_abi_version", "nq_last_error", "nq_create", "nq_destroy", "nq_set_blocks", "nq_set_weight_f32",

@@ -140,7 +140,7 @@ int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t o
         return fail(NQ_ERR_INVALID, "nq_create: unknown format " + std::to_string(format));
     if (in_features <= 0 || out_features <= 0)
         return fail(NQ_ERR_INVALID, "nq_create: IN and OUT must be positive");
-    if (flags & ~NQ_FLAG_NO_TILE_COPY) return fail(NQ_ERR_INVALID, "nq_create: unknown flags");
+    if (flags & ~(NQ_FLAG_NO_TILE_COPY | NQ_FLAG_PREFER_TILE)) return fail(NQ_ERR_INVALID, "nq_create: unknown flags");
     if (format == NQ_FMT_Q4_0) {
         // qlinear.mojo:243-245
         if (in_features % Q4_GROUP != 0)
@@ -164,6 +164,7 @@ int32_t nq_create(nq_handle* out, int32_t format, int32_t in_features, int32_t o
     L->format = format, L->in = in_features, L->out = out_features, L->group = group;
     L->groups = group ? (in_features + group - 1) / group : 0;
     L->no_tile_copy = (flags & NQ_FLAG_NO_TILE_COPY) != 0;
+    L->prefer_tile = (flags & NQ_FLAG_PREFER_TILE) != 0;
     *out = L;
     return NQ_OK;
 }
@@ -395,12 +396,22 @@ void row_view(const nq_layer* L, int r0, int r1, nq_layer* v) {
         default: srow = 0;
     }
     v->d_scales = L->d_scales ? reinterpret_cast<uint8_t*>(L->d_scales) + r0 * srow : nullptr;
+    // the tile-ordered copy is in units of 16 rows: a part that starts on one has its own view of it
+    v->prefer_tile = L->prefer_tile, v->no_tile_copy = L->no_tile_copy;
+    if (L->d_tile16 && r0 % 16 == 0) {
+        const int64_t t0 = (int64_t)(r0 / 16) * L->tile_nj;
+        v->d_tile16 = L->d_tile16 + t0 * 1024;
+        if (L->d_tile16_scales)
+            v->d_tile16_scales = reinterpret_cast<uint8_t*>(L->d_tile16_scales) + t0 * 16 * (L->format == NQ_FMT_W4_GROUP ? 4 : 8);
+        v->tile_nj = L->tile_nj;
+    }
 }
 
 int32_t dispatch(const ForwardArgs& a) {
     if (a.L->glu) {
         // gate | up pairs meet in the epilogue of the kernels whose result layout keeps a pair in one wavefront
         if (a.M == 1 && gemv_m1_applicable(a)) return launch_gemv_m1(a);
+        if (gemm_tile_mt_applicable(a)) return launch_gemm_tile_mt(a);
         if (a.M >= 2 && gemm_a16_applicable(a)) return launch_gemm_a16(a);
         return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no SwiGLU kernel for this shape (IN = " + std::to_string(a.L->in) +
                                             ", M = " + std::to_string(a.M) + "): run gate | up with nq_forward_fused "
@@ -414,6 +425,7 @@ int32_t dispatch(const ForwardArgs& a) {
     if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemv_tile_rows_applicable(a)) return launch_gemv_tile_rows(a);
+    if (gemm_tile_mt_applicable(a)) return launch_gemm_tile_mt(a);
     if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
     if (gemv_tile_applicable(a)) return launch_gemv_tile(a);
     if (gemv_split8_applicable(a)) return launch_gemv_split8(a);
@@ -427,7 +439,8 @@ int32_t dispatch(const ForwardArgs& a) {
 bool places_parts(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_I8) return false;
     if (gemv_fp8_applicable(a) || gemm8_applicable(a)) return false;
-    return gemv_tile_rows_applicable(a) || gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
+    if (gemm_tile_mt_splits_parts(a)) return false;  // wide and narrow parts: each on the kernel of its own layer
+    return gemv_tile_rows_applicable(a) || gemm_tile_mt_applicable(a) || gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
 }
 
 // argument checks shared by nq_forward and nq_forward_fused, then the launch(es)
@@ -527,7 +540,7 @@ int32_t nq_fuse_rows(nq_handle* out, const nq_handle* layers, int32_t n, void* s
     if (!F) return fail(NQ_ERR_INVALID, "nq_fuse_rows: out of host memory");
     F->format = a->format, F->in = a->in, F->out = (int32_t)rows, F->group = a->group, F->groups = a->groups;
     F->scale = a->scale, F->row_bytes = a->row_bytes, F->device = a->device;
-    F->no_tile_copy = a->no_tile_copy;
+    F->no_tile_copy = a->no_tile_copy, F->prefer_tile = a->prefer_tile;
     int32_t rc = bind_device(F);
     if (rc) {
         delete F;
@@ -601,7 +614,8 @@ int32_t nq_fuse_glu(nq_handle* out, nq_handle gate, nq_handle up, void* stream) 
     if (!F) return fail(NQ_ERR_INVALID, "nq_fuse_glu: out of host memory");
     F->format = a->format, F->in = a->in, F->out = 2 * a->out, F->group = a->group, F->groups = a->groups;
     F->scale = a->scale, F->row_bytes = a->row_bytes, F->device = a->device;
-    F->glu = true, F->no_tile_copy = true;  // (the tile kernels keep a pair in two workgroups)
+    F->no_tile_copy = a->no_tile_copy, F->prefer_tile = a->prefer_tile;
+    F->glu = true;  // (of the tile kernels only the M-tile one carries the SwiGLU epilogue: the others check `glu`)
     int32_t rc = bind_device(F);
     if (rc) {
         delete F;
@@ -631,10 +645,12 @@ int32_t nq_fuse_glu(nq_handle* out, nq_handle gate, nq_handle up, void* stream) 
                                  (size_t)F->groups, (size_t)H, hipMemcpyDeviceToDevice, s);
     }
     if (e == hipSuccess) e = hipStreamSynchronize(s);
-    if (e != hipSuccess) {
+    if (e == hipSuccess) rc = build_tile_copy(F, s);
+    if (e == hipSuccess && rc == NQ_OK) e = hipStreamSynchronize(s);
+    if (e != hipSuccess || rc != NQ_OK) {
         free_device(F);
         delete F;
-        return fail_hip(e, "nq_fuse_glu");
+        return e != hipSuccess ? fail_hip(e, "nq_fuse_glu") : rc;
     }
     F->loaded = true;
     *out = F;

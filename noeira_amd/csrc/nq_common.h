@@ -72,6 +72,7 @@ struct nq_layer {
     void* d_tile16_scales = nullptr;
     int32_t tile_nj = 0;
     bool no_tile_copy = false;  // NQ_FLAG_NO_TILE_COPY
+    bool prefer_tile = false;   // NQ_FLAG_PREFER_TILE
     float scale = 1.0f;
     int64_t row_bytes = 0;     // bytes of one row of d_codes
     std::vector<int32_t> seg_end;  // a row-fused layer: the end row of each fused part (else empty)
@@ -170,6 +171,9 @@ bool tile_copy_wanted(const nq_layer* L);
 int32_t build_tile_copy(nq_layer* L, hipStream_t s);
 bool gemv_tile_applicable(const ForwardArgs& a);
 bool gemv_tile_rows_applicable(const ForwardArgs& a);
+bool gemm_tile_mt_applicable(const ForwardArgs& a);
+bool gemm_tile_mt_splits_parts(const ForwardArgs& a);
+int32_t launch_gemm_tile_mt(const ForwardArgs& a);
 int32_t launch_gemv_tile_rows(const ForwardArgs& a);
 int32_t launch_gemv_tile(const ForwardArgs& a);
 

@@ -448,6 +448,225 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
     }
 }
 
+// ---- tens to hundreds of activation rows over 4-bit codes ------------------------------------------------
+// The same scheme over tiles of M: workgroup (x, y) owns the 16 activation rows of M tile y - their A operands for
+// all of K sit in its wavefronts' registers for the whole call - and walks a share of the 16-row weight tiles.
+// KW wavefronts split K (JPW steps of 128 k each) and the 16 / KW groups of them take different weight tiles at the
+// same time; a group's [16 x 16] shares meet in LDS in wave order and 256 of its threads finish the tile (bias,
+// ReLU or SwiGLU, part placement).  fp32 activations are three exact bf16 terms per value, i.e. three A operands
+// and three MFMAs per chunk into one accumulator (JPW = 1 only: beyond, the operands no longer fit the registers).
+// A weight tile is read once per M tile (from L2 after the first), an activation once per workgroup; K, the group
+// count and the sum order follow IN alone, so a row gets the same bits in its own layer and in a row-fused one.
+template <int FMT, bool XF32, int JPW, int TB>
+__global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams pm, const int kw) {
+    const TileParams& p = pm.t;
+    constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
+    constexpr int NT = XF32 ? 3 : 1;
+    constexpr bool XS_REGS = G128 || JPW <= 2;
+    __shared__ __attribute__((aligned(16))) float red[2][16][256];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const int ng = 16 / kw;                      // groups of wavefronts, each on its own weight tile
+    const int grp = wave / kw, kwi = wave - grp * kw;
+    const bool active = grp < ng;
+    const int ntiles = (p.N + 15) / 16;
+    const int J0 = kwi * JPW;
+    const int m0 = blockIdx.y * 16;
+    const int rows = min(16, pm.M - m0);
+    const int xrow = m0 + min(c, rows - 1);
+    uint32_t magic = 0x41804180u;
+    asm volatile("" : "+v"(magic));
+
+    // a group's tiles: first, first + stride, ...; fetched TB at a time, a batch ahead of their use.  (TB = 1 is
+    // what is launched: with 2 or 4 tiles in flight the same calls measured 3 - 10 % slower - the kernel is bound by
+    // the vector ALU's share of a tile (nibbles -> bf16, the scale per chunk), not by the trip to L2.)
+    const int stride = gridDim.x * ng;
+    const int first = blockIdx.x * ng + min(grp, ng - 1);
+    auto fetch = [&](int it0, u32x4 (&wv)[TB][JPW], uint2 (&sc)[TB][JPW]) {
+#pragma unroll
+        for (int t = 0; t < TB; t++) {
+            const int64_t R = min(first + (it0 + t) * stride, ntiles - 1);
+#pragma unroll
+            for (int j = 0; j < JPW; j++) {
+                const int64_t at = R * p.NJ + min(J0 + j, p.NJ - 1);
+                wv[t][j] = p.tile[at * 64 + lane];
+                if constexpr (!G128) sc[t][j] = reinterpret_cast<const uint2*>(p.tscales)[at * 16 + c];
+                else sc[t][j].x = reinterpret_cast<const uint32_t*>(p.tscales)[at * 16 + c], sc[t][j].y = 0;
+            }
+        }
+    };
+    u32x4 wv[TB][JPW], wn[TB][JPW];
+    uint2 sc[TB][JPW], sn[TB][JPW];
+    fetch(0, wv, sc);
+
+    // ---- A operands, once: 16 bytes of bf16 per (term, step, MFMA); rows past M and k past K are zero
+    u32x4 aop[NT][JPW][4];
+#pragma unroll
+    for (int j = 0; j < JPW; j++)
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int k0 = (J0 + j) * 128 + 32 * m + 8 * q;
+            const int k = min(k0, p.K - 8);
+            const uint32_t keep = (c < rows && k0 < p.K && active) ? ~0u : 0u;
+            if constexpr (XF32) {
+                const float* xf = reinterpret_cast<const float*>(p.x) + (int64_t)xrow * p.K + k;
+                const u32x4 r0 = *reinterpret_cast<const u32x4*>(xf), r1 = *reinterpret_cast<const u32x4*>(xf + 4);
+                uint32_t v[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = r0[i] & keep, v[4 + i] = r1[i] & keep;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    // hi + mid + lo = the fp32 value (each split truncates: every residual is exact)
+                    const uint32_t a = v[2 * i], b = v[2 * i + 1];
+                    const float ra = __uint_as_float(a) - __uint_as_float(a & 0xFFFF0000u);
+                    const float rb = __uint_as_float(b) - __uint_as_float(b & 0xFFFF0000u);
+                    const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                    const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                    aop[0][j][m][i] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+                    aop[1][j][m][i] = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+                    aop[2][j][m][i] = __builtin_amdgcn_perm(__float_as_uint(sb), __float_as_uint(sa), 0x07060302u);
+                }
+            } else {
+                u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + (int64_t)xrow * p.K + k);
+#pragma unroll
+                for (int i = 0; i < 4; i++) t[i] &= keep;
+                aop[0][j][m] = t;
+            }
+        }
+    // ---- the rows' sums of x under every chunk (Q4_0, times -24) or group of 128, in the product's layout
+    const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto chunk_sum = [&](int j, int m, f32x4 into) {
+#pragma unroll
+        for (int t = NT - 1; t >= 0; t--)  // (smallest term first)
+            into = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[t][j][m]), as_bf16x8(ones), into, 0, 0, 0);
+        return into;
+    };
+    f32x4 xs[XS_REGS ? JPW : 1][G128 ? 1 : 4];
+    if constexpr (XS_REGS) {
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            if constexpr (G128) {
+                xs[j][0] = zero4;
+#pragma unroll
+                for (int m = 0; m < 4; m++) xs[j][0] = chunk_sum(j, m, xs[j][0]);
+            } else {
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    xs[j][m] = chunk_sum(j, m, zero4);
+#pragma unroll
+                    for (int t = 0; t < 4; t++) xs[j][m][t] *= -24.0f;
+                }
+            }
+        }
+    }
+    // this thread's place in its group's finished tile: token row fr, weight row (column of y) fc
+    const int f = threadIdx.x - grp * kw * 64;
+    const bool finisher = active && f < 256;
+    const int fr = (f >> 4) & 15, fc = f & 15;
+
+    const int iters = (ntiles + stride - 1) / stride;
+    int buf = 0;
+    for (int it0 = 0; it0 < iters; it0 += TB) {
+      const bool more = it0 + TB < iters;
+      if (more) fetch(it0 + TB, wn, sn);  // the next batch is on its way while this one is multiplied
+#pragma unroll
+      for (int tb = 0; tb < TB; tb++) {
+        const int it = it0 + tb;
+        if (it >= iters) break;  // (uniform)
+        const int tile = first + it * stride;
+        const bool have = active && tile < ntiles;
+        uint32_t braw = 0;
+        const int64_t fn = min((int64_t)tile * 16 + fc, (int64_t)p.N - 1);
+        if (p.bias && finisher)
+            braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[fn]
+                                               : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[fn];
+        if (have) {
+            f32x4 acc = zero4;
+#pragma unroll
+            for (int j = 0; j < JPW; j++) {
+                const bool live = J0 + j < p.NJ;  // (a step past K: its A operand is zero; its scale is set to zero too)
+                if constexpr (!G128) {
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        const u32x4 bop = nib_word_to_bf16(wv[tb][j][m], magic);
+                        f32x4 dd;
+                        if constexpr (XS_REGS) {
+                            dd = xs[j][m];
+                        } else {
+                            dd = chunk_sum(j, m, zero4);
+#pragma unroll
+                            for (int t = 0; t < 4; t++) dd[t] *= -24.0f;
+                        }
+#pragma unroll
+                        for (int t = NT - 1; t >= 0; t--)
+                            dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[t][j][m]), as_bf16x8(bop), dd, 0, 0, 0);
+                        const uint32_t sbits = (m < 2 ? sc[tb][j].x : sc[tb][j].y) >> (16 * (m & 1));
+                        const float d = live ? __half2float(__ushort_as_half((uint16_t)(sbits & 0xFFFFu))) : 0.0f;
+#pragma unroll
+                        for (int t = 0; t < 4; t++) acc[t] = fmaf(d, dd[t], acc[t]);
+                    }
+                } else {
+                    const float d = live ? __half2float(__ushort_as_half((uint16_t)(sc[tb][j].x & 0xFFFFu))) : 0.0f;
+                    const float zoff = -(16.0f + (float)(sc[tb][j].x >> 16));
+                    f32x4 dd;
+#pragma unroll
+                    for (int t = 0; t < 4; t++) dd[t] = zoff * xs[j][0][t];
+#pragma unroll
+                    for (int m = 0; m < 4; m++) {
+                        const u32x4 bop = nib_word_to_bf16(wv[tb][j][m], magic);
+#pragma unroll
+                        for (int t = NT - 1; t >= 0; t--)
+                            dd = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[t][j][m]), as_bf16x8(bop), dd, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int t = 0; t < 4; t++) acc[t] = fmaf(d, dd[t], acc[t]);
+                }
+            }
+            *reinterpret_cast<f32x4*>(&red[buf][wave][lane * 4]) = acc;
+        }
+        __syncthreads();
+        // D[v][cc] sits in lane cc + 16 (v / 4), register v % 4: v the token row, cc the weight row
+        if (finisher && have) {
+            const int at = (fc + 16 * (fr >> 2)) * 4 + (fr & 3);
+            const float* r0 = &red[buf][grp * kw][at];  // the group's shares, in wave order
+            float z = r0[0];
+            for (int w = 1; w < kw; w++) z += r0[w * 256];
+            const int n = tile * 16 + fc;
+            if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
+            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+            if (p.epilogue == NQ_EPI_SWIGLU) {  // (uniform) gate in the even column, up one lane over
+                const float other = lane_xor1(z);
+                if ((n & 1) == 0 && n + 1 < p.N && fr < rows) {
+                    const float g = swiglu_f32(other, z);
+                    const int64_t o = (int64_t)(m0 + fr) * (p.N >> 1) + (n >> 1);
+                    if (p.y_dtype == NQ_DT_F32)
+                        reinterpret_cast<float*>(p.seg.y[0])[o] = g;
+                    else
+                        reinterpret_cast<uint16_t*>(p.seg.y[0])[o] = f32_to_bf16_rne(g);
+                }
+            } else if (n < p.N && fr < rows) {
+                void* yp;
+                int width, col;
+                seg_lookup(p.seg, n, yp, width, col);
+                const int64_t o = (int64_t)(m0 + fr) * width + col;
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(yp)[o] = z;
+                else
+                    reinterpret_cast<uint16_t*>(yp)[o] = f32_to_bf16_rne(z);
+            }
+        }
+        buf ^= 1;
+      }
+      if (more) {
+#pragma unroll
+        for (int t = 0; t < TB; t++)
+#pragma unroll
+            for (int j = 0; j < JPW; j++) wv[t][j] = wn[t][j], sc[t][j] = sn[t][j];
+      }
+    }
+}
+
 // ---- int8 codes -----------------------------------------------------------------------------------
 constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: the low byte of (t + MAGIC)'s bits is rne(t) as an int8
 
@@ -576,25 +795,27 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p)
 
 // ---- load time: the tile-ordered copies -------------------------------------------------------------
 // codes [N][nch][4 words] (row order) -> tile[R][J][lane][4 words]; one thread per lane slot
+// (nch: 16-byte chunks per row; a row's last tile may hold fewer than four: the rest is zero codes under zero scales)
 __global__ __launch_bounds__(256) void tile4_repack_kernel(const uint32_t* __restrict__ codes, u32x4* __restrict__ tile,
-                                                           int64_t N, int64_t NJ, int64_t slots) {
+                                                           int64_t N, int64_t NJ, int64_t nch, int64_t slots) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= slots) return;
     const int l = (int)(t & 63), c = l & 15, q = l >> 4;
     const int64_t J = (t >> 6) % NJ, R = (t >> 6) / NJ, row = R * 16 + c;
     u32x4 v = {0, 0, 0, 0};
     if (row < N) {
-        const uint32_t* src = codes + (row * NJ * 4 + J * 4) * 4 + q;  // chunk 4 J of the row, word q
+        const uint32_t* src = codes + (row * nch + J * 4) * 4 + q;  // chunk 4 J of the row, word q
 #pragma unroll
-        for (int m = 0; m < 4; m++) v[m] = src[m * 4];
+        for (int m = 0; m < 4; m++)
+            if (J * 4 + m < nch) v[m] = src[m * 4];
     }
     tile[t] = v;
 }
 
 // Q4_0 scales [N][nch] fp16 -> [R][J][c][4]; groups of 128: scales [N][G] fp16, zps [N][G] -> [R][J][c] u32
 __global__ __launch_bounds__(256) void tile4_scales_kernel(const uint16_t* __restrict__ scales, const uint8_t* __restrict__ zps,
-                                                           uint32_t* __restrict__ out, int64_t N, int64_t NJ, int64_t count,
-                                                           int g128) {
+                                                           uint32_t* __restrict__ out, int64_t N, int64_t NJ, int64_t nch,
+                                                           int64_t count, int g128) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= count) return;
     const int c = (int)(t & 15);
@@ -604,8 +825,11 @@ __global__ __launch_bounds__(256) void tile4_scales_kernel(const uint16_t* __res
     } else {
         uint32_t lo = 0, hi = 0;
         if (row < N) {
-            const uint16_t* s = scales + row * NJ * 4 + J * 4;
-            lo = (uint32_t)s[0] | ((uint32_t)s[1] << 16), hi = (uint32_t)s[2] | ((uint32_t)s[3] << 16);
+            const uint16_t* s = scales + row * nch + J * 4;
+            uint32_t v[4];
+#pragma unroll
+            for (int m = 0; m < 4; m++) v[m] = J * 4 + m < nch ? (uint32_t)s[m] : 0u;
+            lo = v[0] | (v[1] << 16), hi = v[2] | (v[3] << 16);
         }
         out[2 * t] = lo, out[2 * t + 1] = hi;
     }
@@ -693,19 +917,67 @@ int32_t launch4_rows(const TileMrParams& pm, hipStream_t s) {
     return NQ_OK;
 }
 
+// The K split of the M-tile kernel, from IN alone: JPW steps per wavefront, KW wavefronts per group (at least 4, so
+// that a group has the 256 threads that finish its tile), 16 / KW groups; the choice that keeps most of the 16
+// wavefronts busy.
+inline void mt_split(int nj, bool xf32, int& jpw, int& kw) {
+    double best = -1.0;
+    jpw = 0, kw = 0;
+    for (int j = 1; j <= (xf32 ? 1 : 3); j++) {
+        const int w = std::max(4, (nj + j - 1) / j);
+        if (w > 16) continue;
+        const double util = (double)nj / (w * j) * ((16 / w) * w) / 16.0;
+        if (util > best + 1e-9) best = util, jpw = j, kw = w;
+    }
+}
+
+template <int FMT, bool XF32>
+int32_t launch4_mt(const TileMrParams& pm, hipStream_t s) {
+    int jpw, kw;
+    mt_split(pm.t.NJ, XF32, jpw, kw);
+    if (!jpw) return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no M-tile kernel for this IN");
+    int dev = 0, cus = 0;
+    NQ_HIP(hipGetDevice(&dev));
+    NQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int ng = 16 / kw, ntiles = (pm.t.N + 15) / 16, mt = (pm.M + 15) / 16;
+    const int gx = std::max(1, std::min((ntiles + ng - 1) / ng, std::max(cus, 1) / mt));
+    const dim3 grid((unsigned)gx, (unsigned)mt);
+    if constexpr (XF32) {
+        hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, true, 1, 1>), grid, dim3(1024), 0, s, pm, kw);
+    } else {
+        switch (jpw) {
+            case 1: hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 1, 1>), grid, dim3(1024), 0, s, pm, kw); break;
+            case 2: hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 2, 1>), grid, dim3(1024), 0, s, pm, kw); break;
+            default: hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 3, 1>), grid, dim3(1024), 0, s, pm, kw); break;
+        }
+    }
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
 }  // namespace
 
 // Which layers get the tile-ordered copy (a second copy of the codes: 0.5 or 1 byte per weight on top):
 // weights of 4 M codes and more, whose single-row calls are bound by the weight stream.  4-bit: Q4_0 or
 // groups of exactly 128, IN a multiple of 128 in 2048 .. 16384; int8: IN a multiple of 64, at least 1024.
+// 4-bit layers whose rows are at most 6144 codes long get it whatever their size (IN alone decides, so that a
+// row-fused layer and its parts agree): the kernel for tens to hundreds of activation rows reads it.
 bool tile_copy_wanted(const nq_layer* L) {
     if (L->no_tile_copy) return false;
-    if ((int64_t)L->in * ((L->out + 15) / 16 * 16) >= ((int64_t)1 << 32)) return false;  // (32-bit offsets in a tile copy)
+    if ((int64_t)((L->in + 127) / 128 * 128) * ((L->out + 15) / 16 * 16) >= ((int64_t)1 << 32)) return false;  // (32-bit offsets in a tile copy)
+    const bool four = L->format == NQ_FMT_Q4_0 || (L->format == NQ_FMT_W4_GROUP && L->group == 128);
+    if (four && L->in % 32 == 0 && L->in >= 512 && L->in <= 6144) return true;
     if ((int64_t)L->in * L->out < ((int64_t)4 << 20)) return false;
-    if (L->format == NQ_FMT_Q4_0 || (L->format == NQ_FMT_W4_GROUP && L->group == 128))
-        return L->in % 128 == 0 && L->in >= 2048 && L->in <= 16384;
+    if (four) return L->in % 128 == 0 && L->in >= 2048 && L->in <= 16384;
     if (L->format == NQ_FMT_W8_CHANNEL) return L->in % 64 == 0 && L->in >= 1024;
     return false;
+}
+
+// the layers whose single-row (and 2 .. 16 row) calls are bound by the weight stream: 4 M codes and more
+static bool stream_bound_layer(const nq_layer* L) {
+    if ((int64_t)L->in * L->out < ((int64_t)4 << 20)) return false;
+    if (L->format == NQ_FMT_W8_CHANNEL) return true;
+    return L->in % 128 == 0 && L->in >= 2048;
 }
 
 // builds (or drops) the tile-ordered copy from the row-ordered device arrays of a loaded layer
@@ -716,7 +988,7 @@ int32_t build_tile_copy(nq_layer* L, hipStream_t s) {
     if (!tile_copy_wanted(L)) return NQ_OK;
     const int64_t N = L->out, R = (N + 15) / 16;
     const bool w8 = L->format == NQ_FMT_W8_CHANNEL;
-    const int64_t NJ = w8 ? L->in / 64 : L->in / 128;
+    const int64_t NJ = w8 ? L->in / 64 : (L->in + 127) / 128;
     const int64_t slots = R * NJ * 64;
     NQ_HIP(hipMalloc((void**)&L->d_tile16, (size_t)slots * 16));
     if (w8) {
@@ -727,10 +999,11 @@ int32_t build_tile_copy(nq_layer* L, hipStream_t s) {
         const int64_t count = R * NJ * 16;
         NQ_HIP(hipMalloc(&L->d_tile16_scales, (size_t)count * (g128 ? 4 : 8)));
         hipLaunchKernelGGL(tile4_repack_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, s,
-                           reinterpret_cast<const uint32_t*>(L->d_codes), reinterpret_cast<u32x4*>(L->d_tile16), N, NJ, slots);
+                           reinterpret_cast<const uint32_t*>(L->d_codes), reinterpret_cast<u32x4*>(L->d_tile16), N, NJ,
+                           (int64_t)L->in / 32, slots);
         hipLaunchKernelGGL(tile4_scales_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s,
                            reinterpret_cast<const uint16_t*>(L->d_scales), L->d_zps,
-                           reinterpret_cast<uint32_t*>(L->d_tile16_scales), N, NJ, count, (int)g128);
+                           reinterpret_cast<uint32_t*>(L->d_tile16_scales), N, NJ, (int64_t)L->in / 32, count, (int)g128);
     }
     NQ_HIP(hipGetLastError());
     L->tile_nj = (int32_t)NJ;
@@ -739,7 +1012,7 @@ int32_t build_tile_copy(nq_layer* L, hipStream_t s) {
 
 bool gemv_tile_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
-    if (a.M != 1 || !L->d_tile16) return false;
+    if (a.M != 1 || !L->d_tile16 || L->glu || !stream_bound_layer(L)) return false;
     if (a.x_dtype != NQ_DT_BF16 && a.x_dtype != NQ_DT_F32) return false;
     return a.y_dtype == NQ_DT_F32 || a.y_dtype == NQ_DT_BF16;
 }
@@ -749,11 +1022,60 @@ bool gemv_tile_applicable(const ForwardArgs& a) {
 // the kernel spills)
 bool gemv_tile_rows_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
-    if (!L->d_tile16 || L->format == NQ_FMT_W8_CHANNEL || L->tile_nj > 48) return false;
+    if (!L->d_tile16 || L->format == NQ_FMT_W8_CHANNEL || L->tile_nj > 48 || L->glu || !stream_bound_layer(L)) return false;
     if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
     if (a.x_dtype == NQ_DT_BF16) return a.M >= 2 && a.M <= 16;
     if (a.x_dtype == NQ_DT_F32) return a.M >= 2 && a.M <= 5;
     return false;
+}
+
+// 96 .. 256 rows of bf16 activations, or 96 .. 512 of fp32 ones where IN <= 2048, over a wide 4-bit layer with a tile copy.
+// Where it wins over the 16-row tile kernel was measured at IN = 960 / 2560, OUT = 320 .. 5120, M = 17 .. 512: wide
+// layers (it amortises a workgroup's start over many weight tiles; a narrow layer gives it one or two), a hundred
+// rows and more.  Everything but the width:
+static bool mt_shape_ok(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (!L->d_tile16 || L->format == NQ_FMT_W8_CHANNEL || L->tile_nj > 48) return false;
+    if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
+    if ((int64_t)a.M * L->in >= ((int64_t)1 << 31)) return false;
+    if (a.M < 2 || a.M > 512) return false;
+    if (!L->prefer_tile && a.M < 96) return false;
+    if (a.x_dtype == NQ_DT_BF16) return L->prefer_tile || a.M <= 256;
+    return a.x_dtype == NQ_DT_F32 && L->tile_nj <= 16;
+}
+constexpr int MT_WIDE = 2048;
+
+// The width that counts is each part's own: a row-fused layer runs on this kernel in one launch when all its parts
+// are wide, on the other kernel when none is, and part by part when they differ (gemm_tile_mt_splits_parts), so that
+// a part gets the kernel - and the bits - of its own layer's forward.
+bool gemm_tile_mt_applicable(const ForwardArgs& a) {
+    if (!mt_shape_ok(a)) return false;
+    if (a.L->prefer_tile || a.L->glu) return a.L->prefer_tile || a.L->out >= MT_WIDE;
+    for (int i = 0, prev = 0; i < a.seg.nseg; prev = a.seg.end[i], i++)
+        if (a.seg.end[i] - prev < MT_WIDE) return false;
+    return true;
+}
+
+bool gemm_tile_mt_splits_parts(const ForwardArgs& a) {
+    if (a.seg.nseg < 2 || a.L->prefer_tile || !mt_shape_ok(a)) return false;
+    int wide = 0;
+    for (int i = 0, prev = 0; i < a.seg.nseg; prev = a.seg.end[i], i++) wide += a.seg.end[i] - prev >= MT_WIDE;
+    return wide > 0 && wide < a.seg.nseg;
+}
+
+int32_t launch_gemm_tile_mt(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    TileMrParams pm{};
+    TileParams& p = pm.t;
+    p.tile = reinterpret_cast<const u32x4*>(L->d_tile16), p.tscales = L->d_tile16_scales, p.col_scale = nullptr;
+    p.x = a.x, p.bias = a.bias, p.seg = a.seg;
+    p.N = L->out, p.K = L->in, p.NJ = L->tile_nj;
+    p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    pm.M = a.M;
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
+    if (L->format == NQ_FMT_Q4_0)
+        return xf32 ? launch4_mt<NQ_FMT_Q4_0, true>(pm, a.stream) : launch4_mt<NQ_FMT_Q4_0, false>(pm, a.stream);
+    return xf32 ? launch4_mt<NQ_FMT_W4_GROUP, true>(pm, a.stream) : launch4_mt<NQ_FMT_W4_GROUP, false>(pm, a.stream);
 }
 
 int32_t launch_gemv_tile_rows(const ForwardArgs& a) {

@@ -59,12 +59,12 @@ class _Layer:
 
     FORMAT = -1
 
-    def __init__(self, IN: int, OUT: int, group: int = 0, tile_copy: bool = True):
+    def __init__(self, IN: int, OUT: int, group: int = 0, tile_copy: bool = True, prefer_tile: bool = False):
         """tile_copy=False (NQ_FLAG_NO_TILE_COPY): a large layer does not keep the second,
         matrix-core-ordered copy of its codes that its single-row calls stream faster."""
         self.IN, self.OUT, self.group = int(IN), int(OUT), int(group)
         h = C.c_void_p()
-        flags = 0 if tile_copy else L.FLAG_NO_TILE_COPY
+        flags = (0 if tile_copy else L.FLAG_NO_TILE_COPY) | (L.FLAG_PREFER_TILE if prefer_tile else 0)
         L.check(L.lib().nq_create(C.byref(h), self.FORMAT, self.IN, self.OUT, self.group, flags))
         self._h = h
         self._loaded = False
@@ -136,10 +136,10 @@ class QLinear(_Layer):
     FORMAT = L.FMT_Q4_0
     ARITY = 1
 
-    def __init__(self, IN: int, OUT: int, tile_copy: bool = True):
+    def __init__(self, IN: int, OUT: int, tile_copy: bool = True, prefer_tile: bool = False):
         if IN % Q4_GROUP != 0:  # the comptime assert of qlinear.mojo:243-245
             raise L.NQError(L.NQ_ERR_INVALID, "QLinear: IN must be a multiple of 32 (one Q4_0 group)")
-        super().__init__(IN, OUT, Q4_GROUP, tile_copy)
+        super().__init__(IN, OUT, Q4_GROUP, tile_copy, prefer_tile)
         self.W_SIZE = IN * OUT
         self.ROW_BYTES = (IN // Q4_GROUP) * Q4_BLOCK
         self.BYTES = OUT * self.ROW_BYTES
@@ -291,8 +291,8 @@ class W4GroupLinear(_Layer):
 
     FORMAT = L.FMT_W4_GROUP
 
-    def __init__(self, IN, OUT, group=128, tile_copy: bool = True):
-        super().__init__(IN, OUT, group, tile_copy)
+    def __init__(self, IN, OUT, group=128, tile_copy: bool = True, prefer_tile: bool = False):
+        super().__init__(IN, OUT, group, tile_copy, prefer_tile)
         self.G = -(-IN // group)
 
     @classmethod
