@@ -444,9 +444,17 @@ bool places_parts(const ForwardArgs& a) {
 }
 
 // argument checks shared by nq_forward and nq_forward_fused, then the launch(es)
+// (lora: an adapter to fold into the launch, or null; folded only where the M-tile kernel is the one that runs the
+// base call anyway - `*folded` says whether it was)
+struct LoraArgs {
+    const float* a;
+    const float* b;
+    int32_t r;
+    float s;
+};
 int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, const SegTable& seg,
                      int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue,
-                     void* stream) {
+                     void* stream, const LoraArgs* lora = nullptr, bool* folded = nullptr) {
     if (((uintptr_t)x & 15)) return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
     for (int t = 0; t < seg.nseg; t++)
         if (!seg.y[t] || ((uintptr_t)seg.y[t] & 3))
@@ -483,6 +491,12 @@ int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x
         }
     }
     ForwardArgs a{h, x, x_dtype, x_scale, seg.y[0], y_dtype, M, bias, bias_dtype, epilogue, (hipStream_t)stream, seg};
+    if (lora && seg.nseg == 1 && lora->r <= 16 && !h->glu && epilogue == NQ_EPI_NONE && x_dtype != NQ_DT_I8 &&
+        !gemv_fp8_applicable(a) && !gemm8_applicable(a) && !gemv_tile_rows_applicable(a) && gemm_tile_mt_applicable(a) && gemm_tile_mt_lora_foldable(a)) {
+        a.lora_a = lora->a, a.lora_b = lora->b, a.lora_r = lora->r, a.lora_s = lora->s;
+        *folded = true;
+        return launch_gemm_tile_mt(a);
+    }
     if (seg.nseg == 1 || places_parts(a)) return dispatch(a);
     // one launch per part, each on a view of its rows
     const int bias_es = bias_dtype == NQ_DT_F32 ? 4 : 2;
@@ -706,6 +720,32 @@ int32_t nq_grad_input(nq_handle h, const float* gy, float* gx, int32_t M, void* 
     if (M == 0) return NQ_OK;
     if (!gy || !gx) return fail(NQ_ERR_INVALID, "nq_grad_input: null gy or gx");
     return launch_grad_input_q4_0(h, gy, gx, M, (hipStream_t)stream);
+}
+
+int32_t nq_forward_lora(nq_handle h, const void* x, int32_t x_dtype, void* y, int32_t y_dtype, int32_t M,
+                        const void* bias, int32_t bias_dtype, const float* lora_a, const float* lora_b, int32_t r_pad,
+                        float scale, void* stream) {
+    int32_t rc = check_handle(h, "nq_forward_lora");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward_lora: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!x || !y || !lora_a || !lora_b) return fail(NQ_ERR_INVALID, "nq_forward_lora: null pointer");
+    if (r_pad <= 0) return fail(NQ_ERR_INVALID, "nq_forward_lora: R_PAD must be positive");
+    if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "nq_forward_lora: x must be fp32 or bf16");
+    SegTable seg{};
+    seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
+    const LoraArgs lora{lora_a, lora_b, r_pad, scale};
+    bool folded = false;
+    rc = forward_impl(h, x, x_dtype, nullptr, seg, y_dtype, M, bias, bias_dtype, NQ_EPI_NONE, stream, &lora, &folded);
+    if (rc || folded) return rc;
+    // the base call ran on another kernel: the adapter as a launch of its own, into the fp32 output
+    if (y_dtype != NQ_DT_F32)
+        return fail(NQ_ERR_UNSUPPORTED, "nq_forward_lora: for this layer and M the adapter is a second launch that adds "
+                                        "into an fp32 y; ask for fp32 output");
+    return nq_lora_forward_add(lora_a, lora_b, h->in, h->out, r_pad, scale, x, x_dtype, reinterpret_cast<float*>(y), M,
+                               stream);
 }
 
 int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features, int32_t out_features, int32_t r_pad,

@@ -129,6 +129,11 @@ struct ForwardArgs {
     int32_t epilogue;
     hipStream_t stream;
     SegTable seg;  // seg.y[0] == y and seg.end[0] == OUT for an ordinary call
+    // nq_forward_lora: the adapter folded into the launch (only the M-tile kernel reads these)
+    const float* lora_a = nullptr;
+    const float* lora_b = nullptr;
+    int32_t lora_r = 0;
+    float lora_s = 0.0f;
 };
 
 // nq_q4_0.hip
@@ -173,6 +178,7 @@ bool gemv_tile_applicable(const ForwardArgs& a);
 bool gemv_tile_rows_applicable(const ForwardArgs& a);
 bool gemm_tile_mt_applicable(const ForwardArgs& a);
 bool gemm_tile_mt_splits_parts(const ForwardArgs& a);
+bool gemm_tile_mt_lora_foldable(const ForwardArgs& a);
 int32_t launch_gemm_tile_mt(const ForwardArgs& a);
 int32_t launch_gemv_tile_rows(const ForwardArgs& a);
 int32_t launch_gemv_tile(const ForwardArgs& a);

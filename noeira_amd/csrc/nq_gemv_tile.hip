@@ -277,6 +277,11 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
 struct TileMrParams {
     TileParams t;
     int32_t M;
+    // a frozen LoRA adapter folded into the call (the M-tile kernel only; null = none): y += ls * (x la) lb
+    const float* la;  // [IN][lr] fp32
+    const float* lb;  // [lr][OUT] fp32
+    int32_t lr;       // rank as stored (padded), <= 16
+    float ls;
 };
 
 template <int FMT, bool XF32, int JPW>
@@ -457,12 +462,17 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
 // and three MFMAs per chunk into one accumulator (JPW = 1 only: beyond, the operands no longer fit the registers).
 // A weight tile is read once per M tile (from L2 after the first), an activation once per workgroup; K, the group
 // count and the sum order follow IN alone, so a row gets the same bits in its own layer and in a row-fused one.
-template <int FMT, bool XF32, int JPW, int TB>
+// LORA: `y += s (x A) B` of a frozen adapter (noeira/nn/peft/lora.mojo:292-349) in the same launch.  The workgroup
+// holds its rows' x for all of K already, so h = x A [16 x rank] costs it a handful of MFMAs once (A's fp32 values as
+// three exact bf16 terms against the one or three terms of x, products below 2^-24 of the largest left out), summed
+// over the K split through LDS; the threads that finish a tile add s * h[row] . B[:, column] to it before the store.
+// With B = 0 the sum is an exact zero and the base result keeps its bits.
+template <int FMT, bool XF32, int JPW, int TB, bool LORA>
 __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams pm, const int kw) {
     const TileParams& p = pm.t;
     constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
     constexpr int NT = XF32 ? 3 : 1;
-    constexpr bool XS_REGS = G128 || JPW <= 2;
+    constexpr bool XS_REGS = (G128 || JPW <= 2) && !(LORA && !G128 && (XF32 || JPW >= 2));  // (registers: the adapter's operands need them)
     __shared__ __attribute__((aligned(16))) float red[2][16][256];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, q = lane >> 4;
@@ -565,6 +575,60 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
     const bool finisher = active && f < 256;
     const int fr = (f >> 4) & 15, fc = f & 15;
 
+    __shared__ float hfin[LORA ? 4 : 1][16][17];
+    if constexpr (LORA) {
+        // h = x A over this wavefront's share of K: the MFMA's B operand is A[k][r] for 8 consecutive k of column
+        // r = lane % 16 (ranks past lr, and k past K, are zero)
+        // (the groups of a workgroup hold the same x: each forms h over every ng-th chunk and all sixteen shares
+        // are summed, so that the splitting of A into bf16 terms - the vector ALU's work here - is done once)
+        const int rc = min(c, pm.lr - 1);
+        f32x4 hacc = zero4;
+#pragma unroll
+        for (int j = 0; j < JPW; j++)
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const int ci = j * 4 + m;
+                const bool mine = active && (ng == 1 || (ng == 2 && ((ci ^ grp) & 1) == 0) || (ng == 3 && ci % 3 == grp) ||
+                                             (ng == 4 && (ci & 3) == grp));
+                if (!mine) continue;  // (uniform)
+                const int k0 = (J0 + j) * 128 + 32 * m + 8 * q;
+                const uint32_t keep = (c < pm.lr && k0 < p.K && active) ? ~0u : 0u;
+                uint32_t av[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    av[i] = reinterpret_cast<const uint32_t*>(pm.la)[(int64_t)min(k0 + i, p.K - 1) * pm.lr + rc];
+                u32x4 pl[3];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t a0 = av[2 * i] & keep, b0 = av[2 * i + 1] & keep;
+                    const float ra = __uint_as_float(a0) - __uint_as_float(a0 & 0xFFFF0000u);
+                    const float rb = __uint_as_float(b0) - __uint_as_float(b0 & 0xFFFF0000u);
+                    const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                    const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                    pl[0][i] = __builtin_amdgcn_perm(b0, a0, 0x07060302u);
+                    pl[1][i] = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+                    pl[2][i] = __builtin_amdgcn_perm(__float_as_uint(sb), __float_as_uint(sa), 0x07060302u);
+                }
+                auto mm = [&](int xt, int at) {
+                    hacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[xt][j][m]), as_bf16x8(pl[at]), hacc, 0, 0, 0);
+                };
+                if constexpr (XF32) {  // smallest products first
+                    mm(1, 1), mm(2, 0), mm(0, 2), mm(1, 0), mm(0, 1), mm(0, 0);
+                } else {
+                    mm(0, 2), mm(0, 1), mm(0, 0);
+                }
+            }
+        *reinterpret_cast<f32x4*>(&red[0][wave][lane * 4]) = hacc;
+        __syncthreads();
+        if (finisher) {
+            const int at = (fc + 16 * (fr >> 2)) * 4 + (fr & 3);  // D[token fr][rank fc]
+            float hv = red[0][0][at];
+            for (int w = 1; w < ng * kw; w++) hv += red[0][w][at];
+            hfin[grp][fr][fc] = hv;
+        }
+        __syncthreads();
+    }
+
     const int iters = (ntiles + stride - 1) / stride;
     int buf = 0;
     for (int it0 = 0; it0 < iters; it0 += TB) {
@@ -581,6 +645,13 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
         if (p.bias && finisher)
             braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[fn]
                                                : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[fn];
+        float lbv[LORA ? 16 : 1];
+        if constexpr (LORA) {
+            if (finisher) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) lbv[r] = pm.lb[(int64_t)min(r, pm.lr - 1) * p.N + fn];
+            }
+        }
         if (have) {
             f32x4 acc = zero4;
 #pragma unroll
@@ -634,6 +705,12 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
             for (int w = 1; w < kw; w++) z += r0[w * 256];
             const int n = tile * 16 + fc;
             if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
+            if constexpr (LORA) {
+                float ls = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; r++) ls = fmaf(hfin[grp][fr][r], r < pm.lr ? lbv[r] : 0.0f, ls);
+                z = fmaf(pm.ls, ls, z);
+            }
             if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
             if (p.epilogue == NQ_EPI_SWIGLU) {  // (uniform) gate in the even column, up one lane over
                 const float other = lane_xor1(z);
@@ -942,15 +1019,21 @@ int32_t launch4_mt(const TileMrParams& pm, hipStream_t s) {
     const int ng = 16 / kw, ntiles = (pm.t.N + 15) / 16, mt = (pm.M + 15) / 16;
     const int gx = std::max(1, std::min((ntiles + ng - 1) / ng, std::max(cus, 1) / mt));
     const dim3 grid((unsigned)gx, (unsigned)mt);
+#define NQ_MT(XF, J)                                                                                             \
+    if (pm.la) hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, true>), grid, dim3(1024), 0, s, pm, kw);      \
+    else hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, false>), grid, dim3(1024), 0, s, pm, kw);
     if constexpr (XF32) {
-        hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, true, 1, 1>), grid, dim3(1024), 0, s, pm, kw);
+        NQ_MT(true, 1)
     } else {
         switch (jpw) {
-            case 1: hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 1, 1>), grid, dim3(1024), 0, s, pm, kw); break;
-            case 2: hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 2, 1>), grid, dim3(1024), 0, s, pm, kw); break;
-            default: hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 3, 1>), grid, dim3(1024), 0, s, pm, kw); break;
+            case 1: NQ_MT(false, 1) break;
+            case 2: NQ_MT(false, 2) break;
+            default:  // (three steps per wavefront leave no registers for an adapter's operands: lora_foldable says no)
+                hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 3, 1, false>), grid, dim3(1024), 0, s, pm, kw);
+                break;
         }
     }
+#undef NQ_MT
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
@@ -1056,6 +1139,13 @@ bool gemm_tile_mt_applicable(const ForwardArgs& a) {
     return true;
 }
 
+// an adapter can ride along where a wavefront holds at most two steps of K (IN <= 4096)
+bool gemm_tile_mt_lora_foldable(const ForwardArgs& a) {
+    int jpw, kw;
+    mt_split(a.L->tile_nj, a.x_dtype == NQ_DT_F32, jpw, kw);
+    return jpw >= 1 && jpw <= 2;
+}
+
 bool gemm_tile_mt_splits_parts(const ForwardArgs& a) {
     if (a.seg.nseg < 2 || a.L->prefer_tile || !mt_shape_ok(a)) return false;
     int wide = 0;
@@ -1072,6 +1162,7 @@ int32_t launch_gemm_tile_mt(const ForwardArgs& a) {
     p.N = L->out, p.K = L->in, p.NJ = L->tile_nj;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     pm.M = a.M;
+    pm.la = a.lora_a, pm.lb = a.lora_b, pm.lr = a.lora_r, pm.ls = a.lora_s;
     const bool xf32 = a.x_dtype == NQ_DT_F32;
     if (L->format == NQ_FMT_Q4_0)
         return xf32 ? launch4_mt<NQ_FMT_Q4_0, true>(pm, a.stream) : launch4_mt<NQ_FMT_Q4_0, false>(pm, a.stream);

@@ -63,3 +63,24 @@ class LoRAAdapter:
                                             self.R_PAD, C.c_float(self.scale()), _dev_ptr(x), _TORCH_DT[x.dtype],
                                             _dev_ptr(y), T, _stream_ptr()))
         return y
+
+    def forward_with(self, base, x: torch.Tensor, bias: torch.Tensor | None = None,
+                     out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """``base.forward(x)`` and this adapter's share in one call (`nq_forward_lora`): one launch where the base
+        call runs on the kernel that keeps its rows' activations resident, the two of `forward` + `forward_add`
+        elsewhere.  B = 0 returns the bits of ``base.forward(x)``."""
+        if self.merged:
+            return base.forward(x, bias=bias, out_dtype=out_dtype)
+        if x.dtype not in _TORCH_DT or not x.is_cuda or not x.is_contiguous() or x.dim() != 2 or x.shape[1] != self.IN:
+            raise L.NQError(L.NQ_ERR_INVALID, "LoRAAdapter.forward_with: x must be a contiguous fp32/bf16 device [T, IN] tensor")
+        if base.IN != self.IN or base.OUT != self.OUT:
+            raise L.NQError(L.NQ_ERR_INVALID, "LoRAAdapter.forward_with: the adapter and the base layer differ in shape")
+        T = x.shape[0]
+        y = torch.empty((T, self.OUT), dtype=out_dtype, device=x.device)
+        null = C.c_void_p(0)
+        L.check(L.lib().nq_forward_lora(base._h, _dev_ptr(x), _TORCH_DT[x.dtype], _dev_ptr(y), _TORCH_DT[out_dtype], T,
+                                        _dev_ptr(bias) if bias is not None else null,
+                                        _TORCH_DT[bias.dtype] if bias is not None else L.DT_F32,
+                                        _dev_ptr(self.lora_A), _dev_ptr(self.lora_B), self.R_PAD,
+                                        C.c_float(self.scale()), _stream_ptr()))
+        return y

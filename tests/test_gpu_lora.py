@@ -88,3 +88,58 @@ def test_merged_adapter_adds_nothing_and_errors():
         LoRAAdapter(64, 32, 0)
     with pytest.raises(L.NQError, match="expected A"):
         ad.set_params(np.zeros((64, 5), np.float32), np.zeros((4, 32), np.float32))
+
+
+# ---- the adapter folded into the base launch (nq_forward_lora) ---------------------------------------------
+# the reference's shapes again, at T = 7 and at the prefill's 135 tokens, on layers that prefer the kernel the fold
+# rides on (2 .. 512 rows), plus the default dispatch: folded on a wide layer at T = 135, two launches elsewhere
+@pytest.mark.parametrize("IN,OUT,T,R,prefer", [(960, 320, 7, 16, True), (2560, 960, 7, 16, True), (960, 960, 135, 8, True),
+                                                 (960, 2560, 135, 16, False), (960, 2560, 2, 16, True),
+                                                 (960, 320, 135, 16, False), (64, 96, 7, 4, True), (992, 100, 33, 3, True),
+                                                 (4096, 512, 40, 16, True), (4224, 64, 20, 16, True)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_qlora_one_call(IN, OUT, T, R, prefer, xdt):
+    rng = np.random.default_rng(IN + OUT + T + R + 1)
+    w = (rng.standard_normal((OUT, IN)) * 0.05).astype(np.float32)
+    base = QLinear(IN, OUT, prefer_tile=prefer)
+    base.set_weight(w)
+    bias = torch.from_numpy((rng.standard_normal(OUT) * 0.1).astype(np.float32)).cuda()
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).to(xdt).cuda()
+    y_base = base.forward(x, bias=bias)
+    # B = 0: bit for bit the bare QLinear (test_qlora.mojo: b0_fwd_diff == 0)
+    ad0, _, _ = make(rng, IN, OUT, R, zero_b=True)
+    assert torch.equal(ad0.forward_with(base, x, bias=bias), y_base)
+    # nonzero B: LoRA over deq(W), oracle on the same inputs, band 1e-5
+    ad, a, b = make(rng, IN, OUT, R)
+    y = ad.forward_with(base, x, bias=bias)
+    assert torch.equal(ad.forward_with(base, x, bias=bias), y)
+    xf = x.float().cpu().numpy()
+    want = O.qlinear_forward_cpu(base.blocks(), IN, OUT, xf) + bias.cpu().numpy()
+    want = O.lora_forward_add(xf, a, b, ad.scale(), want)
+    assert O.rel_max(y.cpu().numpy(), want) < BAND, O.rel_max(y.cpu().numpy(), want)
+    # the adapter's share alone, against fp64
+    share = 2.0 * (xf.astype(np.float64) @ a.astype(np.float64)) @ b.astype(np.float64)
+    got = y.double().cpu().numpy() - y_base.double().cpu().numpy()
+    assert np.abs(got - share).max() <= 2e-6 * max(np.abs(share).max(), np.abs(want).max())
+    # and the two-launch form gives the same values
+    two = ad.forward_add(x, y_base.clone())
+    assert float((two - y).abs().max()) <= 2e-6 * float(two.abs().max())
+
+
+def test_qlora_one_call_bf16_out_and_errors():
+    rng = np.random.default_rng(5)
+    IN, OUT, T = 960, 2560, 135
+    base = QLinear(IN, OUT)
+    base.set_weight((rng.standard_normal((OUT, IN)) * 0.05).astype(np.float32))
+    ad, a, b = make(rng, IN, OUT, 16)
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).to(torch.bfloat16).cuda()
+    y32 = ad.forward_with(base, x)
+    yb = ad.forward_with(base, x, out_dtype=torch.bfloat16)       # folded: bf16 in, bf16 out
+    assert torch.equal(yb, y32.to(torch.bfloat16))
+    narrow = QLinear(IN, 320)
+    narrow.set_weight((rng.standard_normal((320, IN)) * 0.05).astype(np.float32))
+    adn, _, _ = make(rng, IN, 320, 16)
+    with pytest.raises(L.NQError, match="second launch"):        # not folded here: the adapter adds into fp32 only
+        adn.forward_with(narrow, x, out_dtype=torch.bfloat16)
+    with pytest.raises(L.NQError, match="differ in shape"):
+        adn.forward_with(base, x)
