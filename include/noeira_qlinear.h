@@ -154,10 +154,13 @@ int32_t nq_keep_only_repacked(nq_handle h);
  * The dequantised weight is never materialised.
  * Non-finite activations: products and sums follow IEEE, with one exception.
  * A single F32 / BF16 row (M = 1) over W8_CHANNEL weights of 4 M codes and
- * more is split into int8 terms under the largest magnitude of the row (or of
- * a slice of it; error <= 6e-8 of that magnitude per element); if the row
- * holds a NaN or an infinity, every output of the call is NaN before the
- * epilogue.  The epilogue NQ_EPI_RELU is z > 0 ? z : 0 in every kernel: a NaN
+ * more, or over 4-bit weights (Q4_0, W4_GROUP with groups of 128) of so many
+ * rows that every workgroup on the chip gets three tiles of 16 (OUT >= 24576
+ * up to IN = 4096, >= 12288 up to 8192; any such layer with
+ * NQ_FLAG_PREFER_TILE), is split into int8 terms under the largest magnitude
+ * of the row (or of a slice of it; error <= 6e-8 of that magnitude per
+ * element); if the row holds a NaN or an infinity, every output of the call
+ * is NaN before the epilogue.  The epilogue NQ_EPI_RELU is z > 0 ? z : 0 in every kernel: a NaN
  * pre-activation becomes 0 and -0.0 becomes +0.0 (ops/relu_op.mojo:29-31). */
 int32_t nq_forward(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
                    int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype,

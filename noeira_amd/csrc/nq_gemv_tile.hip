@@ -58,6 +58,7 @@ struct TileParams {
     const void* bias;
     int32_t N, K, NJ;         // NJ steps per row tile (128 k for 4-bit, 64 k for int8)
     int32_t y_dtype, bias_dtype, epilogue;
+    int32_t prefer;           // NQ_FLAG_PREFER_TILE: the int8-matrix-core route for 4-bit codes whatever the layer's size
     SegTable seg;
 };
 
@@ -751,6 +752,211 @@ __device__ __forceinline__ uint32_t pack_low_bytes(uint32_t a0, uint32_t a1, uin
     return __builtin_amdgcn_perm(a1, a0, 0x0c0c0400u) | __builtin_amdgcn_perm(a3, a2, 0x04000c0cu);
 }
 
+// ---- 4-bit codes on the int8 matrix cores ----------------------------------------------------------------
+// The same tile, read as int8: a word of the tile holds eight codes as nibbles, and `w & 0x0F0F0F0F`,
+// `(w >> 4) & 0x0F0F0F0F` are each four of them as bytes (elements 0, 4, 1, 5 and 2, 6, 3, 7 of the word's eight
+// k), so a lane's 16 bytes become the B operands of two v_mfma_i32_16x16x64_i8 with 12 instructions, where the bf16
+// route spends 32 on its four.  x is split per wavefront slice into three int8 terms under one scale, as for int8
+// weights (x = (absmax / 127) (q1 + q2 / 254 + q3 / 254^2) + e, |e| <= 6e-8 absmax; a NaN or infinity in x makes
+// every output NaN), written to LDS in the bytes' own order, and sits in the MFMA's A rows - once per slice, in
+// registers.  Which rows: a word of a lane belongs to ONE chunk of 32 k (word m = chunk m of the tile), so with
+// Q4_0, whose every chunk has its own scale, A row 4 G + t carries term t in word G only and zeros elsewhere: the
+// MFMA's result row 4 G + t is then chunk G's sum for term t, and it lands in lane n + 16 G, register t - each of a
+// weight row's four lanes finishes one chunk: three conversions, the three terms' weights, -8 times the chunk's sum
+// of x (fp32, from the x stage), the chunk's scale.  Groups of 128: rows 0 .. 2 carry the terms in every word, lane
+// n finishes the tile.  A workgroup takes RT row tiles, which share the x stage.
+constexpr int T4I_MAXT = 8;  // row tiles a workgroup walks at most
+template <int FMT, bool XF32, int KW, int JPW>
+__global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p) {
+    constexpr bool EXACT = false;
+    constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
+    constexpr int NO = JPW * 16;  // octets (8 consecutive k) of x per wavefront and round: one per lane
+    static_assert(JPW >= 1 && JPW <= 4, "a lane holds one octet of the slice");
+    __shared__ __attribute__((aligned(16))) uint32_t xq[KW][3][2][NO];  // [term][lo / hi bytes][16 j + 4 q + m]
+    __shared__ float xsum[KW][G128 ? JPW : JPW * 4];
+    __shared__ float red[T4I_MAXT][KW][16];
+    __shared__ RowTail tails[T4I_MAXT][16];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const int NR = (p.N + 15) / 16;
+    // The workgroup walks row tiles blockIdx.x, blockIdx.x + gridDim.x, ... (at most T4I_MAXT); wavefront w keeps the
+    // same slice of K in all of them, so x is split once and its A operands stay in registers, and the next
+    // tile's codes are requested before the current one is multiplied.
+    const int J0 = wave * JPW;
+    auto fetch = [&](int64_t R, u32x4 (&wv)[JPW], uint32_t (&sc)[JPW]) {
+        const int64_t Rr = min(R, (int64_t)NR - 1);
+        const u32x4* const wbase = p.tile + Rr * p.NJ * 64;
+#pragma unroll
+        for (int j = 0; j < JPW; j++) wv[j] = __builtin_nontemporal_load(wbase + (min(J0 + j, p.NJ - 1) * 64 + lane));
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const int64_t at = (Rr * p.NJ + min(J0 + j, p.NJ - 1)) * 16 + c;
+            if constexpr (!G128) sc[j] = reinterpret_cast<const uint16_t*>(p.tscales)[at * 4 + q];  // chunk q's scale
+            else sc[j] = reinterpret_cast<const uint32_t*>(p.tscales)[at];
+        }
+    };
+    u32x4 wv[JPW], wn[JPW];
+    uint32_t sc[JPW], sn[JPW];
+    i32x4 aq[JPW][2];
+    float xz[JPW];
+    float s_x;
+    {
+        // x first, then the first tile's codes and their records, every load from a clamped address
+        const int k0 = J0 * 128 + min(lane, NO - 1) * 8;
+        const int kc = EXACT ? k0 : min(k0, p.K - 8);
+        const bool live = EXACT || k0 < p.K;
+        u32x4 xr[XF32 ? 2 : 1];
+        if constexpr (XF32) {
+            const float* xf = reinterpret_cast<const float*>(p.x) + kc;
+            xr[0] = *reinterpret_cast<const u32x4*>(xf), xr[1] = *reinterpret_cast<const u32x4*>(xf + 4);
+        } else {
+            xr[0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+        }
+        fetch(blockIdx.x, wv, sc);
+        float xf[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if constexpr (XF32) xf[i] = __uint_as_float(xr[i / 4][i % 4]);
+            else xf[i] = (i & 1) ? __uint_as_float(xr[0][i / 2] & 0xFFFF0000u) : __uint_as_float(xr[0][i / 2] << 16);
+            if (!live) xf[i] = 0.0f;
+        }
+        // the slice's largest magnitude as a bit pattern (NaN > inf > finite), over the wavefront
+        uint32_t mbits = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) mbits = max(mbits, __float_as_uint(xf[i]) & 0x7FFFFFFFu);
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0xB1));
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0x4E));
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0x141));
+        mbits = max(mbits, (uint32_t)NQ_DPP(mbits, 0x140));
+        {
+            const auto sw = __builtin_amdgcn_permlane16_swap(mbits, mbits, false, false);
+            mbits = max(sw[0], sw[1]);
+        }
+        {
+            const auto sw = __builtin_amdgcn_permlane32_swap(mbits, mbits, false, false);
+            mbits = max(sw[0], sw[1]);
+        }
+        const bool finite = mbits < 0x7F800000u;
+        const float absmax = __uint_as_float(mbits);
+        const float inv_s = (finite && absmax > 1e-30f) ? 127.0f / absmax : 0.0f;
+        s_x = finite ? (inv_s != 0.0f ? absmax * (1.0f / 127.0f) : 0.0f) : __uint_as_float(0x7FC00000u);
+        uint32_t a1[8], a2[8], a3[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            // round by adding 1.5 * 2^23 (the sum's low byte is the int8) and take every leftover against the very
+            // integer that was packed: no leftover exceeds a half, no term leaves the int8 range
+            const float t = xf[e] * inv_s;
+            const float b1 = t + MAGIC;
+            a1[e] = __float_as_uint(b1);
+            const float r1 = t - (b1 - MAGIC);
+            const float b2 = __builtin_fmaf(r1, 254.0f, MAGIC);
+            a2[e] = __float_as_uint(b2);
+            const float r2 = __builtin_fmaf(r1, 254.0f, MAGIC - b2);
+            a3[e] = __float_as_uint(__builtin_fmaf(r2, 254.0f, MAGIC));
+        }
+        // the sum of x under a chunk (four lanes), under a group of 128 (sixteen): fixed butterflies
+        float ps = ((xf[0] + xf[1]) + (xf[2] + xf[3])) + ((xf[4] + xf[5]) + (xf[6] + xf[7]));
+        ps += NQ_DPP_F32(ps, 0xB1);
+        ps += NQ_DPP_F32(ps, 0x4E);
+        if constexpr (G128) {
+            ps += NQ_DPP_F32(ps, 0x141);
+            ps += NQ_DPP_F32(ps, 0x140);
+        }
+        if (lane < NO) {
+            // octet l of the slice is k = 8 l ..: tile j = l / 16, chunk m = (l / 4) % 4, piece q = l % 4
+            const int at = (lane & ~15) + (lane & 3) * 4 + ((lane >> 2) & 3);
+            xq[wave][0][0][at] = pack_low_bytes(a1[0], a1[4], a1[1], a1[5]), xq[wave][0][1][at] = pack_low_bytes(a1[2], a1[6], a1[3], a1[7]);
+            xq[wave][1][0][at] = pack_low_bytes(a2[0], a2[4], a2[1], a2[5]), xq[wave][1][1][at] = pack_low_bytes(a2[2], a2[6], a2[3], a2[7]);
+            xq[wave][2][0][at] = pack_low_bytes(a3[0], a3[4], a3[1], a3[5]), xq[wave][2][1][at] = pack_low_bytes(a3[2], a3[6], a3[3], a3[7]);
+            if constexpr (!G128) {
+                if ((lane & 3) == 0) xsum[wave][lane >> 2] = -8.0f * ps;
+            } else {
+                if ((lane & 15) == 0) xsum[wave][lane >> 4] = ps;
+            }
+        }
+        // (the region is this wavefront's own and a wavefront's LDS accesses execute in order)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // the A operands of the slice's tiles, and this lane's zero-point terms
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            if constexpr (!G128) {
+                const int G = c >> 2, t = c & 3;  // A row c = 4 G + t
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    uint32_t v = xq[wave][min(t, 2)][h][j * 16 + q * 4 + G];
+                    v = t < 3 ? v : 0u;
+                    aq[j][h] = (i32x4){(int)(G == 0 ? v : 0u), (int)(G == 1 ? v : 0u), (int)(G == 2 ? v : 0u), (int)(G == 3 ? v : 0u)};
+                }
+                xz[j] = xsum[wave][j * 4 + q];
+            } else {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    i32x4 v = *reinterpret_cast<const i32x4*>(&xq[wave][min(c, 2)][h][j * 16 + q * 4]);
+                    if (c >= 3) v = (i32x4){0, 0, 0, 0};
+                    aq[j][h] = v;
+                }
+                xz[j] = xsum[wave][j];
+            }
+        }
+    }
+    int nt = 0;
+    for (int64_t R = blockIdx.x; R < NR && nt < T4I_MAXT; R += gridDim.x, nt++) {
+        if (R + gridDim.x < NR) fetch(R + gridDim.x, wn, sn);
+        if (wave == 0 && q == 0) tails[nt][c] = fetch_tail(p, R, lane);
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const bool live_j = J0 + j < p.NJ;  // (a step past K: its x is zero; its scale is set to zero too)
+            const u32x4 w = wv[j];
+            i32x4 lo, hi;
+#pragma unroll
+            for (int m = 0; m < 4; m++) lo[m] = (int)(w[m] & 0x0F0F0F0Fu), hi[m] = (int)((w[m] >> 4) & 0x0F0F0F0Fu);
+            i32x4 d = {0, 0, 0, 0};
+            d = __builtin_amdgcn_mfma_i32_16x16x64_i8(aq[j][0], lo, d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_i32_16x16x64_i8(aq[j][1], hi, d, 0, 0, 0);
+            // |sum| <= 15 * 127 * 128 < 2^24: exact as fp32
+            const float f = fmaf((float)d[2], 1.0f / 64516.0f, fmaf((float)d[1], 1.0f / 254.0f, (float)d[0]));
+            if constexpr (!G128) {
+                const float ds = live_j ? __half2float(__ushort_as_half((uint16_t)sc[j])) : 0.0f;
+                acc = fmaf(ds, fmaf(s_x, f, xz[j]), acc);
+            } else {
+                const float ds = (live_j && q == 0) ? __half2float(__ushort_as_half((uint16_t)(sc[j] & 0xFFFFu))) : 0.0f;
+                const float z = (float)(sc[j] >> 16);
+                acc = fmaf(ds, fmaf(s_x, f, -z * xz[j]), acc);
+            }
+        }
+        // a row's four lanes (its chunks' shares); the wavefronts' shares meet once, after the last tile
+        acc += __shfl_xor(acc, 16);
+        acc += __shfl_xor(acc, 32);
+        if (q == 0) red[nt][wave][c] = acc;
+#pragma unroll
+        for (int j = 0; j < JPW; j++) wv[j] = wn[j], sc[j] = sn[j];
+    }
+    __syncthreads();
+    // thread (tile i, row r): the wavefronts' shares in wave order, bias, epilogue, placement by part
+    if ((int)threadIdx.x < 16 * nt) {
+        const int i = threadIdx.x >> 4, r = threadIdx.x & 15;
+        float z = red[i][0][r];
+#pragma unroll
+        for (int w = 1; w < KW; w++) z += red[i][w][r];
+        const int64_t n = ((int64_t)blockIdx.x + (int64_t)i * gridDim.x) * 16 + r;
+        if (n < p.N) {
+            const RowTail t = tails[i][r];
+            if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? t.braw : t.braw << 16);
+            if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+            void* yp;
+            int width, col;
+            seg_lookup(p.seg, (int)n, yp, width, col);  // M = 1: the part's row is its only row
+            if (p.y_dtype == NQ_DT_F32)
+                reinterpret_cast<float*>(yp)[col] = z;
+            else
+                reinterpret_cast<uint16_t*>(yp)[col] = f32_to_bf16_rne(z);
+        }
+    }
+}
+
 template <bool XF32, int KW, int JPW, bool EXACT>
 __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p) {
     constexpr int SL = JPW * 64;  // k per wavefront and round
@@ -941,8 +1147,45 @@ int32_t launch4_jpw(const TileParams& p, int jpw, dim3 grid, hipStream_t s) {
     return NQ_OK;
 }
 
+template <int FMT, bool XF32, int KW>
+int32_t launch4i_jpw(const TileParams& p, int jpw, dim3 grid, hipStream_t s) {
+#define NQ_T4I(J_) \
+    case J_: hipLaunchKernelGGL((gemv_tile4i_kernel<FMT, XF32, KW, J_>), grid, dim3(64 * KW), 0, s, p); break;
+    switch (jpw) {
+        NQ_T4I(1) NQ_T4I(2) NQ_T4I(3) NQ_T4I(4)
+        default: return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no tile GEMV for this IN");
+    }
+#undef NQ_T4I
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+// The int8-matrix-core route, K <= 8192: four steps per wavefront at most, 8 wavefronts up to K = 4096, 16 beyond.
+// It is launched where every resident workgroup (1024 threads: one per CU; 512: two) gets three row tiles and more:
+// the workgroups are then persistent and split x once.  (With fewer tiles a static share per workgroup balances
+// worse than the hardware's own hand-out of one workgroup per tile, and launch4 keeps the bf16 route.)
+inline int t4i_resident_wgs(int nj) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+        cus = 256;
+    return std::max(cus, 1) * (nj <= 32 ? 2 : 1);
+}
+template <int FMT, bool XF32>
+int32_t launch4i(const TileParams& p, hipStream_t s) {
+    const int kw = p.NJ <= 32 ? 8 : 16;
+    const int jpw = (p.NJ + kw - 1) / kw;
+    const int nr = (p.N + 15) / 16, res = t4i_resident_wgs(p.NJ);
+    const int gridx = std::min(nr, std::max(res, (nr + T4I_MAXT - 1) / T4I_MAXT));
+    const dim3 grid((unsigned)gridx);
+    return kw == 8 ? launch4i_jpw<FMT, XF32, 8>(p, jpw, grid, s) : launch4i_jpw<FMT, XF32, 16>(p, jpw, grid, s);
+}
+
 template <int FMT, bool XF32>
 int32_t launch4(const TileParams& p, hipStream_t s) {
+    // Which route (measured at 4096 -> 11008 and 8192 -> 28672, cold): the int8 one where its workgroups are persistent
+    // (three row tiles and more each: 24.4 -> 23.0 us for groups of 128, 26.3 -> 23.6 for Q4_0); with a workgroup
+    // per tile it has no x stage to share and is no faster than the bf16 route (6.4 - 7.5 against 6.2 - 6.9 us)
+    if (p.NJ <= 64 && (p.prefer || (p.N + 15) / 16 >= 3 * t4i_resident_wgs(p.NJ))) return launch4i<FMT, XF32>(p, s);
     // about four steps (4 KiB of codes) per wavefront measured best: 8 wavefronts up to K = 4096, 16 beyond
     const int kw = p.NJ <= 32 ? 8 : 16;
     const int jpw = std::min(8, (p.NJ + kw - 1) / kw);
@@ -1192,6 +1435,7 @@ int32_t launch_gemv_tile(const ForwardArgs& a) {
     p.x = a.x, p.bias = a.bias, p.seg = a.seg;
     p.N = L->out, p.K = L->in, p.NJ = L->tile_nj;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    p.prefer = L->prefer_tile;
     const bool xf32 = a.x_dtype == NQ_DT_F32;
     switch (L->format) {
         case NQ_FMT_Q4_0:

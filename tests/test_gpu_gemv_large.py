@@ -272,3 +272,58 @@ def test_tile_relu_rule_and_nonfinite_x():
     w8.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
     assert bool(torch.isnan(w8.forward(x)).all())
     assert torch.equal(w8.forward(x, epilogue="relu"), torch.zeros((1, N), device="cuda"))
+
+
+# ---- 4-bit codes on the int8 matrix cores (the persistent route large layers take at one row) --------------
+def _w4g_layer(rng, K, N, **kw):
+    G = K // 128
+    codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
+    lin = W4GroupLinear(K, N, 128, **kw)
+    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+    return lin
+
+
+def _q4_signed(rng, K, N, **kw):
+    lin = QLinear(K, N, **kw)
+    blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+    bits = (rng.uniform(1e-3, 1e-2, (N, K // 32)) * rng.choice([-1.0, 1.0], (N, K // 32))).astype(np.float16).view(np.uint16)
+    blocks[:, :, 0], blocks[:, :, 1] = bits & 0xFF, bits >> 8
+    lin.set_blocks(blocks.reshape(-1))
+    return lin
+
+
+# default dispatch: layers with three row tiles and more per resident workgroup (N >= 24576 up to K = 4096, >= 12288
+# beyond); with NQ_FLAG_PREFER_TILE: every K split of the kernel on small layers (2 .. 4 steps per wavefront, 8 and 16
+# wavefronts, K not a multiple of the wavefronts' share), one tile per workgroup
+@pytest.mark.parametrize("K,N,prefer", [(2048, 24600, False), (4224, 12400, False), (8192, 12300, False), (2048, 2051, True),
+                                        (2176, 1999, True), (4096, 1100, True), (5504, 800, True), (8192, 1031, True),
+                                        (3072, 1400, True)])
+@pytest.mark.parametrize("fmt", ["q4_0", "w4g"])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_four_bit_single_row_on_the_int8_matrix_cores(K, N, prefer, fmt, xdt):
+    """x enters as three int8 terms under one scale per wavefront slice (error <= 6e-8 of the slice's largest
+    |x| per element), the codes as int8, sums exact in int32: the fp32 band of the reference (1e-5 of the largest
+    reference value) holds for fp32 and bf16 activations alike."""
+    rng = np.random.default_rng(K + N + len(fmt))
+    lin = (_q4_signed if fmt == "q4_0" else _w4g_layer)(rng, K, N, prefer_tile=prefer)
+    deq = lin.dequantized_dev().double()
+    x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    y = lin.forward(x, bias=bias)
+    exact = x.double() @ deq.T + bias.double()
+    assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
+    assert torch.equal(lin.forward(x, bias=bias), y)
+    yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16)
+    want = (x.double() @ deq.T + bias.to(torch.bfloat16).double()).clamp_min(0)
+    assert float((yr.double() - want).abs().max()) <= 2.0 ** -8 * float(want.abs().max()) + 1e-5 * float(exact.abs().max())
+    del deq, exact, want
+    # an outlier sixty times the rest: the terms keep 24 bits under the slice's scale
+    xo = x.clone()
+    xo[0, K // 3] = 60.0
+    yo = lin.forward(xo)
+    eo = xo.double() @ lin.dequantized_dev().double().T
+    assert float((yo.double() - eo).abs().max()) <= 1e-5 * float(eo.abs().max())
+    # a NaN or an infinity in x: every output NaN (the exact result would be NaN or +-inf per row)
+    xn = x.clone()
+    xn[0, 5] = float("inf")
+    assert bool(torch.isnan(lin.forward(xn)).all())
