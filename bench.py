@@ -704,6 +704,16 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_big, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "W4A16 g128, Q4_0 (fp32 x) and W8A16 at 4096->11008, M=1, cold rotation, one call each per step"
+    elif which == "hugegemv":
+        K, N = 8192, 28672
+        wls = [make_w4g(K=K, N=N, M=1, copies=5), make_q4_0(IN=K, OUT=N, M=1, copies=4)]
+
+        def step_huge(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_huge, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "W4A16 g128 and Q4_0 (fp32 x) at 8192->28672 (122 / 132 MB), M=1, cold rotation, one call each per step"
     elif which == "smallm":
         K, N, M = 4096, 11008, 16
         c = max(1, COLD_BYTES // (N * K // 2))
@@ -800,12 +810,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "mfma_peak", "gemm_timeline"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
                          "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
-                         "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, tile8 = int8 and fp8 "
+                         "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, hugegemv = the two 4-bit layers at 8192->28672, M=1, tile8 = int8 and fp8 "
                          "activations at M = 16 .. 512 over 4096 x 4096, manyrows = bf16 / fp32 activations at M = 1120 "
                          "and 4096, mfma_peak = the matrix cores alone (nq_diag_mfma_rate) on constant and random operands, gemm_timeline = the "
                          "config-5 GEMM's workgroups stamping entry / first stage / K loop / stores (nq_diag_gemm8_timeline)")
@@ -828,7 +838,7 @@ def main():
     if a.rows_layout:
         global TILE_COPY
         TILE_COPY = False
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "mfma_peak", "gemm_timeline"):
+    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 
