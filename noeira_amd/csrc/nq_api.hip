@@ -425,6 +425,7 @@ int32_t dispatch(const ForwardArgs& a) {
     if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemv_tile_rows_applicable(a)) return launch_gemv_tile_rows(a);
+    if (gemv_tile8_rows_applicable(a)) return launch_gemv_tile8_rows(a);
     if (gemm_tile_mt_applicable(a)) return launch_gemm_tile_mt(a);
     if (gemm_a16_applicable(a)) return launch_gemm_a16(a);
     if (gemv_tile_applicable(a)) return launch_gemv_tile(a);
@@ -440,7 +441,7 @@ bool places_parts(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_I8) return false;
     if (gemv_fp8_applicable(a) || gemm8_applicable(a)) return false;
     if (gemm_tile_mt_splits_parts(a)) return false;  // wide and narrow parts: each on the kernel of its own layer
-    return gemv_tile_rows_applicable(a) || gemm_tile_mt_applicable(a) || gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
+    return gemv_tile_rows_applicable(a) || gemv_tile8_rows_applicable(a) || gemm_tile_mt_applicable(a) || gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
 }
 
 // argument checks shared by nq_forward and nq_forward_fused, then the launch(es)

@@ -176,6 +176,8 @@ bool tile_copy_wanted(const nq_layer* L);
 int32_t build_tile_copy(nq_layer* L, hipStream_t s);
 bool gemv_tile_applicable(const ForwardArgs& a);
 bool gemv_tile_rows_applicable(const ForwardArgs& a);
+bool gemv_tile8_rows_applicable(const ForwardArgs& a);
+int32_t launch_gemv_tile8_rows(const ForwardArgs& a);
 bool gemm_tile_mt_applicable(const ForwardArgs& a);
 bool gemm_tile_mt_splits_parts(const ForwardArgs& a);
 bool gemm_tile_mt_lora_foldable(const ForwardArgs& a);

@@ -285,6 +285,8 @@ struct TileMrParams {
     float ls;
 };
 
+constexpr int TR_MAXT = 64;  // row tiles per workgroup of the rows kernels: its 1024 threads stage one tile column each
+
 template <int FMT, bool XF32, int JPW>
 __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParams pm) {
     const TileParams& p = pm.t;
@@ -302,19 +304,85 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
     uint32_t magic = 0x41804180u;
     asm volatile("" : "+v"(magic));
 
-    auto fetch = [&](int tile, u32x4 (&wv)[JPW], uint2 (&sc)[JPW]) {
-        const int64_t R = min(tile, ntiles - 1);
+    const int g = gridDim.x;
+    const int fr = threadIdx.x >> 4, fc = threadIdx.x & 15;  // threads 0 .. 255 finish a tile: row fr, column fc
+    // ---- the biases of all of this workgroup's tiles at once (at most TR_MAXT tiles): thread i stages that of column
+    // i % 16 of its tile i / 16.  The oldest load; then the activations, then the first tile.
+    __shared__ float fin_bias[TR_MAXT * 16];
+    uint32_t st_bias = 0;
+    if (p.bias) {  // (as loaded: a shift here would wait for the load)
+        const int64_t n = min(((int64_t)blockIdx.x + (int64_t)fr * g) * 16 + fc, (int64_t)p.N - 1);
+        st_bias = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                              : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
+    }
+    // The tiles' loads and the waits for them are written out: the compiler's own wait counts are exact in straight
+    // code only, and across the loop's back edge they drain the tile requested ahead together with the one about to
+    // be multiplied.  A fetch is 2 JPW loads (codes and scales of every step), so with the next tile under way "all
+    // but the youngest 2 JPW" is the tile about to be multiplied; loads and stores the compiler issues in between
+    // only make that wait longer.  The waits name no registers (nothing is copied ahead of them); the hand-over that
+    // follows them on every path does, so that nothing reads a slot before its wait.  One tile ahead, two register
+    // slots in turn: two tiles ahead measured slower wherever a workgroup has three tiles and more.
+    struct Slot {
+        u32x4 wv[JPW];
+        uint2 sc[JPW];  // (groups of 128: .x only)
+    };
+    auto fetch = [&](int tile, Slot& s) {
+        if (tile >= ntiles) return;
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
-            const int64_t at = R * p.NJ + min(J0 + j, p.NJ - 1);
-            wv[j] = __builtin_nontemporal_load(p.tile + at * 64 + lane);
-            if constexpr (!G128) sc[j] = reinterpret_cast<const uint2*>(p.tscales)[at * 16 + c];
-            else sc[j].x = reinterpret_cast<const uint32_t*>(p.tscales)[at * 16 + c], sc[j].y = 0;
+            const int64_t at = (int64_t)tile * p.NJ + min(J0 + j, p.NJ - 1);
+            const u32x4* const src = p.tile + at * 64 + lane;
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(s.wv[j]) : "v"(src));
+            if constexpr (!G128) {
+                const uint2* const ssrc = reinterpret_cast<const uint2*>(p.tscales) + at * 16 + c;
+                asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(s.sc[j]) : "v"(ssrc));
+            } else {
+                const uint32_t* const ssrc = reinterpret_cast<const uint32_t*>(p.tscales) + at * 16 + c;
+                asm volatile("global_load_dword %0, %1, off" : "=v"(s.sc[j].x) : "v"(ssrc));
+                s.sc[j].y = 0;
+            }
         }
     };
-    u32x4 wv[JPW], wn[JPW];
-    uint2 sc[JPW], sn[JPW];
-    fetch(blockIdx.x, wv, sc);
+    auto arrived = [&](int tile, Slot& s) {  // (the next tile is under way if there is one)
+        if (tile + g < ntiles) {
+            if constexpr (JPW == 1) asm volatile("s_waitcnt vmcnt(2)");
+            if constexpr (JPW == 2) asm volatile("s_waitcnt vmcnt(4)");
+            if constexpr (JPW == 3) asm volatile("s_waitcnt vmcnt(6)");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)");
+        }
+        if constexpr (G128) {
+            if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]), "+v"(s.sc[0].x));
+            if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0].x), "+v"(s.sc[1].x));
+            if constexpr (JPW == 3)
+                asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0].x), "+v"(s.sc[1].x), "+v"(s.sc[2].x));
+        } else {
+            if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]), "+v"(s.sc[0]));
+            if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0]), "+v"(s.sc[1]));
+            if constexpr (JPW == 3)
+                asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0]), "+v"(s.sc[1]), "+v"(s.sc[2]));
+        }
+    };
+
+    // (Q4_0 under fp32 rows at three steps: the first tile is requested after the operands are built, or the
+    // registers run out while both are under way)
+    constexpr bool LATE_FIRST = !G128 && XF32 && JPW == 3;
+    // ---- the activations first (older than the tiles' loads: waiting for them leaves the tiles under way)
+    u32x4 xraw[JPW][4][XF32 ? 2 : 1];
+#pragma unroll
+    for (int j = 0; j < JPW; j++)
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int k = min((J0 + j) * 128 + 32 * m + 8 * q, p.K - 8);
+            if constexpr (XF32) {
+                const float* xf = reinterpret_cast<const float*>(p.x) + (int64_t)xrow * p.K + k;
+                xraw[j][m][0] = *reinterpret_cast<const u32x4*>(xf), xraw[j][m][XF32 ? 1 : 0] = *reinterpret_cast<const u32x4*>(xf + 4);
+            } else {
+                xraw[j][m][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + (int64_t)xrow * p.K + k);
+            }
+        }
+    Slot s0, s1;
+    if constexpr (!LATE_FIRST) fetch(blockIdx.x, s0);
 
     // ---- A operands, once: 16 bytes of bf16 per (step, MFMA); rows past M and steps past K are zero
     u32x4 aop[JPW][4];
@@ -322,11 +390,9 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
     for (int j = 0; j < JPW; j++)
 #pragma unroll
         for (int m = 0; m < 4; m++) {
-            const int k = min((J0 + j) * 128 + 32 * m + 8 * q, p.K - 8);
             u32x4 t;
             if constexpr (XF32) {
-                const float* xf = reinterpret_cast<const float*>(p.x) + (int64_t)xrow * p.K + k;
-                const u32x4 r0 = *reinterpret_cast<const u32x4*>(xf), r1 = *reinterpret_cast<const u32x4*>(xf + 4);
+                const u32x4 r0 = xraw[j][m][0], r1 = xraw[j][m][XF32 ? 1 : 0];
                 uint32_t v[8];
 #pragma unroll
                 for (int i = 0; i < 4; i++) v[i] = r0[i], v[4 + i] = r1[i];
@@ -343,7 +409,7 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
                     t[i] = __builtin_amdgcn_perm(tb, ta, 0x07060302u);
                 }
             } else {
-                t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + (int64_t)xrow * p.K + k);
+                t = xraw[j][m][0];
             }
             const uint32_t keep = (vrow < pm.M && J0 + j < p.NJ) ? ~0u : 0u;
 #pragma unroll
@@ -372,17 +438,20 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
             }
         }
     }
-    // the epilogue's operands of this thread's column (threads 0 .. 255 finish a tile: row = thread / 16)
-    const int fr = threadIdx.x >> 4, fc = threadIdx.x & 15;
+    fin_bias[threadIdx.x] = __uint_as_float(p.bias_dtype == NQ_DT_F32 ? st_bias : st_bias << 16);  // (read after a barrier)
+    if constexpr (LATE_FIRST) {
+#pragma unroll
+        for (int j = 0; j < JPW; j++)
+#pragma unroll
+            for (int m = 0; m < 4; m++) asm volatile("" : "+v"(aop[j][m]));  // (built before the request below)
+        fetch(blockIdx.x, s0);
+    }
 
-    int buf = 0;
-    for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x, buf ^= 1) {
-        fetch(tile + gridDim.x, wn, sn);  // the next tile's codes are on their way while this one is multiplied
-        uint32_t braw = 0;
-        const int64_t fn = min((int64_t)tile * 16 + fc, (int64_t)p.N - 1);
-        if (p.bias && threadIdx.x < 256)
-            braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[fn]
-                                               : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[fn];
+    int buf = 0, nth = 0;  // nth: the tile's place among this workgroup's
+    auto multiply = [&](int tile, Slot& s) {
+        arrived(tile, s);
+        const u32x4(&wv)[JPW] = s.wv;
+        const uint2(&sc)[JPW] = s.sc;
         f32x4 acc = zero4;
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
@@ -437,7 +506,7 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
             }
             const int64_t n = (int64_t)tile * 16 + fc;
             if (n < p.N) {
-                if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
+                z += fin_bias[nth * 16 + fc];
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
                 void* yp;
                 int width, col;
@@ -449,8 +518,15 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
                     reinterpret_cast<uint16_t*>(yp)[o] = f32_to_bf16_rne(z);
             }
         }
-#pragma unroll
-        for (int j = 0; j < JPW; j++) wv[j] = wn[j], sc[j] = sn[j];
+        buf ^= 1, nth++;
+    };
+    for (int tile = blockIdx.x; tile < ntiles;) {
+        fetch(tile + g, s1);
+        multiply(tile, s0);
+        if ((tile += g) >= ntiles) break;
+        fetch(tile + g, s0);
+        multiply(tile, s1);
+        tile += g;
     }
 }
 
@@ -1076,6 +1152,188 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p)
     finish_rows<KW>(p, red, R, tail);
 }
 
+// ---- a few activation rows (2 <= M <= 16, fp32 rows 2 <= M <= 5) over int8 codes -----------------------------
+// As over 4-bit codes: the activation rows are the MFMA's A rows (a bf16 row as it is, an fp32 row as the three bf16
+// rows that sum to it), loaded once per workgroup into registers; the tile's codes become bf16 exactly (one
+// sign-extending conversion per code, one byte permute per pair) and a step of 64 k is two 16x16x32 MFMAs: a lane's 16
+// codes are k = 64 J + 16 q .. + 15 of weight row c, and the first MFMA takes the first eight under the name
+// "k slot (q, i)", the second the other eight, the A operands following the same naming.  One workgroup of 16
+// wavefronts per CU walks the row tiles with the next tile requested ahead of the one being multiplied (two register
+// slots in turn, no copies); the column scales and biases of all its tiles are staged in LDS before the loop, so that
+// nothing a tile needs is requested after younger loads (a wait counts loads in order of issue).  Sums over the
+// wavefronts in wave order: the same bits on every call.
+template <bool XF32, int JPW>
+__global__ __launch_bounds__(1024) void gemv_tile8_rows_kernel(const TileMrParams pm) {
+    const TileParams& p = pm.t;
+    constexpr int KW = 16;
+    constexpr int NT = XF32 ? 3 : 1;
+    __shared__ __attribute__((aligned(16))) float red[2][KW][256];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const int ntiles = (p.N + 15) / 16;
+    const int J0 = wave * JPW;
+    const int vrow = c / NT, vterm = c % NT;  // this lane's A row: activation row and term
+    const int xrow = min(vrow, pm.M - 1);
+    const int fr = threadIdx.x >> 4, fc = threadIdx.x & 15;  // threads 0 .. 255 finish a tile: row fr, column fc
+
+    // ---- what finishing needs, for all of this workgroup's tiles at once (at most TR_MAXT of them): thread i stages
+    // the scale and the bias of column i % 16 of its tile i / 16.  These are the oldest loads; then the activations,
+    // then the first tile: the loop's only loads are tiles' codes.
+    __shared__ float fin_scale[TR_MAXT * 16], fin_bias[TR_MAXT * 16];
+    const int g = gridDim.x;
+    float st_scale = 0.0f;
+    uint32_t st_bias = 0;
+    {
+        const int64_t n = min(((int64_t)blockIdx.x + (int64_t)fr * g) * 16 + fc, (int64_t)p.N - 1);
+        st_scale = p.col_scale[n];
+        if (p.bias)  // (as loaded: a shift here would wait for the load)
+            st_bias = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                                  : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
+    }
+    struct Slot {
+        u32x4 wv[JPW];
+    };
+    // The tiles' loads and the waits for them are written out: the compiler's own wait counts are exact in straight
+    // code only, and across the loop's back edge they drain the tile requested ahead together with the one about to
+    // be multiplied.  A fetch is JPW loads, so with the next tile under way "all but the youngest JPW" is the tile
+    // about to be multiplied; loads and stores the compiler issues in between only make that wait longer.  arrived()
+    // hands the registers on: nothing reads them before the wait.
+    auto fetch = [&](int tile, Slot& s) {
+        if (tile >= ntiles) return;
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const u32x4* const src = p.tile + (((int64_t)tile * p.NJ + min(J0 + j, p.NJ - 1)) * 64 + lane);
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(s.wv[j]) : "v"(src));
+        }
+    };
+    auto arrived = [&](int tile, Slot& s) {  // (the next tile is under way if there is one)
+        // (the waits name no registers, so that nothing is copied ahead of them; the hand-over follows on every path)
+        if (tile + g < ntiles) {
+            if constexpr (JPW == 1) asm volatile("s_waitcnt vmcnt(1)");
+            if constexpr (JPW == 2) asm volatile("s_waitcnt vmcnt(2)");
+            if constexpr (JPW == 3) asm volatile("s_waitcnt vmcnt(3)");
+            if constexpr (JPW == 4) asm volatile("s_waitcnt vmcnt(4)");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)");
+        }
+        if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]));
+        if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]));
+        if constexpr (JPW == 3) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]));
+        if constexpr (JPW == 4) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.wv[3]));
+    };
+    // ---- the activations first (the oldest loads: waiting for them leaves the tiles' loads under way), then two tiles
+    u32x4 xraw[JPW][2][XF32 ? 2 : 1];
+#pragma unroll
+    for (int j = 0; j < JPW; j++)
+#pragma unroll
+        for (int m = 0; m < 2; m++) {
+            const int k = min((J0 + j) * 64 + 16 * q + 8 * m, p.K - 8);
+            if constexpr (XF32) {
+                const float* xf = reinterpret_cast<const float*>(p.x) + (int64_t)xrow * p.K + k;
+                xraw[j][m][0] = *reinterpret_cast<const u32x4*>(xf), xraw[j][m][XF32 ? 1 : 0] = *reinterpret_cast<const u32x4*>(xf + 4);
+            } else {
+                xraw[j][m][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + (int64_t)xrow * p.K + k);
+            }
+        }
+    Slot s0, s1;
+    fetch(blockIdx.x, s0);
+
+    // ---- A operands, once: 16 bytes of bf16 per (step, MFMA); rows past M and steps past K are zero
+    u32x4 aop[JPW][2];
+#pragma unroll
+    for (int j = 0; j < JPW; j++)
+#pragma unroll
+        for (int m = 0; m < 2; m++) {
+            u32x4 t;
+            if constexpr (XF32) {
+                const u32x4 r0 = xraw[j][m][0], r1 = xraw[j][m][XF32 ? 1 : 0];
+                uint32_t v[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = r0[i], v[4 + i] = r1[i];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    // hi + mid + lo = the fp32 value (each split truncates: every residual is exact); this lane keeps one
+                    const uint32_t a = v[2 * i], b = v[2 * i + 1];
+                    const float ra = __uint_as_float(a) - __uint_as_float(a & 0xFFFF0000u);
+                    const float rb = __uint_as_float(b) - __uint_as_float(b & 0xFFFF0000u);
+                    const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                    const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                    const uint32_t ta = vterm == 0 ? a : vterm == 1 ? __float_as_uint(ra) : __float_as_uint(sa);
+                    const uint32_t tb = vterm == 0 ? b : vterm == 1 ? __float_as_uint(rb) : __float_as_uint(sb);
+                    t[i] = __builtin_amdgcn_perm(tb, ta, 0x07060302u);
+                }
+            } else {
+                t = xraw[j][m][0];
+            }
+            const uint32_t keep = (vrow < pm.M && J0 + j < p.NJ) ? ~0u : 0u;
+#pragma unroll
+            for (int i = 0; i < 4; i++) t[i] &= keep;
+            aop[j][m] = t;
+        }
+
+    fin_scale[threadIdx.x] = st_scale;  // (read after a tile's barrier)
+    fin_bias[threadIdx.x] = __uint_as_float(p.bias_dtype == NQ_DT_F32 ? st_bias : st_bias << 16);
+
+    int buf = 0, nth = 0;  // nth: the tile's place among this workgroup's
+    auto multiply = [&](int tile, Slot& s) {
+        arrived(tile, s);
+        f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < JPW; j++)
+#pragma unroll
+            for (int m = 0; m < 2; m++) {
+                u32x4 bop;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const uint32_t w = s.wv[j][2 * m + h];
+                    const float f0 = (float)(int8_t)w, f1 = (float)(int8_t)(w >> 8), f2 = (float)(int8_t)(w >> 16),
+                                f3 = (float)((int32_t)w >> 24);
+                    bop[2 * h] = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+                    bop[2 * h + 1] = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+                }
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(aop[j][m]), as_bf16x8(bop), acc, 0, 0, 0);
+            }
+        *reinterpret_cast<f32x4*>(&red[buf][wave][lane * 4]) = acc;
+        __syncthreads();
+        // D[v][cc] sits in lane cc + 16 (v / 4), register v % 4.  Thread (row fr, column fc) sums its row's terms'
+        // shares, each over the wavefronts in wave order.
+        if (threadIdx.x < 256 && fr < pm.M && (!XF32 || fr < 5)) {
+            float z = 0.0f;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int v = NT * fr + t;
+                const int at = (fc + 16 * (v >> 2)) * 4 + (v & 3);
+                float zt = red[buf][0][at];
+#pragma unroll
+                for (int w = 1; w < KW; w++) zt += red[buf][w][at];
+                z = t == 0 ? zt : z + zt;
+            }
+            const int64_t n = (int64_t)tile * 16 + fc;
+            if (n < p.N) {
+                z = z * fin_scale[nth * 16 + fc] + fin_bias[nth * 16 + fc];
+                if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
+                void* yp;
+                int width, col;
+                seg_lookup(p.seg, (int)n, yp, width, col);
+                const int64_t o = (int64_t)fr * width + col;
+                if (p.y_dtype == NQ_DT_F32)
+                    reinterpret_cast<float*>(yp)[o] = z;
+                else
+                    reinterpret_cast<uint16_t*>(yp)[o] = f32_to_bf16_rne(z);
+            }
+        }
+        buf ^= 1, nth++;
+    };
+    for (int tile = blockIdx.x; tile < ntiles;) {
+        fetch(tile + g, s1);
+        multiply(tile, s0);
+        if ((tile += g) >= ntiles) break;
+        fetch(tile + g, s0);
+        multiply(tile, s1);
+        tile += g;
+    }
+}
+
 // ---- load time: the tile-ordered copies -------------------------------------------------------------
 // codes [N][nch][4 words] (row order) -> tile[R][J][lane][4 words]; one thread per lane slot
 // (nch: 16-byte chunks per row; a row's last tile may hold fewer than four: the rest is zero codes under zero scales)
@@ -1226,7 +1484,7 @@ int32_t launch4_rows(const TileMrParams& pm, hipStream_t s) {
     NQ_HIP(hipGetDevice(&dev));
     NQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     const int ntiles = (pm.t.N + 15) / 16;
-    const dim3 grid((unsigned)std::min(ntiles, std::max(cus, 1)));
+    const dim3 grid((unsigned)std::min(ntiles, std::max(std::max(cus, 1), (ntiles + TR_MAXT - 1) / TR_MAXT)));
     switch (jpw) {
         case 1: hipLaunchKernelGGL((gemv_tile4_rows_kernel<FMT, XF32, 1>), grid, dim3(1024), 0, s, pm); break;
         case 2: hipLaunchKernelGGL((gemv_tile4_rows_kernel<FMT, XF32, 2>), grid, dim3(1024), 0, s, pm); break;
@@ -1353,6 +1611,55 @@ bool gemv_tile_rows_applicable(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_BF16) return a.M >= 2 && a.M <= 16;
     if (a.x_dtype == NQ_DT_F32) return a.M >= 2 && a.M <= 5;
     return false;
+}
+
+// 2 .. 16 rows of bf16 activations, 2 .. 5 of fp32 ones, over an int8 layer that keeps its tile copy, K <= 4096 (four
+// steps of K per wavefront: its A operands and two tiles' codes stay in registers).  Taken where it measured faster
+// than the kernels over the row-ordered codes: rows of 2048 codes and more; up to 4 activation rows always, up to 8
+// from 8 M codes, more from rows of 4096 codes and 8192 of them (every workgroup reads all the activations: with
+// 16 rows and one tile per workgroup that is twice its share of the weights).
+bool gemv_tile8_rows_applicable(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    if (!L->d_tile16 || L->format != NQ_FMT_W8_CHANNEL || L->tile_nj > 64 || L->glu) return false;
+    if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
+    if (a.x_dtype != NQ_DT_BF16 && a.x_dtype != NQ_DT_F32) return false;
+    if (a.M < 2 || a.M > (a.x_dtype == NQ_DT_F32 ? 5 : 16)) return false;
+    if (L->prefer_tile) return true;
+    if (L->tile_nj < 32) return false;
+    if (a.M <= 4) return true;
+    if (a.M <= 8) return (int64_t)L->in * L->out >= ((int64_t)8 << 20);
+    return L->tile_nj == 64 && L->out >= 8192;
+}
+
+int32_t launch_gemv_tile8_rows(const ForwardArgs& a) {
+    const nq_layer* L = a.L;
+    TileMrParams pm{};
+    TileParams& p = pm.t;
+    p.tile = reinterpret_cast<const u32x4*>(L->d_tile16), p.tscales = nullptr;
+    p.col_scale = reinterpret_cast<const float*>(L->d_scales);
+    p.x = a.x, p.bias = a.bias, p.seg = a.seg;
+    p.N = L->out, p.K = L->in, p.NJ = L->tile_nj;
+    p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
+    pm.M = a.M;
+    int dev = 0, cus = 0;
+    NQ_HIP(hipGetDevice(&dev));
+    NQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const int ntiles = (p.N + 15) / 16;
+    const dim3 grid((unsigned)std::min(ntiles, std::max(std::max(cus, 1), (ntiles + TR_MAXT - 1) / TR_MAXT)));
+    const int jpw = (p.NJ + 15) / 16;
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
+#define NQ_T8R(J_)                                                                                                      \
+    case J_:                                                                                                           \
+        if (xf32) hipLaunchKernelGGL((gemv_tile8_rows_kernel<true, J_>), grid, dim3(1024), 0, a.stream, pm);            \
+        else hipLaunchKernelGGL((gemv_tile8_rows_kernel<false, J_>), grid, dim3(1024), 0, a.stream, pm);                \
+        break;
+    switch (jpw) {
+        NQ_T8R(1) NQ_T8R(2) NQ_T8R(3) NQ_T8R(4)
+        default: return fail(NQ_ERR_UNSUPPORTED, "nq_forward: no int8 rows kernel for this IN");
+    }
+#undef NQ_T8R
+    NQ_HIP(hipGetLastError());
+    return NQ_OK;
 }
 
 // 96 .. 256 rows of bf16 activations, or 96 .. 512 of fp32 ones where IN <= 2048, over a wide 4-bit layer with a tile copy.

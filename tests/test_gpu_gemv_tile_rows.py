@@ -100,3 +100,85 @@ def test_few_rows_nonfinite_stay_in_their_row():
     y = lin.forward(x)
     assert bool(torch.isnan(y[2]).all()) and not bool(torch.isnan(y[[0, 1, 3, 5]]).any())
     assert not bool(torch.isfinite(y[4]).any())
+
+
+# ---- int8 codes: the activation rows as the matrix core's A rows, three int8 terms each under the row's own scale
+def w8_layer(rng, K, N, tile_copy=True, prefer_tile=True):
+    # (prefer_tile: the kernel wherever it applies, not only on the long-row layers it is dispatched to by default)
+    from noeira_amd.qlinear import W8Linear
+    w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    w[3, :] = -128  # the one code the symmetric range leaves out
+    s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    lin = W8Linear(K, N, tile_copy=tile_copy, prefer_tile=prefer_tile and tile_copy)
+    lin.set_weight(w, s)
+    return lin, w, s
+
+
+# K = 1024 (one step per wavefront), 1088 (17 steps: a ragged second step), 2048 (two), 3136 (49: four, ragged),
+# 4096 (the most the kernel holds); N off the tile size; fewer tiles than CUs and several tiles per workgroup
+W8_SHAPES = [(1024, 4100), (1088, 3900), (2048, 2051), (3136, 1400), (4096, 1100), (4096, 11008)]
+
+
+@pytest.mark.parametrize("K,N", W8_SHAPES)
+@pytest.mark.parametrize("xdt,M", [(torch.bfloat16, 2), (torch.bfloat16, 7), (torch.bfloat16, 16), (torch.float32, 2),
+                                   (torch.float32, 5), (torch.float32, 16)])
+@pytest.mark.parametrize("prefer", [True, False])
+def test_few_rows_over_int8_tile_copy(K, N, xdt, M, prefer):
+    if not prefer and K < 4096:
+        pytest.skip("the default dispatch differs from the preferred one on rows of 3072 codes and more only")
+    rng = np.random.default_rng(K + N + M)
+    lin, w, s = w8_layer(rng, K, N, prefer_tile=prefer)
+    xh = rng.standard_normal((M, K)).astype(np.float32)
+    xh[M - 1] *= 1e-3  # a quiet row beside loud ones: every row is split under its own scale
+    xh[0, 5] = 40.0    # an outlier 40 sigma out
+    x = torch.from_numpy(xh).to(xdt).cuda()
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    y = lin.forward(x, bias=bias)
+    xe = x.float().cpu().numpy()
+    exact = O.w8_forward_f64(w, s, xe, np.zeros(N, np.float32))
+    assert y.shape == (M, N)
+    got = y.cpu().numpy().astype(np.float64) - bias.cpu().numpy().astype(np.float64)
+    for m in range(M):  # each row to 1e-5 of its own RMS (the north star's bar is 1e-3)
+        assert np.abs(got[m] - exact[m]).max() < 1e-5 * np.sqrt((exact[m] ** 2).mean()) + 1e-7 * np.abs(bias.cpu().numpy()).max()
+    assert torch.equal(lin.forward(x, bias=bias), y)
+    yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16).float().cpu().numpy()
+    want = np.maximum(O.w8_forward_f64(w, s, xe, bias.to(torch.bfloat16).float().cpu().numpy()), 0)
+    rms = np.sqrt((exact ** 2).mean())
+    assert np.abs(yr - want).max() <= 1e-3 * rms + 2.0 ** -8 * np.abs(want).max()
+
+
+def test_few_rows_int8_agree_with_the_row_ordered_kernels_and_with_one_row():
+    rng = np.random.default_rng(31)
+    K, N, M = 4096, 2048, 4
+    a, _, _ = w8_layer(np.random.default_rng(3), K, N)
+    b, _, _ = w8_layer(np.random.default_rng(3), K, N, tile_copy=False)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    ya, yb = a.forward(x), b.forward(x)
+    assert float((ya - yb).abs().max()) <= 1e-5 * float(yb.abs().max())
+    for m in range(M):
+        y1 = a.forward(x[m:m + 1].contiguous())
+        assert float((ya[m] - y1[0]).abs().max()) <= 1e-5 * float(y1.abs().max())
+
+
+def test_few_rows_int8_fused_parts():
+    rng = np.random.default_rng(37)
+    K = 4096
+    parts = [w8_layer(rng, K, n)[0] for n in (1024, 256, 260)]
+    fused = FusedRows(parts)
+    x = torch.from_numpy(rng.standard_normal((3, K)).astype(np.float32)).cuda()
+    for lin, y in zip(parts, fused.forward(x)):
+        want = lin.forward(x)
+        assert y.shape == want.shape
+        assert float((y - want).abs().max()) <= 1e-5 * float(want.abs().max())
+
+
+def test_few_rows_int8_nonfinite_stay_in_their_row():
+    rng = np.random.default_rng(41)
+    K, N, M = 4096, 1040, 6
+    lin, _, _ = w8_layer(rng, K, N)
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    x[2, 100] = float("nan")
+    x[4, 7] = float("inf")
+    y = lin.forward(x)
+    assert bool(torch.isnan(y[2]).all()) and not bool(torch.isnan(y[[0, 1, 3, 5]]).any())
+    assert not bool(torch.isfinite(y[4]).any())
