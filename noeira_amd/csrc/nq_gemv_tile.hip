@@ -858,21 +858,61 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
     // The workgroup walks row tiles blockIdx.x, blockIdx.x + gridDim.x, ... (at most T4I_MAXT); wavefront w keeps the
     // same slice of K in all of them, so x is split once and its A operands stay in registers, and the next
     // tile's codes are requested before the current one is multiplied.
+    // That request and the wait for the current tile are written out (two register slots in turn, no copies): the
+    // compiler's own counts would drain the tile requested ahead at the end of every pass through the loop.  A
+    // fetch is 2 JPW loads (codes and records of every step), so with the next tile under way "all but the youngest
+    // 2 JPW" is the tile about to be multiplied; loads and stores the compiler issues in between only make that wait
+    // longer.  The waits name no registers (nothing is copied ahead of them); the hand-over that follows them on
+    // every path does, so that nothing reads a slot before its wait.
     const int J0 = wave * JPW;
-    auto fetch = [&](int64_t R, u32x4 (&wv)[JPW], uint32_t (&sc)[JPW]) {
-        const int64_t Rr = min(R, (int64_t)NR - 1);
-        const u32x4* const wbase = p.tile + Rr * p.NJ * 64;
-#pragma unroll
-        for (int j = 0; j < JPW; j++) wv[j] = __builtin_nontemporal_load(wbase + (min(J0 + j, p.NJ - 1) * 64 + lane));
+    const int g = gridDim.x;
+    struct Slot {
+        u32x4 wv[JPW];
+        uint32_t sc[JPW];
+    };
+    auto fetch = [&](int64_t R, Slot& s) {
+        const u32x4* const wbase = p.tile + R * p.NJ * 64;
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
-            const int64_t at = (Rr * p.NJ + min(J0 + j, p.NJ - 1)) * 16 + c;
-            if constexpr (!G128) sc[j] = reinterpret_cast<const uint16_t*>(p.tscales)[at * 4 + q];  // chunk q's scale
-            else sc[j] = reinterpret_cast<const uint32_t*>(p.tscales)[at];
+            const u32x4* const src = wbase + (min(J0 + j, p.NJ - 1) * 64 + lane);
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(s.wv[j]) : "v"(src));
+        }
+#pragma unroll
+        for (int j = 0; j < JPW; j++) {
+            const int64_t at = (R * p.NJ + min(J0 + j, p.NJ - 1)) * 16 + c;
+            if constexpr (!G128) {
+                const uint16_t* const src = reinterpret_cast<const uint16_t*>(p.tscales) + (at * 4 + q);  // chunk q's scale
+                asm volatile("global_load_ushort %0, %1, off" : "=v"(s.sc[j]) : "v"(src));
+            } else {
+                const uint32_t* const src = reinterpret_cast<const uint32_t*>(p.tscales) + at;
+                asm volatile("global_load_dword %0, %1, off" : "=v"(s.sc[j]) : "v"(src));
+            }
         }
     };
-    u32x4 wv[JPW], wn[JPW];
-    uint32_t sc[JPW], sn[JPW];
+    auto arrived = [&](bool next_under_way, Slot& s) {
+        if (next_under_way) {
+            if constexpr (JPW == 1) asm volatile("s_waitcnt vmcnt(2)");
+            if constexpr (JPW == 2) asm volatile("s_waitcnt vmcnt(4)");
+            if constexpr (JPW == 3) asm volatile("s_waitcnt vmcnt(6)");
+            if constexpr (JPW == 4) asm volatile("s_waitcnt vmcnt(8)");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)");
+        }
+        if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]), "+v"(s.sc[0]));
+        if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0]), "+v"(s.sc[1]));
+        if constexpr (JPW == 3)
+            asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0]), "+v"(s.sc[1]), "+v"(s.sc[2]));
+        if constexpr (JPW == 4)
+            asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.wv[3]), "+v"(s.sc[0]), "+v"(s.sc[1]),
+                         "+v"(s.sc[2]), "+v"(s.sc[3]));
+    };
+    // what finishing needs, for all of this workgroup's tiles: thread (tile i, row r) requests it first of all
+    RowTail my_tail{};
+    if ((int)threadIdx.x < 16 * T4I_MAXT) {
+        const int64_t Rt = (int64_t)blockIdx.x + (int64_t)(threadIdx.x >> 4) * g;
+        if (Rt < NR) my_tail = fetch_tail(p, Rt, threadIdx.x & 15);
+    }
+    Slot s0, s1;
     i32x4 aq[JPW][2];
     float xz[JPW];
     float s_x;
@@ -888,7 +928,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
         } else {
             xr[0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
         }
-        fetch(blockIdx.x, wv, sc);
+        fetch(blockIdx.x, s0);
         float xf[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -977,10 +1017,11 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
             }
         }
     }
-    int nt = 0;
-    for (int64_t R = blockIdx.x; R < NR && nt < T4I_MAXT; R += gridDim.x, nt++) {
-        if (R + gridDim.x < NR) fetch(R + gridDim.x, wn, sn);
-        if (wave == 0 && q == 0) tails[nt][c] = fetch_tail(p, R, lane);
+    if ((int)threadIdx.x < 16 * T4I_MAXT) tails[threadIdx.x >> 4][threadIdx.x & 15] = my_tail;  // (read after the barrier)
+    auto multiply = [&](int nt, bool next_under_way, Slot& s) {
+        arrived(next_under_way, s);
+        const u32x4(&wv)[JPW] = s.wv;
+        const uint32_t(&sc)[JPW] = s.sc;
         float acc = 0.0f;
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
@@ -1007,8 +1048,20 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
         acc += __shfl_xor(acc, 16);
         acc += __shfl_xor(acc, 32);
         if (q == 0) red[nt][wave][c] = acc;
-#pragma unroll
-        for (int j = 0; j < JPW; j++) wv[j] = wn[j], sc[j] = sn[j];
+    };
+    int nt = 0;
+    // (one tile ahead: requesting the tile after next as well measured slower, here as in the rows kernels)
+    for (int64_t R = blockIdx.x;;) {
+        bool more = R + g < NR && nt + 1 < T4I_MAXT;
+        if (more) fetch(R + g, s1);
+        multiply(nt++, more, s0);
+        if (!more) break;
+        R += g;
+        more = R + g < NR && nt + 1 < T4I_MAXT;
+        if (more) fetch(R + g, s0);
+        multiply(nt++, more, s1);
+        if (!more) break;
+        R += g;
     }
     __syncthreads();
     // thread (tile i, row r): the wavefronts' shares in wave order, bias, epilogue, placement by part
@@ -1441,7 +1494,7 @@ int32_t launch4i(const TileParams& p, hipStream_t s) {
 template <int FMT, bool XF32>
 int32_t launch4(const TileParams& p, hipStream_t s) {
     // Which route (measured at 4096 -> 11008 and 8192 -> 28672, cold): the int8 one where its workgroups are persistent
-    // (three row tiles and more each: 24.4 -> 23.0 us for groups of 128, 26.3 -> 23.6 for Q4_0); with a workgroup
+    // (three row tiles and more each: 24.4 -> 21.3 us for groups of 128, 26.3 -> 22.3 for Q4_0); with a workgroup
     // per tile it has no x stage to share and is no faster than the bf16 route (6.4 - 7.5 against 6.2 - 6.9 us)
     if (p.NJ <= 64 && (p.prefer || (p.N + 15) / 16 >= 3 * t4i_resident_wgs(p.NJ))) return launch4i<FMT, XF32>(p, s);
     // about four steps (4 KiB of codes) per wavefront measured best: 8 wavefronts up to K = 4096, 16 beyond
