@@ -73,9 +73,10 @@ extern "C" {
                                   codes; 4-bit layers with 512 <= IN <= 6144 keep it too, for calls with a
                                   hundred activation rows and more over wide layers; this flag saves that memory
                                   (0.5 or 1 byte per weight) */
-#define NQ_FLAG_PREFER_TILE 2  /* take the kernels that read the tile-ordered copy wherever they apply (2 .. 512
-                                  activation rows, any width), not only where they were measured to win: for
-                                  tuning on other shapes, and for tests that walk every instantiation */
+#define NQ_FLAG_PREFER_TILE 2  /* take the kernels that read the tile-ordered copy wherever they apply (4-bit layers:
+                                  2 .. 512 activation rows, any width; int8 layers: 2 .. 16 rows up to IN = 4096),
+                                  not only where they were measured to win: for tuning on other shapes, and for
+                                  tests that walk every instantiation */
 
 /* epilogues (LinearAct's, noeira/nn/primitives/linear_act.mojo:81-115) */
 #define NQ_EPI_NONE 0
