@@ -14,6 +14,7 @@ from __future__ import annotations
 import argparse
 import concurrent.futures as cf
 import os
+import re
 import subprocess
 import sys
 
@@ -36,6 +37,27 @@ FLAGS = [
 EXTRA_FLAGS = {"nq_gptq.hip": ["-ffp-contract=off"]}
 
 
+# Kernels that request a tile ahead with `global_load` instructions in inline assembly and wait for it with an explicit
+# `s_waitcnt`: the compiler takes the registers those loads write for valid from the load on, so a spill (or a copy made
+# to free a register) between request and wait would store what has not arrived yet.  Their register budgets are
+# chosen so that none is needed; the build refuses an object in which one of them uses scratch memory.
+NO_SPILL = {"nq_gemv_tile.hip": ("gemv_tile4i_kernel", "gemv_tile4_rows_kernel", "gemv_tile8_rows_kernel")}
+
+
+def _spilling_kernels(remarks: str, names) -> list:
+    """From the compiler's kernel-resource-usage remarks: the kernels among `names` with scratch memory or spills."""
+    out, cur = [], None
+    for l in remarks.splitlines():
+        m = re.search(r"remark: Function Name: (\S+)", l)
+        if m:
+            cur = m.group(1) if any(n in m.group(1) for n in names) else None
+            continue
+        m = re.search(r"remark:\s+(ScratchSize \[bytes/lane\]|SGPRs Spill|VGPRs Spill): (\d+)", l)
+        if m and cur and int(m.group(2)) > 0 and m.group(1) != "SGPRs Spill" and cur not in out:
+            out.append(cur)
+    return out
+
+
 def _deps():
     hs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     hs.append(os.path.join(ROOT, "include", "noeira_qlinear.h"))
@@ -48,11 +70,19 @@ def _compile(src: str, force: bool) -> str:
     newest = max(os.path.getmtime(p) for p in [path] + _deps())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj
-    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", path, "-o", obj]
+    guarded = NO_SPILL.get(src)
+    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + (["-Rpass-analysis=kernel-resource-usage"] if guarded else []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
-    warn = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    err = r.stderr
+    if guarded:
+        spilled = _spilling_kernels(err, guarded)
+        err = "\n".join(l for l in err.splitlines() if "kernel-resource-usage" not in l and not re.match(r"^\s+(\d+ \||\|)", l))
+        if spilled:
+            os.remove(obj)
+            raise RuntimeError(f"{src}: kernels that keep loads under way in registers must not spill: {spilled}")
+    warn = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l and l.strip())
     if warn:
         sys.stderr.write(warn + "\n")
     return obj
