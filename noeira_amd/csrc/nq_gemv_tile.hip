@@ -544,6 +544,18 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
 // three exact bf16 terms against the one or three terms of x, products below 2^-24 of the largest left out), summed
 // over the K split through LDS; the threads that finish a tile add s * h[row] . B[:, column] to it before the store.
 // With B = 0 the sum is an exact zero and the base result keeps its bits.
+// the sum of N wavefronts' shares of one output (256 floats apart), in wave order: all reads issued, then the additions
+template <int N>
+__device__ __forceinline__ float sum_shares(const float* r0) {
+    float v[N];
+#pragma unroll
+    for (int w = 0; w < N; w++) v[w] = r0[w * 256];
+    float z = v[0];
+#pragma unroll
+    for (int w = 1; w < N; w++) z += v[w];
+    return z;
+}
+
 template <int FMT, bool XF32, int JPW, int TB, bool LORA>
 __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams pm, const int kw) {
     const TileParams& p = pm.t;
@@ -565,8 +577,11 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
     asm volatile("" : "+v"(magic));
 
     // a group's tiles: first, first + stride, ...; fetched TB at a time, a batch ahead of their use.  (TB = 1 is
-    // what is launched: with 2 or 4 tiles in flight the same calls measured 3 - 10 % slower - the kernel is bound by
-    // the vector ALU's share of a tile (nibbles -> bf16, the scale per chunk), not by the trip to L2.)
+    // what is launched: with 2 or 4 tiles in flight the same calls measured 3 - 10 % slower, and the hand-written
+    // request and wait of the rows kernels, which keeps exactly one tile under way across the loop's back edge,
+    // changed nothing here (960 -> 2560 at 256 rows: 9.35 against 9.48 us): a pass is not waiting for its codes.
+    // Of that call's 8.9 us, finishing is 2.0 - 1.2 of them the stores of y in 64-byte row segments - the rest is the
+    // launch, the operands' set-up and five passes of unpack, MFMA, LDS and barrier.)
     const int stride = gridDim.x * ng;
     const int first = blockIdx.x * ng + min(grp, ng - 1);
     auto fetch = [&](int it0, u32x4 (&wv)[TB][JPW], uint2 (&sc)[TB][JPW]) {
@@ -647,7 +662,9 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
             }
         }
     }
-    // this thread's place in its group's finished tile: token row fr, weight row (column of y) fc
+    // this thread's place in its group's finished tile: token row fr, weight row (column of y) fc.  (Finishing the
+    // groups' neighbouring tiles side by side, a wavefront's stores covering whole 128-byte lines of y instead of
+    // 64-byte halves, measured slower: 9.4 against 8.9 us on 960 -> 2560 at 256 rows.)
     const int f = threadIdx.x - grp * kw * 64;
     const bool finisher = active && f < 256;
     const int fr = (f >> 4) & 15, fc = f & 15;
@@ -778,8 +795,22 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
         if (finisher && have) {
             const int at = (fc + 16 * (fr >> 2)) * 4 + (fr & 3);
             const float* r0 = &red[buf][grp * kw][at];  // the group's shares, in wave order
-            float z = r0[0];
-            for (int w = 1; w < kw; w++) z += r0[w * 256];
+            float z;
+            switch (kw) {  // (uniform; a loop over a run-time count would wait for every read before the next)
+                case 4: z = sum_shares<4>(r0); break;
+                case 5: z = sum_shares<5>(r0); break;
+                case 6: z = sum_shares<6>(r0); break;
+                case 7: z = sum_shares<7>(r0); break;
+                case 8: z = sum_shares<8>(r0); break;
+                case 9: z = sum_shares<9>(r0); break;
+                case 10: z = sum_shares<10>(r0); break;
+                case 11: z = sum_shares<11>(r0); break;
+                case 12: z = sum_shares<12>(r0); break;
+                case 13: z = sum_shares<13>(r0); break;
+                case 14: z = sum_shares<14>(r0); break;
+                case 15: z = sum_shares<15>(r0); break;
+                default: z = sum_shares<16>(r0); break;
+            }
             const int n = tile * 16 + fc;
             if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
             if constexpr (LORA) {
