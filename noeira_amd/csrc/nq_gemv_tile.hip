@@ -273,7 +273,9 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4_kernel(const TileParams p)
 // lane's 16 bytes of row lane % 16), and stay there, and so do the zero-point terms: the sum of x under a
 // chunk, per row, comes out of the matrix core in the product's own register layout when the B operand is all
 // ones (Q4_0: times -24 and used as the product MFMA's C operand; groups of 128: times -(16 + z) first).  The
-// next tile's codes are requested before the current tile is multiplied.  The 16 wavefronts' [16 x 16] shares
+// next tile's codes are requested before the current tile is multiplied - by hand: loads in inline assembly into two
+// register slots in turn and an explicit wait, see the kernel - and the biases of all of a workgroup's tiles are
+// staged in LDS before the loop, so that its only loads are the codes.  The 16 wavefronts' [16 x 16] shares
 // meet in LDS in wave order (two buffers, one barrier per tile); thread (row, column) adds bias and epilogue.
 struct TileMrParams {
     TileParams t;
