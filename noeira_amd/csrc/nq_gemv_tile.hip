@@ -544,8 +544,8 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
 // LORA: `y += s (x A) B` of a frozen adapter (noeira/nn/peft/lora.mojo:292-349) in the same launch.  The workgroup
 // holds its rows' x for all of K already, so h = x A [16 x rank] costs it a handful of MFMAs once (A's fp32 values as
 // three exact bf16 terms against the one or three terms of x, products below 2^-24 of the largest left out), summed
-// over the K split through LDS; the threads that finish a tile add s * h[row] . B[:, column] to it before the store.
-// With B = 0 the sum is an exact zero and the base result keeps its bits.
+// over the K split through LDS; s * h . B[:, columns] then enters each tile as four fp32 MFMAs into the accumulator of
+// the group's first wavefront.  With B = 0 that adds exact zeros and the base result keeps its bits.
 // the sum of N wavefronts' shares of one output (256 floats apart), in wave order: all reads issued, then the additions
 template <int N>
 __device__ __forceinline__ float sum_shares(const float* r0) {
@@ -741,6 +741,19 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
         }
         __syncthreads();
     }
+    // The adapter's share of a tile, s h B[:, columns], is four fp32 MFMAs of 16x16x4 (rank 16 as four k-extents) into
+    // the accumulator of each group's first wavefront before the K split's shares meet: its A operand is s h (token
+    // lane % 16, rank 4 m + lane / 16), kept in registers for the whole call; its B operand B[rank][column lane % 16],
+    // four loads per lane and tile.  (The threads that finish a tile used to do it: sixteen loads of B, sixteen LDS
+    // reads of h and sixteen FMAs per output.)
+    float hA[LORA ? 4 : 1];
+    if constexpr (LORA) {
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int r = 4 * m + q;
+            hA[m] = (kwi == 0 && active && r < pm.lr) ? pm.ls * hfin[grp][c][r] : 0.0f;
+        }
+    }
 
     const int iters = (ntiles + stride - 1) / stride;
     int buf = 0;
@@ -758,11 +771,12 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
         if (p.bias && finisher)
             braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[fn]
                                                : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[fn];
-        float lbv[LORA ? 16 : 1];
+        float lbf[LORA ? 4 : 1];
         if constexpr (LORA) {
-            if (finisher) {
+            if (kwi == 0 && active) {  // (uniform per wavefront)
+                const int64_t nb = min((int64_t)tile * 16 + c, (int64_t)p.N - 1);
 #pragma unroll
-                for (int r = 0; r < 16; r++) lbv[r] = pm.lb[(int64_t)min(r, pm.lr - 1) * p.N + fn];
+                for (int m = 0; m < 4; m++) lbf[m] = pm.lb[(int64_t)min(4 * m + q, pm.lr - 1) * p.N + nb];
             }
         }
         if (have) {
@@ -807,6 +821,12 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
                     for (int t = 0; t < 4; t++) acc[t] = fmaf(d, dd[t], acc[t]);
                 }
             }
+            if constexpr (LORA) {
+                if (kwi == 0) {
+#pragma unroll
+                    for (int m = 0; m < 4; m++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(hA[m], lbf[m], acc, 0, 0, 0);
+                }
+            }
             *reinterpret_cast<f32x4*>(&red[buf][wave][lane * 4]) = acc;
         }
         __syncthreads();
@@ -817,12 +837,6 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
             float z = sum_shares_n(r0, kw);
             const int n = tile * 16 + fc;
             if (p.bias) z += __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
-            if constexpr (LORA) {
-                float ls = 0.0f;
-#pragma unroll
-                for (int r = 0; r < 16; r++) ls = fmaf(hfin[grp][fr][r], r < pm.lr ? lbv[r] : 0.0f, ls);
-                z = fmaf(pm.ls, ls, z);
-            }
             if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
             if (p.epilogue == NQ_EPI_SWIGLU) {  // (uniform) gate in the even column, up one lane over
                 const float other = lane_xor1(z);
