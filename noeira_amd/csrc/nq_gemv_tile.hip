@@ -581,7 +581,7 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
     const TileParams& p = pm.t;
     constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
     constexpr int NT = XF32 ? 3 : 1;
-    constexpr bool XS_REGS = (G128 || JPW <= 2) && !(LORA && !G128 && (XF32 || JPW >= 2));  // (registers: the adapter's operands need them)
+    constexpr bool XS_REGS = (G128 || JPW <= 2) && !(LORA && !G128 && JPW >= 2);  // (registers: the adapter's operands need them)
     __shared__ __attribute__((aligned(16))) float red[2][16][256];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, q = lane >> 4;
