@@ -1774,20 +1774,37 @@ static bool mt_shape_ok(const ForwardArgs& a) {
     if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
     if ((int64_t)a.M * L->in >= ((int64_t)1 << 31)) return false;
     if (a.M < 2 || a.M > 512) return false;
-    if (!L->prefer_tile && a.M < 96) return false;
+    if (!L->prefer_tile && a.M < 17) return false;
     if (a.x_dtype == NQ_DT_BF16) return L->prefer_tile || a.M <= 256;
-    return a.x_dtype == NQ_DT_F32 && L->tile_nj <= 16;
+    return a.x_dtype == NQ_DT_F32 && L->tile_nj <= 16 && (L->prefer_tile || a.M >= 96);
 }
 constexpr int MT_WIDE = 2048;
 
-// The width that counts is each part's own: a row-fused layer runs on this kernel in one launch when all its parts
-// are wide, on the other kernel when none is, and part by part when they differ (gemm_tile_mt_splits_parts), so that
-// a part gets the kernel - and the bits - of its own layer's forward.
+// ... and the width, which is each part's own.  A hundred rows and more: 2048 columns.  Below (17 .. 95 rows of bf16
+// activations; the 16-row tile kernel re-reads and re-unpacks the weights per 16 rows) only over large layers whose
+// split of K leaves a wavefront at most two steps, by these measurements (us, 16-row tile kernel / this one):
+//   2048 -> 11008: M = 17 11.4 / 9.2, 64 17.1 / 13.7, 95 26.2 / 19.7     2048 -> 8192: 17 7.0 / 7.7, 48 13.0 / 11.2
+//   4096 -> 11008: 17 17.1 / 13.9, 64 26.2 / 22.6                        4096 -> 8192: 32 10.5 / 12.1, 48 19.8 / 17.5
+//   4096 ->  6144: 32 9.9 / 10.6, 48 19.1 / 14.6                         4096 -> 4096: 48 10.9 / 12.3
+//   3072 ->  8192 and 5120 -> 6912 (three steps per wavefront): the 16-row tile kernel at every M
+static bool mt_part_ok(const ForwardArgs& a, int width) {
+    if (width < MT_WIDE) return false;
+    if (a.M >= 96) return true;
+    int jpw, kw;
+    mt_split(a.L->tile_nj, a.x_dtype == NQ_DT_F32, jpw, kw);
+    if (jpw < 1 || jpw > 2) return false;
+    return width >= 10240 || (a.M >= 48 && (int64_t)a.L->in * width >= ((int64_t)(jpw == 1 ? 16 : 24) << 20));
+}
+
+// A row-fused layer runs on this kernel in one launch when all its parts pass, on the other kernel when none does,
+// and part by part when they differ (gemm_tile_mt_splits_parts), so that a part gets the kernel - and the bits - of
+// its own layer's forward.
 bool gemm_tile_mt_applicable(const ForwardArgs& a) {
     if (!mt_shape_ok(a)) return false;
-    if (a.L->prefer_tile || a.L->glu) return a.L->prefer_tile || a.L->out >= MT_WIDE;
+    if (a.L->prefer_tile) return true;
+    if (a.L->glu) return mt_part_ok(a, a.L->out);
     for (int i = 0, prev = 0; i < a.seg.nseg; prev = a.seg.end[i], i++)
-        if (a.seg.end[i] - prev < MT_WIDE) return false;
+        if (!mt_part_ok(a, a.seg.end[i] - prev)) return false;
     return true;
 }
 
@@ -1802,7 +1819,7 @@ bool gemm_tile_mt_lora_foldable(const ForwardArgs& a) {
 bool gemm_tile_mt_splits_parts(const ForwardArgs& a) {
     if (a.seg.nseg < 2 || a.L->prefer_tile || !mt_shape_ok(a)) return false;
     int wide = 0;
-    for (int i = 0, prev = 0; i < a.seg.nseg; prev = a.seg.end[i], i++) wide += a.seg.end[i] - prev >= MT_WIDE;
+    for (int i = 0, prev = 0; i < a.seg.nseg; prev = a.seg.end[i], i++) wide += mt_part_ok(a, a.seg.end[i] - prev);
     return wide > 0 && wide < a.seg.nseg;
 }
 

@@ -121,3 +121,25 @@ def test_default_dispatch_keeps_fused_parts_bitwise():
             parts = [mk(n) for n in widths]
             for part, y in zip(parts, FusedRows(parts).forward(x)):
                 assert torch.equal(y, part.forward(x))
+
+
+def test_default_dispatch_below_a_hundred_rows_over_large_layers():
+    """17 .. 95 rows of bf16 activations take the M-tile kernel by default over large layers whose split of K leaves
+    a wavefront at most two steps (2048 -> 11008 here; 2048 -> 2048 stays on the 16-row tile kernel): against fp64
+    over the dequantised weights, and a row-fused layer of a large and a small part returns the bits of each part's
+    own forward."""
+    rng = np.random.default_rng(83)
+    K, M = 2048, 33
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+    big, small = QLinear(K, 11008), QLinear(K, 2048)
+    for lin in (big, small):
+        blocks = rng.integers(0, 256, (lin.OUT, K // 32, 18), dtype=np.uint8)
+        sc = rng.uniform(1e-3, 1e-2, (lin.OUT, K // 32)).astype(np.float16).view(np.uint16)
+        blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+        lin.set_blocks(blocks.reshape(-1))
+        y = lin.forward(x)
+        exact = x.double() @ lin.dequantized_dev().double().T
+        assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
+        assert torch.equal(lin.forward(x), y)
+    for part, y in zip((big, small), FusedRows([big, small]).forward(x)):
+        assert torch.equal(y, part.forward(x))
