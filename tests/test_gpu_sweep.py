@@ -49,8 +49,10 @@ def _check(tag, y, exact, out_bf16, tol=1e-3):
     assert not bool((err > allow).any()), (tag, float(err.max()) / rms)
 
 
-@pytest.mark.parametrize("seed", [11, 12])
-def test_random_shapes(seed):
+@pytest.mark.parametrize("seed,prefer", [(11, False), (12, False), (21, True), (22, True)])
+def test_random_shapes(seed, prefer):
+    """prefer: the layers ask for the kernels over their tile-ordered copy wherever those can run
+    (NQ_FLAG_PREFER_TILE), so the same ragged shapes reach them below the sizes they take by default."""
     rng = np.random.default_rng(seed)
     for case in range(150):
         fmt = ["q4_0", "w8", "w4g", "fp8", "w8a8"][case % 5]
@@ -61,27 +63,28 @@ def test_random_shapes(seed):
         use_bias = int(rng.integers(0, 3))  # 0 none, 1 fp32, 2 bf16
         epi = "relu" if rng.integers(0, 3) == 0 else "none"
         w = None
+        hi = 8192 if (prefer and rng.integers(0, 3) == 0) else 4096  # (the tile kernels' own K ranges end at 4096 .. 8192)
         if fmt == "q4_0":
-            K = _pick_k(rng, 32)
-            lin = QLinear(K, N)
+            K = _pick_k(rng, 32, hi)
+            lin = QLinear(K, N, prefer_tile=prefer)
             blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
             sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
             blocks[:, :, 0] = sc & 0xFF
             blocks[:, :, 1] = sc >> 8
             lin.set_blocks(blocks.reshape(-1))
         elif fmt in ("w8", "w8a8"):
-            K = _pick_k(rng, 128 if (fmt == "w8a8" and rng.integers(0, 2)) else 16)
-            lin = W8Linear(K, N)
+            K = _pick_k(rng, 128 if (fmt == "w8a8" and rng.integers(0, 2)) else 16, hi)
+            lin = W8Linear(K, N, prefer_tile=prefer)
             w = rng.integers(-127, 128, (N, K), dtype=np.int8)
             lin.set_weight(w, rng.uniform(1e-3, 1e-2, N).astype(np.float32))
         elif fmt == "w4g":
             group = int(rng.choice([128, 128, 64, 32]))
-            K = _pick_k(rng, 32)
+            K = _pick_k(rng, 32, hi)
             G = -(-K // group)
             q = rng.integers(0, 16, (N, K), dtype=np.uint8)
             z = rng.integers(0, 16, (N, G), dtype=np.uint8)
             codes, zps = F.pack_w4g(q, z)
-            lin = W4GroupLinear(K, N, group)
+            lin = W4GroupLinear(K, N, group, prefer_tile=prefer)
             lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
         else:
             K = _pick_k(rng, 16)
