@@ -96,7 +96,8 @@ def test_merged_adapter_adds_nothing_and_errors():
 @pytest.mark.parametrize("IN,OUT,T,R,prefer", [(960, 320, 7, 16, True), (2560, 960, 7, 16, True), (960, 960, 135, 8, True),
                                                  (960, 2560, 135, 16, False), (960, 2560, 2, 16, True),
                                                  (960, 320, 135, 16, False), (64, 96, 7, 4, True), (992, 100, 33, 3, True),
-                                                 (4096, 512, 40, 16, True), (4224, 64, 20, 16, True)])
+                                                 (4096, 512, 40, 16, True), (4224, 64, 20, 16, True),
+                                                 (2048, 10240, 33, 16, False)])  # (folded by default: bf16 x over a large layer)
 @pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
 def test_qlora_one_call(IN, OUT, T, R, prefer, xdt):
     rng = np.random.default_rng(IN + OUT + T + R + 1)
