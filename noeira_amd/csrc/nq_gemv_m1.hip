@@ -168,7 +168,6 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     float rs[RPL], rsn[RPL];
     uint32_t rbias[RPL], rbiasn[RPL];
     const float tscale = (FMT == NQ_FMT_FP8_E4M3) ? p.tscale * (p.x_scale ? p.x_scale[0] : 1.0f) : 1.0f;
-    fetch(row_begin, wv, cs, cz, rs, rbias);
 
     // ---- this lane's slice of x, loaded once
     uint32_t xr[CPL][XR];  // fp32 bits, or bf16 pairs when DOT2
@@ -176,23 +175,49 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
     // piece v (16 bytes) of chunk c sits at c * 128 + (v ^ (c / 2) % 8) * 16: 16 lanes reading the same piece
     // of 16 consecutive chunks then touch every LDS bank once
     auto xslot = [](int c, int v) { return c * 128 + ((v ^ ((c >> 1) & 7)) << 4); };
+    // Every load of the first batch is issued before anything waits, x first: it comes from L2 and is widened and
+    // summed while the weights are still on their way from memory (loads return in the order of issue, so with the
+    // weights first the wait for x would be the wait for them).  The scheduling barrier below keeps the loads
+    // above it and their uses beneath: left to itself the compiler put the weights' loads after the wait for x in
+    // about half of the variants - a second, and with a scale in between a third, round trip to memory per call.
+    constexpr int XRAW = STAGE_X ? 2 * CPL : DOT2 ? EPC / 8 : XDT == NQ_DT_F32 ? EPC / 4 : XDT == NQ_DT_BF16 ? EPC / 8 : EPC / 16;
+    u32x4 xraw[STAGE_X ? 1 : CPL][XRAW];
+    if constexpr (STAGE_X) {
+        // (at most 64 CPL chunks of 8 pieces: 2 CPL per thread)
+        const int npieces = p.nch * 8;
+#pragma unroll
+        for (int v = 0; v < XRAW; v++) {
+            const int e = min((int)threadIdx.x + 256 * v, npieces - 1);
+            xraw[0][v] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.x) + (size_t)e * 16);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < CPL; i++) {
+            // clamped, unconditional loads; the product of a chunk past the end of the row is dropped below
+            const int64_t k0 = (int64_t)min(lj + i * lpr, p.nch - 1) * EPC;
+            const char* xb = reinterpret_cast<const char*>(p.x) + k0 * (XDT == NQ_DT_F32 ? 4 : XDT == NQ_DT_BF16 ? 2 : 1);
+#pragma unroll
+            for (int v = 0; v < XRAW; v++) xraw[i][v] = *reinterpret_cast<const u32x4*>(xb + 16 * v);
+        }
+    }
+    fetch(row_begin, wv, cs, cz, rs, rbias);
+    __builtin_amdgcn_sched_barrier(0);
     if constexpr (STAGE_X) {
         const int npieces = p.nch * 8;
-        for (int e = threadIdx.x; e < npieces; e += 256) {
-            const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.x) + (size_t)e * 16);
-            *reinterpret_cast<u32x4*>(xstage + xslot(e >> 3, e & 7)) = t;
+#pragma unroll
+        for (int v = 0; v < XRAW; v++) {
+            const int e = (int)threadIdx.x + 256 * v;
+            if (e < npieces) *reinterpret_cast<u32x4*>(xstage + xslot(e >> 3, e & 7)) = xraw[0][v];
         }
         __syncthreads();
     }
 #pragma unroll
     for (int i = 0; i < CPL; i++) {
-        // clamped, unconditional loads; the product of a chunk past the end of the row is dropped below
-        const int64_t k0 = (int64_t)min(lj + i * lpr, p.nch - 1) * EPC;
         float s = 0.0f;
         if constexpr (DOT2) {
 #pragma unroll
             for (int v = 0; v < EPC / 8; v++) {
-                const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
+                const u32x4 t = xraw[i][v];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     xr[i][4 * v + e] = t[e];
@@ -211,20 +236,21 @@ __global__ __launch_bounds__(256) void gemv_m1_kernel(const M1Params p) {
             } else if constexpr (XDT == NQ_DT_F32) {
 #pragma unroll
                 for (int v = 0; v < EPC / 4; v++) {
-                    const float4 t = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.x) + k0 + 4 * v);
-                    f[4 * v] = t.x, f[4 * v + 1] = t.y, f[4 * v + 2] = t.z, f[4 * v + 3] = t.w;
+                    const u32x4 t = xraw[i][v];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) f[4 * v + e] = __uint_as_float(t[e]);
                 }
             } else if constexpr (XDT == NQ_DT_BF16) {
 #pragma unroll
                 for (int v = 0; v < EPC / 8; v++) {
-                    const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + k0 + 8 * v);
+                    const u32x4 t = xraw[i][v];
 #pragma unroll
                     for (int e = 0; e < 4; e++) f[8 * v + 2 * e] = bf16lo(t[e]), f[8 * v + 2 * e + 1] = bf16hi(t[e]);
                 }
             } else {  // fp8 e4m3
 #pragma unroll
                 for (int v = 0; v < EPC / 16; v++) {
-                    const u32x4 t = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint8_t*>(p.x) + k0 + 16 * v);
+                    const u32x4 t = xraw[i][v];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)t[e], false);
