@@ -41,7 +41,8 @@ EXTRA_FLAGS = {"nq_gptq.hip": ["-ffp-contract=off"]}
 # `s_waitcnt`: the compiler takes the registers those loads write for valid from the load on, so a spill (or a copy made
 # to free a register) between request and wait would store what has not arrived yet.  Their register budgets are
 # chosen so that none is needed; the build refuses an object in which one of them uses scratch memory.
-NO_SPILL = {"nq_gemv_tile.hip": ("gemv_tile4i_kernel", "gemv_tile4_rows_kernel", "gemv_tile8_rows_kernel")}
+NO_SPILL = {"nq_gemv_tile.hip": ("gemv_tile4i_kernel", "gemv_tile4_rows_kernel", "gemv_tile8_rows_kernel"),
+            "nq_gemv_fp8.hip": ("tile8_kernel",)}
 
 
 def _spilling_kernels(remarks: str, names) -> list:
@@ -55,6 +56,40 @@ def _spilling_kernels(remarks: str, names) -> list:
         m = re.search(r"remark:\s+(ScratchSize \[bytes/lane\]|SGPRs Spill|VGPRs Spill): (\d+)", l)
         if m and cur and int(m.group(2)) > 0 and m.group(1) != "SGPRs Spill" and cur not in out:
             out.append(cur)
+    return out
+
+
+# Straight-line prefetches marked in the source: loads in inline assembly whose text ends in `; pf`, waited for by
+# an `s_waitcnt ... ; pfw`.  Between the two no instruction may name a register such a load writes (a copy or a
+# reuse there would take what has not arrived yet): checked on the kernels' assembly.
+PREFETCH_MARKED = ("nq_gemv_fp8.hip",)
+
+
+def _early_uses_of_prefetched(asm: str) -> list:
+    """(kernel, instruction) pairs that touch a `; pf` load's destination before that kernel's `; pfw` wait."""
+    out = []
+    parts = re.split(r"\n(_Z\S+): ; @\S*\n", asm)
+    for k in range(1, len(parts), 2):
+        body = parts[k + 1].split(".Lfunc_end")[0]
+        if "; pf" not in body:
+            continue
+        regs, waited = set(), False
+        for line in body.split("\n"):
+            t = line.strip()
+            if t.startswith("global_load") and t.endswith("; pf"):
+                regs.add(re.match(r"global_load_\w+ (v\d+),", t).group(1))
+                continue
+            if "; pfw" in t:
+                waited = True
+                break
+            if regs and t and not t.startswith(";"):
+                named = set(re.findall(r"\bv\d+\b", t))
+                for a, b in re.findall(r"v\[(\d+):(\d+)\]", t):
+                    named |= {"v%d" % x for x in range(int(a), int(b) + 1)}
+                if named & regs:
+                    out.append((parts[k], t))
+        if not waited:
+            out.append((parts[k], "no `; pfw` wait after the prefetch"))
     return out
 
 
@@ -82,6 +117,17 @@ def _compile(src: str, force: bool) -> str:
         if spilled:
             os.remove(obj)
             raise RuntimeError(f"{src}: kernels that keep loads under way in registers must not spill: {spilled}")
+    if src in PREFETCH_MARKED:
+        cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["--cuda-device-only", "-S", path, "-o", obj + ".s"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc -S failed on {src}:\n{r.stdout}\n{r.stderr}")
+        with open(obj + ".s") as f:
+            early = _early_uses_of_prefetched(f.read())
+        os.remove(obj + ".s")
+        if early:
+            os.remove(obj)
+            raise RuntimeError(f"{src}: a prefetched register is named before its wait: {early[:4]}")
     warn = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l and l.strip())
     if warn:
         sys.stderr.write(warn + "\n")

@@ -107,6 +107,41 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
     uint8_t* scr = stage[wave];
     auto lds16 = [&](uint32_t off) -> u32x4& { return *reinterpret_cast<u32x4*>(scr + off); };
 
+    // What the finishing threads need besides the sums - channel scale, bias, the rows' activation scales - is
+    // requested here, ahead of the K loop: asked for where it is used, after the barrier, it was one more trip to
+    // memory at the end of every call.  Thread t finishes outputs t, t + 64 KW, ... of a [16 x 16 NT] tile.
+    constexpr int FIT = (NT * 256 + 64 * KW - 1) / (64 * KW);
+    // (loads in inline assembly: the compiler would move its own down to their use.  Unconditional and in straight
+    // code - an operand the call does not have is read from the weights' first bytes and ignored - because a load
+    // under a branch gets its register copied at the join, before the data has landed.  They are the oldest loads of
+    // the wavefront and the wait for them stands after the K loop, before the first barrier.)
+    // From two activation tiles per workgroup on, where every tile's finish paid that trip (4096 x 4096 int8 at 63
+    // rows: 10.6 -> 10.0 us, 1024 x 1024: 4.8 -> 4.2); with one tile the registers these operands hold through the
+    // K loop cost a streaming call more than the trip (4096 -> 11008 at 2 .. 16 rows: 9.4 -> 10.6 us).  And not
+    // where 16 wavefronts hold four activation tiles each: there the registers run out, and a register spilled while
+    // its load is under way is saved before the data has landed.  The build refuses spills in these kernels.
+    constexpr bool PF = MT >= 2 && !(KW == 16 && MT == 4);
+    uint32_t f_cs[FIT], f_xs[MT][FIT], f_b32[FIT], f_b16[FIT];
+    const bool scaled = I8 && p.y_dtype != NQ_DT_I32;
+    const bool b32 = p.bias && p.bias_dtype == NQ_DT_F32, b16 = p.bias && p.bias_dtype != NQ_DT_F32;
+#pragma unroll
+    for (int it = 0; PF && it < FIT; it++) {
+        const int t = min((int)threadIdx.x + it * 64 * KW, NT * 256 - 1);
+        const int n = min(n_base + 16 * (t >> 8) + (t & 15), p.N - 1);
+        const void* const a_cs = scaled ? (const void*)(p.col_scale + n) : (const void*)p.w;
+        const void* const a_b32 = b32 ? (const void*)(reinterpret_cast<const uint32_t*>(p.bias) + n) : (const void*)p.w;
+        const void* const a_b16 = b16 ? (const void*)(reinterpret_cast<const uint16_t*>(p.bias) + n) : (const void*)p.w;
+        asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_cs[it]) : "v"(a_cs));
+        asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_b32[it]) : "v"(a_b32));
+        asm volatile("global_load_ushort %0, %1, off ; pf" : "=v"(f_b16[it]) : "v"(a_b16));
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            const void* const a_xs = scaled ? (const void*)(p.x_scale + min(m_base + 16 * i + ((t & 255) >> 4), p.M - 1))
+                                            : (!I8 ? (const void*)p.x_scale : (const void*)p.w);  // (fp8: per tensor)
+            asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_xs[i][it]) : "v"(a_xs));
+        }
+    }
+
     acc_t acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; i++)
@@ -187,6 +222,13 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
         }
     }
 
+    if constexpr (PF) asm volatile("s_waitcnt vmcnt(0) ; pfw");  // the finishing operands requested at the top (nothing else is under way here)
+#pragma unroll
+    for (int it = 0; PF && it < FIT; it++) {
+        asm volatile("" : "+v"(f_cs[it]), "+v"(f_b32[it]), "+v"(f_b16[it]));
+#pragma unroll
+        for (int i = 0; i < MT; i++) asm volatile("" : "+v"(f_xs[i][it]));
+    }
     // D layout: lane holds column n = lane % 16, rows m = 4 (lane / 16) + r.  The K-slices of one
     // activation tile (all its NT weight tiles) at a time are summed in wave order (fixed, so results
     // repeat bit for bit).
@@ -200,7 +242,10 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
                 red[wave][j * 256 + (4 * kb + r) * 16 + ln] =
                     I8 ? (uint32_t)acc[i][j][r] : __float_as_uint((float)acc[i][j][r]);
         __syncthreads();
-        for (int t = threadIdx.x; t < NT * 256; t += 64 * KW) {
+#pragma unroll
+        for (int it = 0; it < FIT; it++) {
+            const int t = (int)threadIdx.x + it * 64 * KW;
+            if (t >= NT * 256) break;
             const int m = m_base + 16 * i + ((t & 255) >> 4), n = n_base + 16 * (t >> 8) + (t & 15);
             if (m < p.M && n < p.N) {
                 const int64_t o = (int64_t)m * p.N + n;
@@ -213,17 +258,20 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
                         reinterpret_cast<int32_t*>(p.y)[o] = sum;
                         continue;
                     }
-                    z = (float)sum * (p.x_scale[m] * p.col_scale[n]);
+                    z = PF ? (float)sum * (__uint_as_float(f_xs[i][it]) * __uint_as_float(f_cs[it]))
+                           : (float)sum * (p.x_scale[m] * p.col_scale[n]);
                 } else {
                     z = __uint_as_float(red[0][t]);
 #pragma unroll
                     for (int w = 1; w < KW; w++) z += __uint_as_float(red[w][t]);
-                    z *= p.tscale * p.x_scale[0];
+                    z *= p.tscale * (PF ? __uint_as_float(f_xs[0][0]) : p.x_scale[0]);
                 }
-                if (p.bias)
-                    z += (p.bias_dtype == NQ_DT_F32)
-                             ? reinterpret_cast<const float*>(p.bias)[n]
+                if constexpr (PF) {
+                    if (p.bias) z += __uint_as_float(b32 ? f_b32[it] : f_b16[it] << 16);
+                } else if (p.bias) {
+                    z += b32 ? reinterpret_cast<const float*>(p.bias)[n]
                              : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
+                }
                 if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
                 if (p.y_dtype == NQ_DT_F32)
                     reinterpret_cast<float*>(p.y)[o] = z;

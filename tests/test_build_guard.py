@@ -32,4 +32,35 @@ def test_guarded_kernels_exist_where_they_are_listed():
         for n in names:
             assert f"void {n}(" in text, (src, n)
             # each of them waits by hand for loads written in inline assembly
-        assert 'asm volatile("global_load_dwordx4' in text and 's_waitcnt vmcnt(' in text
+        assert 'asm volatile("global_load_' in text and 's_waitcnt vmcnt(' in text
+
+
+ASM = """\t.text
+_ZN2nq4goodEv: ; @_ZN2nq4goodEv
+\tglobal_load_dword v7, v[2:3], off ; pf
+\tglobal_load_ushort v9, v[4:5], off ; pf
+\tv_add_u32_e32 v1, s2, v0
+\tglobal_load_dwordx4 v[10:13], v[2:3], off
+\ts_waitcnt vmcnt(0) ; pfw
+\tv_mov_b32_e32 v20, v7
+.Lfunc_end0:
+_ZN2nq3badEv: ; @_ZN2nq3badEv
+\tglobal_load_dword v7, v[2:3], off ; pf
+\tv_mov_b32_e32 v20, v7
+\tscratch_store_dwordx2 off, v[6:7], off
+\ts_waitcnt vmcnt(0) ; pfw
+.Lfunc_end1:
+_ZN2nq6nowaitEv: ; @_ZN2nq6nowaitEv
+\tglobal_load_dword v7, v[2:3], off ; pf
+\ts_endpgm
+.Lfunc_end2:
+"""
+
+
+def test_a_prefetched_register_named_before_its_wait_is_reported():
+    early = B._early_uses_of_prefetched(ASM)
+    assert [k for k, _ in early] == ["_ZN2nq3badEv", "_ZN2nq3badEv", "_ZN2nq6nowaitEv"]
+    assert "v_mov_b32_e32 v20, v7" in early[0][1] and "scratch_store" in early[1][1]
+    for src in B.PREFETCH_MARKED:
+        text = open(os.path.join(B.CSRC, src)).read()
+        assert "; pf\"" in text and "; pfw\"" in text, src

@@ -127,6 +127,26 @@ def test_qlora_one_call(IN, OUT, T, R, prefer, xdt):
     assert float((two - y).abs().max()) <= 2e-6 * float(two.abs().max())
 
 
+@pytest.mark.parametrize("R,pad", [(8, 8), (3, 1), (16, 16)])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_qlora_one_call_rank_as_stored(R, pad, xdt):
+    """The folded call reads A [IN, R_PAD] in 16-byte pieces when R_PAD is 16 and element by element otherwise (R_PAD
+    8 and 3 here): the same values either way, B = 0 bit for bit the base."""
+    rng = np.random.default_rng(R * 31 + pad)
+    IN, OUT, T = 960, 2560, 135
+    base = QLinear(IN, OUT)
+    base.set_weight((rng.standard_normal((OUT, IN)) * 0.05).astype(np.float32))
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).to(xdt).cuda()
+    y_base = base.forward(x)
+    ad0, _, _ = make(rng, IN, OUT, R, pad=pad, zero_b=True)
+    assert torch.equal(ad0.forward_with(base, x), y_base)
+    ad, a, b = make(rng, IN, OUT, R, pad=pad)
+    y = ad.forward_with(base, x)
+    xf = x.float().cpu().numpy()
+    want = O.lora_forward_add(xf, a, b, ad.scale(), O.qlinear_forward_cpu(base.blocks(), IN, OUT, xf))
+    assert O.rel_max(y.cpu().numpy(), want) < BAND
+
+
 def test_qlora_one_call_bf16_out_and_errors():
     rng = np.random.default_rng(5)
     IN, OUT, T = 960, 2560, 135
