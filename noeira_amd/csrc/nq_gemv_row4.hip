@@ -116,23 +116,51 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row4_kernel(const Row4Params 
         }
     };
 
-    // all of this wavefront's rows are requested now: their latency is paid once, under the staging of x
+    // x first (it is staged first, and loads return in the order of issue), then all of this wavefront's rows: their
+    // latency is paid once, under the staging of x.  The scheduling barrier keeps every load above the first wait.
+    constexpr int XIT = (KPAD / 8 + NTHR - 1) / NTHR;  // staging steps per thread
+    u32x4 xraw[XIT][XF32 ? 2 : 1];
+#pragma unroll
+    for (int it = 0; it < XIT; it++) {
+        const int kc = min(min(tid + it * NTHR, KPAD / 8 - 1) * 8, p.K - 8);
+        if constexpr (XF32) {
+            xraw[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc);
+            xraw[it][XF32 ? 1 : 0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc + 4);
+        } else {
+            xraw[it][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+        }
+    }
     u32x4 wv[RPW][CPL];
     uint2 meta[RPW][CPL];
 #pragma unroll
     for (int rr = 0; rr < RPW; rr++) fetch(row_first + rr, wv[rr], meta[rr]);
+    // the epilogue's operand travels with the codes (raw: widening a bf16 bias here would wait for it)
+    uint32_t braw[RPW];
+#pragma unroll
+    for (int rr = 0; rr < RPW; rr++) {
+        braw[rr] = 0;
+        if (p.bias) {
+            const int64_t n = min(row_first + rr, (int64_t)p.N - 1);
+            braw[rr] = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[n]
+                                                   : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n];
+        }
+    }
+
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- x -> LDS: 8 values per thread and step; 4 consecutive threads cover one chunk
-    for (int e = tid; e < KPAD / 8; e += NTHR) {
-        const int k0 = e * 8, kc = min(k0, p.K - 8);
+#pragma unroll
+    for (int it = 0; it < XIT; it++) {
+        const int e = tid + it * NTHR;
+        if (e >= KPAD / 8) break;  // (uniform over a wavefront)
+        const int k0 = e * 8;
         const uint32_t keep = k0 < p.K ? ~0u : 0u;
         const int ch = e >> 2, blk = ch >> 6, cin = ch & 63;
         // byte offset in a plane: MFMA m = cin % 4 of the block reads one KiB, lane (c = cin / 4, q = e % 4) its 16 bytes
         const int at = blk * 4096 + (cin & 3) * 1024 + ((cin >> 2) + 16 * (e & 3)) * 16;
         float part;
         if constexpr (XF32) {
-            const u32x4 r0 = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc);
-            const u32x4 r1 = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc + 4);
+            const u32x4 r0 = xraw[it][0], r1 = xraw[it][XF32 ? 1 : 0];
             uint32_t v[8];
 #pragma unroll
             for (int i = 0; i < 4; i++) v[i] = r0[i] & keep, v[4 + i] = r1[i] & keep;
@@ -155,7 +183,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row4_kernel(const Row4Params 
             part = ((__uint_as_float(v[0]) + __uint_as_float(v[1])) + (__uint_as_float(v[2]) + __uint_as_float(v[3]))) +
                    ((__uint_as_float(v[4]) + __uint_as_float(v[5])) + (__uint_as_float(v[6]) + __uint_as_float(v[7])));
         } else {
-            u32x4 r0 = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+            u32x4 r0 = xraw[it][0];
 #pragma unroll
             for (int i = 0; i < 4; i++) r0[i] &= keep;
             *reinterpret_cast<u32x4*>(plane + at) = r0;
@@ -193,14 +221,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row4_kernel(const Row4Params 
 #pragma unroll
     for (int rr = 0; rr < RPW; rr++) {
         const int64_t row = row_first + rr;
-        // the epilogue's operand travels with the codes
-        float bias = 0.0f;
-        if (p.bias) {
-            const int64_t n = min(row, (int64_t)p.N - 1);
-            bias = (p.bias_dtype == NQ_DT_F32)
-                       ? reinterpret_cast<const float*>(p.bias)[n]
-                       : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[n] << 16);
-        }
+        const float bias = __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw[rr] : braw[rr] << 16);
         const u32x4(&w)[CPL] = wv[rr];
         const uint2(&mt)[CPL] = meta[rr];
         float acc = 0.0f;
