@@ -55,27 +55,44 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row8_kernel(const Row8Params 
     const int64_t r = min(row, (int64_t)p.N - 1);
     const u32x4* wq = reinterpret_cast<const u32x4*>(p.codes) + r * p.nch;
 
-    // the row, requested before anything else (unconditional loads from clamped chunk indices)
+    // Every load is issued before anything waits: x first (it is staged first, and loads return in the order of
+    // issue), then the row (unconditional loads from clamped chunk indices), its scale and the bias as stored
+    // (widening a bf16 bias here would wait for it).  The scheduling barrier keeps the loads above the first wait.
+    constexpr int XIT = (KPAD / 4 + NTHR - 1) / NTHR;  // staging steps per thread
+    u32x4 xraw[XIT];
+#pragma unroll
+    for (int it = 0; it < XIT; it++) {
+        const int kc = min(min(tid + it * NTHR, KPAD / 4 - 1) * 4, p.K - 4);
+        if constexpr (XF32) {
+            xraw[it] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc);
+        } else {
+            const uint2 h = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
+            xraw[it][0] = h.x, xraw[it][1] = h.y;
+        }
+    }
     u32x4 wv[CPL];
 #pragma unroll
     for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wq + min(j * 64 + lane, p.nch - 1));
     const float scale = FMT == NQ_FMT_W8_CHANNEL ? p.scales[r] : p.tscale * (p.x_scale ? p.x_scale[0] : 1.0f);
-    float bias = 0.0f;
+    uint32_t braw = 0;
     if (p.bias)
-        bias = (p.bias_dtype == NQ_DT_F32)
-                   ? reinterpret_cast<const float*>(p.bias)[r]
-                   : __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[r] << 16);
+        braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[r]
+                                           : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[r];
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- x -> LDS as fp32: unit u = 4 consecutive k; unit t of chunk ch goes to ((4 (ch / 64) + t) 64 + ch % 64)
-    for (int u = tid; u < KPAD / 4; u += NTHR) {
-        const int k0 = u * 4, kc = min(k0, p.K - 4);
+#pragma unroll
+    for (int it = 0; it < XIT; it++) {
+        const int u = tid + it * NTHR;
+        if (u >= KPAD / 4) break;  // (uniform over a wavefront)
+        const int k0 = u * 4;
         const uint32_t keep = k0 < p.K ? ~0u : 0u;
         u32x4 v;
         if constexpr (XF32) {
-            v = *reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p.x) + kc);
+            v = xraw[it];
         } else {
-            const uint2 h = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.x) + kc);
-            v[0] = h.x << 16, v[1] = h.x & 0xFFFF0000u, v[2] = h.y << 16, v[3] = h.y & 0xFFFF0000u;
+            const uint32_t hx = xraw[it][0], hy = xraw[it][1];
+            v[0] = hx << 16, v[1] = hx & 0xFFFF0000u, v[2] = hy << 16, v[3] = hy & 0xFFFF0000u;
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) v[i] &= keep;
@@ -125,7 +142,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_row8_kernel(const Row8Params 
         v = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
     }
     if (lane == 0 && row < p.N) {
-        float z = v * scale + bias;
+        float z = v * scale + __uint_as_float(p.bias_dtype == NQ_DT_F32 ? braw : braw << 16);
         if (p.epilogue == NQ_EPI_RELU) z = z > 0.0f ? z : 0.0f;
         void* yp;
         int width, col;
