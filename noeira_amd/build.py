@@ -77,7 +77,9 @@ def _early_uses_of_prefetched(asm: str) -> list:
         for line in body.split("\n"):
             t = line.strip()
             if t.startswith("global_load") and t.endswith("; pf"):
-                regs.add(re.match(r"global_load_\w+ (v\d+),", t).group(1))
+                m = re.match(r"global_load_\w+ v(\d+|\[(\d+):(\d+)\]),", t)
+                lo, hi = (int(m.group(2)), int(m.group(3))) if m.group(2) else (int(m.group(1)), int(m.group(1)))
+                regs |= {"v%d" % x for x in range(lo, hi + 1)}
                 continue
             if "; pfw" in t:
                 waited = True

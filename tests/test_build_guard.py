@@ -50,6 +50,11 @@ _ZN2nq3badEv: ; @_ZN2nq3badEv
 \tscratch_store_dwordx2 off, v[6:7], off
 \ts_waitcnt vmcnt(0) ; pfw
 .Lfunc_end1:
+_ZN2nq4wideEv: ; @_ZN2nq4wideEv
+\tglobal_load_dwordx4 v[8:11], v[2:3], off ; pf
+\tv_add_f32_e32 v1, v10, v0
+\ts_waitcnt vmcnt(0) ; pfw
+.Lfunc_end3:
 _ZN2nq6nowaitEv: ; @_ZN2nq6nowaitEv
 \tglobal_load_dword v7, v[2:3], off ; pf
 \ts_endpgm
@@ -59,7 +64,7 @@ _ZN2nq6nowaitEv: ; @_ZN2nq6nowaitEv
 
 def test_a_prefetched_register_named_before_its_wait_is_reported():
     early = B._early_uses_of_prefetched(ASM)
-    assert [k for k, _ in early] == ["_ZN2nq3badEv", "_ZN2nq3badEv", "_ZN2nq6nowaitEv"]
+    assert [k for k, _ in early] == ["_ZN2nq3badEv", "_ZN2nq3badEv", "_ZN2nq4wideEv", "_ZN2nq6nowaitEv"]
     assert "v_mov_b32_e32 v20, v7" in early[0][1] and "scratch_store" in early[1][1]
     for src in B.PREFETCH_MARKED:
         text = open(os.path.join(B.CSRC, src)).read()
