@@ -38,6 +38,7 @@ namespace nq {
 namespace {
 
 typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int MAXT = 16;  // 16-channel tiles per layer (OUT <= 256)
 constexpr int MAXS = 4;   // 64-wide k-steps per layer (IN <= 256)
@@ -47,7 +48,6 @@ struct MlpLayer {
     const float* sw;      // [N]
     const float* bias;    // [N] or null
     int32_t N, K;
-    int32_t vec;          // N % 4 == 0 and sw, bias 16-byte aligned: four channels' scales or biases per load
 };
 
 struct MlpParams {
@@ -77,7 +77,6 @@ constexpr int HROW = 256 + 16;     // LDS row stride of the int8 hand-over buffe
 template <int TPW>
 struct LayerRegs {
     i32x4 a[TPW][MAXS];
-    float swv[TPW][4], bsv[TPW][4];
 };
 
 template <int TPW>
@@ -92,29 +91,16 @@ __device__ __forceinline__ void layer_load(const MlpLayer& L, int wave, int ln, 
             if (s < steps && 16 * j < L.N)  // uniform over the wavefront; one contiguous KiB per instruction
                 R.a[u][s] = *reinterpret_cast<const i32x4*>(L.w + ((j * steps + s) * 1024 + 16 * (16 * kb + ln)));
         }
-        if (L.vec) {  // uniform: the lane's four channels with one load each for scales and biases
-            const int n0 = min(16 * j + 4 * kb, L.N - 4);
-            const float4 sv = *reinterpret_cast<const float4*>(L.sw + n0);
-            R.swv[u][0] = sv.x, R.swv[u][1] = sv.y, R.swv[u][2] = sv.z, R.swv[u][3] = sv.w;
-            float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (L.bias) bv = *reinterpret_cast<const float4*>(L.bias + n0);
-            R.bsv[u][0] = bv.x, R.bsv[u][1] = bv.y, R.bsv[u][2] = bv.z, R.bsv[u][3] = bv.w;
-        } else {
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int n = min(16 * j + 4 * kb + r, L.N - 1);
-                R.swv[u][r] = L.sw[n];
-                R.bsv[u][r] = L.bias ? L.bias[n] : 0.0f;
-            }
-        }
     }
 }
 
 // `bop[s]` is the B operand of k-step s (16 int8 of the lane's token), `sx` the token's scale.
 // z[u][r] = fp32 output for channel 16 (TPW w + u) + 4 kb + r of the lane's token (0 beyond N).
+// `sb` = the layer's [scales | biases] in LDS, 256 floats each (zeros beyond N and for a missing bias).
 template <int TPW>
-__device__ __forceinline__ void layer_forward(const MlpLayer& L, const LayerRegs<TPW>& R, const i32x4 (&bop)[MAXS],
-                                              float sx, bool relu, int wave, int ln, int kb, float (&z)[TPW][4]) {
+__device__ __forceinline__ void layer_forward(const MlpLayer& L, const LayerRegs<TPW>& R, const float* sb,
+                                              const i32x4 (&bop)[MAXS], float sx, bool relu, int wave, int ln, int kb,
+                                              float (&z)[TPW][4]) {
     const int steps = (L.K + 63) >> 6;
 #pragma unroll
     for (int u = 0; u < TPW; u++) {
@@ -127,10 +113,12 @@ __device__ __forceinline__ void layer_forward(const MlpLayer& L, const LayerRegs
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(R.a[u][s], bop[s], acc, 0, 0, 0);
             }
         }
+        const f32x4 sv = *reinterpret_cast<const f32x4*>(sb + 16 * j + 4 * kb);
+        const f32x4 bv = *reinterpret_cast<const f32x4*>(sb + 256 + 16 * j + 4 * kb);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int n = 16 * j + 4 * kb + r;
-            float v = (float)acc[r] * (sx * R.swv[u][r]) + R.bsv[u][r];
+            float v = (float)acc[r] * (sx * sv[r]) + bv[r];
             if (relu) v = v > 0.0f ? v : 0.0f;
             z[u][r] = (n < L.N) ? v : 0.0f;
         }
@@ -173,6 +161,7 @@ __global__ __launch_bounds__(64 * WAVES) void mlp3_w8a8_kernel(const MlpParams p
     __shared__ __attribute__((aligned(16))) uint8_t hq[2][16 * HROW];
     __shared__ float amax_part[2][16 * WAVES];
     __shared__ __attribute__((aligned(16))) float xsh[16][256 + 4];
+    __shared__ __attribute__((aligned(16))) float sbs[3][2 * 256];  // per layer [scales | biases]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int ln = lane & 15, kb = lane >> 4;
     const int m = blockIdx.x * 16 + ln;          // this lane's token
@@ -199,11 +188,26 @@ __global__ __launch_bounds__(64 * WAVES) void mlp3_w8a8_kernel(const MlpParams p
     layer_load<TPW>(p.l[0], wave, ln, kb, R0);
     layer_load<TPW>(p.l[1], wave, ln, kb, R1);
     layer_load<TPW>(p.l[2], wave, ln, kb, R2);
+    // Channel scales and biases: one element per thread and layer (thread t: array t / 256, channel t % 256, clamped
+    // loads, zero beyond N and for a missing bias), handed round through LDS under the barrier that x needs anyway.
+    // As two 16-byte loads per 16-channel tile and wavefront they were 96 of a workgroup's ~176 load instructions,
+    // and an instruction costs the CU's address unit the same whatever it fetches.
+    static_assert(WAVES == 8, "one scale or bias element per thread");
+    float sbr[3];
+#pragma unroll
+    for (int l = 0; l < 3; l++) {
+        const int ch = threadIdx.x & 255;
+        const float* const src = (threadIdx.x >> 8) ? p.l[l].bias : p.l[l].sw;
+        const float v = (src ? src : p.l[l].sw)[min(ch, p.l[l].N - 1)];
+        sbr[l] = (src && ch < p.l[l].N) ? v : 0.0f;
+    }
 #pragma unroll
     for (int n = 0; n < XU; n++) {
         const int i = (int)threadIdx.x + n * 64 * WAVES;
         if (i < units) *reinterpret_cast<float4*>(&xsh[(4 * i) / K0][(4 * i) % K0]) = xr[n];
     }
+#pragma unroll
+    for (int l = 0; l < 3; l++) sbs[l][threadIdx.x] = sbr[l];
     __syncthreads();
     float xv[MAXS][16];
     float amax = 0.0f;
@@ -238,11 +242,11 @@ __global__ __launch_bounds__(64 * WAVES) void mlp3_w8a8_kernel(const MlpParams p
     // channels its layer does not produce, because z is 0 there)
 
     float z[TPW][4];
-    layer_forward<TPW>(p.l[0], R0, bop, sx, true, wave, ln, kb, z);
+    layer_forward<TPW>(p.l[0], R0, sbs[0], bop, sx, true, wave, ln, kb, z);
     requantize<TPW>(z, hq[0], amax_part[0], wave, ln, kb, bop, sx);
-    layer_forward<TPW>(p.l[1], R1, bop, sx, true, wave, ln, kb, z);
+    layer_forward<TPW>(p.l[1], R1, sbs[1], bop, sx, true, wave, ln, kb, z);
     requantize<TPW>(z, hq[1], amax_part[1], wave, ln, kb, bop, sx);
-    layer_forward<TPW>(p.l[2], R2, bop, sx, p.final_relu != 0, wave, ln, kb, z);
+    layer_forward<TPW>(p.l[2], R2, sbs[2], bop, sx, p.final_relu != 0, wave, ln, kb, z);
 
     if (m >= p.M) return;
     const int N2 = p.l[2].N;
@@ -269,7 +273,6 @@ int32_t launch_mlp3_w8a8(const nq_layer* l1, const nq_layer* l2, const nq_layer*
         p.l[i].sw = reinterpret_cast<const float*>(ls[i]->d_scales);
         p.l[i].bias = bs[i];
         p.l[i].N = ls[i]->out, p.l[i].K = ls[i]->in;
-        p.l[i].vec = ls[i]->out % 4 == 0 && ((uintptr_t)p.l[i].sw & 15) == 0 && ((uintptr_t)bs[i] & 15) == 0;
     }
     p.x = x, p.y = y, p.M = M, p.final_relu = final_relu;
     // eight wavefronts: with four the three layers' operands do not fit the registers (10.3 us against 8.7), with
