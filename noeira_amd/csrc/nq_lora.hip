@@ -139,12 +139,170 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_add_kernel(const void* __r
     }
 }
 
+// ---- the usual case: R = 16 as stored, IN a multiple of 32, OUT a multiple of 4, 16-byte aligned operands --------
+// The kernel above is bound by its load instructions (a dword per lane and k of A: IN / 4 of them per wavefront, and
+// an instruction costs the CU's address unit the same whatever it fetches) and by the fp32 matrix cores (a sixteenth
+// of the bf16 rate): 5.8 us at 960 -> 2560 for one token, 12.8 us at IN = 2560, 16.4 at 4096.  Here A's rows (16
+// ranks = 64 bytes, so a chunk of 32 k is 2 KiB in one piece) are fetched 16 bytes per lane and turned into the
+// MFMA's operand through the wavefront's own 2 KiB of LDS (the 16-byte quarter of row k sits at quarter ^ (k / 8) % 4:
+// the four k-pieces of a rank then read different banks); h = x A runs on the bf16 matrix cores with A as three exact
+// bf16 terms against the one (bf16 x) or three (fp32 x) terms of the activations, products below 2^-24 of the largest
+// left out - the arithmetic of the adapter folded into the base call (nq_gemv_tile.hip); the tiles of B and y are
+// fetched 16 bytes per lane as well, B through LDS.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+constexpr int L16_NB = 4;  // chunks of 32 k whose loads are in flight together, per wavefront
+
+template <bool XBF16>
+__global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* __restrict__ xv, const float* __restrict__ A,
+                                                                   const float* __restrict__ B, float* __restrict__ y, int T,
+                                                                   int IN, int OUT, float s) {
+    constexpr int NT = XBF16 ? 1 : 3;
+    __shared__ float part[LR_WAVES][LR_ROWS][LR_R + 1];
+    __shared__ __attribute__((aligned(16))) float h[LR_ROWS][LR_R];
+    __shared__ __attribute__((aligned(16))) float sta[LR_WAVES][2][256];  // a chunk of A per wavefront, turned
+    __shared__ __attribute__((aligned(16))) float bt[LR_R][LR_COLS];      // the tile of B
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, q = lane >> 4;
+    const int m0 = blockIdx.y * LR_ROWS, n0 = blockIdx.x * LR_COLS;
+    // second phase: thread (column quad cq, row pair rp) owns y[m0 + 2 rp .. + 1][n0 + 4 cq .. + 3]
+    const int cq = tid & 63, rp = tid >> 6;
+    const bool cols_in = n0 + 4 * cq < OUT;  // (OUT is a multiple of 4: a quad is inside or outside)
+    const int ncl = min(n0 + 4 * cq, OUT - 4);
+    // requested first, used last: the tile of y and the tile of B (rows 2 rp, 2 rp + 1 of it per thread)
+    f32x4 yv[2], bv[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        yv[i] = *reinterpret_cast<const f32x4*>(y + (int64_t)min(m0 + 2 * rp + i, T - 1) * OUT + ncl);
+        bv[i] = *reinterpret_cast<const f32x4*>(B + (int64_t)(2 * rp + i) * OUT + ncl);
+    }
+
+    // ---- h = x A: wavefront w takes the chunks w, w + 8, ... of 32 k, L16_NB of them under way at a time
+    const int nch = IN >> 5;
+    const int mrow = min(m0 + c, T - 1);
+    f32x4 hacc = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int c0 = wave; c0 < nch; c0 += LR_WAVES * L16_NB) {
+        u32x4 ar[L16_NB][2], xr[L16_NB][XBF16 ? 1 : 2];
+#pragma unroll
+        for (int b = 0; b < L16_NB; b++) {
+            const int k0 = min(c0 + b * LR_WAVES, nch - 1) << 5;  // (a chunk past K: read again, not used)
+            if constexpr (XBF16) {
+                xr[b][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(xv) + (int64_t)mrow * IN + k0 + 8 * q);
+            } else {
+                const float* xf = reinterpret_cast<const float*>(xv) + (int64_t)mrow * IN + k0 + 8 * q;
+                xr[b][0] = *reinterpret_cast<const u32x4*>(xf), xr[b][XBF16 ? 0 : 1] = *reinterpret_cast<const u32x4*>(xf + 4);
+            }
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                ar[b][t] = *reinterpret_cast<const u32x4*>(A + (int64_t)(k0 + 16 * t + (lane >> 2)) * LR_R + 4 * (lane & 3));
+        }
+        __builtin_amdgcn_sched_barrier(0);  // every load of the batch ahead of the first wait
+#pragma unroll
+        for (int b = 0; b < L16_NB; b++) {
+            if (c0 + b * LR_WAVES >= nch) break;  // (uniform over the wavefront)
+            // A's chunk [32 k][16 ranks] -> 8 consecutive k of rank c per lane
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const int row = lane >> 2, kq = (2 * t + (row >> 3)) & 3;  // k / 8 of row 16 t + row
+                *reinterpret_cast<u32x4*>(&sta[wave][t][row * 16 + 4 * ((lane & 3) ^ kq)]) = ar[b][t];
+            }
+            uint32_t av[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                av[i] = __float_as_uint(sta[wave][q >> 1][(8 * (q & 1) + i) * 16 + 4 * ((c >> 2) ^ q) + (c & 3)]);
+            // hi + mid + lo = the fp32 value (each split truncates: every residual is exact)
+            u32x4 pl[3], xt[NT];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t a0 = av[2 * i], b0 = av[2 * i + 1];
+                const float ra = __uint_as_float(a0) - __uint_as_float(a0 & 0xFFFF0000u);
+                const float rb = __uint_as_float(b0) - __uint_as_float(b0 & 0xFFFF0000u);
+                const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                pl[0][i] = __builtin_amdgcn_perm(b0, a0, 0x07060302u);
+                pl[1][i] = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+                pl[2][i] = __builtin_amdgcn_perm(__float_as_uint(sb), __float_as_uint(sa), 0x07060302u);
+            }
+            if constexpr (XBF16) {
+                xt[0] = xr[b][0];
+            } else {
+                uint32_t v[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = xr[b][0][i], v[4 + i] = xr[b][XBF16 ? 0 : 1][i];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t a0 = v[2 * i], b0 = v[2 * i + 1];
+                    const float ra = __uint_as_float(a0) - __uint_as_float(a0 & 0xFFFF0000u);
+                    const float rb = __uint_as_float(b0) - __uint_as_float(b0 & 0xFFFF0000u);
+                    const float sa = ra - __uint_as_float(__float_as_uint(ra) & 0xFFFF0000u);
+                    const float sb = rb - __uint_as_float(__float_as_uint(rb) & 0xFFFF0000u);
+                    xt[0][i] = __builtin_amdgcn_perm(b0, a0, 0x07060302u);
+                    xt[NT / 2][i] = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+                    xt[NT - 1][i] = __builtin_amdgcn_perm(__float_as_uint(sb), __float_as_uint(sa), 0x07060302u);
+                }
+            }
+            auto mm = [&](int xi, int ai) {
+                hacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xt[xi]), __builtin_bit_cast(bf16x8, pl[ai]),
+                                                               hacc, 0, 0, 0);
+            };
+            if constexpr (XBF16) {  // smallest products first
+                mm(0, 2), mm(0, 1), mm(0, 0);
+            } else {
+                mm(NT / 2, 1), mm(NT - 1, 0), mm(0, 2), mm(NT / 2, 0), mm(0, 1), mm(0, 0);  // (x term, A term): 1 1, 2 0, 0 2, ...
+            }
+        }
+    }
+    // D[token 4 (lane / 16) + v][rank lane % 16]: the wavefronts' shares, summed in wave order
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[wave][4 * q + v][c] = hacc[v];
+#pragma unroll
+    for (int i = 0; i < 2; i++) *reinterpret_cast<f32x4*>(&bt[2 * rp + i][4 * cq]) = bv[i];
+    __syncthreads();
+    if (tid < LR_ROWS * LR_R) {
+        const int m = tid >> 4, rr = tid & 15;
+        float t = 0.0f;
+#pragma unroll
+        for (int w = 0; w < LR_WAVES; w++) t += part[w][m][rr];
+        h[m][rr] = t;
+    }
+    __syncthreads();
+    // ---- y[m][n] += s sum_r h[m][r] B[r][n], r ascending
+    f32x4 out[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+    for (int r4 = 0; r4 < LR_R; r4 += 4) {
+        const f32x4 h0 = *reinterpret_cast<const f32x4*>(&h[2 * rp][r4]), h1 = *reinterpret_cast<const f32x4*>(&h[2 * rp + 1][r4]);
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+            const f32x4 bq = *reinterpret_cast<const f32x4*>(&bt[r4 + rr][4 * cq]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) out[0][e] = fmaf(h0[rr], bq[e], out[0][e]), out[1][e] = fmaf(h1[rr], bq[e], out[1][e]);
+        }
+    }
+    if (cols_in) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (m0 + 2 * rp + i >= T) break;
+            f32x4 z;
+#pragma unroll
+            for (int e = 0; e < 4; e++) z[e] = fmaf(s, out[i][e], yv[i][e]);
+            *reinterpret_cast<f32x4*>(y + (int64_t)(m0 + 2 * rp + i) * OUT + ncl) = z;
+        }
+    }
+}
+
 }  // namespace
 
 int32_t launch_lora_add(const void* x, int32_t x_dtype, const float* A, const float* B, float* y, int32_t T, int32_t IN,
                         int32_t OUT, int32_t R, float s, hipStream_t stream) {
     dim3 grid((OUT + LR_COLS - 1) / LR_COLS, (T + LR_ROWS - 1) / LR_ROWS);
     const bool bf = x_dtype == NQ_DT_BF16;
+    const auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    if (R == LR_R && IN % 32 == 0 && OUT % 4 == 0 && al16(x) && al16(A) && al16(B) && al16(y)) {
+        if (bf) hipLaunchKernelGGL((lora_add16_kernel<true>), grid, dim3(64 * LR_WAVES), 0, stream, x, A, B, y, T, IN, OUT, s);
+        else hipLaunchKernelGGL((lora_add16_kernel<false>), grid, dim3(64 * LR_WAVES), 0, stream, x, A, B, y, T, IN, OUT, s);
+        NQ_HIP(hipGetLastError());
+        return NQ_OK;
+    }
     const bool vec = IN % 4 == 0 && ((uintptr_t)x & 15) == 0;
 #define NQ_LORA(BF, VEC) \
     hipLaunchKernelGGL((lora_add_kernel<BF, VEC>), grid, dim3(64 * LR_WAVES), 0, stream, x, A, B, y, T, IN, OUT, R, s)
