@@ -4,7 +4,8 @@
 // layer's forward with the same x and y.  The reference runs two GEMMs (and, off NVIDIA, a
 // third kernel for the accumulation) through a [T, R] scratch; here it is one launch and no
 // scratch: a workgroup owns 16 tokens x 256 output columns, forms h = x A for its 16 tokens
-// itself (on the fp32 matrix cores, k split eight ways over the wavefronts and reduced through
+// itself (the general kernel: on the fp32 matrix cores; R = 16 as stored has its own further down, on the bf16 ones
+// with exact three-term splits; either way k split eight ways over the wavefronts and reduced through
 // LDS; recomputed by each column tile, which costs less than a launch) and then adds s * h B
 // to its tile of y with coalesced read-modify-writes.  fp32 throughout; x may be bf16.
 //
