@@ -1789,10 +1789,16 @@ constexpr int MT_WIDE = 2048;
 //   3072 ->  8192 and 5120 -> 6912 (three steps per wavefront): the 16-row tile kernel at every M
 static bool mt_part_ok(const ForwardArgs& a, int width) {
     if (width < MT_WIDE) return false;
-    if (a.M >= 96) return true;
     int jpw, kw;
     mt_split(a.L->tile_nj, a.x_dtype == NQ_DT_F32, jpw, kw);
-    if (jpw < 1 || jpw > 2) return false;
+    // Three steps per wavefront (IN = 2560, 3072, 5120 ..): against the medium-M kernel this one loses over layers less
+    // than 4096 wide (2560 x 2560 at M = 135 15.1 against 12.5 us, 3072 x 3072 18.0 against 15.0) and, with Q4_0's
+    // per-chunk row sums no longer in registers, ties or loses over wider ones (2560 -> 5120 at M = 100 / 135 / 256
+    // 20.0 / 22.4 / 32.5 against 18.2 / 23.5 / 30.5); with groups of 128 it wins there (3072 -> 8192 22.7 / 26.8 /
+    // 38.2 against 25.9 / 32.3 / 50.7, 5120 x 5120 24.5 / 30.0 / 44.8 against 27.8 / 35.6 / 48.9).
+    if (jpw < 1 || jpw > 3) return false;
+    if (jpw == 3) return a.M >= 96 && width >= 4096 && a.L->format == NQ_FMT_W4_GROUP;
+    if (a.M >= 96) return true;
     return width >= 10240 || (a.M >= 48 && (int64_t)a.L->in * width >= ((int64_t)(jpw == 1 ? 16 : 24) << 20));
 }
 
