@@ -1064,6 +1064,12 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     // wider tiles leave the chip waiting for the last round; the 16 x 32 tile in twice as many
     // workgroups is faster)
     if (!xf32 && nsteps <= 8 && (mw * nw == 4) && wgs_of(mw, nw) >= 300 && wgs_of(mw, nw) < 1000) mw = 1, nw = 2;
+    // (longer K, 4-bit codes, bf16 activations: one workgroup of these tiles fits a CU, so 257 .. 512 of them are a
+    // full round and a part of one; the 32 x 64 tile then does the call in one round - 1536 x 1536 at M = 176 9.3 ->
+    // 8.0 us, 2560 x 2560 at M = 100 12.0 -> 10.1, 2560 -> 960 at M = 300 12.1 -> 10.1, 4096 x 4096 at M = 96 18.0 -> 14.8)
+    else if (!xf32 && four_bit && nsteps > 8 && mw * nw == 4 && wgs_of(mw, nw) > 256 && wgs_of(mw, nw) <= 512 &&
+             wgs_of(2, 4) <= 256)
+        mw = 2, nw = 4;
     // K split: 8 wavefronts when there are more than 4 k-steps.  It follows K alone: the K split fixes
     // the order in which an output's sum is formed, and a row must get the same bits whichever
     // layer (its own, or a row-fused one) it is computed in.

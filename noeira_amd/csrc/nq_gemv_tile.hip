@@ -1798,7 +1798,16 @@ static bool mt_part_ok(const ForwardArgs& a, int width) {
     // 38.2 against 25.9 / 32.3 / 50.7, 5120 x 5120 24.5 / 30.0 / 44.8 against 27.8 / 35.6 / 48.9).
     if (jpw < 1 || jpw > 3) return false;
     if (jpw == 3) return a.M >= 96 && width >= 4096 && a.L->format == NQ_FMT_W4_GROUP;
-    if (a.M >= 96) return true;
+    if (a.M >= 96) {
+        // Where the medium-M kernel covers the call with one round of its 32 x 64 tiles (a workgroup of them per CU,
+        // 256 CUs) it is the faster one from IN = 1280 on - 1280 -> 2560 at M = 135 8.0 against 9.5 us, 4096 x 4096 at
+        // M = 96 .. 128 15 against 18.6, 2048 -> 2560 at M = 160 .. 192 9.7 - 10.1 against 11.1 - 12.3 (and 9.4 against
+        // 8.7 at M = 100 .. 128) - beyond that round this kernel is (4096 x 4096 at M = 135 22.1 against 26.1, 4096 ->
+        // 11008 48 against 60, 960 -> 5120 10.2 against 11.7).
+        const int64_t a16_wgs = (int64_t)((a.M + 31) / 32) * ((width + 63) / 64);
+        if (a.x_dtype == NQ_DT_BF16 && a.L->tile_nj > 8 && a16_wgs <= 256) return false;
+        return true;
+    }
     return width >= 10240 || (a.M >= 48 && (int64_t)a.L->in * width >= ((int64_t)(jpw == 1 ? 16 : 24) << 20));
 }
 
