@@ -143,3 +143,26 @@ def test_default_dispatch_below_a_hundred_rows_over_large_layers():
         assert torch.equal(lin.forward(x), y)
     for part, y in zip((big, small), FusedRows([big, small]).forward(x)):
         assert torch.equal(y, part.forward(x))
+
+
+@pytest.mark.parametrize("M", [100, 135, 200])
+def test_default_dispatch_at_a_hundred_rows_follows_each_parts_own_rule(M):
+    """From a hundred rows on the choice between the M-tile kernel and the medium-M one follows each part's own width
+    and the row count (one round of 32 x 64 tiles, a three-step split of K): a row-fused layer whose parts fall on
+    different sides - IN = 2048 with parts 2560 and 8192 wide, and IN = 2560 (three steps) with 2560 and 5120 - returns
+    the bits of each part's own forward, and those are within the band of the fp64 product."""
+    rng = np.random.default_rng(91 + M)
+    for K, outs in ((2048, (2560, 8192)), (2560, (2560, 5120))):
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+        parts = [QLinear(K, n) for n in outs]
+        for lin in parts:
+            blocks = rng.integers(0, 256, (lin.OUT, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (lin.OUT, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+            y = lin.forward(x)
+            exact = x.double() @ lin.dequantized_dev().double().T
+            assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
+            assert torch.equal(lin.forward(x), y)
+        for part, y in zip(parts, FusedRows(parts).forward(x)):
+            assert torch.equal(y, part.forward(x))
