@@ -220,3 +220,41 @@ def test_single_row_fp32_x_through_lds(fmt):
         assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max()), tag
         assert torch.equal(y, lin.forward(x)), tag + ": a repeated call differs"
         del lin
+
+
+def test_random_large_layers():
+    """Layers of 8 M to 100 M weights with ragged OUT, at every row count from 1 to 300: the kernels over the
+    tile-ordered copy and the row-ordered ones (tile copy and preference drawn per case), bias + ReLU, fp32 or bf16
+    out, against the fp64 product of the dequantised weights; a repeated call returns the same bits."""
+    rng = np.random.default_rng(2026)
+    for case in range(60):
+        fmt = ["q4_0", "w4g", "w8"][case % 3]
+        K = int(rng.choice([2048, 2176, 2560, 3072, 4096, 4224, 5120, 6144, 8192]))
+        N = int(rng.integers(4000, 12500))
+        M = int(rng.choice([1, 2, 3, 5, 6, 8, 11, 16, 17, 24, 33, 48, 64, 95, 96, 100, 135, 200, 256, 300]))
+        prefer, tc = bool(rng.integers(0, 2)), bool(rng.integers(0, 4))
+        xdt = torch.bfloat16 if rng.integers(0, 3) else torch.float32
+        odt = torch.float32 if rng.integers(0, 2) else torch.bfloat16
+        if fmt == "q4_0":
+            lin = QLinear(K, N, tile_copy=tc, prefer_tile=prefer)
+            blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0] = sc & 0xFF
+            blocks[:, :, 1] = sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+        elif fmt == "w4g":
+            G = -(-K // 128)
+            codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
+            lin = W4GroupLinear(K, N, 128, tile_copy=tc, prefer_tile=prefer)
+            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+        else:
+            lin = W8Linear(K, N, tile_copy=tc, prefer_tile=prefer)
+            lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+        tag = "%s M=%d K=%d N=%d x=%s y=%s prefer=%d tile_copy=%d" % (fmt, M, K, N, str(xdt)[6:], str(odt)[6:], prefer, tc)
+        deq = lin.dequantized_dev().double()
+        bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
+        y = lin.forward(x, bias=bias, epilogue="relu", out_dtype=odt)
+        _check(tag, y, (x.double() @ deq.T + bias.double()).clamp_min(0), odt == torch.bfloat16)
+        assert torch.equal(lin.forward(x, bias=bias, epilogue="relu", out_dtype=odt), y), tag + ": a repeated call differs"
+        del lin, deq
