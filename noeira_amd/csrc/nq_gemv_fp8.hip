@@ -131,14 +131,17 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
         const void* const a_cs = scaled ? (const void*)(p.col_scale + n) : (const void*)p.w;
         const void* const a_b32 = b32 ? (const void*)(reinterpret_cast<const uint32_t*>(p.bias) + n) : (const void*)p.w;
         const void* const a_b16 = b16 ? (const void*)(reinterpret_cast<const uint16_t*>(p.bias) + n) : (const void*)p.w;
-        asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_cs[it]) : "v"(a_cs));
+        if constexpr (I8) asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_cs[it]) : "v"(a_cs));
+        else f_cs[it] = 0;  // (fp8: one scale per tensor, below)
         asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_b32[it]) : "v"(a_b32));
         asm volatile("global_load_ushort %0, %1, off ; pf" : "=v"(f_b16[it]) : "v"(a_b16));
 #pragma unroll
         for (int i = 0; i < MT; i++) {
             const void* const a_xs = scaled ? (const void*)(p.x_scale + min(m_base + 16 * i + ((t & 255) >> 4), p.M - 1))
                                             : (!I8 ? (const void*)p.x_scale : (const void*)p.w);  // (fp8: per tensor)
-            asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_xs[i][it]) : "v"(a_xs));
+            // (a condition on unrolled indices: decided at compile time, no branch)
+            if (I8 || (i == 0 && it == 0)) asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(f_xs[i][it]) : "v"(a_xs));
+            else f_xs[i][it] = 0;
         }
     }
 
