@@ -150,6 +150,8 @@ int32_t launch_w4g_repack(uint8_t* codes, int64_t nchunks, hipStream_t s);
 // nq_gemm_a16.hip: medium-M dequant GEMM on the bf16 matrix cores
 bool gemm_a16_applicable(const ForwardArgs& a);
 int32_t launch_gemm_a16(const ForwardArgs& a);
+// the medium-M kernel's tile shape for a call (M >= 2, below the many-rows kernel's range) and its estimated time
+float gemm_a16_estimate_us(int32_t format, bool xf32, int M, int N, int K, int* mw_out, int* nw_out);
 
 // nq_gemv.hip: dequant-GEMV for small M (also the any-M fallback)
 int32_t launch_gemv(const ForwardArgs& a);

@@ -983,6 +983,63 @@ int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipSt
 
 }  // namespace
 
+// Tile shape of the medium-M kernel (wavefront tiles of 16 rows x 16 columns: mw x nw of them per workgroup) and what
+// the call will take.  One workgroup of any shape fits a CU at a time, so a call runs in ceil(workgroups / 256)
+// rounds, and a round costs a fixed part and a part per k-step that both grow with the tile: measured over K = 512 ..
+// 6144, N = 320 .. 4096 and M = 17 .. 500 for each format and activation type (five shapes each, 3000 calls), a call
+// takes
+//     t = F + rounds * (p0 + p1 * k-steps)   microseconds
+// within 3 - 6 % on average, with the constants below.  The shape with the least estimate is taken: over those calls
+// that is within 1 % of always taking the fastest shape (the rules it replaces - the widest tile that still gave 128
+// workgroups, none with two M tiles for an odd count of them - were 5 - 18 % off: with fp32 activations two M tiles
+// per wavefront are never worth their registers, 4096 x 4096 int8 codes at M = 256 67 -> 47 us, and with bf16 ones an
+// odd count of M tiles is worth padding, 2048 x 2048 at M = 135 9.4 -> 7.9 us).  The shape changes which workgroup
+// computes an output, not the order of its sum.
+float gemm_a16_estimate_us(int32_t format, bool xf32, int M, int N, int K, int* mw_out, int* nw_out) {
+    struct ShapeCost {
+        int mw, nw;
+        float f, p0, p1;
+    };
+    static const ShapeCost costs[6][5] = {
+        // 8-bit codes (int8, e4m3), bf16 activations
+        {{2, 4, 1.18f, 2.773f, 0.1292f}, {2, 2, 2.56f, 0.495f, 0.0795f}, {1, 4, 2.52f, 0.579f, 0.0972f},
+         {1, 2, 2.41f, 0.256f, 0.0518f}, {1, 1, 2.36f, 0.205f, 0.0318f}},
+        // 8-bit codes, fp32 activations (the 2 x 4 shape does not fit the registers)
+        {{2, 4, 0, 0, 0}, {2, 2, 1.10f, 1.796f, 0.1967f}, {1, 4, 2.55f, 0.536f, 0.1604f},
+         {1, 2, 2.44f, 0.232f, 0.1084f}, {1, 1, 2.53f, 0.133f, 0.0788f}},
+        // Q4_0, bf16 activations
+        {{2, 4, 1.68f, 2.926f, 0.2849f}, {2, 2, 1.70f, 1.690f, 0.1809f}, {1, 4, 1.90f, 1.621f, 0.2214f},
+         {1, 2, 2.82f, 0.333f, 0.1093f}, {1, 1, 2.59f, 0.190f, 0.0722f}},
+        // Q4_0, fp32 activations
+        {{2, 4, 0, 0, 0}, {2, 2, 2.03f, 1.825f, 0.3953f}, {1, 4, 1.99f, 1.759f, 0.3347f},
+         {1, 2, 2.17f, 0.711f, 0.2540f}, {1, 1, 2.80f, 0.198f, 0.1620f}},
+        // 4-bit codes in groups with zero points, bf16 activations
+        {{2, 4, 1.69f, 2.576f, 0.2536f}, {2, 2, 1.75f, 1.402f, 0.1698f}, {1, 4, 2.08f, 1.169f, 0.2006f},
+         {1, 2, 2.69f, 0.302f, 0.0984f}, {1, 1, 2.54f, 0.162f, 0.0667f}},
+        // 4-bit codes in groups with zero points, fp32 activations
+        {{2, 4, 0, 0, 0}, {2, 2, 2.03f, 1.446f, 0.3875f}, {1, 4, 1.96f, 1.469f, 0.3212f},
+         {1, 2, 2.15f, 0.562f, 0.2366f}, {1, 1, 2.70f, 0.142f, 0.1565f}},
+    };
+    const bool four_bit = format != NQ_FMT_W8_CHANNEL && format != NQ_FMT_FP8_E4M3;
+    const int mt = (M + 15) / 16;
+    const int kstep = four_bit ? 128 : 64;
+    const int nsteps = (K + kstep - 1) / kstep;
+    const ShapeCost* row = costs[(!four_bit ? 0 : format == NQ_FMT_Q4_0 ? 2 : 4) + (xf32 ? 1 : 0)];
+    int mw = 1, nw = 1;
+    float least = 0.0f;
+    for (int c = 0; c < 5; c++) {
+        const ShapeCost& sc = row[c];
+        if (sc.mw * sc.nw == 8 && xf32) continue;
+        if (sc.mw == 2 && mt == 1) continue;  // a second M tile of padding only
+        const int64_t wgs = (int64_t)((mt + sc.mw - 1) / sc.mw) * ((N + 16 * sc.nw - 1) / (16 * sc.nw));
+        const float t = sc.f + (float)((wgs + 255) / 256) * (sc.p0 + sc.p1 * (float)nsteps);
+        if (least == 0.0f || t < least) least = t, mw = sc.mw, nw = sc.nw;
+    }
+    if (mw_out) *mw_out = mw;
+    if (nw_out) *nw_out = nw;
+    return least;
+}
+
 bool gemm_a16_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (a.x_dtype != NQ_DT_F32 && a.x_dtype != NQ_DT_BF16) return false;
@@ -1035,41 +1092,10 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
                             : launch_big<NQ_FMT_FP8_E4M3, false, false>(p, big, bnw, a.stream);
         }
     }
-    // Tile shape: as wide in N as still leaves enough workgroups to occupy the chip (the
-    // activations are the operand that is re-read per N tile), two M tiles per wavefront only
-    // when that costs no extra padded rows
-    // (measured at M = 100..256: the 2 x 4 tile only pays once there is work for several
-    // rounds of workgroups, and below ~128 workgroups a narrower tile wins)
-    // (and that over a weight too large to stay in the caches a workgroup per CU is the least to ask for)
-    const bool big = (int64_t)L->in * L->out >= ((int64_t)4 << 20);
-    static const int shapes[5][2] = {{2, 4}, {2, 2}, {1, 4}, {1, 2}, {1, 1}};
     int mw = 1, nw = 1;
-    const int mt = (a.M + 15) / 16;
-    for (int c = 0; c < 5; c++) {
-        mw = shapes[c][0], nw = shapes[c][1];
-        // (an odd count of 16-row tiles: two per wavefront pads one tile.  With bf16 activations over 4-bit codes
-        // that is worth it from seven tiles on - 2560 -> 960 at T = 135 7.7 -> 6.8 us, 960 -> 960 5.6 -> 5.0, 2560 x
-        // 2560 13.8 -> 12.0 - the same shapes with fp32 activations or int8 codes measured 5 - 15 % slower for it)
-        if (mw == 2 && (mt & 1) && mt < 16 && !(four_bit && !xf32 && mt >= 7)) continue;
-        if (mw * nw == 8 && xf32) continue;  // would not fit the register budget
-        const int64_t wgs = (int64_t)((mt + mw - 1) / mw) * ((L->out + 16 * nw - 1) / (16 * nw));
-        if (wgs >= (mw * nw == 8 ? 2048 : big ? 160 : 128)) break;
-    }
+    gemm_a16_estimate_us(L->format, xf32, a.M, L->out, L->in, &mw, &nw);
     const int kstep = four_bit ? 128 : 64;
     const int nsteps = (L->in + kstep - 1) / kstep;
-    auto wgs_of = [&](int mw_, int nw_) {
-        return (int64_t)((mt + mw_ - 1) / mw_) * ((L->out + 16 * nw_ - 1) / (16 * nw_));
-    };
-    // (measured with bf16 activations and short K, at most 8 k-steps: a few hundred workgroups of the
-    // wider tiles leave the chip waiting for the last round; the 16 x 32 tile in twice as many
-    // workgroups is faster)
-    if (!xf32 && nsteps <= 8 && (mw * nw == 4) && wgs_of(mw, nw) >= 300 && wgs_of(mw, nw) < 1000) mw = 1, nw = 2;
-    // (longer K, 4-bit codes, bf16 activations: one workgroup of these tiles fits a CU, so 257 .. 512 of them are a
-    // full round and a part of one; the 32 x 64 tile then does the call in one round - 1536 x 1536 at M = 176 9.3 ->
-    // 8.0 us, 2560 x 2560 at M = 100 12.0 -> 10.1, 2560 -> 960 at M = 300 12.1 -> 10.1, 4096 x 4096 at M = 96 18.0 -> 14.8)
-    else if (!xf32 && four_bit && nsteps > 8 && mw * nw == 4 && wgs_of(mw, nw) > 256 && wgs_of(mw, nw) <= 512 &&
-             wgs_of(2, 4) <= 256)
-        mw = 2, nw = 4;
     // K split: 8 wavefronts when there are more than 4 k-steps.  It follows K alone: the K split fixes
     // the order in which an output's sum is formed, and a row must get the same bits whichever
     // layer (its own, or a row-fused one) it is computed in.

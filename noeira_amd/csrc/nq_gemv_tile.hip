@@ -1764,51 +1764,56 @@ int32_t launch_gemv_tile8_rows(const ForwardArgs& a) {
     return NQ_OK;
 }
 
-// 96 .. 256 rows of bf16 activations, or 96 .. 512 of fp32 ones where IN <= 2048, over a wide 4-bit layer with a tile copy.
-// Where it wins over the 16-row tile kernel was measured at IN = 960 / 2560, OUT = 320 .. 5120, M = 17 .. 512: wide
-// layers (it amortises a workgroup's start over many weight tiles; a narrow layer gives it one or two), a hundred
-// rows and more.  Everything but the width:
+// 17 .. 511 rows of bf16 activations, or of fp32 ones where IN <= 2048, over a wide 4-bit layer with a tile copy.
+// Everything but the width:
 static bool mt_shape_ok(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (!L->d_tile16 || L->format == NQ_FMT_W8_CHANNEL || L->tile_nj > 48) return false;
     if (a.y_dtype != NQ_DT_F32 && a.y_dtype != NQ_DT_BF16) return false;
     if ((int64_t)a.M * L->in >= ((int64_t)1 << 31)) return false;
     if (a.M < 2 || a.M > 512) return false;
-    if (!L->prefer_tile && a.M < 17) return false;
-    if (a.x_dtype == NQ_DT_BF16) return L->prefer_tile || a.M <= 256;
-    return a.x_dtype == NQ_DT_F32 && L->tile_nj <= 16 && (L->prefer_tile || a.M >= 96);
+    if (!L->prefer_tile && (a.M < 17 || a.M > 511)) return false;  // (from 512 rows on: the many-rows kernel)
+    if (a.x_dtype == NQ_DT_BF16) return true;
+    return a.x_dtype == NQ_DT_F32 && L->tile_nj <= 16;
 }
 constexpr int MT_WIDE = 2048;
 
-// ... and the width, which is each part's own.  A hundred rows and more: 2048 columns.  Below (17 .. 95 rows of bf16
-// activations; the 16-row tile kernel re-reads and re-unpacks the weights per 16 rows) only over large layers whose
-// split of K leaves a wavefront at most two steps, by these measurements (us, 16-row tile kernel / this one):
-//   2048 -> 11008: M = 17 11.4 / 9.2, 64 17.1 / 13.7, 95 26.2 / 19.7     2048 -> 8192: 17 7.0 / 7.7, 48 13.0 / 11.2
-//   4096 -> 11008: 17 17.1 / 13.9, 64 26.2 / 22.6                        4096 -> 8192: 32 10.5 / 12.1, 48 19.8 / 17.5
-//   4096 ->  6144: 32 9.9 / 10.6, 48 19.1 / 14.6                         4096 -> 4096: 48 10.9 / 12.3
-//   3072 ->  8192 and 5120 -> 6912 (three steps per wavefront): the 16-row tile kernel at every M
+// What a call of this kernel takes, in microseconds.  Its workgroups (M tiles x column groups, at most one per CU)
+// run in one round and each walks `iters` sets of weight tiles; over IN = 512 .. 6144, OUT = 960 .. 11008 and
+// M = 17 .. 384 (2000 calls) a call took F + iters * q within 4 - 5 % on average, F and q by format, activation type
+// and the steps of K per wavefront.
+static float mt_estimate_us(const ForwardArgs& a, int width) {
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
+    int jpw, kw;
+    mt_split(a.L->tile_nj, xf32, jpw, kw);
+    if (jpw < 1 || jpw > 3) return 0.0f;
+    static const float fq[2][4][2] = {
+        // Q4_0: bf16 activations with 1, 2, 3 steps per wavefront; fp32 activations
+        {{4.15f, 0.938f}, {5.51f, 1.660f}, {6.84f, 2.559f}, {6.19f, 0.905f}},
+        // groups of 128 with zero points
+        {{4.15f, 0.860f}, {5.46f, 1.454f}, {7.18f, 1.835f}, {6.11f, 0.846f}},
+    };
+    const float* c = fq[a.L->format == NQ_FMT_Q4_0 ? 0 : 1][xf32 ? 3 : jpw - 1];
+    const int ng = 16 / kw, sets = ((width + 15) / 16 + ng - 1) / ng, mt = (a.M + 15) / 16;
+    const int gx = std::max(1, std::min(sets, 256 / mt));
+    return c[0] + (float)((sets + gx - 1) / gx) * c[1];
+}
+
+// ... and the width, which is each part's own: 2048 columns and more (a narrower layer gives a workgroup one or two
+// weight tiles to amortise its start over), and wherever this kernel's estimate is below the medium-M kernel's for the
+// same part.  Measured side by side over the calls above, the pair of estimates picks the slower kernel by more than
+// a tenth in 70 of 2000 calls and costs 0.3 - 1.3 % in total against always picking the faster one (the rules
+// it replaces - row counts from 96, a round of the other kernel's widest tile, three steps of K only over groups of
+// 128 - cost 0.5 - 3.1 %, and up to 50 % where they did not look: fp32 activations below 96 rows over the widest
+// layers, 2048 -> 11008 at M = 33 24 -> 15 us, groups of 128 at IN = 2560 .. 3072 and a hundred rows, 2560 -> 4096
+// 13.7 -> 8.9 us).
 static bool mt_part_ok(const ForwardArgs& a, int width) {
     if (width < MT_WIDE) return false;
-    int jpw, kw;
-    mt_split(a.L->tile_nj, a.x_dtype == NQ_DT_F32, jpw, kw);
-    // Three steps per wavefront (IN = 2560, 3072, 5120 ..): against the medium-M kernel this one loses over layers less
-    // than 4096 wide (2560 x 2560 at M = 135 15.1 against 12.5 us, 3072 x 3072 18.0 against 15.0) and, with Q4_0's
-    // per-chunk row sums no longer in registers, ties or loses over wider ones (2560 -> 5120 at M = 100 / 135 / 256
-    // 20.0 / 22.4 / 32.5 against 18.2 / 23.5 / 30.5); with groups of 128 it wins there (3072 -> 8192 22.7 / 26.8 /
-    // 38.2 against 25.9 / 32.3 / 50.7, 5120 x 5120 24.5 / 30.0 / 44.8 against 27.8 / 35.6 / 48.9).
-    if (jpw < 1 || jpw > 3) return false;
-    if (jpw == 3) return a.M >= 96 && width >= 4096 && a.L->format == NQ_FMT_W4_GROUP;
-    if (a.M >= 96) {
-        // Where the medium-M kernel covers the call with one round of its 32 x 64 tiles (a workgroup of them per CU,
-        // 256 CUs) it is the faster one from IN = 1280 on - 1280 -> 2560 at M = 135 8.0 against 9.5 us, 4096 x 4096 at
-        // M = 96 .. 128 15 against 18.6, 2048 -> 2560 at M = 160 .. 192 9.7 - 10.1 against 11.1 - 12.3 (and 9.4 against
-        // 8.7 at M = 100 .. 128) - beyond that round this kernel is (4096 x 4096 at M = 135 22.1 against 26.1, 4096 ->
-        // 11008 48 against 60, 960 -> 5120 10.2 against 11.7).
-        const int64_t a16_wgs = (int64_t)((a.M + 31) / 32) * ((width + 63) / 64);
-        if (a.x_dtype == NQ_DT_BF16 && a.L->tile_nj > 8 && a16_wgs <= 256) return false;
-        return true;
-    }
-    return width >= 10240 || (a.M >= 48 && (int64_t)a.L->in * width >= ((int64_t)(jpw == 1 ? 16 : 24) << 20));
+    const float mine = mt_estimate_us(a, width);
+    if (mine == 0.0f) return false;
+    // (estimates within a tenth of each other go to this kernel: it is the one that can carry an adapter in the same
+    // launch, and over the measured calls that margin costs 0.1 - 0.2 % more)
+    return mine < 1.10f * gemm_a16_estimate_us(a.L->format, a.x_dtype == NQ_DT_F32, a.M, width, a.L->in, nullptr, nullptr);
 }
 
 // A row-fused layer runs on this kernel in one launch when all its parts pass, on the other kernel when none does,
