@@ -256,8 +256,8 @@ int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features,
  * `QLoRALinear.forward` makes, tests/nn/quant/qlora_common.mojo).  Where the base call runs on the kernel that keeps
  * its rows' activations resident (4-bit layers with 512 <= IN <= 4096 whose split of K leaves a wavefront at most two
  * steps of 128: IN <= 1280, 1537..2048 and 3073..4096; fp32 activations: IN <= 2048 - at 2..512 rows when made with
- * NQ_FLAG_PREFER_TILE, else a hundred rows and more over layers at least 2048 wide and 17 rows and more of bf16
- * activations over the largest ones, wherever nq_forward itself takes that kernel; R_PAD <= 16)
+ * NQ_FLAG_PREFER_TILE, else 17 .. 511 rows over layers at least 2048 wide, wherever nq_forward itself takes that
+ * kernel: where its estimated time is the lower one, e.g. 960 -> 2560 at 135 rows; R_PAD <= 16)
  * the adapter is folded into that launch: h = x A is formed once per 16 rows from the activations the workgroup
  * already holds, and s * h B is added before the store; y may then be fp32 or bf16.  Elsewhere it is nq_forward
  * followed by nq_lora_forward_add (y fp32).  Either way B = 0 returns the bits of nq_forward on the same arguments. */

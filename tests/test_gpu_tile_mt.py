@@ -109,9 +109,10 @@ def test_row_fused_parts_and_glu(M, xdt):
 
 
 def test_default_dispatch_keeps_fused_parts_bitwise():
-    """By default the M-tile kernel takes wide layers at a hundred rows and more, and a row-fused layer by its
-    narrowest part: gate | up (2560 | 2560) and each of the two alone run on it, q | k | v (960 | 320 | 320) and its parts do
-    not; either way every part of the fused launch carries the bits of its own forward."""
+    """By default the M-tile kernel takes layers 2048 wide and more where its estimated time is the lower one, and a
+    row-fused layer part by part: gate | up (2560 | 2560) and each of the two alone run on it at T = 135, q | k | v
+    (960 | 320 | 320) and its parts do not; either way every part of the fused launch carries the bits of its own
+    forward."""
     rng = np.random.default_rng(77)
     M, IN = 135, 960
     mk = lambda n: QLinear.from_linear((rng.standard_normal((IN, n)) * 0.05).astype(np.float32))
@@ -124,10 +125,9 @@ def test_default_dispatch_keeps_fused_parts_bitwise():
 
 
 def test_default_dispatch_below_a_hundred_rows_over_large_layers():
-    """17 .. 95 rows of bf16 activations take the M-tile kernel by default over large layers whose split of K leaves
-    a wavefront at most two steps (2048 -> 11008 here; 2048 -> 2048 stays on the 16-row tile kernel): against fp64
-    over the dequantised weights, and a row-fused layer of a large and a small part returns the bits of each part's
-    own forward."""
+    """Below a hundred rows the M-tile kernel takes a call by default over the widest layers (2048 -> 11008 here;
+    2048 -> 2048 stays on the 16-row tile kernel): against fp64 over the dequantised weights, and a row-fused layer of
+    a large and a small part returns the bits of each part's own forward."""
     rng = np.random.default_rng(83)
     K, M = 2048, 33
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
@@ -147,10 +147,10 @@ def test_default_dispatch_below_a_hundred_rows_over_large_layers():
 
 @pytest.mark.parametrize("M", [100, 135, 200])
 def test_default_dispatch_at_a_hundred_rows_follows_each_parts_own_rule(M):
-    """From a hundred rows on the choice between the M-tile kernel and the medium-M one follows each part's own width
-    and the row count (one round of 32 x 64 tiles, a three-step split of K): a row-fused layer whose parts fall on
-    different sides - IN = 2048 with parts 2560 and 8192 wide, and IN = 2560 (three steps) with 2560 and 5120 - returns
-    the bits of each part's own forward, and those are within the band of the fp64 product."""
+    """The choice between the M-tile kernel and the medium-M one follows each part's own width and the row count
+    (the two kernels' estimated times): a row-fused layer whose parts may fall on different sides - IN = 2048 with
+    parts 2560 and 8192 wide, and IN = 2560 (three steps of K per wavefront) with 2560 and 5120 - returns the bits of
+    each part's own forward, and those are within the band of the fp64 product."""
     rng = np.random.default_rng(91 + M)
     for K, outs in ((2048, (2560, 8192)), (2560, (2560, 5120))):
         x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
@@ -166,3 +166,41 @@ def test_default_dispatch_at_a_hundred_rows_follows_each_parts_own_rule(M):
             assert torch.equal(lin.forward(x), y)
         for part, y in zip(parts, FusedRows(parts).forward(x)):
             assert torch.equal(y, part.forward(x))
+
+
+@pytest.mark.parametrize("fmt,K,N,M,xdt", [
+    ("q4_0", 2048, 11008, 33, torch.float32),    # fp32 activations below a hundred rows over the widest layers
+    ("w4g", 1280, 8192, 48, torch.float32),
+    ("q4_0", 960, 8192, 384, torch.bfloat16),    # bf16 activations beyond 256 rows
+    ("w4g", 2048, 11008, 500, torch.bfloat16),
+    ("w4g", 2560, 4096, 96, torch.bfloat16),     # three steps of K per wavefront at a hundred rows
+    ("q4_0", 3072, 5120, 160, torch.bfloat16),
+    ("q4_0", 960, 2560, 511, torch.float32),     # the last row count before the many-rows kernel
+])
+def test_default_dispatch_by_estimate(fmt, K, N, M, xdt):
+    """Calls whose kernel changed when the dispatch went from row-count and width thresholds to the two kernels'
+    estimated times: whichever takes them, the result is within the fp32 band of the fp64 product over the
+    dequantised weights, repeats bit for bit, and a row-fused layer of two such parts returns each part's own bits."""
+    rng = np.random.default_rng(K + N + M)
+    def layer(n):
+        if fmt == "q4_0":
+            lin = QLinear(K, n)
+            blocks = rng.integers(0, 256, (n, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (n, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+            return lin
+        G = -(-K // 128)
+        codes, zps = F.pack_w4g(rng.integers(0, 16, (n, K), dtype=np.uint8), rng.integers(0, 16, (n, G), dtype=np.uint8))
+        lin = W4GroupLinear(K, n, 128)
+        lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (n, G)).astype(np.float16), zps)
+        return lin
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
+    big, small = layer(N), layer(960)
+    for lin in (big, small):
+        y = lin.forward(x)
+        exact = x.double() @ lin.dequantized_dev().double().T
+        assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
+        assert torch.equal(lin.forward(x), y)
+    for part, y in zip((big, small), FusedRows([big, small]).forward(x)):
+        assert torch.equal(y, part.forward(x))
