@@ -23,6 +23,9 @@ batched-env actor at M = 4096, in TOPS); `roofline_mfma` is the large-M fp8 GEMM
 (config 5) beside what the matrix cores alone sustain on the same GPU
 (`mfma_only`: back-to-back MFMAs on register operands, constant and random data).
 
+`--only a16_shapes --a16-class C` re-derives the constants by which the library picks the tile shape of its
+kernel for tens to hundreds of activation rows (a grid of calls timed under each shape, nq_diag_a16_shape).
+
 `cpu_baseline` times the CPU oracle's restatement of the reference's CPU
 forward (a fresh dequantize to an fp32 scratch, then the serial triple loop;
 noeira/nn/quant/qlinear.mojo:416-426, noeira/nn/core/cpu_gemm.mojo:88-98) on
@@ -805,12 +808,96 @@ def cpu_baseline(budget_s=12.0):
                       f"fp32 [OUT, IN] scratch then the serial triple loop, single thread, {dt:.1f} s"}
 
 
+def a16_shapes(cls="w4g"):
+    """Times a grid of medium-M calls of one weight format / activation type under each of the 16-row tile kernel's
+    five tile shapes (`nq_diag_a16_shape`) and under the library's own choice, and re-derives the constants of
+    the estimate the library chooses by: t = F + ceil(workgroups / 256) * (p0 + p1 * k-steps) microseconds per
+    shape, by least squares on relative errors.  Reports the constants, the fit's mean error, what always taking
+    the shape of least estimate costs against always taking the fastest, and the same for the library's choice."""
+    import numpy as np
+    import torch
+
+    from noeira_amd import _lib as L
+    from noeira_amd import formats as F
+    from noeira_amd.qlinear import QLinear, W4GroupLinear, W8Linear
+
+    xf32, kind = cls.endswith("f"), cls.rstrip("f")
+    kstep = 64 if kind == "w8" else 128
+    rng = np.random.default_rng(1)
+    shapes = [(2, 4), (2, 2), (1, 4), (1, 2), (1, 1)]
+    rows = []
+    for K in ((512, 2048, 4096) if kind == "w8" else (960, 2048, 4096)):
+        for N in (512, 2048, 4096):
+            if kind == "q4":
+                lin = QLinear(K, N, tile_copy=False)
+                blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+                sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+                blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+                lin.set_blocks(blocks.reshape(-1))
+            elif kind == "w4g":
+                G = -(-K // 128)
+                codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
+                lin = W4GroupLinear(K, N, 128, tile_copy=False)
+                lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+            else:
+                lin = W8Linear(K, N, tile_copy=False)
+                lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+            for M in (17, 64, 100, 135, 256, 384, 500):
+                x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda()
+                x = x if xf32 else x.to(torch.bfloat16)
+                y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+                step = lambda i: lin.forward(x, out=y)
+                median_per_call(step, 20)  # (clocks up before the first timed shape)
+                ts = []
+                for mw, nw in shapes + [(0, 0)]:
+                    L.check(L.lib().nq_diag_a16_shape(mw, nw))
+                    ts.append(float("nan") if (xf32 and mw * nw == 8) else median_per_call(step, 20) * 1e6)
+                rows.append((K, N, M, ts))
+    L.check(L.lib().nq_diag_a16_shape(0, 0))
+
+    def feats(K, N, M, mw, nw):
+        mt = (M + 15) // 16
+        wgs = ((mt + mw - 1) // mw) * ((N + 16 * nw - 1) // (16 * nw))
+        return -(-wgs // 256), (K + kstep - 1) // kstep
+
+    consts, errs = {}, {}
+    for si, (mw, nw) in enumerate(shapes):
+        A, t = [], []
+        for K, N, M, ts in rows:
+            if ts[si] == ts[si]:
+                R, ns = feats(K, N, M, mw, nw)
+                A.append([1.0, R, R * ns])
+                t.append(ts[si])
+        if not A:
+            continue
+        A, t = np.array(A), np.array(t)
+        c = np.linalg.lstsq(A / t[:, None], np.ones(len(t)), rcond=None)[0]
+        consts[(mw, nw)] = c
+        errs[(mw, nw)] = float(np.mean(np.abs(A @ c - t) / t))
+    by_estimate = fastest = library = 0.0
+    for K, N, M, ts in rows:
+        est = {}
+        for si, sh in enumerate(shapes):
+            if sh in consts and not (sh[0] == 2 and M <= 16):
+                R, ns = feats(K, N, M, *sh)
+                est[si] = consts[sh][0] + R * (consts[sh][1] + consts[sh][2] * ns)
+        by_estimate += ts[min(est, key=est.get)]
+        fastest += min(v for v in ts[:5] if v == v)
+        library += ts[5]
+    return {"only": "a16_shapes", "class": cls, "calls": len(rows),
+            "constants_F_p0_p1": {f"{mw}x{nw}": [round(float(v), 4) for v in c] for (mw, nw), c in consts.items()},
+            "fit_mean_rel_err": {f"{mw}x{nw}": round(e, 4) for (mw, nw), e in errs.items()},
+            "least_estimate_vs_fastest": round(by_estimate / fastest, 4),
+            "library_choice_vs_fastest": round(library / fastest, 4)}
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline", "a16_shapes"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
@@ -823,6 +910,8 @@ def main():
     ap.add_argument("--rows-layout", action="store_true",
                     help="large layers keep only their row-ordered codes (NQ_FLAG_NO_TILE_COPY): the single-row kernels "
                          "that read them, for a before / after comparison with the tile-ordered copy")
+    ap.add_argument("--a16-class", default="w4g", choices=["w8", "w8f", "q4", "q4f", "w4g", "w4gf"],
+                    help="with --only a16_shapes: int8 codes, Q4_0 or groups of 128 with zero points; f: fp32 activations")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     a = ap.parse_args()
@@ -838,6 +927,9 @@ def main():
     if a.rows_layout:
         global TILE_COPY
         TILE_COPY = False
+    if a.only == "a16_shapes":
+        print(json.dumps(a16_shapes(a.a16_class)))
+        return
     if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return

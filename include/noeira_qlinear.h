@@ -343,6 +343,13 @@ int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream);
 int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
                                int32_t y_dtype, int32_t M, uint64_t* stamps, int64_t max_tiles, void* stream);
 
+/* The tile shape of the 16-row tile kernel that takes 2 .. 511 rows of fp32 / bf16 activations (no counterpart in
+ * the reference): mw x nw wavefront tiles of 16 x 16 per workgroup, one of 1 x 1, 1 x 2, 1 x 4, 2 x 2, 2 x 4, for
+ * every later call in the process until (0, 0) gives the choice back to the library.  The library picks the shape
+ * of least estimated time; `bench.py --only a16_shapes` times a grid of calls under each shape with this switch and
+ * re-derives the estimate's constants from them.  The shape never changes a result's bits. */
+int32_t nq_diag_a16_shape(int32_t mw, int32_t nw);
+
 #ifdef __cplusplus
 }
 #endif

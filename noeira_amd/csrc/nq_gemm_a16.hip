@@ -39,6 +39,8 @@
 #include <algorithm>
 
 
+#include <atomic>
+
 #include "nq_common.h"
 
 namespace nq {
@@ -983,6 +985,9 @@ int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipSt
 
 }  // namespace
 
+// the shape nq_diag_a16_shape asked for (mw << 4 | nw), 0: none
+static std::atomic<int> g_diag_shape{0};
+
 // Tile shape of the medium-M kernel (wavefront tiles of 16 rows x 16 columns: mw x nw of them per workgroup) and what
 // the call will take.  One workgroup of any shape fits a CU at a time, so a call runs in ceil(workgroups / 256)
 // rounds, and a round costs a fixed part and a part per k-step that both grow with the tile: measured over K = 512 ..
@@ -1094,6 +1099,10 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     }
     int mw = 1, nw = 1;
     gemm_a16_estimate_us(L->format, xf32, a.M, L->out, L->in, &mw, &nw);
+    if (const int forced = g_diag_shape.load(std::memory_order_relaxed)) {
+        // nq_diag_a16_shape: a measurement asked for one shape (2 x 4 does not exist for fp32 activations)
+        if (!(xf32 && forced == 0x24)) mw = forced >> 4, nw = forced & 15;
+    }
     const int kstep = four_bit ? 128 : 64;
     const int nsteps = (L->in + kstep - 1) / kstep;
     // K split: 8 wavefronts when there are more than 4 k-steps.  It follows K alone: the K split fixes
@@ -1123,3 +1132,14 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
 }
 
 }  // namespace nq
+
+extern "C" int32_t nq_diag_a16_shape(int32_t mw, int32_t nw) {
+    if (mw == 0 && nw == 0) {
+        nq::g_diag_shape.store(0);
+        return NQ_OK;
+    }
+    if ((mw != 1 && mw != 2) || (nw != 1 && nw != 2 && nw != 4) || (mw == 2 && nw == 1))
+        return nq::fail(NQ_ERR_INVALID, "nq_diag_a16_shape: shapes are 1 x 1, 1 x 2, 1 x 4, 2 x 2, 2 x 4 (0, 0: the library's own choice)");
+    nq::g_diag_shape.store(mw << 4 | nw);
+    return NQ_OK;
+}

@@ -372,3 +372,27 @@ def test_stream_read_diagnostic_really_reads():
     us = e0.elapsed_time(e1) * 1e3 / 12
     assert us > 33.5, f"a plain read of 256 MiB took {us:.1f} us: the loads were not issued"
     assert us < 200
+
+
+def test_a16_shape_switch_changes_no_bits():
+    """nq_diag_a16_shape fixes the tile shape of the 16-row tile kernel for the calls that follow (bench.py times a
+    grid of calls under each shape with it).  A shape decides which workgroup computes an output, not the order of
+    its sum: every shape returns the bits of the library's own choice, for each format and activation type; shapes
+    that do not exist are refused, and (0, 0) gives the choice back."""
+    lib = L.lib()
+    rng = np.random.default_rng(61)
+    try:
+        for fmt, K, N, M in (("q4_0", 960, 1000, 135), ("w4g", 2560, 520, 40), ("w8", 3200, 512, 100), ("w4g64", 992, 300, 77)):
+            lin = _make(fmt, K, N, rng, False)
+            for xdt in (torch.float32, torch.bfloat16):
+                x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
+                L.check(lib.nq_diag_a16_shape(0, 0))
+                want = lin.forward(x)
+                for mw, nw in ((1, 1), (1, 2), (1, 4), (2, 2), (2, 4)):
+                    L.check(lib.nq_diag_a16_shape(mw, nw))
+                    assert torch.equal(lin.forward(x).view(torch.int32), want.view(torch.int32)), (fmt, xdt, mw, nw)
+        for mw, nw in ((2, 1), (3, 2), (1, 3), (0, 1), (-1, -1)):
+            assert lib.nq_diag_a16_shape(mw, nw) == L.NQ_ERR_INVALID
+            assert "shapes are" in L.last_error()
+    finally:
+        L.check(lib.nq_diag_a16_shape(0, 0))
