@@ -47,6 +47,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
 MFMA_PEAK_TOPS = {"fp8": 5000.0, "int8": 5000.0, "bf16": 2500.0}
 SAMPLES, COLD_BYTES = 7, 512 << 20
+SETTLE_S = 0.05  # warm-up replays before the samples of a row (see median_per_call)
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (fetched + written), scaled by
 # what the same counters read for a plain copy of known size; None until measured
 HEADLINE_TRAFFIC = 1804544      # mean of the two linears' launches (1.66 MB algorithmic)
@@ -109,15 +110,23 @@ def capture(fn, n):
 
 
 def median_per_call(fn, calls, graph=True):
-    """The reference's protocol (warm once, SAMPLES samples of `calls` calls between two
-    synchronisations, median sample / calls), with the calls of a sample replayed from a graph."""
+    """The reference's protocol (warm up, SAMPLES samples of `calls` calls between two
+    synchronisations, median sample / calls), with the calls of a sample replayed from a graph.
+    The warm-up lasts SETTLE_S of replays, not one call: after an idle spell (the host building the next
+    workload) the matrix-core-bound calls need 30 - 40 ms to reach their steady rate - config 5's GEMM runs at
+    117, then 136, then 104 - 105 us per launch, where it stays - and a sample taken earlier times the power
+    management's transient, not the kernel.  The memory-bound calls show no such transient."""
     import torch
 
     tm = Timer()
     if graph:
         g = capture(fn, calls)
-        g.replay()
-        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while True:
+            g.replay()
+            torch.cuda.synchronize()
+            if time.perf_counter() - t0 >= SETTLE_S:
+                break
         ts = [tm.run(lambda i: g.replay(), 1) / calls for _ in range(SAMPLES)]
     else:
         fn(0)
