@@ -485,8 +485,10 @@ def mfma_only(iters=4096, reps=5):
         def go(_i=0):
             L.check(lib.nq_diag_mfma_rate(k, C.c_void_p(d.data_ptr()), d.numel(), iters, wgs, C.c_void_p(stamps.data_ptr()), stream))
 
-        for _ in range(3):
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 2 * SETTLE_S:  # (steady clocks: see median_per_call)
             go()
+            torch.cuda.synchronize()
         sec = Timer().run(go, reps) / reps
         ops = wgs * 4 * iters * 16 * (131072 if k == 0 else 65536)
         st = stamps.cpu().numpy().astype(np.float64)
@@ -518,7 +520,12 @@ def gemm_timeline(N=4096, K=4096, M=8192):
     null = C.c_void_p(0)
     t = None
     for _ in range(7):  # single launches differ by a few percent with the clock the chip happens to be at: the fastest
-        for i in range(3):
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 2 * SETTLE_S:  # the stamped launch follows a steady run (see median_per_call)
+            for i in range(50):
+                wl["step"](i)
+            torch.cuda.synchronize()
+        for i in range(20):
             wl["step"](i)
         L.check(L.lib().nq_diag_gemm8_timeline(layers[0]._h, C.c_void_p(a.data_ptr()), L.DT_FP8_E4M3,
                                                 C.c_void_p(sa.data_ptr()), C.c_void_p(y.data_ptr()), L.DT_BF16, M,
