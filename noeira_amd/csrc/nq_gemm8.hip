@@ -38,6 +38,11 @@
 // clock, so what is left to gain is energy per stage (bytes moved, instructions
 // issued), not issue slots.  MFMAs alone, on random data, are held to 3.7 - 3.9
 // PFLOP/s by the same limit; this loop delivers 2.4 of them.
+// (All of the above was timed within milliseconds of an idle spell.  The board's power
+// management needs 30 - 40 ms of load to settle, and then leaves more clock: MFMAs alone
+// on random data 4.28 PFLOP/s at 2.08 GHz, a stage of this loop 1.28 us, the call 101 -
+// 110 us, 2.5 - 2.7 PFLOP/s.  The proportions hold: the loop is at 78 % of what the
+// matrix cores alone sustain on such data.)
 //
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= (row >> 1) & 7.  Rows r and r + 1 then sit 128 B apart in
