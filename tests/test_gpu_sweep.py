@@ -223,15 +223,16 @@ def test_single_row_fp32_x_through_lds(fmt):
 
 
 def test_random_large_layers():
-    """Layers of 8 M to 100 M weights with ragged OUT, at every row count from 1 to 300: the kernels over the
+    """Layers of 4 M to 100 M weights with ragged OUT, at row counts from 1 to 512 (every kernel's range of rows and
+    the counts either side of each hand-over): the kernels over the
     tile-ordered copy and the row-ordered ones (tile copy and preference drawn per case), bias + ReLU, fp32 or bf16
     out, against the fp64 product of the dequantised weights; a repeated call returns the same bits."""
     rng = np.random.default_rng(2026)
-    for case in range(60):
+    for case in range(90):
         fmt = ["q4_0", "w4g", "w8"][case % 3]
-        K = int(rng.choice([2048, 2176, 2560, 3072, 4096, 4224, 5120, 6144, 8192]))
-        N = int(rng.integers(4000, 12500))
-        M = int(rng.choice([1, 2, 3, 5, 6, 8, 11, 16, 17, 24, 33, 48, 64, 95, 96, 100, 135, 200, 256, 300]))
+        K = int(rng.choice([1536, 2048, 2176, 2560, 3072, 4096, 4224, 5120, 6144, 8192]))
+        N = int(rng.integers(2100, 12500))
+        M = int(rng.choice([1, 2, 3, 5, 6, 8, 11, 16, 17, 24, 33, 48, 64, 95, 96, 100, 135, 200, 256, 257, 300, 384, 500, 511, 512]))
         prefer, tc = bool(rng.integers(0, 2)), bool(rng.integers(0, 4))
         xdt = torch.bfloat16 if rng.integers(0, 3) else torch.float32
         odt = torch.float32 if rng.integers(0, 2) else torch.bfloat16
