@@ -441,6 +441,8 @@ bool places_parts(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_I8) return false;
     if (gemv_fp8_applicable(a) || gemm8_applicable(a)) return false;
     if (gemm_tile_mt_splits_parts(a)) return false;  // wide and narrow parts: each on the kernel of its own layer
+    // (the same between the medium-M and the many-rows kernel, where neither tile kernel takes the call)
+    if (!gemv_tile_rows_applicable(a) && !gemv_tile8_rows_applicable(a) && !gemm_tile_mt_applicable(a) && gemm_a16_splits_parts(a)) return false;
     return gemv_tile_rows_applicable(a) || gemv_tile8_rows_applicable(a) || gemm_tile_mt_applicable(a) || gemm_a16_applicable(a) || gemv_tile_applicable(a) || gemv_split8_applicable(a) || gemv_row4_applicable(a) || gemv_row8_applicable(a) || gemv_m1_applicable(a);
 }
 

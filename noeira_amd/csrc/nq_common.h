@@ -152,6 +152,10 @@ bool gemm_a16_applicable(const ForwardArgs& a);
 int32_t launch_gemm_a16(const ForwardArgs& a);
 // the medium-M kernel's tile shape for a call (M >= 2, below the many-rows kernel's range) and its estimated time
 float gemm_a16_estimate_us(int32_t format, bool xf32, int M, int N, int K, int* mw_out, int* nw_out);
+// ... the lower of that and the many-rows kernel's estimate (from 256 rows on)
+float gemm_a16_best_estimate_us(int32_t format, bool xf32, int M, int N, int K);
+// a row-fused layer of 256 .. 511 rows whose parts differ in which of the two kernels they take: part by part
+bool gemm_a16_splits_parts(const ForwardArgs& a);
 
 // nq_gemv.hip: dequant-GEMV for small M (also the any-M fallback)
 int32_t launch_gemv(const ForwardArgs& a);

@@ -1045,6 +1045,60 @@ float gemm_a16_estimate_us(int32_t format, bool xf32, int M, int N, int K, int* 
     return least;
 }
 
+bool gemm_a16_applicable(const ForwardArgs& a);
+
+// What the many-rows kernel (a weight unpacked once per 64 or 128 rows) will take, in microseconds, or 0 where it
+// does not apply: below 256 rows, or with fewer than 64 workgroups of 64 rows.  Measured against the medium-M kernel
+// over K = 512 .. 4096, N = 1024 .. 11008 and M = 256 .. 1024 for each format and activation type (960 pairs of calls):
+// t = F + rounds * (c0 + c1 * k-steps), rounds of 256 workgroups, twice the cost per round with 128 rows per
+// workgroup, within 5 - 9 % on average.  Taking this kernel where its estimate is below the medium-M kernel's is
+// within 1 - 3 % of always taking the faster of the two; the thresholds before (512 rows and 192 such workgroups, 256
+// with fp32 activations) were 6 - 13 % off over those calls.  mt_out: 32-row tiles per workgroup (2 or 4).
+static float big_estimate_us(int32_t format, bool xf32, int M, int N, int K, int* mt_out) {
+    static const float consts[6][3] = {
+        {5.64f, 0.684f, 0.3934f}, {12.26f, -2.602f, 1.0247f},   // 8-bit codes: bf16, fp32 activations
+        {6.49f, -0.439f, 1.1383f}, {14.01f, -3.669f, 2.6569f},  // Q4_0
+        {5.46f, 0.237f, 0.9032f}, {10.55f, -1.821f, 2.1478f},   // 4-bit codes in groups with zero points
+    };
+    const bool four_bit = format != NQ_FMT_W8_CHANNEL && format != NQ_FMT_FP8_E4M3;
+    const int64_t wgs64 = (int64_t)((N + 127) / 128) * ((M + 63) / 64);
+    const int mt = (!xf32 && K >= 4096 && wgs64 >= 384) ? 4 : 2;  // 128 rows per workgroup over a long K
+    if (mt_out) *mt_out = mt;
+    if (M < 256 || wgs64 < 64) return 0.0f;
+    const float* c = consts[(!four_bit ? 0 : format == NQ_FMT_Q4_0 ? 2 : 4) + (xf32 ? 1 : 0)];
+    const int64_t wgs = (int64_t)((N + 127) / 128) * ((M + 32 * mt - 1) / (32 * mt));
+    const int nsteps = (K + (four_bit ? 128 : 64) - 1) / (four_bit ? 128 : 64);
+    return c[0] + (float)((wgs + 255) / 256) * (float)(mt / 2) * (c[1] + c[2] * (float)nsteps);
+}
+
+// the many-rows kernel for a layer (or a part of a row-fused one) `width` columns wide
+static bool big_wins(const ForwardArgs& a, int width) {
+    const bool xf32 = a.x_dtype == NQ_DT_F32;
+    const float big = big_estimate_us(a.L->format, xf32, a.M, width, a.L->in, nullptr);
+    return big > 0.0f && big < gemm_a16_estimate_us(a.L->format, xf32, a.M, width, a.L->in, nullptr, nullptr);
+}
+
+static int big_parts(const ForwardArgs& a) {
+    int n = 0;
+    for (int i = 0, prev = 0; i < a.seg.nseg; prev = a.seg.end[i], i++) n += big_wins(a, a.seg.end[i] - prev);
+    return n;
+}
+
+// Below 512 rows a part of a row-fused layer gets the kernel - and so the bits - of its own layer's forward: all
+// parts on the many-rows kernel, none, or (this) part by part.  From 512 rows on the whole layer's width decides.
+bool gemm_a16_splits_parts(const ForwardArgs& a) {
+    if (a.seg.nseg < 2 || a.M < 256 || a.M >= 512 || !gemm_a16_applicable(a)) return false;
+    const int n = big_parts(a);
+    return n > 0 && n < a.seg.nseg;
+}
+
+// the lower of the two kernels' estimates (what the M-tile kernel's estimate is held against)
+float gemm_a16_best_estimate_us(int32_t format, bool xf32, int M, int N, int K) {
+    const float medium = gemm_a16_estimate_us(format, xf32, M, N, K, nullptr, nullptr);
+    const float big = big_estimate_us(format, xf32, M, N, K, nullptr);
+    return big > 0.0f && big < medium ? big : medium;
+}
+
 bool gemm_a16_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     if (a.x_dtype != NQ_DT_F32 && a.x_dtype != NQ_DT_BF16) return false;
@@ -1070,14 +1124,15 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     p.s_pairs = L->format != NQ_FMT_Q4_0 ? 0 : (L->in / 32) % 4 == 0 ? 2 : (L->in / 32) % 2 == 0 ? 1 : 0;
     p.nch = L->in / (four_bit ? 32 : 16);
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
-    // Many rows: the kernel that unpacks a weight once per 64 or 128 rows, wherever its workgroups fill
-    // the chip (measured over 960 .. 4096-wide layers and M = 512 .. 4096: it wins from about 192
-    // workgroups of 64 rows on, 256 with fp32 activations, and is 2 x faster at M = 4096).  Its sums
-    // are formed in another order than the medium-M kernel's, and the choice follows N: from 512
-    // rows on, a row's bits in a row-fused layer may differ from those in its own layer.
-    const int64_t wgs64 = (int64_t)((L->out + 127) / 128) * ((a.M + 63) / 64);
-    if (a.M >= 512 && wgs64 >= (xf32 ? 256 : 192)) {
-        const int big = (!xf32 && L->in >= 4096 && wgs64 >= 384) ? 4 : 2;  // 128 rows per workgroup over a long K
+    // Many rows: the kernel that unpacks a weight once per 64 or 128 rows, from 256 rows on wherever its estimated
+    // time is the lower one.  Its sums are formed in another order than the medium-M kernel's.  Below 512 rows a
+    // row-fused layer takes it only when every part would on its own (a mix runs part by part:
+    // gemm_a16_splits_parts); from 512 rows on the whole layer's width decides, and a row's bits in a row-fused
+    // layer may differ from those in its own layer.
+    const bool use_big = (a.M >= 512 || a.seg.nseg < 2) ? big_wins(a, L->out) : big_parts(a) == a.seg.nseg;
+    if (use_big) {
+        int big = 2;
+        big_estimate_us(L->format, xf32, a.M, L->out, L->in, &big);
         const int bnw = xf32 ? 4 : 2;                                      // four or eight wavefronts
         switch (L->format) {
             case NQ_FMT_Q4_0:

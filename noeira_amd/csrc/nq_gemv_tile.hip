@@ -1813,7 +1813,7 @@ static bool mt_part_ok(const ForwardArgs& a, int width) {
     if (mine == 0.0f) return false;
     // (estimates within a tenth of each other go to this kernel: it is the one that can carry an adapter in the same
     // launch, and over the measured calls that margin costs 0.1 - 0.2 % more)
-    return mine < 1.10f * gemm_a16_estimate_us(a.L->format, a.x_dtype == NQ_DT_F32, a.M, width, a.L->in, nullptr, nullptr);
+    return mine < 1.10f * gemm_a16_best_estimate_us(a.L->format, a.x_dtype == NQ_DT_F32, a.M, width, a.L->in);
 }
 
 // A row-fused layer runs on this kernel in one launch when all its parts pass, on the other kernel when none does,

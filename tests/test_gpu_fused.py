@@ -149,3 +149,37 @@ def test_fuse_rows_errors():
         f.forward(x, outs=[torch.empty((2, 24), dtype=torch.float32, device="cuda")])
     with pytest.raises(L.NQError, match="between 1 and 4"):
         FusedRows([a, a, a, a, a])
+
+
+@pytest.mark.parametrize("M", [256, 300, 400, 511])
+def test_parts_keep_their_bits_between_the_medium_and_the_many_rows_kernel(M):
+    """From 256 rows on the many-rows kernel takes a layer where its estimated time is the lower one: wide layers
+    first.  Below 512 rows a row-fused layer follows its parts: a wide and a narrow part run part by part, two wide
+    ones in one launch, and every part returns the bits of its own layer's forward (and those agree with the fp64
+    product of the dequantised weights)."""
+    rng = np.random.default_rng(M)
+    K = 1024
+    x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(torch.bfloat16).cuda()
+
+    def w8(n):
+        lin = W8Linear(K, n)
+        lin.set_weight(rng.integers(-127, 128, (n, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, n).astype(np.float32))
+        return lin
+
+    def q4(n):
+        lin = QLinear(K, n, tile_copy=False)
+        blocks = rng.integers(0, 256, (n, K // 32, 18), dtype=np.uint8)
+        sc = rng.uniform(1e-3, 1e-2, (n, K // 32)).astype(np.float16).view(np.uint16)
+        blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+        lin.set_blocks(blocks.reshape(-1))
+        return lin
+
+    for make in (w8, q4):
+        for widths in ((8192, 512), (8192, 6144), (512, 640)):
+            parts = [make(n) for n in widths]
+            outs = FusedRows(parts).forward(x)
+            for part, y in zip(parts, outs):
+                own = part.forward(x)
+                assert torch.equal(y, own), (make.__name__, widths, part.OUT)
+                exact = x.double() @ part.dequantized_dev().double().T
+                assert float((own.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
