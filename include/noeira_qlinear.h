@@ -198,7 +198,8 @@ int32_t nq_fused_parts(nq_handle h);
  * kernel, hence the order of a row's sum, may follow the total row count).
  * n_ys must equal nq_fused_parts(h).  bias, if any, is [sum OUT].  One launch
  * where the kernel for the shape can place rows by part (bf16/fp32
- * activations at any M), otherwise one launch per part. */
+ * activations at any M; at 17 .. 511 rows only where all parts take the same
+ * kernel on their own), otherwise one launch per part. */
 int32_t nq_forward_fused(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale,
                          void* const* ys, int32_t n_ys, int32_t y_dtype, int32_t M, const void* bias,
                          int32_t bias_dtype, int32_t epilogue, void* stream);
