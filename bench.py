@@ -24,7 +24,9 @@ batched-env actor at M = 4096, in TOPS); `roofline_mfma` is the large-M fp8 GEMM
 (`mfma_only`: back-to-back MFMAs on register operands, constant and random data).
 
 `--only a16_shapes --a16-class C` re-derives the constants by which the library picks the tile shape of its
-kernel for tens to hundreds of activation rows (a grid of calls timed under each shape, nq_diag_a16_shape).
+kernel for tens to hundreds of activation rows (a grid of calls timed under each shape, nq_diag_a16_shape);
+`--only mid_dispatch --a16-class C` times the kernels that compete for those calls side by side and the library's
+choice between them.
 
 `cpu_baseline` times the CPU oracle's restatement of the reference's CPU
 forward (a fresh dequantize to an fp32 scratch, then the serial triple loop;
@@ -908,12 +910,62 @@ def a16_shapes(cls="w4g"):
 
 
 
+def mid_dispatch(cls="w4g"):
+    """Which kernel takes a call of tens to hundreds of rows over a 4-bit layer, checked from outside: a grid of
+    calls timed on a layer made with NQ_FLAG_PREFER_TILE (the M-tile kernel wherever the shape allows it), on one
+    made without the tile-ordered copy (the 16-row tile kernel, or the many-rows kernel from 256 rows) and on a
+    plain one (the library's choice between them).  Reports the library's total against always taking the faster
+    of the two, and the calls where it is more than a tenth slower."""
+    import numpy as np
+    import torch
+
+    from noeira_amd import formats as F
+    from noeira_amd.qlinear import QLinear, W4GroupLinear
+
+    xf32, kind = cls.endswith("f"), cls.rstrip("f")
+    rng = np.random.default_rng(1)
+
+    def layer(K, N, **kw):
+        if kind == "q4":
+            lin = QLinear(K, N, **kw)
+            blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+            sc = rng.uniform(1e-3, 1e-2, (N, K // 32)).astype(np.float16).view(np.uint16)
+            blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+            lin.set_blocks(blocks.reshape(-1))
+            return lin
+        G = -(-K // 128)
+        codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
+        lin = W4GroupLinear(K, N, 128, **kw)
+        lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+        return lin
+
+    rows, slow = [], []
+    for K in ((960, 2048) if xf32 else (960, 2048, 4096)):
+        for N in (2560, 5120, 11008):
+            ls = [layer(K, N, prefer_tile=True), layer(K, N, tile_copy=False), layer(K, N)]
+            for M in (33, 100, 135, 256, 384, 511):
+                x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda()
+                x = x if xf32 else x.to(torch.bfloat16)
+                y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+                ts = [median_per_call((lambda l: (lambda i: l.forward(x, out=y)))(l), 20) * 1e6 for l in ls]
+                rows.append(ts)
+                if ts[2] > 1.1 * min(ts[:2]):
+                    slow.append({"K": K, "N": N, "M": M, "m_tile_us": round(ts[0], 2), "other_us": round(ts[1], 2),
+                                 "library_us": round(ts[2], 2)})
+            del ls
+    lib, best = sum(t[2] for t in rows), sum(min(t[:2]) for t in rows)
+    return {"only": "mid_dispatch", "class": cls, "calls": len(rows), "library_vs_faster_kernel": round(lib / best, 4),
+            "always_m_tile_vs_faster": round(sum(t[0] for t in rows) / best, 4),
+            "never_m_tile_vs_faster": round(sum(t[1] for t in rows) / best, 4), "more_than_a_tenth_slower": slow}
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline", "a16_shapes"],
+    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline", "a16_shapes", "mid_dispatch"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
                          "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
@@ -945,6 +997,11 @@ def main():
         TILE_COPY = False
     if a.only == "a16_shapes":
         print(json.dumps(a16_shapes(a.a16_class)))
+        return
+    if a.only == "mid_dispatch":
+        if a.a16_class.startswith("w8"):
+            sys.exit("bench.py: --only mid_dispatch is about the 4-bit formats (--a16-class q4, q4f, w4g or w4gf)")
+        print(json.dumps(mid_dispatch(a.a16_class)))
         return
     if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
