@@ -177,9 +177,16 @@ def test_parts_keep_their_bits_between_the_medium_and_the_many_rows_kernel(M):
     for make in (w8, q4):
         for widths in ((8192, 512), (8192, 6144), (512, 640)):
             parts = [make(n) for n in widths]
-            outs = FusedRows(parts).forward(x)
+            fused = FusedRows(parts)
+            outs = fused.forward(x)
             for part, y in zip(parts, outs):
                 own = part.forward(x)
                 assert torch.equal(y, own), (make.__name__, widths, part.OUT)
                 exact = x.double() @ part.dequantized_dev().double().T
                 assert float((own.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
+            if make is w8:  # bias and ReLU travel with each part when the call runs part by part
+                bias = torch.from_numpy(rng.standard_normal(sum(widths)).astype(np.float32)).cuda()
+                r0 = 0
+                for part, y in zip(parts, fused.forward(x, bias=bias, epilogue="relu")):
+                    assert torch.equal(y, part.forward(x, bias=bias[r0:r0 + part.OUT].contiguous(), epilogue="relu"))
+                    r0 += part.OUT
