@@ -470,8 +470,10 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
         }
     };
 
-    auto emit = [&](auto kind) {
+    auto emit = [&](auto kind, auto plain) {
         constexpr int KIND = decltype(kind)::value;  // 0: fp32, 1: bf16, 2: raw int32
+        // PLAIN: one scale for the whole tensor and no bias (fp8 x fp8 without a bias): no channel operands at all
+        constexpr bool PLAIN = decltype(plain)::value;
         constexpr int ES = (KIND == 1) ? 2 : 4;      // bytes per output element
         constexpr int IP = (KIND == 1) ? 2 : 1;      // token tiles (of 32) staged per pass
         constexpr int ROWB = WN * ES + 16;           // staged row: the wavefront's channels + pad (bank spread)
@@ -495,7 +497,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
                 float cs[4][4], cb[4][4];
-                if constexpr (KIND != 2) {
+                if constexpr (KIND != 2 && !PLAIN) {
 #pragma unroll
                     for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8, zero);
                 }
@@ -518,7 +520,9 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
                         for (int g = 0; g < 4; g++)
 #pragma unroll
                             for (int r = 0; r < 4; r++) {
-                                if constexpr (FP8)
+                                if constexpr (PLAIN)
+                                    z[ii][g][r] = acc[ip + ii][j][4 * g + r] * fp8_scale + 0.0f;  // (+ 0.0f: the bits of the general path, -0.0 included)
+                                else if constexpr (FP8)
                                     z[ii][g][r] = acc[ip + ii][j][4 * g + r] * fp8_scale + cb[g][r];
                                 else
                                     z[ii][g][r] = (float)acc[ip + ii][j][4 * g + r] * (rscale[ii] * cs[g][r]) + cb[g][r];
@@ -587,7 +591,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     };
-    emit(std::integral_constant<int, KIND_>{});
+    if constexpr (FP8 && KIND_ != 2) {
+        if (!p.bias) emit(std::integral_constant<int, KIND_>{}, std::true_type{});
+        else emit(std::integral_constant<int, KIND_>{}, std::false_type{});
+    } else {
+        emit(std::integral_constant<int, KIND_>{}, std::false_type{});
+    }
     if (p.stamps) {  // (uniform) entry, first stage landed, loop done, stores acknowledged
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (tid == 0) {
