@@ -472,8 +472,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 
     auto emit = [&](auto kind, auto plain) {
         constexpr int KIND = decltype(kind)::value;  // 0: fp32, 1: bf16, 2: raw int32
-        // PLAIN: one scale for the whole tensor and no bias (fp8 x fp8 without a bias): no channel operands at all
-        constexpr bool PLAIN = decltype(plain)::value;
+        // MODE (uniform over the launch, so chosen once and not per channel tile: a branch around a load makes the
+        // wavefront wait for that load where the branches meet).  0: one scale for the whole tensor and no bias (fp8 x
+        // fp8): no channel operands at all; 1 .. 3: the lane's four channels adjacent and aligned, one load per
+        // operand - no bias, fp32 bias, bf16 bias; 4: channel by channel
+        constexpr int MODE = decltype(plain)::value;
+        constexpr bool PLAIN = MODE == 0;
         constexpr int ES = (KIND == 1) ? 2 : 4;      // bytes per output element
         constexpr int IP = (KIND == 1) ? 2 : 1;      // token tiles (of 32) staged per pass
         constexpr int ROWB = WN * ES + 16;           // staged row: the wavefront's channels + pad (bank spread)
@@ -494,10 +498,47 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
                 rscale[ii] = 1.0f;
                 if constexpr (!FP8 && KIND != 2) rscale[ii] = p.row_scale[min(wm0 + 32 * (ip + ii) + lm, p.M - 1)];
             }
+            // modes 1 .. 3: the operands of channel tile j + 1 are requested before tile j is worked on
+            auto fetch = [&](int j, float (&cs)[4][4], float (&cb)[4][4]) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int nb = min(wn0 + 32 * j + 8 * g + 4 * lh, p.N - 4) + zero;
+                    if constexpr (!FP8) {
+                        const float4 sv = *reinterpret_cast<const float4*>(p.col_scale + nb);
+                        cs[g][0] = sv.x, cs[g][1] = sv.y, cs[g][2] = sv.z, cs[g][3] = sv.w;
+                    } else {
+                        cs[g][0] = cs[g][1] = cs[g][2] = cs[g][3] = 1.0f;
+                    }
+                    if constexpr (MODE == 2) {
+                        const float4 bv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + nb);
+                        cb[g][0] = bv.x, cb[g][1] = bv.y, cb[g][2] = bv.z, cb[g][3] = bv.w;
+                    } else if constexpr (MODE == 3) {
+                        const uint2 bv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.bias) + nb);
+                        cb[g][0] = __uint_as_float(bv.x << 16), cb[g][1] = __uint_as_float(bv.x & 0xFFFF0000u);
+                        cb[g][2] = __uint_as_float(bv.y << 16), cb[g][3] = __uint_as_float(bv.y & 0xFFFF0000u);
+                    } else {
+                        cb[g][0] = cb[g][1] = cb[g][2] = cb[g][3] = 0.0f;
+                    }
+                }
+            };
+            // (not for int8 with fp32 output: its four passes of one token tile leave no registers for a second set)
+            constexpr bool VEC = KIND != 2 && MODE >= 1 && MODE <= 3;
+            constexpr bool AHEAD = VEC && !(KIND == 0 && !FP8);
+            float ncs[4][4], ncb[4][4];
+            if constexpr (AHEAD) fetch(0, ncs, ncb);
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
                 float cs[4][4], cb[4][4];
-                if constexpr (KIND != 2 && !PLAIN) {
+                if constexpr (AHEAD) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) cs[g][r] = ncs[g][r], cb[g][r] = ncb[g][r];
+                    if (j + 1 < TJ) fetch(j + 1, ncs, ncb);
+                } else if constexpr (VEC) {
+                    fetch(j, cs, cb);
+                }
+                if constexpr (KIND != 2 && MODE == 4) {
 #pragma unroll
                     for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8, zero);
                 }
@@ -591,11 +632,15 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     };
-    if constexpr (FP8 && KIND_ != 2) {
-        if (!p.bias) emit(std::integral_constant<int, KIND_>{}, std::true_type{});
-        else emit(std::integral_constant<int, KIND_>{}, std::false_type{});
+    using kind_t = std::integral_constant<int, KIND_>;
+    if constexpr (KIND_ == 2) {
+        emit(kind_t{}, std::integral_constant<int, 4>{});
     } else {
-        emit(std::integral_constant<int, KIND_>{}, std::false_type{});
+        if (FP8 && !p.bias) emit(kind_t{}, std::integral_constant<int, 0>{});
+        else if (!p.chan_vec) emit(kind_t{}, std::integral_constant<int, 4>{});
+        else if (!p.bias) emit(kind_t{}, std::integral_constant<int, 1>{});
+        else if (p.bias_dtype == NQ_DT_F32) emit(kind_t{}, std::integral_constant<int, 2>{});
+        else emit(kind_t{}, std::integral_constant<int, 3>{});
     }
     if (p.stamps) {  // (uniform) entry, first stage landed, loop done, stores acknowledged
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
