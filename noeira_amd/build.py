@@ -41,8 +41,11 @@ EXTRA_FLAGS = {"nq_gptq.hip": ["-ffp-contract=off"]}
 # `s_waitcnt`: the compiler takes the registers those loads write for valid from the load on, so a spill (or a copy made
 # to free a register) between request and wait would store what has not arrived yet.  Their register budgets are
 # chosen so that none is needed; the build refuses an object in which one of them uses scratch memory.
+# (the large-tile GEMM is held to the same rule for its speed: 256 accumulators per lane leave its epilogue a tight
+# budget, and a variant that spills there has cost 60 % of the call before)
 NO_SPILL = {"nq_gemv_tile.hip": ("gemv_tile4i_kernel", "gemv_tile4_rows_kernel", "gemv_tile8_rows_kernel"),
-            "nq_gemv_fp8.hip": ("tile8_kernel",)}
+            "nq_gemv_fp8.hip": ("tile8_kernel",),
+            "nq_gemm8.hip": ("gemm8_kernel",)}
 
 
 def _spilling_kernels(remarks: str, names) -> list:
