@@ -41,11 +41,11 @@ EXTRA_FLAGS = {"nq_gptq.hip": ["-ffp-contract=off"]}
 # `s_waitcnt`: the compiler takes the registers those loads write for valid from the load on, so a spill (or a copy made
 # to free a register) between request and wait would store what has not arrived yet.  Their register budgets are
 # chosen so that none is needed; the build refuses an object in which one of them uses scratch memory.
-# (the large-tile GEMM is held to the same rule for its speed: 256 accumulators per lane leave its epilogue a tight
-# budget, and a variant that spills there has cost 60 % of the call before)
 NO_SPILL = {"nq_gemv_tile.hip": ("gemv_tile4i_kernel", "gemv_tile4_rows_kernel", "gemv_tile8_rows_kernel"),
-            "nq_gemv_fp8.hip": ("tile8_kernel",),
-            "nq_gemm8.hip": ("gemm8_kernel",)}
+            "nq_gemv_fp8.hip": ("tile8_kernel",)}
+# The large-tile GEMM is held to the same rule for its speed: 256 accumulators per lane leave its epilogue a tight
+# budget, and a variant that spills there has cost 60 % of the call before.
+NO_SPILL_FOR_SPEED = {"nq_gemm8.hip": ("gemm8_kernel",)}
 
 
 def _spilling_kernels(remarks: str, names) -> list:
@@ -110,7 +110,7 @@ def _compile(src: str, force: bool) -> str:
     newest = max(os.path.getmtime(p) for p in [path] + _deps())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj
-    guarded = NO_SPILL.get(src)
+    guarded = NO_SPILL.get(src) or NO_SPILL_FOR_SPEED.get(src)
     cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + (["-Rpass-analysis=kernel-resource-usage"] if guarded else []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -121,7 +121,8 @@ def _compile(src: str, force: bool) -> str:
         err = "\n".join(l for l in err.splitlines() if "kernel-resource-usage" not in l and not re.match(r"^\s+(\d+ \||\|)", l))
         if spilled:
             os.remove(obj)
-            raise RuntimeError(f"{src}: kernels that keep loads under way in registers must not spill: {spilled}")
+            raise RuntimeError(f"{src}: kernels that keep loads under way in registers, or whose register budget is tuned, "
+                               f"must not spill: {spilled}")
     if src in PREFETCH_MARKED:
         cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["--cuda-device-only", "-S", path, "-o", obj + ".s"]
         r = subprocess.run(cmd, capture_output=True, text=True)
