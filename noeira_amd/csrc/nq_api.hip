@@ -973,7 +973,8 @@ int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq
 
 int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_bytes, int32_t iters, int32_t workgroups,
                           int64_t* stamps, void* stream) {
-    if (kind != 0 && kind != 1) return fail(NQ_ERR_INVALID, "nq_diag_mfma_rate: kind must be 0 (fp8) or 1 (int8)");
+    if (kind < 0 || kind > 3)
+        return fail(NQ_ERR_INVALID, "nq_diag_mfma_rate: kind must be 0 / 1 (fp8 / int8, 32 x 32) or 2 / 3 (fp8 / int8, 16 x 16)");
     if (!operands || operand_bytes < 4096 || ((uintptr_t)operands & 3))
         return fail(NQ_ERR_INVALID, "nq_diag_mfma_rate: at least 4096 bytes of 4-byte aligned operands are needed");
     if (iters <= 0 || workgroups <= 0 || !stamps)
@@ -997,9 +998,16 @@ int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, cons
         return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: 8-bit activations, M >= 64 and a stamp buffer are needed");
     const int64_t tiles = (int64_t)((M + 255) / 256) * ((h->out + 255) / 256);
     if (tiles > max_tiles) return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: the stamp buffer is smaller than the tile count");
-    gemm8_set_stamps(reinterpret_cast<unsigned long long*>(stamps));
-    rc = nq_forward(h, x, x_dtype, x_scale, y, y_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_NONE, stream);
-    gemm8_set_stamps(nullptr);
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    if (!x || !y || !x_scale || (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16))
+        return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: x, its scale(s) and an fp32 or bf16 y are needed");
+    SegTable seg{};
+    seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
+    ForwardArgs a{h, x, x_dtype, x_scale, y, y_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_NONE, (hipStream_t)stream, seg};
+    if (!gemm8_applicable(a))
+        return fail(NQ_ERR_UNSUPPORTED, "nq_diag_gemm8_timeline: the large-tile GEMM does not take this layer (format, IN % 128)");
+    a.diag_stamps = reinterpret_cast<unsigned long long*>(stamps);
+    rc = launch_gemm8(a);
     if (rc) return rc;
     NQ_HIP(hipStreamSynchronize((hipStream_t)stream));
     return NQ_OK;

@@ -26,9 +26,6 @@ int32_t fail_hip(hipError_t e, const char* what);
         if (_e != hipSuccess) return nq::fail_hip(_e, #expr); \
     } while (0)
 
-// nq_gemm8.hip: per-workgroup clock readings of the next large-tile GEMM launches (a diagnostic; null = off)
-void gemm8_set_stamps(unsigned long long* buf);
-
 // nq_diag.hip: the matrix cores' own rate (a diagnostic)
 int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s);
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
@@ -134,6 +131,8 @@ struct ForwardArgs {
     const float* lora_b = nullptr;
     int32_t lora_r = 0;
     float lora_s = 0.0f;
+    // nq_diag_gemm8_timeline: where the large-tile GEMM writes its per-tile clock readings (null: none)
+    unsigned long long* diag_stamps = nullptr;
 };
 
 // nq_q4_0.hip

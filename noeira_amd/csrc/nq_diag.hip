@@ -57,6 +57,47 @@ void mfma_rate_kernel(const int* __restrict__ seed, int seed_words, int iters, i
     if (threadIdx.x == 0) stamps[2 * blockIdx.x] = c1 - c0, stamps[2 * blockIdx.x + 1] = w1 - w0;
 }
 
+// The same yardstick for the 16 x 16 shapes: KIND 2: v_mfma_f32_16x16x128_f8f6f4, 3: v_mfma_i32_16x16x64_i8.  Eight A and
+// eight B fragments per wavefront (a 128 x 128 register tile as 8 x 8 results of 16 x 16): 64 MFMAs per iteration, twice
+// the operations of the 32 x 32 kernels' 16.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+template <int KIND>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void mfma16_rate_kernel(const int* __restrict__ seed, int seed_words, int iters, int64_t* __restrict__ stamps, float* sink) {
+    i32x8 a[8], b[8];
+#pragma unroll
+    for (int o = 0; o < 8; o++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            a[o][i] = seed[(threadIdx.x * 8 + i + 2048 * o) % seed_words];
+            b[o][i] = seed[(threadIdx.x * 8 + i + 2048 * o + 1024) % seed_words];
+        }
+    typedef typename std::conditional<KIND == 2, f32x4, i32x4>::type acc_t;
+    acc_t acc[64];
+#pragma unroll
+    for (int j = 0; j < 64; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[j][r] = 0;
+    const int64_t c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            if constexpr (KIND == 2)
+                acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b[j % 8], a[j / 8], acc[j], 0, 0, 0, 0, 0, 0);
+            else
+                acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4){b[j % 8][0], b[j % 8][1], b[j % 8][2], b[j % 8][3]},
+                                                               (i32x4){a[j / 8][0], a[j / 8][1], a[j / 8][2], a[j / 8][3]},
+                                                               acc[j], 0, 0, 0);
+        }
+    }
+    const int64_t c1 = clock64(), w1 = wall_clock64();
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 64; j++) s += (float)acc[j][0];
+    if (s == 12345.678f) sink[0] = s;  // (keeps the accumulators alive)
+    if (threadIdx.x == 0) stamps[2 * blockIdx.x] = c1 - c0, stamps[2 * blockIdx.x + 1] = w1 - w0;
+}
+
 // A second yardstick: a kernel that only READS `kib` KiB (one 1 KiB load instruction per wavefront and KiB, four
 // in flight per wavefront, eight wavefronts per workgroup) and computes nothing.  What it takes for the bytes
 // of a GEMV's weight is the floor of that GEMV on this GPU: launch + the stream.
@@ -87,7 +128,11 @@ int32_t launch_stream_read(const void* src, int64_t kib, hipStream_t s) {
 
 int32_t launch_mfma_rate(int kind, const int* seed, int seed_words, int iters, int blocks, int64_t* stamps, float* sink,
                          hipStream_t s) {
-    if (kind == 0)
+    if (kind == 2)
+        hipLaunchKernelGGL(mfma16_rate_kernel<2>, dim3(blocks), dim3(256), 0, s, seed, seed_words, iters, stamps, sink);
+    else if (kind == 3)
+        hipLaunchKernelGGL(mfma16_rate_kernel<3>, dim3(blocks), dim3(256), 0, s, seed, seed_words, iters, stamps, sink);
+    else if (kind == 0)
         hipLaunchKernelGGL(mfma_rate_kernel<0>, dim3(blocks), dim3(256), 0, s, seed, seed_words, iters, stamps, sink);
     else
         hipLaunchKernelGGL(mfma_rate_kernel<1>, dim3(blocks), dim3(256), 0, s, seed, seed_words, iters, stamps, sink);

@@ -61,6 +61,7 @@
 // gets one contiguous run of tiles, and runs walk the tile grid in bands of 8
 // row tiles, so the ~32 tiles resident on an XCD share 8 x-tiles and 4 w-tiles
 // in that XCD's L2 instead of 32 + 32.
+#include <cstdlib>
 #include <type_traits>
 
 #include "nq_common.h"
@@ -71,8 +72,6 @@ namespace {
 
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(16))) int i32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -100,18 +99,89 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float v) {
     return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
 }
 
-// BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with
-// BK = 128 (a 256 x 128, BK = 64 variant with two workgroups per CU measured slower: its stage is
-// too short for a transfer to land in).
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(static_cast<F&&>(f));
+    }
+}
+
+// ---- the issue order of one phase (64 MFMAs of one k-extent: row i = 0..7 of token fragments, column j = 0..7 of
+// channel fragments, MFMA m = 8 i + j), as the waits' model.  Slot m = right after MFMA m.  A phase requests what
+// the NEXT phase multiplies: the token fragment x_i into the registers row i has just finished with (one MFMA
+// later, so that no request follows the last reader directly), the channel fragments into the second set; x_7
+// is read at the start of the phase that uses it.  Nothing is requested in rows 0 and 1: where the next phase lies
+// in the other stage buffer, the stage's barrier stands at the start of row 2, and the requests a barrier-free
+// phase could have made earlier are kept where they are, so that every phase has one order.
+//   event e:   0     1    2    3    4    5    6    7    8    9    10   11   12   13   14   15
+//   brings:    x7'   x0   x1   w0   w1   w2   x2   w3   x3   w4   x4   w5   x5   w6   x6   w7   (x7': this phase's own)
+__host__ __device__ constexpr int ev_slot(int e) {
+    constexpr int s[16] = {0, 16, 17, 18, 19, 20, 24, 27, 32, 35, 40, 43, 48, 51, 56, 59};
+    return s[e];
+}
+__host__ __device__ constexpr int ev_of_x(int i) {  // i <= 6: the event of the previous phase that brought x_i
+    constexpr int e[7] = {1, 2, 6, 8, 10, 12, 14};
+    return e[i];
+}
+__host__ __device__ constexpr int ev_of_w(int j) {
+    constexpr int e[8] = {3, 4, 5, 7, 9, 11, 13, 15};
+    return e[j];
+}
+// the event (or -1) in slot m
+__host__ __device__ constexpr int ev_at(int m) {
+    for (int e = 0; e < 16; e++)
+        if (ev_slot(e) == m) return e;
+    return -1;
+}
+// The wait in front of MFMA m = 8 i + j, as the number of reads (fragments x reads per fragment) that may still be
+// under way, or -1 where what the MFMA needs has landed by an earlier wait of the phase.  Events are numbered
+// 0 .. 15 (the phase before) and 16 .. 31 (this phase); LDS returns in the order of issue, so a wait that leaves
+// `a` events in flight proves every older one landed.  A phase starts knowing nothing (conservative: a stage's
+// barrier waits for everything, but not every phase follows one).  lgkmcnt counts to 15.
+__host__ __device__ constexpr int lds_wait(int m_want, int reads_per_fragment, bool barrier_at_16) {
+    int landed = 0;  // events 0 .. landed - 1 are known to have landed
+    for (int m = 0; m < 64; m++) {
+        const int i = m / 8, j = m % 8;
+        int issued = 16;
+        for (int e = 0; e < 16; e++)
+            if (ev_slot(e) < m) issued++;
+        const int nx = (i == 7) ? 16 : ev_of_x(i), nw = ev_of_w(j);
+        const int need = nx > nw ? nx : nw;
+        int w = -1;
+        if (barrier_at_16 && m == 16) {
+            landed = issued;  // (the barrier's own wait is lgkmcnt(0))
+        } else if (need >= landed) {
+            int a = issued - 1 - need;                       // events younger than the needed one
+            const int cap = 15 / reads_per_fragment;
+            if (a > cap) a = cap;
+            w = a * reads_per_fragment;
+            landed = issued - a;
+        }
+        if (m == m_want) return w;
+    }
+    return -1;
+}
+// a stage's 16 transfers per wavefront leave in pairs, in these slots of the stage's last phase (after the barrier, in
+// slots that hold no request): the first transfer of the pair in slot m, or -1
+__host__ __device__ constexpr int dma_at(int m) {
+    constexpr int s[8] = {21, 22, 25, 26, 29, 30, 33, 34};
+    for (int t = 0; t < 8; t++)
+        if (s[t] == m) return 2 * t;
+    return -1;
+}
+
+// BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with BK = 128.
 // KIND: the output type the epilogue is built for (0 fp32, 1 bf16, 2 raw int32 accumulators); one
 // kernel per kind, because with all three in one function the register allocator spills.
 template <bool FP8, int KIND_, int BN, int BK>
 __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int STAGE_BYTES = (BM + BN) * BK;
     constexpr int SLOTS = BK / 16;     // 16-byte slots per LDS row
-    constexpr int SWZ = SLOTS - 1;     // slot ^= (row >> 1) & SWZ
     constexpr int WN = BN / 2;         // channels per wavefront
-    constexpr int TJ = WN / 32;        // weight fragments (MFMA tiles along N) per wavefront
+    constexpr int TI = 8, TJ = WN / 16;  // fragments of 16 rows: token rows i, channel columns j
+    static_assert(BM == 256 && BN == 256 && BK == 128 && TJ == 8, "the phase model is written for this tile");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const unsigned long long t_entry = wall_clock64();
     const int tid = threadIdx.x;
@@ -134,14 +204,18 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     const int tn = in_band / band_rows;
     const int m0 = tm * BM, n0 = tn * BN;
 
+    // the slot permutation of an LDS row (see the header): rows 16 f + r of any fragment f share it
+    auto swz = [](int row) { return (((row >> 1) & 7) + 6) & 7; };
+
     // ---- global -> LDS, direct (global_load_lds_dwordx4): no register round trip.  One
     // instruction fills 1 KiB of LDS, lane l at byte 16 l, i.e. 1024 / BK rows; wavefront w owns
-    // a quarter of the rows of both tiles.  The slot swizzle is applied on the global side: the
+    // a quarter of the rows of both tiles.  The slot permutation is applied on the global side: the
     // lane that lands in physical slot s of its row fetches logical slot s ^ swz(row).
     typedef __attribute__((address_space(3))) void lptr_t;
     constexpr int DROWS = 1024 / BK;           // rows per instruction
     constexpr int DA = BM / 4 / DROWS;         // instructions per wavefront and stage, x tile
     constexpr int DB = BN / 4 / DROWS;         // ... w tile
+    static_assert(DA + DB == 16, "dma_at() places 16 transfers per wavefront and stage");
     // addresses as a uniform 64-bit tile base (advanced by k0) plus a 32-bit per-lane offset, and
     // the LDS destination as a scalar: two instructions per transfer (set M0, issue)
     const uint8_t* const abase = p.a + (int64_t)m0 * p.K;
@@ -150,13 +224,13 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 #pragma unroll
     for (int t = 0; t < DA; t++) {
         const int row = wave * (BM / 4) + t * DROWS + lane / SLOTS;
-        const int slot = (lane % SLOTS) ^ ((row >> 1) & SWZ);
+        const int slot = (lane % SLOTS) ^ swz(row);
         doff[t] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.K + slot * 16;
     }
 #pragma unroll
     for (int t = 0; t < DB; t++) {
         const int row = wave * (BN / 4) + t * DROWS + lane / SLOTS;
-        const int slot = (lane % SLOTS) ^ ((row >> 1) & SWZ);
+        const int slot = (lane % SLOTS) ^ swz(row);
         doff[DA + t] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.K + slot * 16;
     }
     // transfer t (0 .. DA+DB-1) of a stage: M0 = the LDS address of the 1 KiB the instruction
@@ -185,205 +259,135 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     } while (0)
     const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;  // requested now, used in the epilogue
 
-    typedef typename std::conditional<FP8, f32x16, i32x16>::type acc_t;
-    acc_t acc[4][TJ];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+    typedef typename std::conditional<FP8, f32x4, i32x4>::type acc_t;
+    acc_t acc[TI][TJ];
 
-    // Fragment addressing.  fp8: a 64-byte k-step, this lane supplies bytes [32 h, 32 h + 32) of
-    // its row (h = lane / 32), i.e. slots 4 s + 2 h and 4 s + 2 h + 1.  int8: a 32-byte k-step,
-    // bytes [16 h, 16 h + 16), slot 2 s + h.  Tile bases are multiples of 32 rows, so the swizzle
-    // term depends on the row within the tile only.
-    const int frow = lane & 31;
-    const int fh = lane >> 5;
-    const int fsw = (frow >> 1) & SWZ;
-
-    // ---- main loop, software-pipelined by hand, with the LDS reads and their waits written out.
-    // Measured on this GPU: an MFMA 32x32x64 occupies the matrix core for 64 cycles and other
-    // instructions of the same wavefront issue in its shadow, about seven of them; past that
-    // every extra instruction delays the next MFMA.  With one wavefront per SIMD the loop is
-    // therefore laid out so that no gap between two MFMAs holds more than a handful of
-    // instructions, and nothing in it waits longer than it must:
-    //   - the compiler's own s_waitcnt before a use of loaded data is lgkmcnt(0) here (it waits
-    //     for every read in flight), so the fragment reads are inline-asm ds_read_b128 whose
-    //     latency the compiler does not see, and each MFMA is preceded by s_waitcnt lgkmcnt(N)
-    //     with N from a compile-time model of the issue order (Sched): "all but the N youngest
-    //     reads have landed";
-    //   - per stage of G = 4 SPS groups (a group = the TJ MFMAs of one x fragment): the x
-    //     fragment of group g+2 is requested in group g (four register sets in rotation), the
-    //     w fragments of the next sub-step in the first two groups of the current one (two
-    //     sets), each after the group's first MFMA;
-    //   - the stage's only barrier sits at the start of its last-but-one group, with vmcnt(0)
-    //     (this wavefront's part of the next stage has landed) and lgkmcnt(0) (its reads of
-    //     this stage are done: the buffer may be overwritten); the two groups after it request
-    //     the next stage's first fragments and issue the global -> LDS transfers of the stage
-    //     after next into the buffer just freed, two or three between consecutive MFMAs, so a
-    //     transfer has a whole stage to land;
-    //   - the K loop is unrolled by two stages so that buffer addresses are loop invariants.
-    // __builtin_amdgcn_sched_barrier(0) pins the order against the instruction scheduler.
-    constexpr int KE = FP8 ? 64 : 32;       // bytes of K one MFMA consumes
-    constexpr int SPS = BK / KE;             // sub-steps (one MFMA k-extent each) per stage
-    constexpr int G = 4 * SPS;               // groups per stage
+    // ---- fragments.  fp8 (v_mfma_f32_16x16x128_f8f6f4): the whole 128-byte k-extent of a stage is ONE phase; lane
+    // l supplies bytes [32 c, 32 c + 32) of row l % 16, c = l / 16: slots 2 c and 2 c + 1, two 128-bit reads.  int8
+    // (v_mfma_i32_16x16x64_i8): two phases of 64 bytes per stage, bytes [16 c, 16 c + 16) of the phase's half: slot
+    // 4 u + c, one read.  A fragment is 16 rows x 128 B = 2 KiB of a tile: the immediate offset of the read.
+    constexpr int PH = FP8 ? 1 : 2;          // phases per stage
     constexpr int R = FP8 ? 2 : 1;           // 128-bit reads per fragment
-    constexpr int HB = TJ / 2;               // w fragments requested per group (in the groups that request any)
-    static_assert(SPS % 2 == 0 && TJ == 4, "register-set rotation and transfer slots assume this tile");
-
-    struct Sched {
-        // reads requested in group g (after its first MFMA): the x fragment of group g+2, then w fragments
-        static constexpr int wfrags(int g) {
-            const int sub = g / 4, i = g % 4;
-            return (sub < SPS - 1) ? (i < 2 ? HB : 0) : (i >= 2 ? HB : 0);
-        }
-        static constexpr int reads(int g) { return R * (1 + wfrags(g)); }
-        static constexpr int before(int g) {  // reads requested in groups 0..g-1 of a stage
-            int n = 0;
-            for (int t = 0; t < g; t++) n += reads(t);
-            return n;
-        }
-        static constexpr int total() { return before(G); }
-        // position (reads since the start of the stage, negative = previous stage) of the LAST read of ...
-        static constexpr int pos_a(int g) {  // ... the x fragment group g consumes
-            return g >= 2 ? before(g - 2) + R - 1 : before(G + g - 2) + R - 1 - total();
-        }
-        static constexpr int pos_b(int sub, int j) {  // ... w fragment j of sub-step sub
-            const int g = sub >= 1 ? (sub - 1) * 4 + j / HB : (SPS - 1) * 4 + 2 + j / HB;
-            const int pos = before(g) + R + (j % HB) * R + R - 1;
-            return sub >= 1 ? pos : pos - total();
-        }
-        // reads that may still be in flight when MFMA j of group g issues
-        static constexpr int allow(int g, int j) {
-            const int issued = before(g) + (j >= 1 ? reads(g) : 0);
-            const int pa = pos_a(g), pb = pos_b(g / 4, j);
-            const int n = issued - 1 - (pa > pb ? pa : pb);
-            return n > 15 ? 15 : n;
-        }
-    };
-
-    // LDS byte addresses (32-bit) of this lane's reads: [buffer][sub-step][half of the fragment];
-    // the fragment index t is the instruction's immediate offset
-    uint32_t aaddr[2][SPS][R], baddr[2][SPS][R];
+    const int frow = lane & 15, fc = lane >> 4;
+    const int fsw = swz(frow);
+    // LDS byte addresses of this lane's reads: [buffer][u], u = half of the fragment (fp8) or phase of the stage (int8)
+    uint32_t aaddr[2][2], baddr[2][2];
 #pragma unroll
     for (int buf = 0; buf < 2; buf++)
 #pragma unroll
-        for (int sub = 0; sub < SPS; sub++)
-#pragma unroll
-            for (int e = 0; e < R; e++) {
-                const uint32_t so = FP8 ? (uint32_t)(((4 * sub + 2 * fh + e) ^ fsw) << 4)
-                                        : (uint32_t)(((2 * sub + fh) ^ fsw) << 4);
-                aaddr[buf][sub][e] = lds_addr0 + buf * STAGE_BYTES + (wm * 128 + frow) * BK + so;
-                baddr[buf][sub][e] = lds_addr0 + buf * STAGE_BYTES + BM * BK + (wn * WN + frow) * BK + so;
-            }
-
-    i32x4 af[4][R], bf[2][TJ][R];
+        for (int u = 0; u < 2; u++) {
+            const uint32_t so = (uint32_t)(((FP8 ? 2 * fc + u : 4 * u + fc) ^ fsw) << 4);
+            aaddr[buf][u] = lds_addr0 + buf * STAGE_BYTES + (wm * 128 + frow) * BK + so;
+            baddr[buf][u] = lds_addr0 + buf * STAGE_BYTES + BM * BK + (wn * WN + frow) * BK + so;
+        }
+    i32x4 xf[TI][R], wf[2][TJ][R];
 #define NQ_LDS_READ(dst, addr, imm) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm))
 #define NQ_LDS_WAIT(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n))
-    auto mma = [&](int i, int j, const i32x4(&a)[R], const i32x4(&b)[R]) {
+    // zc: the accumulator's first MFMA of the tile (C = 0)
+    auto mma = [&](auto zc, int i, int j, const i32x4(&a)[R], const i32x4(&b)[R]) {
+        constexpr bool ZERO = decltype(zc)::value;
         if constexpr (FP8) {
             const i32x8 av = {a[0][0], a[0][1], a[0][2], a[0][3], a[1][0], a[1][1], a[1][2], a[1][3]};
             const i32x8 bv = {b[0][0], b[0][1], b[0][2], b[0][3], b[1][0], b[1][1], b[1][2], b[1][3]};
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, acc[i][j], 0, 0, 0, 0, 0, 0);
+            if constexpr (ZERO)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc_t{}, 0, 0, 0, 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[i][j], 0, 0, 0, 0, 0, 0);
         } else {
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], acc[i][j], 0, 0, 0);
+            // (inline assembly with the accumulator tied to itself: for this four-pass MFMA the compiler keeps result
+            // and addend apart, and with all 256 accumulator registers live that turns into a rotation through the
+            // vector registers, two copies per MFMA.  Consecutive MFMAs never share an accumulator, and the
+            // operands come from LDS reads whose wait stands in front, so no hazard is hidden from the compiler.)
+            auto& c = acc;
+            if constexpr (ZERO)
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(c[i][j]) : "v"(b[0]), "v"(a[0]));
+            else
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[i][j]) : "v"(b[0]), "v"(a[0]));
         }
     };
-    // the requests of group g of the stage in buffer BUF, in Sched's order (a request that would
-    // belong to a stage past K reads stale LDS into registers nobody uses)
-    auto requests = [&](auto gc, auto bufc) {
-        constexpr int g = decltype(gc)::value, BUF = decltype(bufc)::value;
-        auto& afr = af;  // (named outside the asm statements so that the lambda captures them)
-        auto& bfr = bf;
-        constexpr int sub = g / 4, i = g % 4;
-        constexpr int g2 = (g + 2) % G;                       // the group whose x fragment is requested
-        constexpr int abuf = (g + 2 >= G) ? BUF ^ 1 : BUF;    // ... in the next stage's buffer when it wraps
+    // token fragment i / channel fragment j of (buffer, phase) into the given registers
+    auto read_x = [&](auto ic, auto bufc, auto phc) {
+        constexpr int i = decltype(ic)::value, BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
+        auto& x = xf;  // (named outside the asm statements so that the lambda captures them)
 #pragma unroll
         for (int e = 0; e < R; e++) {
-            const uint32_t addr = aaddr[abuf][g2 / 4][e];
-            NQ_LDS_READ(afr[(g + 2) % 4][e], addr, (g2 % 4) * 32 * BK);
-        }
-        if constexpr (Sched::wfrags(g) > 0) {
-            constexpr bool nb = sub == SPS - 1;  // the w fragments are the next stage's first sub-step
-            constexpr int first = (nb ? i - 2 : i) * HB;
-            constexpr int set = (sub + 1) & 1, bsub = nb ? 0 : sub + 1, bbuf = nb ? BUF ^ 1 : BUF;
-#pragma unroll
-            for (int f = 0; f < HB; f++)
-#pragma unroll
-                for (int e = 0; e < R; e++) {
-                    const uint32_t addr = baddr[bbuf][bsub][e];
-                    NQ_LDS_READ(bfr[set][first + f][e], addr, (first + f) * 32 * BK);
-                }
+            const uint32_t addr = aaddr[BUF][FP8 ? e : PHI];
+            NQ_LDS_READ(x[i][e], addr, i * 16 * BK);
         }
     };
-    // transfers of the stage after next, issued from groups G-2 and G-1 in three slots each
-    constexpr int ND = DA + DB, DPG = ND / 2;
-    static_assert(ND == 16, "transfer slots below are written for 16 transfers per wavefront and stage");
-#define NQ_DMA_SLOT(g, slot, buf, srca, srcb)                                                      \
-    if constexpr ((g) >= G - 2) {                                                                  \
-        if (have2) {                                                                               \
-            constexpr int t0 = ((g) - (G - 2)) * DPG + (slot) * 3;                                 \
-            NQ_DMA(t0, buf, srca, srcb);                                                           \
-            NQ_DMA(t0 + 1, buf, srca, srcb);                                                       \
-            if constexpr ((slot) < 2) NQ_DMA(t0 + 2, buf, srca, srcb);                             \
-        }                                                                                          \
-    }
-#define NQ_GROUP(g, BUF)                                                                           \
-    if constexpr ((g) < G) {                                                                       \
-        constexpr int sub_ = (g) / 4, i_ = (g) % 4, set_ = sub_ & 1;                               \
-        constexpr int w0_ = ((g) == G - 2) ? 0 : Sched::allow((g), 0);                             \
-        if constexpr ((g) == G - 2) {                                                              \
-            /* this wavefront's share of the next stage has landed and its reads of this stage */ \
-            /* are done; past the barrier that holds for every wavefront */                        \
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");                            \
-            __builtin_amdgcn_s_barrier();                                                          \
-        } else {                                                                                   \
-            NQ_LDS_WAIT(w0_);                                                                      \
-        }                                                                                          \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        mma(i_, 0, af[(g) % 4], bf[set_][0]);                                                      \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        requests(std::integral_constant<int, (g)>{}, std::integral_constant<int, BUF>{});          \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        /* later MFMAs of the group wait again only where their w fragment is younger */           \
-        constexpr int b1_ = w0_ + Sched::reads((g));                                               \
-        constexpr int w1_ = Sched::allow((g), 1) < b1_ ? Sched::allow((g), 1) : b1_;               \
-        if constexpr (w1_ < b1_) NQ_LDS_WAIT(w1_);                                                 \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        mma(i_, 1, af[(g) % 4], bf[set_][1]);                                                      \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        NQ_DMA_SLOT((g), 0, BUF, srca, srcb)                                                       \
-        constexpr int w2_ = Sched::allow((g), 2) < w1_ ? Sched::allow((g), 2) : w1_;               \
-        if constexpr (w2_ < w1_) NQ_LDS_WAIT(w2_);                                                 \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        mma(i_, 2, af[(g) % 4], bf[set_][2]);                                                      \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        NQ_DMA_SLOT((g), 1, BUF, srca, srcb)                                                       \
-        constexpr int w3_ = Sched::allow((g), 3) < w2_ ? Sched::allow((g), 3) : w2_;               \
-        if constexpr (w3_ < w2_) NQ_LDS_WAIT(w3_);                                                 \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        mma(i_, 3, af[(g) % 4], bf[set_][3]);                                                      \
-        __builtin_amdgcn_sched_barrier(0);                                                         \
-        NQ_DMA_SLOT((g), 2, BUF, srca, srcb)                                                       \
-    }
-    // one stage, read from buffer BUF; its groups G-2 and G-1 refill BUF with stage st+2
-#define NQ_STAGE(BUF)                                                                              \
-    {                                                                                              \
-        const bool have2 = st + 2 < KT;                                                            \
-        const uint8_t* const srca = abase + (int64_t)(st + 2) * BK;                                \
-        const uint8_t* const srcb = bbase + (int64_t)(st + 2) * BK;                                \
-        NQ_GROUP(0, BUF) NQ_GROUP(1, BUF) NQ_GROUP(2, BUF) NQ_GROUP(3, BUF) NQ_GROUP(4, BUF)       \
-        NQ_GROUP(5, BUF) NQ_GROUP(6, BUF) NQ_GROUP(7, BUF) NQ_GROUP(8, BUF) NQ_GROUP(9, BUF)       \
-        NQ_GROUP(10, BUF) NQ_GROUP(11, BUF) NQ_GROUP(12, BUF) NQ_GROUP(13, BUF) NQ_GROUP(14, BUF)  \
-        NQ_GROUP(15, BUF)                                                                          \
-    }
+    auto read_w = [&](auto setc, auto jc, auto bufc, auto phc) {
+        constexpr int SET = decltype(setc)::value, j = decltype(jc)::value, BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
+        auto& w = wf;
+#pragma unroll
+        for (int e = 0; e < R; e++) {
+            const uint32_t addr = baddr[BUF][FP8 ? e : PHI];
+            NQ_LDS_READ(w[SET][j][e], addr, j * 16 * BK);
+        }
+    };
+    using std::integral_constant;
+    // One phase: the 64 MFMAs of (buffer BUF, phase PHI of its stage) with the requests for the next phase, and in a
+    // stage's last phase its barrier (start of row 2: this wavefront's share of the next stage has landed, its reads
+    // of this stage are done) followed by the transfers of the stage after next into the buffer just freed.
+    // ZERO: the tile's first phase (accumulators start from a literal zero).
+    auto phase = [&](auto bufc, auto phc, auto zeroc, bool have2, const uint8_t* srca, const uint8_t* srcb) {
+        constexpr int BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
+        constexpr bool LAST = PHI == PH - 1;
+        constexpr int NBUF = LAST ? BUF ^ 1 : BUF, NPH = LAST ? 0 : PHI + 1;
+        constexpr int WS = FP8 ? BUF : PHI;  // the set of channel fragments this phase multiplies
+        static_for<64>([&](auto mc) {
+            constexpr int m = decltype(mc)::value, i = m / 8, j = m % 8;
+            if constexpr (LAST && m == 16) {
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+            } else {
+                constexpr int al = lds_wait(m, R, LAST);
+                if constexpr (al >= 0) NQ_LDS_WAIT(al);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mma(zeroc, i, j, xf[i], wf[WS][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            constexpr int e = ev_at(m);
+            if constexpr (e == 0) {
+                read_x(integral_constant<int, 7>{}, bufc, phc);
+            } else if constexpr (e > 0) {
+                constexpr bool isx = e == 1 || e == 2 || e == 6 || e == 8 || e == 10 || e == 12 || e == 14;
+                if constexpr (isx) {
+                    constexpr int xi = e == 1 ? 0 : e == 2 ? 1 : e == 6 ? 2 : e == 8 ? 3 : e == 10 ? 4 : e == 12 ? 5 : 6;
+                    read_x(integral_constant<int, xi>{}, integral_constant<int, NBUF>{}, integral_constant<int, NPH>{});
+                } else {
+                    constexpr int wj = e == 3 ? 0 : e == 4 ? 1 : e == 5 ? 2 : e == 7 ? 3 : e == 9 ? 4 : e == 11 ? 5 : e == 13 ? 6 : 7;
+                    read_w(integral_constant<int, WS ^ 1>{}, integral_constant<int, wj>{}, integral_constant<int, NBUF>{},
+                           integral_constant<int, NPH>{});
+                }
+            }
+            if constexpr (LAST && dma_at(m) >= 0) {
+                // (one branch per pair of transfers; the requests above and below stand in straight code, so that no
+                // register with a read under way meets a copy where branches join)
+                if (have2) {
+                    constexpr int t = dma_at(m);
+                    NQ_DMA(t, BUF, srca, srcb);
+                    NQ_DMA(t + 1, BUF, srca, srcb);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    // one stage, read from buffer BUF; its last phase refills BUF with stage st + 2
+    auto stage = [&](auto bufc, auto zeroc, int st, int KT) {
+        const bool have2 = st + 2 < KT;
+        const uint8_t* const srca = abase + (int64_t)(st + 2) * BK;
+        const uint8_t* const srcb = bbase + (int64_t)(st + 2) * BK;
+        if constexpr (PH == 1) {
+            phase(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
+        } else {
+            phase(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
+            phase(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
+        }
+    };
 
     const int KT = p.K / BK;
     {
         // stage 0 now, stage 1 on its way during all of stage 0
-        const bool have2 = true;
-        (void)have2;
         const uint8_t* srca = abase;
         const uint8_t* srcb = bbase;
 #define NQ_DMA_ALL(buf)                                                                            \
@@ -403,64 +407,42 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 #undef NQ_DMA_ALL
     }
     const unsigned long long t_first = wall_clock64();  // stage 0 has landed
-    // what groups G-2 and G-1 of a previous stage (in buffer 1) would have requested
-    requests(std::integral_constant<int, G - 2>{}, std::integral_constant<int, 1>{});
-    requests(std::integral_constant<int, G - 1>{}, std::integral_constant<int, 1>{});
-    int st = 0;
-    for (; st + 1 < KT; st++) {
-        NQ_STAGE(0)
-        st++;
-        NQ_STAGE(1)
+    // what a phase before the first would have requested: all fragments of (buffer 0, phase 0)
+    static_for<TI>([&](auto ic) { read_x(ic, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
+    static_for<TJ>([&](auto jc) { read_w(integral_constant<int, 0>{}, jc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
+    NQ_LDS_WAIT(0);
+    stage(integral_constant<int, 0>{}, std::true_type{}, 0, KT);
+    {
+        int st = 1;
+        for (; st + 1 < KT; st += 2) {
+            stage(integral_constant<int, 1>{}, std::false_type{}, st, KT);
+            stage(integral_constant<int, 0>{}, std::false_type{}, st + 1, KT);
+        }
+        if (st < KT) stage(integral_constant<int, 1>{}, std::false_type{}, st, KT);  // an even number of stages
     }
-    if (st < KT) NQ_STAGE(0)  // an odd number of stages: the last one, in buffer 0 again
     NQ_LDS_WAIT(0);  // requests past the last stage still target registers: let them land
+    __syncthreads();  // every wavefront is done with the stage buffers: the epilogue stages through them
     const unsigned long long t_loop = wall_clock64();
-#undef NQ_STAGE
-#undef NQ_GROUP
-#undef NQ_DMA_SLOT
 #undef NQ_DMA
 #undef NQ_LDS_READ
 #undef NQ_LDS_WAIT
 
-    // ---- epilogue.  The MFMA was issued with the weight tile as its first operand, so in
-    // acc[i][j] a lane holds ONE token m = 32 i + lane % 32 (MFMA column) and, for g = 0..3, the
-    // four consecutive channels n = 32 j + 8 g + 4 (lane / 32) + 0..3 (MFMA rows, registers 4g..4g+3).
-    // Per-token work is lane-local and four outputs of a row of y are adjacent.  Each wavefront
-    // stages its results through its own LDS region (free now: the loop ended on a barrier) as
-    // [token][channel] rows, and writes them out as 128-bit stores, 256 B (bf16) or 512 B (fp32 /
-    // int32) contiguous per row of y.
+    // ---- epilogue.  The MFMA was issued with the weight fragment as its first operand, so in acc[i][j] a lane
+    // holds ONE token m = 16 i + lane % 16 (MFMA column) and the four consecutive channels n = 16 j + 4 (lane / 16)
+    // + 0..3 (MFMA rows, registers 0..3).  Per-token work is lane-local and four outputs of a row of y are adjacent.
+    // Each wavefront stages its results through its own LDS region as [token][channel] rows, and writes them out as
+    // 128-bit stores, 256 B (bf16) or 512 B (fp32 / int32) contiguous per row of y.
     const int wm0 = m0 + wm * 128, wn0 = n0 + wn * WN;
-    const int lm = lane & 31, lh = lane >> 5;
+    const int lm = lane & 15, lq = lane >> 4;
     // whole 16-byte stores wherever the tile's columns all exist and rows of y stay 16-byte aligned
     // (a tile that only M cuts short just skips the rows past M)
     const bool full_cols = (n0 + BN <= p.N) && (p.N % 8 == 0) && (((uintptr_t)p.y & 15) == 0);
 
-    // channel scale and bias for the lane's channels of tile j, group g (needs n < N: clamped)
-    auto chan = [&](int j, int g, float (&cs)[4], float (&cb)[4], bool need_scale, int zero) {
-        if (p.chan_vec) {  // uniform: the lane's four channels are adjacent, one load per operand
-            const int nb = min(wn0 + 32 * j + 8 * g + 4 * lh, p.N - 4) + zero;
-            if (need_scale) {
-                const float4 sv = *reinterpret_cast<const float4*>(p.col_scale + nb);
-                cs[0] = sv.x, cs[1] = sv.y, cs[2] = sv.z, cs[3] = sv.w;
-            } else {
-                cs[0] = cs[1] = cs[2] = cs[3] = 1.0f;
-            }
-            cb[0] = cb[1] = cb[2] = cb[3] = 0.0f;
-            if (p.bias) {
-                if (p.bias_dtype == NQ_DT_F32) {
-                    const float4 bv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + nb);
-                    cb[0] = bv.x, cb[1] = bv.y, cb[2] = bv.z, cb[3] = bv.w;
-                } else {
-                    const uint2 bv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.bias) + nb);
-                    cb[0] = __uint_as_float(bv.x << 16), cb[1] = __uint_as_float(bv.x & 0xFFFF0000u);
-                    cb[2] = __uint_as_float(bv.y << 16), cb[3] = __uint_as_float(bv.y & 0xFFFF0000u);
-                }
-            }
-            return;
-        }
+    // channel scale and bias for the lane's channels of fragment j (needs n < N: clamped)
+    auto chan = [&](int j, float (&cs)[4], float (&cb)[4], bool need_scale, int zero) {
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int n = min(wn0 + 32 * j + 8 * g + 4 * lh + r, p.N - 1) + zero;
+            const int n = min(wn0 + 16 * j + 4 * lq + r, p.N - 1) + zero;
             cs[r] = need_scale ? p.col_scale[n] : 1.0f;
             cb[r] = 0.0f;
             if (p.bias)
@@ -472,127 +454,92 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 
     auto emit = [&](auto kind, auto plain) {
         constexpr int KIND = decltype(kind)::value;  // 0: fp32, 1: bf16, 2: raw int32
-        // MODE (uniform over the launch, so chosen once and not per channel tile: a branch around a load makes the
-        // wavefront wait for that load where the branches meet).  0: one scale for the whole tensor and no bias (fp8 x
-        // fp8): no channel operands at all; 1 .. 3: the lane's four channels adjacent and aligned, one load per
-        // operand - no bias, fp32 bias, bf16 bias; 4: channel by channel
+        // MODE (uniform over the launch, so chosen once and not per channel fragment: a branch around a load makes
+        // the wavefront wait for that load where the branches meet).  0: one scale for the whole tensor and no bias
+        // (fp8 x fp8): no channel operands at all; 1 .. 3: the lane's four channels adjacent and aligned, one load
+        // per operand - no bias, fp32 bias, bf16 bias; 4: channel by channel
         constexpr int MODE = decltype(plain)::value;
         constexpr bool PLAIN = MODE == 0;
         constexpr int ES = (KIND == 1) ? 2 : 4;      // bytes per output element
-        constexpr int IP = (KIND == 1) ? 2 : 1;      // token tiles (of 32) staged per pass
+        constexpr int IP = (KIND == 1) ? 4 : 2;      // token fragments (of 16) staged per pass
         constexpr int ROWB = WN * ES + 16;           // staged row: the wavefront's channels + pad (bank spread)
-        uint8_t* stage = lds + wave * (32 * IP * ROWB);
+        uint8_t* stg = lds + wave * (16 * IP * ROWB);
 #pragma unroll
-        for (int ip = 0; ip < 4; ip += IP) {
-            // ---- registers -> LDS (this wavefront's region only).  Channel scales and biases are
-            // fetched per channel tile j; the compiler barrier keeps it from hoisting all 16 (j, g)
-            // sets above the loop, which would spill.
+        for (int ip = 0; ip < TI; ip += IP) {
+            // ---- registers -> LDS (this wavefront's region only).
             // (a zero the compiler cannot see through, new in every pass: the channel operands do not depend on
-            // the pass, and kept across all four passes of the fp32 epilogue they cost 129 spilled registers and
-            // 60 % of the call's time; they are re-read from L1 per pass instead)
+            // the pass, and kept across the passes they spill; they are re-read from L1 per pass instead)
             int zero = 0;
             asm volatile("" : "+v"(zero));
             float rscale[IP];
 #pragma unroll
             for (int ii = 0; ii < IP; ii++) {
                 rscale[ii] = 1.0f;
-                if constexpr (!FP8 && KIND != 2) rscale[ii] = p.row_scale[min(wm0 + 32 * (ip + ii) + lm, p.M - 1)];
+                if constexpr (!FP8 && KIND != 2) rscale[ii] = p.row_scale[min(wm0 + 16 * (ip + ii) + lm, p.M - 1)];
             }
-            // modes 1 .. 3: the operands of channel tile j + 1 are requested before tile j is worked on
-            auto fetch = [&](int j, float (&cs)[4][4], float (&cb)[4][4]) {
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int nb = min(wn0 + 32 * j + 8 * g + 4 * lh, p.N - 4) + zero;
-                    if constexpr (!FP8) {
-                        const float4 sv = *reinterpret_cast<const float4*>(p.col_scale + nb);
-                        cs[g][0] = sv.x, cs[g][1] = sv.y, cs[g][2] = sv.z, cs[g][3] = sv.w;
-                    } else {
-                        cs[g][0] = cs[g][1] = cs[g][2] = cs[g][3] = 1.0f;
-                    }
-                    if constexpr (MODE == 2) {
-                        const float4 bv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + nb);
-                        cb[g][0] = bv.x, cb[g][1] = bv.y, cb[g][2] = bv.z, cb[g][3] = bv.w;
-                    } else if constexpr (MODE == 3) {
-                        const uint2 bv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.bias) + nb);
-                        cb[g][0] = __uint_as_float(bv.x << 16), cb[g][1] = __uint_as_float(bv.x & 0xFFFF0000u);
-                        cb[g][2] = __uint_as_float(bv.y << 16), cb[g][3] = __uint_as_float(bv.y & 0xFFFF0000u);
-                    } else {
-                        cb[g][0] = cb[g][1] = cb[g][2] = cb[g][3] = 0.0f;
-                    }
+            auto fetch = [&](int j, float (&cs)[4], float (&cb)[4]) {
+                const int nb = min(wn0 + 16 * j + 4 * lq, p.N - 4) + zero;
+                if constexpr (!FP8) {
+                    const float4 sv = *reinterpret_cast<const float4*>(p.col_scale + nb);
+                    cs[0] = sv.x, cs[1] = sv.y, cs[2] = sv.z, cs[3] = sv.w;
+                } else {
+                    cs[0] = cs[1] = cs[2] = cs[3] = 1.0f;
+                }
+                if constexpr (MODE == 2) {
+                    const float4 bv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.bias) + nb);
+                    cb[0] = bv.x, cb[1] = bv.y, cb[2] = bv.z, cb[3] = bv.w;
+                } else if constexpr (MODE == 3) {
+                    const uint2 bv = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p.bias) + nb);
+                    cb[0] = __uint_as_float(bv.x << 16), cb[1] = __uint_as_float(bv.x & 0xFFFF0000u);
+                    cb[2] = __uint_as_float(bv.y << 16), cb[3] = __uint_as_float(bv.y & 0xFFFF0000u);
+                } else {
+                    cb[0] = cb[1] = cb[2] = cb[3] = 0.0f;
                 }
             };
-            // (not for int8 with fp32 output: its four passes of one token tile leave no registers for a second set)
             constexpr bool VEC = KIND != 2 && MODE >= 1 && MODE <= 3;
-            constexpr bool AHEAD = VEC && !(KIND == 0 && !FP8);
-            float ncs[4][4], ncb[4][4];
-            if constexpr (AHEAD) fetch(0, ncs, ncb);
+            // modes 1 .. 3: the operands of two channel fragments are requested together, a pair ahead
+            float ncs[2][4], ncb[2][4];
+            if constexpr (VEC) fetch(0, ncs[0], ncb[0]), fetch(1, ncs[1], ncb[1]);
 #pragma unroll
             for (int j = 0; j < TJ; j++) {
-                float cs[4][4], cb[4][4];
-                if constexpr (AHEAD) {
+                float cs[4], cb[4];
+                if constexpr (VEC) {
 #pragma unroll
-                    for (int g = 0; g < 4; g++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++) cs[g][r] = ncs[g][r], cb[g][r] = ncb[g][r];
-                    if (j + 1 < TJ) fetch(j + 1, ncs, ncb);
-                } else if constexpr (VEC) {
-                    fetch(j, cs, cb);
+                    for (int r = 0; r < 4; r++) cs[r] = ncs[j & 1][r], cb[r] = ncb[j & 1][r];
+                    if (j + 2 < TJ) fetch(j + 2, ncs[j & 1], ncb[j & 1]);
                 }
-                if constexpr (KIND != 2 && MODE == 4) {
+                if constexpr (KIND != 2 && MODE == 4) chan(j, cs, cb, !FP8, zero);
 #pragma unroll
-                    for (int g = 0; g < 4; g++) chan(j, g, cs[g], cb[g], !FP8, zero);
-                }
-                if constexpr (KIND == 2) {
+                for (int ii = 0; ii < IP; ii++) {
+                    const int i = ip + ii;
+                    uint8_t* dst = stg + (16 * ii + lm) * ROWB + (16 * j + 4 * lq) * ES;
+                    if constexpr (KIND == 2) {
+                        *reinterpret_cast<i32x4*>(dst) = (i32x4){(int)acc[i][j][0], (int)acc[i][j][1], (int)acc[i][j][2], (int)acc[i][j][3]};
+                    } else {
+                        float z[4];
 #pragma unroll
-                    for (int ii = 0; ii < IP; ii++) {
-                        const int i = ip + ii;
+                        for (int r = 0; r < 4; r++) {
+                            if constexpr (PLAIN)
+                                z[r] = acc[i][j][r] * fp8_scale + 0.0f;  // (+ 0.0f: the bits of the general path, -0.0 included)
+                            else if constexpr (FP8)
+                                z[r] = acc[i][j][r] * fp8_scale + cb[r];
+                            else
+                                z[r] = (float)acc[i][j][r] * (rscale[ii] * cs[r]) + cb[r];
+                        }
+                        if (p.epilogue == NQ_EPI_RELU) {
+                            // a real (uniform) branch: one v_max per value when asked for, nothing otherwise
+                            asm volatile("" ::: "memory");
 #pragma unroll
-                        for (int g = 0; g < 4; g++) {
-                            uint8_t* dst = stage + (32 * ii + lm) * ROWB + (32 * j + 8 * g + 4 * lh) * ES;
-                            *reinterpret_cast<i32x4*>(dst) = (i32x4){(int)acc[i][j][4 * g], (int)acc[i][j][4 * g + 1],
-                                                                      (int)acc[i][j][4 * g + 2], (int)acc[i][j][4 * g + 3]};
+                            for (int r = 0; r < 4; r++) z[r] = z[r] > 0.0f ? z[r] : 0.0f;
+                        }
+                        if constexpr (KIND == 0) {
+                            *reinterpret_cast<float4*>(dst) = make_float4(z[0], z[1], z[2], z[3]);
+                        } else {
+                            // v_cvt_pk_bf16_f32: round to nearest even in hardware
+                            const bf16x4 pk = __builtin_convertvector((f32x4){z[0], z[1], z[2], z[3]}, bf16x4);
+                            *reinterpret_cast<bf16x4*>(dst) = pk;
                         }
                     }
-                } else {
-                    float z[IP][4][4];
-#pragma unroll
-                    for (int ii = 0; ii < IP; ii++)
-#pragma unroll
-                        for (int g = 0; g < 4; g++)
-#pragma unroll
-                            for (int r = 0; r < 4; r++) {
-                                if constexpr (PLAIN)
-                                    z[ii][g][r] = acc[ip + ii][j][4 * g + r] * fp8_scale + 0.0f;  // (+ 0.0f: the bits of the general path, -0.0 included)
-                                else if constexpr (FP8)
-                                    z[ii][g][r] = acc[ip + ii][j][4 * g + r] * fp8_scale + cb[g][r];
-                                else
-                                    z[ii][g][r] = (float)acc[ip + ii][j][4 * g + r] * (rscale[ii] * cs[g][r]) + cb[g][r];
-                            }
-                    if (p.epilogue == NQ_EPI_RELU) {
-                        // a real (uniform) branch: one v_max per value when asked for, nothing otherwise
-                        asm volatile("" ::: "memory");
-#pragma unroll
-                        for (int ii = 0; ii < IP; ii++)
-#pragma unroll
-                            for (int g = 0; g < 4; g++)
-#pragma unroll
-                                for (int r = 0; r < 4; r++) z[ii][g][r] = z[ii][g][r] > 0.0f ? z[ii][g][r] : 0.0f;
-                    }
-#pragma unroll
-                    for (int ii = 0; ii < IP; ii++)
-#pragma unroll
-                        for (int g = 0; g < 4; g++) {
-                            uint8_t* dst = stage + (32 * ii + lm) * ROWB + (32 * j + 8 * g + 4 * lh) * ES;
-                            if constexpr (KIND == 0) {
-                                *reinterpret_cast<float4*>(dst) =
-                                    make_float4(z[ii][g][0], z[ii][g][1], z[ii][g][2], z[ii][g][3]);
-                            } else {
-                                // v_cvt_pk_bf16_f32: round to nearest even in hardware
-                                const bf16x4 pk = __builtin_convertvector(
-                                    (f32x4){z[ii][g][0], z[ii][g][1], z[ii][g][2], z[ii][g][3]}, bf16x4);
-                                *reinterpret_cast<bf16x4*>(dst) = pk;
-                            }
-                        }
                 }
                 asm volatile("" ::: "memory");
             }
@@ -602,13 +549,13 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             // ---- LDS -> global: 16 bytes per lane, rows of y contiguous
-            constexpr int LPRW = WN * ES / 16;           // lanes per staged row (8, 16 or 32)
+            constexpr int LPRW = WN * ES / 16;           // lanes per staged row (16 or 32)
             constexpr int RPI = 64 / LPRW;               // rows per wavefront instruction
 #pragma unroll
-            for (int t = 0; t < 32 * IP / RPI; t++) {
+            for (int t = 0; t < 16 * IP / RPI; t++) {
                 const int row = t * RPI + lane / LPRW, c16 = lane % LPRW;
-                const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * ROWB + c16 * 16);
-                const int m = wm0 + 32 * ip + row;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(stg + row * ROWB + c16 * 16);
+                const int m = wm0 + 16 * ip + row;
                 const int n = wn0 + c16 * (16 / ES);
                 if (full_cols) {
                     if (m < p.M)
@@ -668,12 +615,6 @@ int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int bn, in
 
 }  // namespace
 
-namespace {
-unsigned long long* g_stamps = nullptr;  // set by the timeline diagnostic around one call, null otherwise
-}
-
-void gemm8_set_stamps(unsigned long long* buf) { g_stamps = buf; }
-
 bool gemm8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
     const bool fp8 = (a.x_dtype == NQ_DT_FP8_E4M3 && L->format == NQ_FMT_FP8_E4M3);
@@ -694,7 +635,7 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + 255) / 256;
-    p.stamps = g_stamps;
+    p.stamps = a.diag_stamps;
     const bool i8 = a.x_dtype == NQ_DT_I8;
     p.chan_vec = L->out % 4 == 0 && L->out >= 4 && (!i8 || a.y_dtype == NQ_DT_I32 || (uintptr_t)p.col_scale % 16 == 0) &&
                  (!a.bias || (uintptr_t)a.bias % (a.bias_dtype == NQ_DT_F32 ? 16 : 8) == 0);
