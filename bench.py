@@ -24,7 +24,7 @@ batched-env actor at M = 4096, in TOPS); `roofline_mfma` is the large-M fp8 GEMM
 (`mfma_only`: back-to-back MFMAs on register operands, constant and random data).
 
 `--only a16_shapes --a16-class C` re-derives the constants by which the library picks the tile shape of its
-kernel for tens to hundreds of activation rows (a grid of calls timed under each shape, nq_diag_a16_shape);
+kernel for tens to hundreds of activation rows (a grid of calls timed under each shape, nq_diag_forward_a16);
 `--only mid_dispatch --a16-class C` times the kernels that compete for those calls side by side and the library's
 choice between them.
 
@@ -828,10 +828,12 @@ def cpu_baseline(budget_s=12.0):
 
 def a16_shapes(cls="w4g"):
     """Times a grid of medium-M calls of one weight format / activation type under each of the 16-row tile kernel's
-    five tile shapes (`nq_diag_a16_shape`) and under the library's own choice, and re-derives the constants of
+    five tile shapes (`nq_diag_forward_a16`) and under the library's own choice, and re-derives the constants of
     the estimate the library chooses by: t = F + ceil(workgroups / 256) * (p0 + p1 * k-steps) microseconds per
     shape, by least squares on relative errors.  Reports the constants, the fit's mean error, what always taking
     the shape of least estimate costs against always taking the fastest, and the same for the library's choice."""
+    import ctypes as C
+
     import numpy as np
     import torch
 
@@ -866,12 +868,15 @@ def a16_shapes(cls="w4g"):
                 y = torch.empty((M, N), dtype=torch.float32, device="cuda")
                 step = lambda i: lin.forward(x, out=y)
                 median_per_call(step, 20)  # (clocks up before the first timed shape)
+                xc = L.DT_F32 if xf32 else L.DT_BF16
                 ts = []
                 for mw, nw in shapes + [(0, 0)]:
-                    L.check(L.lib().nq_diag_a16_shape(mw, nw))
-                    ts.append(float("nan") if (xf32 and mw * nw == 8) else median_per_call(step, 20) * 1e6)
+                    def shaped(i, mw=mw, nw=nw):
+                        L.check(L.lib().nq_diag_forward_a16(lin._h, C.c_void_p(x.data_ptr()), xc, C.c_void_p(y.data_ptr()), L.DT_F32, M,
+                                                             mw, nw, C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+                    fn = step if (mw, nw) == (0, 0) else shaped
+                    ts.append(float("nan") if (xf32 and mw * nw == 8) else median_per_call(fn, 20) * 1e6)
                 rows.append((K, N, M, ts))
-    L.check(L.lib().nq_diag_a16_shape(0, 0))
 
     def feats(K, N, M, mw, nw):
         mt = (M + 15) // 16

@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define NQ_ABI_VERSION 4
+#define NQ_ABI_VERSION 5
 
 /* status codes */
 #define NQ_OK 0
@@ -141,6 +141,14 @@ int32_t nq_get_blocks(nq_handle h, uint8_t* out_host, int64_t nbytes);
 /* `QLinear.keep_only_repacked` (qlinear.mojo:342-356): drop the host copy of
  * the logical blocks; only the device layout the forward reads is kept. */
 int32_t nq_keep_only_repacked(nq_handle h);
+
+/* Device memory the layer's weights occupy, in bytes: codes, scales, zero points and every copy of them in another
+ * order that a kernel reads (no counterpart in the reference, whose `keep_only_repacked` documents the one-copy rule,
+ * qlinear.mojo:342-356; this is how a caller checks it).  0 for an unloaded layer or a null handle.  Q4_0: 0.5625
+ * bytes per weight; a 4-bit layer at least 2048 columns wide (or made with NQ_FLAG_PREFER_TILE) and a layer of 4 M
+ * weights and more keep a second, tile-ordered copy of their codes unless made with NQ_FLAG_NO_TILE_COPY: 1.06 bytes
+ * per weight, 1.16 where IN = 960 pads to 1024 in tile order (int8: 2.0). */
+int64_t nq_device_bytes(nq_handle h);
 
 /* ---- compute ------------------------------------------------------------ */
 
@@ -316,40 +324,9 @@ int32_t nq_set_weight_gptq(nq_handle h, const float* w_host, int64_t n_values, n
 int32_t nq_q4_0_objective(nq_handle h, const float* w_host, int64_t n_values, nq_hessian hess,
                           double* out, void* stream);
 
-/* ---- diagnostics ---------------------------------------------------------------------------- */
-
-/* What the matrix cores alone sustain on this GPU (no counterpart in the reference; bench.py reports it
- * beside the 8-bit GEMM so that the GEMM's fraction of the published peak can be read against what the chip's
- * power limit leaves): `workgroups` workgroups of four wavefronts issue 16 * iters MFMAs of 32 x 32 each, back
- * to back, on register operands taken from `operands` (device, operand_bytes >= 4096; what the bytes are,
- * constant or random codes, is the caller's choice).  kind 0: v_mfma_f32_32x32x64_f8f6f4 on e4m3 codes
- * (131072 operations each), kind 1: v_mfma_i32_32x32x32_i8 (65536 each).  stamps: device int64
- * [workgroups][2] = the loop's duration in shader clocks and in ticks of the constant 100 MHz clock. */
-int32_t nq_diag_mfma_rate(int32_t kind, const void* operands, int64_t operand_bytes, int32_t iters, int32_t workgroups,
-                          int64_t* stamps, void* stream);
-
-/* The floor of a weight-streaming call (no counterpart in the reference): a kernel that only reads the first
- * nbytes / 1024 KiB of `src` (device, 16-byte aligned) with 1 KiB load instructions and computes nothing.
- * bench.py times it on the bytes of each large GEMV's weight: launch + stream, what no GEMV over those bytes
- * can beat on this GPU. */
-int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream);
-
-/* Where the time of a large-tile 8-bit GEMM goes (no counterpart in the reference): nq_forward with 8-bit
- * activations and M >= 64 rows, with every workgroup of the 256 x 256 tile kernel reporting four readings of
- * the GPU's constant 100 MHz clock - entry, first K stage landed, K loop done, stores acknowledged - into
- * stamps (device uint64 [tiles][4], tiles = ceil(M / 256) * ceil(OUT / 256) <= max_tiles, else NQ_ERR_INVALID).
- * The arguments are nq_forward's for that case (x: int8 with per-row x_scale, or e4m3 codes with one scale; no
- * bias).  Synchronises the stream before it returns; calls of nq_forward from other threads meanwhile would
- * write stamps too. */
-int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
-                               int32_t y_dtype, int32_t M, uint64_t* stamps, int64_t max_tiles, void* stream);
-
-/* The tile shape of the 16-row tile kernel that takes 2 .. 511 rows of fp32 / bf16 activations (no counterpart in
- * the reference): mw x nw wavefront tiles of 16 x 16 per workgroup, one of 1 x 1, 1 x 2, 1 x 4, 2 x 2, 2 x 4, for
- * every later call in the process until (0, 0) gives the choice back to the library.  The library picks the shape
- * of least estimated time; `bench.py --only a16_shapes` times a grid of calls under each shape with this switch and
- * re-derives the estimate's constants from them.  The shape never changes a result's bits. */
-int32_t nq_diag_a16_shape(int32_t mw, int32_t nw);
+/* (The measurement helpers bench.py uses - the matrix cores alone, a plain read, a GEMM call's timeline, a forward
+ * under a given tile shape - are declared in noeira_qlinear_diag.h: a caller of the operator needs none of them, and
+ * none of them changes what any other call does.) */
 
 #ifdef __cplusplus
 }

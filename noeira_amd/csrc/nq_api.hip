@@ -66,7 +66,7 @@ void free_device(nq_layer* L) {
     if (L->d_tile16) (void)hipFree(L->d_tile16);
     if (L->d_tile16_scales) (void)hipFree(L->d_tile16_scales);
     L->d_codes = nullptr, L->d_scales = nullptr, L->d_zps = nullptr, L->d_tiled = nullptr;
-    L->d_tile16 = nullptr, L->d_tile16_scales = nullptr, L->tile_nj = 0;
+    L->d_tile16 = nullptr, L->d_tile16_scales = nullptr, L->tile_nj = 0, L->tiled_bytes = 0;
 }
 
 int32_t check_handle(nq_handle h, const char* what) {
@@ -274,6 +274,7 @@ int32_t nq_set_weight_i8(nq_handle h, const int8_t* w_host, const float* scales_
     hipError_t e = hipMalloc((void**)&h->d_codes, n + 16);
     if (e == hipSuccess) e = hipMalloc(&h->d_scales, (size_t)h->out * 4 + 16);
     if (e == hipSuccess && !tiled.empty()) e = hipMalloc((void**)&h->d_tiled, tiled.size());
+    h->tiled_bytes = (int64_t)tiled.size();
     if (e == hipSuccess) e = hipMemcpyAsync(h->d_codes, w_host, n, hipMemcpyHostToDevice, s);
     if (e == hipSuccess) e = hipMemcpyAsync(h->d_scales, scales_host, (size_t)h->out * 4, hipMemcpyHostToDevice, s);
     if (e == hipSuccess && !tiled.empty())
@@ -368,6 +369,25 @@ int32_t nq_get_blocks(nq_handle h, uint8_t* out_host, int64_t nbytes) {
     if (!out_host) return fail(NQ_ERR_INVALID, "nq_get_blocks: null buffer");
     std::memcpy(out_host, h->host_blocks.data(), (size_t)nbytes);
     return NQ_OK;
+}
+
+int64_t nq_device_bytes(nq_handle h) {
+    if (!h || !h->loaded) return 0;
+    const int64_t rows = h->out;
+    int64_t n = rows * h->row_bytes;
+    switch (h->format) {
+        case NQ_FMT_Q4_0: n += rows * (h->in / Q4_GROUP) * 2; break;
+        case NQ_FMT_W4_GROUP: n += rows * h->groups * 3; break;  // fp16 scale + one byte of zero point per group
+        case NQ_FMT_W8_CHANNEL: n += rows * 4; break;
+        default: break;
+    }
+    if (h->d_tiled) n += h->tiled_bytes;
+    if (h->d_tile16) {
+        const int64_t tiles = (rows + 15) / 16 * h->tile_nj;
+        n += tiles * 1024;
+        if (h->d_tile16_scales) n += tiles * 16 * (h->format == NQ_FMT_W4_GROUP ? 4 : 8);
+    }
+    return n;
 }
 
 int32_t nq_keep_only_repacked(nq_handle h) {
@@ -1011,6 +1031,26 @@ int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, cons
     if (rc) return rc;
     NQ_HIP(hipStreamSynchronize((hipStream_t)stream));
     return NQ_OK;
+}
+
+int32_t nq_diag_forward_a16(nq_handle h, const void* x, int32_t x_dtype, void* y, int32_t y_dtype, int32_t M,
+                            int32_t mw, int32_t nw, void* stream) {
+    int32_t rc = check_handle(h, "nq_diag_forward_a16");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    if ((mw != 1 && mw != 2) || (nw != 1 && nw != 2 && nw != 4) || (mw == 2 && nw == 1) ||
+        (mw == 2 && nw == 4 && x_dtype == NQ_DT_F32))
+        return fail(NQ_ERR_INVALID, "nq_diag_forward_a16: shapes are 1 x 1, 1 x 2, 1 x 4, 2 x 2, 2 x 4 (2 x 4 with bf16 activations only)");
+    if (!x || !y || ((uintptr_t)x & 15) || ((uintptr_t)y & 3) || (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16))
+        return fail(NQ_ERR_INVALID, "nq_diag_forward_a16: x (16-byte aligned) and an fp32 or bf16 y (4-byte aligned) are needed");
+    SegTable seg{};
+    seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
+    ForwardArgs a{h, x, x_dtype, nullptr, y, y_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_NONE, (hipStream_t)stream, seg};
+    if (h->glu || !h->seg_end.empty() || !gemm_a16_applicable(a))
+        return fail(NQ_ERR_UNSUPPORTED, "nq_diag_forward_a16: the 16-row tile kernel does not take this call (fp32 / bf16 "
+                                        "activations, M >= 2, an ordinary layer)");
+    a.diag_a16_shape = mw << 4 | nw;
+    return launch_gemm_a16(a);
 }
 
 int32_t nq_quantize_rows_i8(const void* x, int32_t x_dtype, int8_t* q, float* scales, int32_t M, int32_t K,

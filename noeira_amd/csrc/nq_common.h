@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "../../include/noeira_qlinear.h"
+#include "../../include/noeira_qlinear_diag.h"
 
 namespace nq {
 
@@ -63,6 +64,7 @@ struct nq_layer {
     // W8_CHANNEL layers of at most 256 x 256: a second copy of the codes as MFMA operand tiles for the fused MLP
     // (tile (j, s) = rows 16 j .., k = 64 s .. is 1 KiB, lane l's 16 bytes at 16 l; zeros beyond OUT and IN)
     uint8_t* d_tiled = nullptr;
+    int64_t tiled_bytes = 0;
     // large layers (nq_gemv_tile.hip): a second copy of the codes in the matrix core's operand order for 16 rows
     // at a time, and (4-bit) of the group records in the same order; tile_nj = steps of K per row tile
     uint8_t* d_tile16 = nullptr;
@@ -133,6 +135,8 @@ struct ForwardArgs {
     float lora_s = 0.0f;
     // nq_diag_gemm8_timeline: where the large-tile GEMM writes its per-tile clock readings (null: none)
     unsigned long long* diag_stamps = nullptr;
+    // nq_diag_forward_a16: the 16-row tile kernel's shape for this launch, mw << 4 | nw (0: the library's choice)
+    int32_t diag_a16_shape = 0;
 };
 
 // nq_q4_0.hip

@@ -985,8 +985,6 @@ int32_t launch_tile(const A16Params& p, int mw, int nw, int kw, dim3 grid, hipSt
 
 }  // namespace
 
-// the shape nq_diag_a16_shape asked for (mw << 4 | nw), 0: none
-static std::atomic<int> g_diag_shape{0};
 
 // Tile shape of the medium-M kernel (wavefront tiles of 16 rows x 16 columns: mw x nw of them per workgroup) and what
 // the call will take.  One workgroup of any shape fits a CU at a time, so a call runs in ceil(workgroups / 256)
@@ -1129,7 +1127,7 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     // row-fused layer takes it only when every part would on its own (a mix runs part by part:
     // gemm_a16_splits_parts); from 512 rows on the whole layer's width decides, and a row's bits in a row-fused
     // layer may differ from those in its own layer.
-    const bool use_big = (a.M >= 512 || a.seg.nseg < 2) ? big_wins(a, L->out) : big_parts(a) == a.seg.nseg;
+    const bool use_big = !a.diag_a16_shape && ((a.M >= 512 || a.seg.nseg < 2) ? big_wins(a, L->out) : big_parts(a) == a.seg.nseg);
     if (use_big) {
         int big = 2;
         big_estimate_us(L->format, xf32, a.M, L->out, L->in, &big);
@@ -1154,10 +1152,7 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
     }
     int mw = 1, nw = 1;
     gemm_a16_estimate_us(L->format, xf32, a.M, L->out, L->in, &mw, &nw);
-    if (const int forced = g_diag_shape.load(std::memory_order_relaxed)) {
-        // nq_diag_a16_shape: a measurement asked for one shape (2 x 4 does not exist for fp32 activations)
-        if (!(xf32 && forced == 0x24)) mw = forced >> 4, nw = forced & 15;
-    }
+    if (const int forced = a.diag_a16_shape) mw = forced >> 4, nw = forced & 15;  // nq_diag_forward_a16
     const int kstep = four_bit ? 128 : 64;
     const int nsteps = (L->in + kstep - 1) / kstep;
     // K split: 8 wavefronts when there are more than 4 k-steps.  It follows K alone: the K split fixes
@@ -1187,14 +1182,3 @@ int32_t launch_gemm_a16(const ForwardArgs& a) {
 }
 
 }  // namespace nq
-
-extern "C" int32_t nq_diag_a16_shape(int32_t mw, int32_t nw) {
-    if (mw == 0 && nw == 0) {
-        nq::g_diag_shape.store(0);
-        return NQ_OK;
-    }
-    if ((mw != 1 && mw != 2) || (nw != 1 && nw != 2 && nw != 4) || (mw == 2 && nw == 1))
-        return nq::fail(NQ_ERR_INVALID, "nq_diag_a16_shape: shapes are 1 x 1, 1 x 2, 1 x 4, 2 x 2, 2 x 4 (0, 0: the library's own choice)");
-    nq::g_diag_shape.store(mw << 4 | nw);
-    return NQ_OK;
-}

@@ -1643,16 +1643,26 @@ int32_t launch4_mt(const TileMrParams& pm, hipStream_t s) {
 
 }  // namespace
 
-// Which layers get the tile-ordered copy (a second copy of the codes: 0.5 or 1 byte per weight on top):
-// weights of 4 M codes and more, whose single-row calls are bound by the weight stream.  4-bit: Q4_0 or
-// groups of exactly 128, IN a multiple of 128 in 2048 .. 16384; int8: IN a multiple of 64, at least 1024.
-// 4-bit layers whose rows are at most 6144 codes long get it whatever their size (IN alone decides, so that a
-// row-fused layer and its parts agree): the kernel for tens to hundreds of activation rows reads it.
+// Which layers get the tile-ordered copy (a second copy of the codes: 0.5 or 1 byte per weight on top): those whose
+// default dispatch has a kernel that reads it.
+//   - weights of 4 M codes and more, whose single-row calls are bound by the weight stream.  4-bit: Q4_0 or groups of
+//     exactly 128, IN a multiple of 128 in 2048 .. 16384; int8: IN a multiple of 64, at least 1024;
+//   - 4-bit layers whose rows are at most 6144 codes long and which are (or, row-fused, hold a part) at least MT_WIDE
+//     columns wide: the kernel for tens to hundreds of activation rows takes those parts.  A narrower layer's calls
+//     all run on the row-ordered codes, and a copy nobody reads would double its device memory for nothing
+//     (960 -> 960 or 2560 -> 960: 0.5625 bytes per weight, not 1.06);
+//   - any 4-bit layer of such rows made with NQ_FLAG_PREFER_TILE.
+constexpr int MT_WIDE = 2048;
 bool tile_copy_wanted(const nq_layer* L) {
     if (L->no_tile_copy) return false;
     if ((int64_t)((L->in + 127) / 128 * 128) * ((L->out + 15) / 16 * 16) >= ((int64_t)1 << 32)) return false;  // (32-bit offsets in a tile copy)
     const bool four = L->format == NQ_FMT_Q4_0 || (L->format == NQ_FMT_W4_GROUP && L->group == 128);
-    if (four && L->in % 32 == 0 && L->in >= 512 && L->in <= 6144) return true;
+    if (four && L->in % 32 == 0 && L->in >= 512 && L->in <= 6144) {
+        int widest = L->seg_end.empty() ? L->out : 0;
+        for (size_t i = 0, prev = 0; i < L->seg_end.size(); prev = (size_t)L->seg_end[i], i++)
+            widest = std::max(widest, (int)(L->seg_end[i] - (int32_t)prev));
+        if (L->prefer_tile || widest >= MT_WIDE) return true;
+    }
     if ((int64_t)L->in * L->out < ((int64_t)4 << 20)) return false;
     if (four) return L->in % 128 == 0 && L->in >= 2048 && L->in <= 16384;
     if (L->format == NQ_FMT_W8_CHANNEL) return L->in % 64 == 0 && L->in >= 1024;
@@ -1776,8 +1786,6 @@ static bool mt_shape_ok(const ForwardArgs& a) {
     if (a.x_dtype == NQ_DT_BF16) return true;
     return a.x_dtype == NQ_DT_F32 && L->tile_nj <= 16;
 }
-constexpr int MT_WIDE = 2048;
-
 // What a call of this kernel takes, in microseconds.  Its workgroups (M tiles x column groups, at most one per CU)
 // run in one round and each walks `iters` sets of weight tiles; over IN = 512 .. 6144, OUT = 960 .. 11008 and
 // M = 17 .. 384 (2000 calls) a call took F + iters * q within 4 - 5 % on average, F and q by format, activation type

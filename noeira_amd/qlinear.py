@@ -115,6 +115,11 @@ class _Layer:
                                    _dev_ptr(bias), b_dt, epi, _stream_ptr()))
         return out
 
+    def device_bytes(self) -> int:
+        """Device memory the layer's weights occupy: codes, scales, zero points and every re-ordered copy a kernel
+        reads (nq_device_bytes); 0 before a weight is set."""
+        return int(L.lib().nq_device_bytes(self._h))
+
     def dequantized_dev(self, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """deq(W) [OUT, IN] fp32 on the device (`dequant_q4_0_kernel`, q4_0.mojo:242-266).  Without `out` it is
         written into the buffer handed to `share_scratch`, if any (its first OUT*IN values, returned as a
@@ -378,6 +383,10 @@ class FusedRows:
     `forward` writes one dense [M, OUT_t] output per part, what each part's own
     forward writes, in one launch where the kernel allows it."""
 
+    def device_bytes(self) -> int:
+        """Device memory of the fused copy of the parts' weights (nq_device_bytes); the parts keep their own."""
+        return int(L.lib().nq_device_bytes(self._h))
+
     def __init__(self, layers):
         layers = list(layers)
         arr = (C.c_void_p * len(layers))(*[l._h for l in layers])
@@ -436,6 +445,10 @@ class FusedGLU:
     (noeira/deep_agents/smolvla/fused.mojo:337-353).  `forward` returns up(x) * silu(gate(x)) as [M, OUT];
     with bf16 in and `out_dtype=torch.bfloat16` nothing of the MLP's first half leaves the GPU's registers in
     fp32 (the bf16 flow the reference lists as unbuilt, peft-quant.mdx:215-216)."""
+
+    def device_bytes(self) -> int:
+        """Device memory of the fused copy of the parts' weights (nq_device_bytes); the parts keep their own."""
+        return int(L.lib().nq_device_bytes(self._h))
 
     def __init__(self, gate, up):
         h = C.c_void_p()

@@ -1,6 +1,6 @@
 """The C-ABI shared library on a machine without a GPU: it loads through the
 same dlopen/dlsym mechanics the reference's `OwnedDLHandle.get_function` uses,
-exports every symbol include/noeira_qlinear.h declares, and its host-side
+exports every symbol include/noeira_qlinear.h and include/noeira_qlinear_diag.h declare, and its host-side
 argument checks raise the reference's sentences.  No compute call is made."""
 import ctypes as C
 import os
@@ -15,7 +15,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "noeira_qlinear.h")).read()
+    text = "".join(open(os.path.join(ROOT, "include", f)).read() for f in ("noeira_qlinear.h", "noeira_qlinear_diag.h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(nq_[a-z0-9_]+)\s*\(", text)))
 
@@ -25,7 +25,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     names = declared_symbols()
     assert len(names) >= 19
     for n in names:
-        assert hasattr(lib, n), f"{n} is declared in include/noeira_qlinear.h but not exported"
+        assert hasattr(lib, n), f"{n} is declared in include/ but not exported"
     assert sorted(L.EXPORTS) == names
     assert lib.nq_abi_version() == L.ABI_VERSION
 
@@ -34,7 +34,7 @@ def test_header_is_plain_c(tmp_path):
     """The header compiles as C99 on its own (no C++ or torch types in it)."""
     import subprocess
     src = tmp_path / "t.c"
-    src.write_text('#include "noeira_qlinear.h"\nint main(void){return NQ_ABI_VERSION - 1;}\n')
+    src.write_text('#include "noeira_qlinear.h"\n#include "noeira_qlinear_diag.h"\nint main(void){return NQ_ABI_VERSION - 1;}\n')
     subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"),
                            "-c", str(src), "-o", str(tmp_path / "t.o")])
 

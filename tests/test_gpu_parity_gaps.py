@@ -2,6 +2,7 @@
 bit for bit against the oracle (other tests use it as their reference), the ReLU rule of every kernel family on
 the values that tell its variants apart, the path from a blocks file to a forward, the loaders that take
 `Linear`'s [IN, OUT] parameters, and the shared dequantise scratch."""
+import ctypes as C
 import os
 
 import numpy as np
@@ -374,25 +375,57 @@ def test_stream_read_diagnostic_really_reads():
     assert us < 200
 
 
-def test_a16_shape_switch_changes_no_bits():
-    """nq_diag_a16_shape fixes the tile shape of the 16-row tile kernel for the calls that follow (bench.py times a
-    grid of calls under each shape with it).  A shape decides which workgroup computes an output, not the order of
-    its sum: every shape returns the bits of the library's own choice, for each format and activation type; shapes
-    that do not exist are refused, and (0, 0) gives the choice back."""
+def test_a16_shape_changes_no_bits():
+    """nq_diag_forward_a16 runs one forward on the 16-row tile kernel under a tile shape of the caller's choice
+    (bench.py times a grid of calls under each shape with it).  A shape decides which workgroup computes an output,
+    not the order of its sum: every shape returns the bits of nq_forward's own choice, for each format and
+    activation type; shapes that do not exist are refused, and nothing of the call outlasts it (the forward that
+    follows is the library's own again)."""
     lib = L.lib()
     rng = np.random.default_rng(61)
-    try:
-        for fmt, K, N, M in (("q4_0", 960, 1000, 135), ("w4g", 2560, 520, 40), ("w8", 3200, 512, 100), ("w4g64", 992, 300, 77)):
-            lin = _make(fmt, K, N, rng, False)
-            for xdt in (torch.float32, torch.bfloat16):
-                x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
-                L.check(lib.nq_diag_a16_shape(0, 0))
-                want = lin.forward(x)
-                for mw, nw in ((1, 1), (1, 2), (1, 4), (2, 2), (2, 4)):
-                    L.check(lib.nq_diag_a16_shape(mw, nw))
-                    assert torch.equal(lin.forward(x).view(torch.int32), want.view(torch.int32)), (fmt, xdt, mw, nw)
-        for mw, nw in ((2, 1), (3, 2), (1, 3), (0, 1), (-1, -1)):
-            assert lib.nq_diag_a16_shape(mw, nw) == L.NQ_ERR_INVALID
-            assert "shapes are" in L.last_error()
-    finally:
-        L.check(lib.nq_diag_a16_shape(0, 0))
+    null = C.c_void_p(0)
+    for fmt, K, N, M in (("q4_0", 960, 1000, 135), ("w4g", 2560, 520, 40), ("w8", 3200, 512, 100), ("w4g64", 992, 300, 77)):
+        lin = _make(fmt, K, N, rng, False)
+        for xdt, xc in ((torch.float32, L.DT_F32), (torch.bfloat16, L.DT_BF16)):
+            x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
+            want = lin.forward(x)
+            for mw, nw in ((1, 1), (1, 2), (1, 4), (2, 2), (2, 4)):
+                y = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+                rc = lib.nq_diag_forward_a16(lin._h, C.c_void_p(x.data_ptr()), xc, C.c_void_p(y.data_ptr()), L.DT_F32, M, mw, nw, null)
+                if xdt == torch.float32 and (mw, nw) == (2, 4):
+                    assert rc == L.NQ_ERR_INVALID and "shapes are" in L.last_error()
+                    continue
+                L.check(rc)
+                assert torch.equal(y.view(torch.int32), want.view(torch.int32)), (fmt, xdt, mw, nw)
+            assert torch.equal(lin.forward(x).view(torch.int32), want.view(torch.int32))
+    x = torch.zeros((4, 960), dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((4, 1000), dtype=torch.float32, device="cuda")
+    lin = _make("q4_0", 960, 1000, rng, False)
+    for mw, nw in ((2, 1), (3, 2), (1, 3), (0, 1), (-1, -1), (0, 0)):
+        assert lib.nq_diag_forward_a16(lin._h, C.c_void_p(x.data_ptr()), L.DT_BF16, C.c_void_p(y.data_ptr()), L.DT_F32, 4, mw, nw, null) == L.NQ_ERR_INVALID
+        assert "shapes are" in L.last_error()
+    assert lib.nq_diag_forward_a16(lin._h, C.c_void_p(x.data_ptr()), L.DT_BF16, C.c_void_p(y.data_ptr()), L.DT_F32, 1, 1, 1, null) == L.NQ_ERR_UNSUPPORTED
+
+
+def test_device_bytes_one_copy_where_no_kernel_reads_a_second():
+    """`keep_only_repacked` keeps exactly one device copy of the weights in the reference (qlinear.mojo:342-356; "int4
+    buys memory", docs-site/src/content/docs/nn/peft-quant.mdx:194-199).  Here a second, tile-ordered copy exists only
+    where a kernel of the default dispatch reads it: nq_device_bytes bounds it.  The narrow SmolVLA projections
+    (q, k, v, o, down) hold 0.5625 bytes per weight, the wide ones (gate, up: the M-tile kernel's) 1.16 (IN = 960 pads to 1024 in tile order) unless made
+    with NQ_FLAG_NO_TILE_COPY; the forward's bits do not depend on keep_only_repacked."""
+    rng = np.random.default_rng(77)
+    for K, N, wide in ((960, 960, False), (960, 320, False), (2560, 960, False), (960, 2560, True)):
+        lin = _make("q4_0", K, N, rng, True)
+        x = torch.from_numpy(rng.standard_normal((135, K)).astype(np.float32)).cuda()
+        before = {T: lin.forward(x[:T]).clone() for T in (135, 16, 7, 1)}
+        per_weight = lin.device_bytes() / (K * N)
+        assert (1.0 < per_weight < 1.17) if wide else (0.5625 <= per_weight <= 0.60), (K, N, per_weight)
+        lin.keep_only_repacked()
+        assert lin.device_bytes() / (K * N) == per_weight
+        for T, want in before.items():
+            assert torch.equal(lin.forward(x[:T]).view(torch.int32), want.view(torch.int32)), (K, N, T)
+        lean = _make("q4_0", K, N, rng, False)  # NQ_FLAG_NO_TILE_COPY
+        assert 0.5625 <= lean.device_bytes() / (K * N) <= 0.60
+    assert QLinear(960, 320).device_bytes() == 0  # nothing loaded
+    w8 = _make("w8", 3200, 512, rng, True)
+    assert 1.0 <= w8.device_bytes() / (3200 * 512) <= 1.01
