@@ -4,24 +4,25 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--no-sweep]
 
 Prints ONE JSON line.  Configs are numbered 1 .. 5 as BASELINE.md numbers them (config n is
-BASELINE.json's configs[n - 1]).  The headline workload is config 2 at M = 1: the ACT-style policy MLP's two W8A16 linears (512 -> 3200 and
-3200 -> 512, bf16 activations, int8 weights with per-channel fp32 scales, bf16
-bias, fp32 output).  A step is one pass over both linears.  Weights, inputs
-and outputs are resident in HBM before the timed region.  Because a 1.6 MB
-weight sits in the 256 MB Infinity Cache, the step rotates through enough
-distinct copies of the two layers (>= 512 MB) that every call streams from
-HBM ("cold"); the warm figure (one copy, the reference's own protocol,
-benchmarks/quant/bench_qlinear_smolvla.mojo:37-38,89-137) is reported beside
-it.  `value` is algorithmic GB/s: every operand counted once (weights, scales,
-bias, x, y), no scratch, no padding.
+BASELINE.json's configs[n - 1]).  The headline workload is the largest single-GPU M = 1 configuration, config 5's
+GEMV: e4m3 weights [11008, 4096] with a per-tensor scale under one e4m3 activation row, fp32 accumulate, bf16
+out - 45 MB per launch, the size at which a fraction of the HBM roofline means something (config 2's 1.66 MB
+layers are launch-bound by construction and stay a row of `results`).  A step is one launch.  Weights, inputs
+and outputs are resident in HBM before the timed region; the step rotates through enough distinct copies of
+the layer (>= 512 MB) that every call streams from HBM ("cold").  `value` is algorithmic GB/s: every operand
+counted once (weights, scale, x, y), no scratch, no padding.
 
-`results` carries every other BASELINE config measured with the reference's
-protocol (warm-up, 7 samples of N calls between two synchronisations, median
-sample / N), each with its own roofline fraction; `roofline` is the headline
-workload's kernel, and its `m4096` entry the metric's other half (config 4, the
-batched-env actor at M = 4096, in TOPS); `roofline_mfma` is the large-M fp8 GEMM
-(config 5) beside what the matrix cores alone sustain on the same GPU
-(`mfma_only`: back-to-back MFMAs on register operands, constant and random data).
+`results` carries every BASELINE config measured with the reference's protocol (warm-up, 7 samples of N calls
+between two synchronisations, median sample / N; benchmarks/quant/bench_qlinear_smolvla.mojo:37-38,89-137), each
+with its own roofline fraction.  The warm-up is 50 ms of replays (the matrix-core-bound calls need 30 - 40 ms
+after an idle spell to reach their steady rate); the large matrix-core-bound rows also carry the figure taken
+the reference's way, after ONE warm call (`us_per_call_one_warm_call`), so that a kernel's gain can be told from
+the warm-up's.  `roofline` is the headline kernel, with `frac` from the HIP events of this run and
+`frac_profiled` from the kernel's average duration in the committed rocprofv3 trace of the same loop (the
+profiler brackets every dispatch, so its per-kernel time is the longer one); `roofline_m4096` is the metric's
+other half (config 4, the batched-env actor at M = 4096, in TOPS); `roofline_mfma` the large-M fp8 GEMM (config
+5) under both protocols, beside what the matrix cores alone sustain on the same GPU (`mfma_only`: back-to-back
+MFMAs on register operands, constant and random data, both MFMA shapes).
 
 `--only a16_shapes --a16-class C` re-derives the constants by which the library picks the tile shape of its
 kernel for tens to hundreds of activation rows (a grid of calls timed under each shape, nq_diag_forward_a16);
@@ -52,9 +53,13 @@ SAMPLES, COLD_BYTES = 7, 512 << 20
 SETTLE_S = 0.05  # warm-up replays before the samples of a row (see median_per_call)
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (fetched + written), scaled by
 # what the same counters read for a plain copy of known size; None until measured
-HEADLINE_TRAFFIC = 1804544      # mean of the two linears' launches (1.66 MB algorithmic)
+HEADLINE_TRAFFIC = 1804544      # config 2's pair: mean of the two linears' launches (1.66 MB algorithmic)
 FP8_GEMV_TRAFFIC = 45185024     # K=4096, N=11008 (45.09 MB algorithmic)
 FP8_GEMM_TRAFFIC = 269343334    # M=8192, K=4096, N=4096 (117.4 MB algorithmic; the re-reads hit the Infinity Cache)
+# average kernel durations of the committed rocprofv3 kernel traces of the same loops (profiles/), nanoseconds: what
+# `frac_profiled` is computed from.  The profiler brackets every dispatch, so these run longer than the un-profiled
+# launches timed here; a reader can hold either against the other.
+PROFILED_NS = {"fp8_gemv_11008": 8902.0, "fp8_gemm_4096": 109100.0, "actor_fused": None}
 
 
 def ensure_built():
@@ -109,6 +114,22 @@ def capture(fn, n):
         for i in range(n):
             fn(i)
     return g
+
+
+def median_both(fn, calls):
+    """(one warm call then the samples - the reference's own protocol -, the same after SETTLE_S of replays):
+    seconds per call each.  The first is taken right after the workload was built, i.e. after an idle spell."""
+    import torch
+
+    tm = Timer()
+    g = capture(fn, calls)  # (capture makes the one warm call)
+    ref = statistics.median([tm.run(lambda i: g.replay(), 1) / calls for _ in range(SAMPLES)])
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < SETTLE_S:
+        g.replay()
+        torch.cuda.synchronize()
+    settled = statistics.median([tm.run(lambda i: g.replay(), 1) / calls for _ in range(SAMPLES)])
+    return ref, settled
 
 
 def median_per_call(fn, calls, graph=True):
@@ -481,22 +502,25 @@ def mfma_only(iters=4096, reps=5):
     stamps = torch.zeros((wgs, 2), dtype=torch.int64, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = []
+    names = {0: "v_mfma_f32_32x32x64_f8f6f4", 1: "v_mfma_i32_32x32x32_i8", 2: "v_mfma_f32_16x16x128_f8f6f4 (the GEMM's)",
+             3: "v_mfma_i32_16x16x64_i8 (the GEMM's)"}
+    ops_per_iter = {0: 16 * 131072, 1: 16 * 65536, 2: 64 * 65536, 3: 64 * 32768}
     for (kind, what), d in data.items():
-        k = 0 if kind == "fp8" else 1
+        for k in ((0, 2) if kind == "fp8" else (1, 3)):
+            its = iters if k < 2 else iters // 2  # (the 16 x 16 kernels issue twice the operations per iteration)
 
-        def go(_i=0):
-            L.check(lib.nq_diag_mfma_rate(k, C.c_void_p(d.data_ptr()), d.numel(), iters, wgs, C.c_void_p(stamps.data_ptr()), stream))
+            def go(_i=0):
+                L.check(lib.nq_diag_mfma_rate(k, C.c_void_p(d.data_ptr()), d.numel(), its, wgs, C.c_void_p(stamps.data_ptr()), stream))
 
-        t0 = time.perf_counter()
-        while time.perf_counter() - t0 < 2 * SETTLE_S:  # (steady clocks: see median_per_call)
-            go()
-            torch.cuda.synchronize()
-        sec = Timer().run(go, reps) / reps
-        ops = wgs * 4 * iters * 16 * (131072 if k == 0 else 65536)
-        st = stamps.cpu().numpy().astype(np.float64)
-        out.append({"mfma": "v_mfma_f32_32x32x64_f8f6f4" if k == 0 else "v_mfma_i32_32x32x32_i8", "operands": what,
-                    "TOPS": round(ops / sec / 1e12, 1), "shader_clock_GHz": round(st[:, 0].mean() / (st[:, 1].mean() * 10.0), 3),
-                    "cycles_per_mfma": round(st[:, 0].mean() / (iters * 16), 2), "workgroups": wgs})
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < 2 * SETTLE_S:  # (steady clocks: see median_per_call)
+                go()
+                torch.cuda.synchronize()
+            sec = Timer().run(go, reps) / reps
+            ops = wgs * 4 * its * ops_per_iter[k]
+            st = stamps.cpu().numpy().astype(np.float64)
+            out.append({"mfma": names[k], "operands": what, "TOPS": round(ops / sec / 1e12, 1),
+                        "shader_clock_GHz": round(st[:, 0].mean() / (st[:, 1].mean() * 10.0), 3), "workgroups": wgs})
     return out
 
 
@@ -573,7 +597,7 @@ def make_read(nbytes, copies):
     return dict(step=step, bytes=nbytes, ops=0, launches=1, keep=(buf,))
 
 
-def report(name, wl, seconds, bound, peak_key=None):
+def report(name, wl, seconds, bound, peak_key=None, seconds_ref=None):
     gbps = wl["bytes"] / seconds / 1e9
     tops = wl["ops"] / seconds / 1e12
     r = {"workload": name, "us_per_call": round(seconds * 1e6, 3), "GBps": round(gbps, 2), "TOPS": round(tops, 4),
@@ -582,6 +606,9 @@ def report(name, wl, seconds, bound, peak_key=None):
         r["frac_of_roofline"] = round(gbps / HBM_PEAK_GBPS, 4)
     else:
         r["frac_of_roofline"] = round(tops / MFMA_PEAK_TOPS[peak_key], 4)
+    if seconds_ref is not None:  # the reference's protocol: samples right after one warm call
+        r["us_per_call_one_warm_call"] = round(seconds_ref * 1e6, 3)
+        r["frac_of_roofline_one_warm_call"] = round(wl["ops"] / seconds_ref / 1e12 / MFMA_PEAK_TOPS[peak_key], 4)
     return r
 
 
@@ -591,7 +618,7 @@ def sweep(skip_large=False):
 
     out = []
 
-    def run(name, maker, bound, peak_key=None, calls=50, **kw):
+    def run(name, maker, bound, peak_key=None, calls=50, both=False, **kw):
         wl = maker(**kw)
         copies = kw.get("copies", 1)
         # a replay is timed from the host's launch of the graph: with fewer than ~60 calls in it that start-up
@@ -600,12 +627,19 @@ def sweep(skip_large=False):
         n = max(calls, copies)
         if copies > 1:
             n = copies * max(1, -(-60 // copies))
-        t = median_per_call(wl["step"], n)
-        out.append(report(name, wl, t, bound, peak_key))
+        if both:
+            t_ref, t = median_both(wl["step"], n)
+            out.append(report(name, wl, t, bound, peak_key, t_ref))
+        else:
+            t = median_per_call(wl["step"], n)
+            out.append(report(name, wl, t, bound, peak_key))
         del wl
         torch.cuda.empty_cache()
 
     run("cfg1 W8A32 256->256 M=1 (warm)", make_w8a32, "hbm")
+    c2 = -(-COLD_BYTES // (2 * 512 * 3200))
+    run("cfg2 W8A16 ACT MLP pair M=1 (cold, two launches per call)", make_act_w8a16, "hbm", M=1, copies=c2, calls=c2)
+    run("cfg2 W8A16 ACT MLP pair M=1 (warm: one copy, resident in L2 / Infinity Cache)", make_act_w8a16, "hbm", M=1, copies=1, calls=200)
     run("cfg2 W8A16 ACT MLP M=100 (warm)", make_act_w8a16, "hbm", M=100, copies=1)
     for (K, N) in [(960, 960), (960, 2560), (2560, 960)]:
         c = max(1, COLD_BYTES // (N * K // 2))
@@ -639,12 +673,12 @@ def sweep(skip_large=False):
         c = max(1, COLD_BYTES // (N * 4096))
         run(f"cfg5 fp8 GEMV K=4096 N={N} M=1 (cold)", make_fp8, "hbm", M=1, N=N, copies=c, calls=max(c, 20))
         if not skip_large:
-            run(f"cfg5 fp8 GEMM M=8192 K=4096 N={N}", make_fp8, "mfma", "fp8", M=8192, N=N, copies=1, calls=10)
+            run(f"cfg5 fp8 GEMM M=8192 K=4096 N={N}", make_fp8, "mfma", "fp8", M=8192, N=N, copies=1, calls=10, both=True)
     if not skip_large:
         run("W8A8 int8 GEMM M=8192 K=4096 N=4096 (scales + bias epilogue, bf16 out)", make_w8a8_gemm, "mfma", "int8",
-            M=8192, N=4096, calls=10)
+            M=8192, N=4096, calls=10, both=True)
         # thousands of rows with 16-bit activations (prefill over a 4-bit or 8-bit weight)
-        run("W4A16 g128 M=4096 K=4096 N=4096 (warm)", make_w4g, "mfma", "bf16", K=4096, N=4096, M=4096, copies=1, calls=10)
+        run("W4A16 g128 M=4096 K=4096 N=4096 (warm)", make_w4g, "mfma", "bf16", K=4096, N=4096, M=4096, copies=1, calls=10, both=True)
         run("ref Q4_0 g32 960->2560 M=4096 fp32 (warm)", make_q4_0, "mfma", "bf16", IN=960, OUT=2560, M=4096, copies=1,
             calls=10)
         c8 = max(1, COLD_BYTES // (4096 * 11008))
@@ -697,6 +731,10 @@ def only_loop(which, steps, warmup):
         dst = torch.empty_like(src)
         wl = dict(step=lambda i: dst.copy_(src), bytes=2 * n, ops=0, keep=(src, dst))
         name = "plain device copy, 256 MiB read + 256 MiB written"
+    elif which == "act":
+        c = -(-COLD_BYTES // (2 * 512 * 3200))
+        wl = make_act_w8a16(1, c)
+        name = f"cfg2 W8A16 ACT MLP pair M=1, cold rotation over {c} copies of the two layers"
     elif which == "fp8gemv":
         N = 11008
         c = max(1, COLD_BYTES // (N * 4096))
@@ -786,23 +824,24 @@ def only_loop(which, steps, warmup):
 
 
 def cpu_baseline(budget_s=12.0):
-    """The oracle's restatement of the reference's CPU forward, one core, on the
-    headline workload's two linears (M = 1) for about `budget_s` seconds."""
+    """The oracle's restatement of the reference's CPU forward, one core, on the headline workload (config 5's GEMV:
+    e4m3 weights [11008, 4096] under one e4m3 row) for about `budget_s` seconds: a fresh dequantize of the weight to
+    an fp32 [OUT, IN] scratch, then the serial triple loop."""
     import numpy as np
+    import torch
 
     from oracle import oracle as O
 
     rng = np.random.default_rng(2)
-    dims = [(512, 3200), (3200, 512)]
-    ws = [(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32)) for K, N in dims]
-    xs = [bf16_t(rng.standard_normal((1, K))).float().numpy() for K, _ in dims]
-    bs = [bf16_t(rng.standard_normal(N) * 0.02).float().numpy() for _, N in dims]
-    nbytes = sum(N * K + 4 * N + 2 * N + 2 * K + 4 * N for K, N in dims)
-    O.w8_qlinear_forward_cpu(ws[0][0], ws[0][1], xs[0], bs[0])
+    K, N = 4096, 11008
+    g = torch.Generator().manual_seed(6)
+    w = torch.randn((N, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    x = torch.randn((1, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    nbytes = N * K + K + 2 * N + 8
+    O.fp8_qlinear_forward_cpu(w, 1.0 / 16, x, 1.0 / 16)
     n, t0 = 0, time.perf_counter()
     while True:
-        for (w, s), x, b in zip(ws, xs, bs):
-            O.w8_qlinear_forward_cpu(w, s, x, b)
+        O.fp8_qlinear_forward_cpu(w, 1.0 / 16, x, 1.0 / 16)
         n += 1
         dt = time.perf_counter() - t0
         if dt >= budget_s and n >= 3:
@@ -822,8 +861,8 @@ def cpu_baseline(budget_s=12.0):
             q4.append({"layer": f"Q4_0 {IN}->{OUT}", "M": M, "ms_per_call": round((time.perf_counter() - t1) / calls * 1e3, 3)})
     return {"value": round(nbytes * n / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "ms_per_step": round(dt / n * 1e3, 3), "q4_0_reference_shapes": q4,
-            "sample": f"{n} steps of the headline workload (both W8 linears at M=1): a fresh dequantize to an "
-                      f"fp32 [OUT, IN] scratch then the serial triple loop, single thread, {dt:.1f} s"}
+            "sample": f"{n} steps of the headline workload (e4m3 [11008, 4096] under one e4m3 row): a fresh dequantize to "
+                      f"an fp32 [OUT, IN] scratch then the serial triple loop, single thread, {dt:.1f} s"}
 
 
 def a16_shapes(cls="w4g"):
@@ -970,9 +1009,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline", "a16_shapes", "mid_dispatch"],
-                    help="run one loop only and print a short JSON line (for rocprofv3 runs): act = the "
-                         "headline loop, fp8gemv / fp8gemm = config 5 at N=11008 / N=4096, mid = the M=100..256 "
+    ap.add_argument("--only", default="", choices=["", "headline", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline", "a16_shapes", "mid_dispatch"],
+                    help="run one loop only and print a short JSON line (for rocprofv3 runs): headline = the "
+                         "headline line alone (graph replays), act = config 2's pair of linears at M=1, fp8gemv / fp8gemm = "
+                         "config 5 at N=11008 (the headline's kernel, launched call by call) / N=4096, mid = the M=100..256 "
                          "calls of configs 1, 2 and the reference's T=135 shapes, actor = config 3 fused, "
                          "copy = a plain 256 MiB device copy (the counter calibration kernel), biggemv / smallm = the "
                          "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, hugegemv = the two 4-bit layers at 8192->28672, M=1, tile8 = int8 and fp8 "
@@ -1008,20 +1048,22 @@ def main():
             sys.exit("bench.py: --only mid_dispatch is about the 4-bit formats (--a16-class q4, q4f, w4g or w4gf)")
         print(json.dumps(mid_dispatch(a.a16_class)))
         return
-    if a.only in ("fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"):
+    if a.only in ("act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 
-    per_pair = 2 * 512 * 3200
-    copies = -(-COLD_BYTES // per_pair)
-    wl = make_act_w8a16(1, copies)
+    # ---- headline: config 5's GEMV, e4m3 x e4m3, K = 4096, N = 11008, M = 1, every call from HBM
+    K_H, N_H = 4096, 11008
+    copies = max(1, -(-COLD_BYTES // (N_H * K_H)))
+    wl = make_fp8(1, N_H, K=K_H, copies=copies)
     tm = Timer()
     for i in range(a.warmup):
         wl["step"](i)
-    # The timed region is EXACTLY a.steps steps.  They are replayed from a HIP graph holding g
-    # consecutive steps of the rotation (g = the largest divisor of steps that is <= the number
-    # of weight copies), a.steps / g replays back to back, bracketed by synchronisations.
-    g_steps = max(d for d in range(1, min(a.steps, copies) + 1) if a.steps % d == 0)
+    # The timed region is EXACTLY a.steps steps.  They are replayed from a HIP graph holding g consecutive steps
+    # of the rotation (g = the largest divisor of steps that is <= 200: a replay is timed from the host's launch of
+    # the graph, and in a graph of a dozen calls that start-up is a visible share of every call), a.steps / g
+    # replays back to back, bracketed by synchronisations.  The events sit on the stream the kernels run on.
+    g_steps = max(d for d in range(1, min(a.steps, 200) + 1) if a.steps % d == 0)
     if a.only and a.eager:
         sec = tm.run(wl["step"], a.steps)
     else:
@@ -1029,38 +1071,38 @@ def main():
         graph.replay()
         sec = tm.run(lambda i: graph.replay(), a.steps // g_steps)
     ms_per_step = sec / a.steps * 1e3
-    value = wl["bytes"] / (sec / a.steps) / 1e9
-    launch_s = sec / (a.steps * wl["launches"])
-    achieved = (wl["bytes"] / wl["launches"]) / launch_s / 1e9
+    launch_s = sec / a.steps
+    value = wl["bytes"] / launch_s / 1e9
     eager_sec = tm.run(wl["step"], a.steps)
-
-    warm = make_act_w8a16(1, 1)
-    warm_s = median_per_call(warm["step"], 200)
+    prof = PROFILED_NS["fp8_gemv_11008"]
 
     line = {
         "metric": "qlinear GB/s at M=1 and TOPS at M=4096, as % of MI355X roofline",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "BASELINE config 2 (configs[1]), ACT-style policy MLP W8A16 at M=1: linears 512->3200 and "
-                               "3200->512, int8 weights + per-channel fp32 scales, bf16 x, bf16 bias, fp32 y; "
-                               f"cold: rotating over {copies} distinct weight copies ({copies * per_pair >> 20} MiB); "
-                               f"launched as HIP-graph replays of {g_steps} steps",
-                   "arithmetic": "int8 codes and bf16 activations widened to fp32, fp32 products and sums",
-                   "algorithmic_bytes_per_step": wl["bytes"], "launches_per_step": wl["launches"]},
+        "config": {"workload": "BASELINE config 5 (configs[4]) at M=1, the largest single-GPU M=1 configuration: fp8 e4m3 "
+                               f"weights [{N_H}, {K_H}] with a per-tensor fp32 scale under one e4m3 activation row, fp32 "
+                               f"accumulate, bf16 out; cold: rotating over {copies} distinct weight copies "
+                               f"({copies * N_H * K_H >> 20} MiB); launched as HIP-graph replays of {g_steps} steps",
+                   "arithmetic": "e4m3 x e4m3 products on the fp8 matrix cores, fp32 sums",
+                   "algorithmic_bytes_per_step": wl["bytes"], "launches_per_step": 1},
         "pct_of_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 3),
         "eager": {"GBps": round(wl["bytes"] * a.steps / eager_sec / 1e9, 2),
                   "us_per_step": round(eager_sec / a.steps * 1e6, 3),
                   "note": "the same steps launched one by one from Python through ctypes (host-bound)"},
-        "warm": {"GBps": round(warm["bytes"] / warm_s / 1e9, 2), "us_per_step": round(warm_s * 1e6, 3),
-                 "note": "one weight copy, resident in L2 / Infinity Cache (the reference's protocol)"},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 5), "traffic": HEADLINE_TRAFFIC,
-                     "kernel": "nq::gemv_m1_kernel<W8_CHANNEL>", "avg_launch_us": round(launch_s * 1e6, 3),
-                     "note": "1.66 MB per launch: at 8 TB/s the transfer is 0.21 us, less than the 1.4 us an "
-                             "empty kernel takes on this GPU, so this workload is launch-latency-bound; the "
-                             "HBM-bound GEMV figures are the config-5 rows of `results`"},
+        "roofline": {"bound": "hbm", "achieved": round(value, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(value / HBM_PEAK_GBPS, 5), "traffic": FP8_GEMV_TRAFFIC,
+                     "kernel": "nq::gemv8_row_kernel<fp8>", "avg_launch_us": round(launch_s * 1e6, 3),
+                     "frac_profiled": round(wl["bytes"] / (prof * 1e-9) / 1e9 / HBM_PEAK_GBPS, 5) if prof else None,
+                     "profiled_avg_kernel_ns": prof,
+                     "note": "frac: algorithmic bytes / this run's launch time (HIP events around graph replays); "
+                             "frac_profiled: the same bytes / the kernel's average duration in the committed rocprofv3 "
+                             "kernel trace of `bench.py --only fp8gemv` (launched call by call under the profiler, which "
+                             "brackets every dispatch)"},
     }
+    del wl
+    torch.cuda.empty_cache()
     if a.only:
         print(json.dumps(line))
         return
@@ -1069,30 +1111,31 @@ def main():
     actor = make_actor_fused()
     actor_s = median_per_call(actor["step"], 20)
     actor_tops = actor["ops"] / actor_s / 1e12
-    line["roofline"]["m4096"] = {"workload": "BASELINE config 4 (configs[3]): W8A8 actor 64->256->256->8, M=4096, one fused launch",
-                                 "kernel": "nq::mlp3_w8a8_kernel", "us_per_call": round(actor_s * 1e6, 3),
-                                 "bound": "mfma", "achieved": round(actor_tops, 3), "peak": MFMA_PEAK_TOPS["int8"],
-                                 "unit": "TOP/s", "frac": round(actor_tops / MFMA_PEAK_TOPS["int8"], 5),
-                                 "note": "launch- and latency-bound by construction (see results for the MFMA-bound GEMMs)"}
+    line["roofline_m4096"] = {"workload": "BASELINE config 4 (configs[3]): W8A8 actor 64->256->256->8, M=4096, one fused launch",
+                              "kernel": "nq::mlp3_w8a8_kernel", "us_per_call": round(actor_s * 1e6, 3),
+                              "bound": "mfma", "achieved": round(actor_tops, 3), "peak": MFMA_PEAK_TOPS["int8"],
+                              "unit": "TOP/s", "frac": round(actor_tops / MFMA_PEAK_TOPS["int8"], 5),
+                              "note": "launch- and latency-bound by construction (see results for the MFMA-bound GEMMs)"}
     del actor
     if not a.no_sweep:
         line["results"] = sweep()
         mf = [r for r in line["results"] if "fp8 GEMM" in r["workload"]]
         if mf:
             best = next((r for r in mf if "N=4096" in r["workload"]), mf[0])  # the shape the traffic figure is for
+            pg = PROFILED_NS["fp8_gemm_4096"]
             line["roofline_mfma"] = {"bound": "mfma", "achieved": best["TOPS"], "peak": MFMA_PEAK_TOPS["fp8"],
                                      "unit": "TFLOP/s", "frac": round(best["TOPS"] / MFMA_PEAK_TOPS["fp8"], 5),
+                                     "frac_one_warm_call": best.get("frac_of_roofline_one_warm_call"),
+                                     "frac_profiled": round(2 * 8192 * 4096 * 4096 / (pg * 1e-9) / 1e12 / MFMA_PEAK_TOPS["fp8"], 5) if pg else None,
+                                     "profiled_avg_kernel_ns": pg,
                                      "traffic": FP8_GEMM_TRAFFIC, "kernel": "nq::gemm8_kernel<fp8>",
                                      "workload": best["workload"], "avg_launch_us": best["us_per_call"],
+                                     "avg_launch_us_one_warm_call": best.get("us_per_call_one_warm_call"),
+                                     "note": "frac: after 50 ms of the same launches (steady clocks); frac_one_warm_call: the "
+                                             "reference's protocol, samples right after one warm call (the power "
+                                             "management's transient after an idle spell); frac_profiled: from the committed "
+                                             "rocprofv3 trace of a long run of `bench.py --only fp8gemm`",
                                      "mfma_only": mfma_only()}
-        gv = [r for r in line["results"] if "cfg5 fp8 GEMV" in r["workload"]]
-        if gv:
-            # config 5's own GEMV (N = 11008: the shape the traffic figure was counted on); the 235 MB rows of
-            # `results` show the same kernel where a call's fixed part no longer counts
-            best = next((r for r in gv if "N=11008" in r["workload"]), gv[0])
-            line["roofline_gemv"] = {"bound": "hbm", "achieved": best["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                                     "frac": round(best["GBps"] / HBM_PEAK_GBPS, 5), "traffic": FP8_GEMV_TRAFFIC,
-                                     "kernel": "nq::gemv8_row_kernel<fp8>", "workload": best["workload"]}
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

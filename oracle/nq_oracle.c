@@ -793,3 +793,27 @@ int nqo_w8_qlinear_forward_cpu(const int8_t* w, const float* s, int64_t N, int64
     free(deq);
     return NQO_OK;
 }
+
+/* The reference's CPU forward (qlinear.mojo:416-426: a FRESH dequantize to an fp32 [OUT, IN] scratch, then the
+ * serial gemm_cpu) restated for an e4m3 weight under e4m3 activations with per-tensor scales: deq[n,k] =
+ * decode(w[n,k]) * sb, x decoded and scaled by sa, y = x @ deq^T in fp32, then rounded to bf16 (config 5's
+ * output type; out_bf16 may be NULL).  Used as the single-core CPU baseline of the fp8 workloads; pinned against
+ * nqo_fp8_forward_f64 and exact small-integer products in tests/test_oracle_ext.py. */
+int nqo_fp8_qlinear_forward_cpu(const uint8_t* w, float sb, int64_t N, int64_t K, const uint8_t* a, float sa,
+                                int64_t M, float* y, uint16_t* out_bf16) {
+    float* deq = (float*)malloc(sizeof(float) * (size_t)(N * K));
+    float* xs = (float*)malloc(sizeof(float) * (size_t)(M * K));
+    if (!deq || !xs) {
+        free(deq);
+        free(xs);
+        return NQO_ENOMEM;
+    }
+    for (int64_t i = 0; i < N * K; i++) deq[i] = nqo_e4m3_decode(w[i]) * sb;
+    for (int64_t i = 0; i < M * K; i++) xs[i] = nqo_e4m3_decode(a[i]) * sa;
+    nqo_gemm_cpu(0, 1, M, N, K, 1.0f, xs, K, deq, K, 0.0f, y, N);
+    if (out_bf16)
+        for (int64_t i = 0; i < M * N; i++) out_bf16[i] = nqo_f32_to_bf16_bits(y[i]);
+    free(deq);
+    free(xs);
+    return NQO_OK;
+}

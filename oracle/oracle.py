@@ -98,6 +98,8 @@ def lib() -> C.CDLL:
         L.nqo_e4m3_encode.argtypes = [f32]
         L.nqo_fp8_forward_f64.restype = None
         L.nqo_fp8_forward_f64.argtypes = [p, p, i64, i64, i64, f32, f32, p, p]
+        L.nqo_fp8_qlinear_forward_cpu.restype = C.c_int
+        L.nqo_fp8_qlinear_forward_cpu.argtypes = [p, f32, i64, i64, p, f32, i64, p, p]
         L.nqo_e4m3_dequantize.restype = None
         L.nqo_e4m3_dequantize.argtypes = [p, i64, p]
         L.nqo_w8_qlinear_forward_cpu.restype = C.c_int
@@ -492,3 +494,17 @@ def fp8_forward_f64(a, b, sa, sb, want_bf16=True):
     ob = np.empty((M, N), np.uint16) if want_bf16 else None
     lib().nqo_fp8_forward_f64(_ptr(a), _ptr(b), M, N, K, sa, sb, _ptr(y64), _ptr(ob))
     return y64, ob
+
+
+def fp8_qlinear_forward_cpu(w, sb, a, sa, want_bf16=False):
+    """Dequantize-to-scratch then serial GEMM, as QLinear.forward["cpu"] does, for e4m3 weights and activations."""
+    w = _c(w, np.uint8)
+    a = _c(a, np.uint8)
+    N, K = w.shape
+    M = a.size // K
+    y = np.empty((M, N), np.float32)
+    ob = np.empty((M, N), np.uint16) if want_bf16 else None
+    rc = lib().nqo_fp8_qlinear_forward_cpu(_ptr(w), sb, N, K, _ptr(a), sa, M, _ptr(y), _ptr(ob))
+    if rc:
+        raise MemoryError("fp8_qlinear_forward_cpu")
+    return (y, ob) if want_bf16 else y

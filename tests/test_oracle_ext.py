@@ -261,3 +261,30 @@ def test_swiglu_is_u_times_v_sigmoid_v():
     s32 = np.float32(1) / (np.float32(1) + np.exp(-v).astype(np.float32))
     regroup = (u * v) * s32
     assert np.abs(got - regroup).max() <= 2e-7 * np.abs(want).max()
+
+
+def test_fp8_cpu_forward_restatement_pinned():
+    """`fp8_qlinear_forward_cpu` (the CPU baseline bench.py times: dequantize to an fp32 scratch, then the serial
+    gemm_cpu, qlinear.mojo:416-426 / cpu_gemm.mojo:88-98, for e4m3 operands) against what fixes it: small-integer
+    codes whose products and sums are exact in fp32 (so any order of summation gives the same bits as numpy's integer
+    matmul), and the fp64 forward on random codes within fp32 summation error; a transposed operand or a dropped
+    scale fails both."""
+    rng = np.random.default_rng(5)
+    table = O.e4m3_decode_table()
+    ints = np.array([c for c in range(256) if np.isfinite(table[c]) and table[c] == np.round(table[c]) and abs(table[c]) <= 8], np.uint8)
+    M, N, K = 3, 7, 64
+    a = ints[rng.integers(0, len(ints), (M, K))]
+    w = ints[rng.integers(0, len(ints), (N, K))]
+    y = O.fp8_qlinear_forward_cpu(w, 2.0, a, 0.5)
+    want = (table[a].astype(np.int64) @ table[w].astype(np.int64).T).astype(np.float32)  # 2.0 * 0.5 = 1
+    assert np.array_equal(y, want)
+    # random codes (NaN codes excluded), scales that are not powers of two
+    codes = np.array([c for c in range(256) if np.isfinite(table[c])], np.uint8)
+    M, N, K = 2, 33, 4096
+    a = codes[rng.integers(0, len(codes), (M, K))]
+    w = codes[rng.integers(0, len(codes), (N, K))]
+    sa, sb = 0.013, 0.07
+    y, ob = O.fp8_qlinear_forward_cpu(w, sb, a, sa, want_bf16=True)
+    y64, _ = O.fp8_forward_f64(a, w, sa, sb, want_bf16=False)
+    assert np.abs(y - y64).max() <= 2e-5 * np.abs(y64).max()
+    assert np.array_equal(ob, O.bf16_bits(y))
