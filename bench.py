@@ -54,12 +54,12 @@ SETTLE_S = 0.05  # warm-up replays before the samples of a row (see median_per_c
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (fetched + written), scaled by
 # what the same counters read for a plain copy of known size; None until measured
 HEADLINE_TRAFFIC = 1804544      # config 2's pair: mean of the two linears' launches (1.66 MB algorithmic)
-FP8_GEMV_TRAFFIC = 45185024     # K=4096, N=11008 (45.09 MB algorithmic)
-FP8_GEMM_TRAFFIC = 269343334    # M=8192, K=4096, N=4096 (117.4 MB algorithmic; the re-reads hit the Infinity Cache)
+FP8_GEMV_TRAFFIC = 45199360     # K=4096, N=11008 (45.11 MB algorithmic)
+FP8_GEMM_TRAFFIC = 269149440    # M=8192, K=4096, N=4096 (117.4 MB algorithmic; the re-reads hit the Infinity Cache)
 # average kernel durations of the committed rocprofv3 kernel traces of the same loops (profiles/), nanoseconds: what
 # `frac_profiled` is computed from.  The profiler brackets every dispatch, so these run longer than the un-profiled
 # launches timed here; a reader can hold either against the other.
-PROFILED_NS = {"fp8_gemv_11008": 8902.0, "fp8_gemm_4096": 109100.0, "actor_fused": None}
+PROFILED_NS = {"fp8_gemv_11008": 8795.1, "fp8_gemm_4096": 100250.0, "actor_fused": 8006.7}
 
 
 def ensure_built():
@@ -1115,6 +1115,8 @@ def main():
                               "kernel": "nq::mlp3_w8a8_kernel", "us_per_call": round(actor_s * 1e6, 3),
                               "bound": "mfma", "achieved": round(actor_tops, 3), "peak": MFMA_PEAK_TOPS["int8"],
                               "unit": "TOP/s", "frac": round(actor_tops / MFMA_PEAK_TOPS["int8"], 5),
+                              "frac_profiled": round(actor["ops"] / (PROFILED_NS["actor_fused"] * 1e-9) / 1e12 / MFMA_PEAK_TOPS["int8"], 5),
+                              "profiled_avg_kernel_ns": PROFILED_NS["actor_fused"],
                               "note": "launch- and latency-bound by construction (see results for the MFMA-bound GEMMs)"}
     del actor
     if not a.no_sweep:
