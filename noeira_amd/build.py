@@ -72,6 +72,12 @@ def _spilling_kernels(remarks: str, names, allow_bytes: int = 0) -> list:
 # an `s_waitcnt ... ; pfw`.  Between the two no instruction may name a register such a load writes (a copy or a
 # reuse there would take what has not arrived yet): checked on the kernels' assembly.
 PREFETCH_MARKED = ("nq_gemv_fp8.hip",)
+# Prefetches across a loop's back edge, two register slots in turn (the persistent tile kernels): `; pf` loads, and an
+# empty `; pfh <registers>` statement after the hand-written wait on every path.  While a slot may be in flight no
+# move, accumulator copy, swap or spill may take one of its registers as a source: _inflight_violations, a may-analysis
+# over the control-flow graph of the kernels' assembly.  (Established with the hipcc of ROCm 7.2.0; the check runs at
+# every build, so another compiler that starts copying those registers fails the build instead of the numbers.)
+INFLIGHT_MARKED = ("nq_gemv_tile.hip",)
 
 
 def _early_uses_of_prefetched(asm: str) -> list:
@@ -101,6 +107,93 @@ def _early_uses_of_prefetched(asm: str) -> list:
                     out.append((parts[k], t))
         if not waited:
             out.append((parts[k], "no `; pfw` wait after the prefetch"))
+    return out
+
+
+_COPY_LIKE = ("v_mov_b", "v_pk_mov", "v_swap_b", "v_accvgpr_write", "v_accvgpr_mov", "scratch_store")
+
+
+def _vregs(text: str) -> set:
+    out = {int(a) for a in re.findall(r"\bv(\d+)\b", text)}
+    for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+        out |= set(range(int(a), int(b) + 1))
+    return out
+
+
+def _inflight_violations(asm: str) -> list:
+    """(kernel, instruction) pairs that name a vector register while a marked load into it may still be under way.
+
+    Marks, written in the source's inline assembly: a load whose text ends in `; pf` puts its destination registers in
+    flight; a statement `; pfh <registers>` (an empty assembly statement that follows the hand-written wait on every
+    path and names the slot's registers) takes those out of flight; `; pfw` (a wait for everything) takes all out.
+    Between the two the compiler must not copy or spill the registers - a copy made to free or to coalesce one would
+    take what has not arrived, silently.  The check is a forward may-analysis over the kernel's control-flow graph
+    (a loop whose second slot is requested in a block that stands later in the text is followed the way it runs),
+    and it looks at the instructions a compiler adds unasked: moves, accumulator copies, swaps and spills.  (Branch
+    conditions are not followed, so an instruction that merely computes in a slot's registers after the loop's last
+    tile - where the slot was in fact never requested - is not held against the kernel.)"""
+    out = []
+    parts = re.split(r"\n(_Z\S+): ; @\S*\n", asm)
+    for k in range(1, len(parts), 2):
+        body = parts[k + 1].split(".Lfunc_end")[0]
+        if "; pf" not in body:
+            continue
+        # ---- basic blocks
+        blocks, cur, label_of = [[]], 0, {}
+        for raw in body.split("\n"):
+            t = raw.strip()
+            m = re.match(r"(\.LBB\d+_\d+):", t)
+            if m:
+                if blocks[-1]:
+                    blocks.append([])
+                label_of[m.group(1)] = len(blocks) - 1
+                continue
+            if not t or t.startswith(".") or (t.startswith(";") and not t.startswith("; pfh") and "pfw" not in t):
+                continue
+            blocks[-1].append(t)
+            if re.match(r"s_(c?branch\w*|endpgm|setpc)", t):
+                blocks.append([])
+        succ = []
+        for i, b in enumerate(blocks):
+            s_ = []
+            last = b[-1] if b else ""
+            m = re.match(r"s_(c?branch\w*)\s+(\.LBB\d+_\d+)", last)
+            if m:
+                if m.group(2) in label_of:
+                    s_.append(label_of[m.group(2)])
+                if m.group(1) != "branch" and i + 1 < len(blocks):
+                    s_.append(i + 1)
+            elif not last.startswith("s_endpgm") and i + 1 < len(blocks):
+                s_.append(i + 1)
+            succ.append(s_)
+        # ---- fixpoint
+        IN = [set() for _ in blocks]
+        work = list(range(len(blocks)))
+        bad = {}
+        while work:
+            i = work.pop(0)
+            live = set(IN[i])
+            for t in blocks[i]:
+                if t.startswith("; pfh"):
+                    live -= _vregs(t)
+                    continue
+                if "pfw" in t:
+                    live = set()
+                    continue
+                if t.endswith("; pf"):
+                    live |= _vregs(t.partition(",")[0])
+                    continue
+                # what the compiler inserts on its own where registers are short or values meet: copies and spills
+                if live and t.startswith(_COPY_LIKE):
+                    src = t if t.startswith("scratch_store") else t.partition(",")[2]
+                    if _vregs(src) & live:
+                        bad[(i, t)] = True
+            for j in succ[i]:
+                if not live <= IN[j]:
+                    IN[j] |= live
+                    if j not in work:
+                        work.append(j)
+        out += [(parts[k], t) for (_, t) in bad]
     return out
 
 
@@ -157,17 +250,22 @@ def _compile(src: str, force: bool) -> str:
         if inside:
             os.remove(obj)
             raise RuntimeError(f"{src}: scratch memory is accessed, or a register copied, between the first and the last MFMA of {inside}")
-    if src in PREFETCH_MARKED:
+    if src in PREFETCH_MARKED or src in INFLIGHT_MARKED:
         cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["--cuda-device-only", "-S", path, "-o", obj + ".s"]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc -S failed on {src}:\n{r.stdout}\n{r.stderr}")
         with open(obj + ".s") as f:
-            early = _early_uses_of_prefetched(f.read())
+            text = f.read()
         os.remove(obj + ".s")
+        early = _early_uses_of_prefetched(text) if src in PREFETCH_MARKED else []
+        if src in INFLIGHT_MARKED:
+            if text.count("; pfh") == 0:
+                early.append((src, "no `; pfh` hand-over found: the marks are gone from the source"))
+            early += _inflight_violations(text)
         if early:
             os.remove(obj)
-            raise RuntimeError(f"{src}: a prefetched register is named before its wait: {early[:4]}")
+            raise RuntimeError(f"{src}: a prefetched register is named, copied or spilled before its wait: {early[:4]}")
     warn = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l and l.strip())
     if warn:
         sys.stderr.write(warn + "\n")

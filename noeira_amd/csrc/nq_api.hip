@@ -98,6 +98,7 @@ int32_t bind_device(nq_layer* L) {
         return fail(NQ_ERR_INVALID, "layer was loaded on device " + std::to_string(L->device) +
                                         " but the current device is " + std::to_string(dev));
     L->device = dev;
+    hinv_dev_setup();  // (set-up of the entry point that allocates nothing: its scratch array's address on this device)
     return NQ_OK;
 }
 
@@ -477,7 +478,7 @@ struct LoraArgs {
 };
 int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, const SegTable& seg,
                      int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue,
-                     void* stream, const LoraArgs* lora = nullptr, bool* folded = nullptr) {
+                     void* stream, const LoraArgs* lora = nullptr, bool* folded = nullptr, bool fold_or_fail = false) {
     if (((uintptr_t)x & 15)) return fail(NQ_ERR_INVALID, "nq_forward: x must be 16-byte aligned and y 4-byte aligned");
     for (int t = 0; t < seg.nseg; t++)
         if (!seg.y[t] || ((uintptr_t)seg.y[t] & 3))
@@ -520,6 +521,11 @@ int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x
         *folded = true;
         return launch_gemm_tile_mt(a);
     }
+    // (decided before anything is launched: a caller whose y cannot take a second, adding launch gets its answer
+    // with y untouched)
+    if (lora && fold_or_fail)
+        return fail(NQ_ERR_UNSUPPORTED, "nq_forward_lora: for this layer and M the adapter is a second launch that adds "
+                                        "into an fp32 y; ask for fp32 output");
     if (seg.nseg == 1 || places_parts(a)) return dispatch(a);
     // one launch per part, each on a view of its rows
     const int bias_es = bias_dtype == NQ_DT_F32 ? 4 : 2;
@@ -761,12 +767,10 @@ int32_t nq_forward_lora(nq_handle h, const void* x, int32_t x_dtype, void* y, in
     seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
     const LoraArgs lora{lora_a, lora_b, r_pad, scale};
     bool folded = false;
-    rc = forward_impl(h, x, x_dtype, nullptr, seg, y_dtype, M, bias, bias_dtype, NQ_EPI_NONE, stream, &lora, &folded);
+    rc = forward_impl(h, x, x_dtype, nullptr, seg, y_dtype, M, bias, bias_dtype, NQ_EPI_NONE, stream, &lora, &folded,
+                      /*fold_or_fail=*/y_dtype != NQ_DT_F32);
     if (rc || folded) return rc;
     // the base call ran on another kernel: the adapter as a launch of its own, into the fp32 output
-    if (y_dtype != NQ_DT_F32)
-        return fail(NQ_ERR_UNSUPPORTED, "nq_forward_lora: for this layer and M the adapter is a second launch that adds "
-                                        "into an fp32 y; ask for fp32 output");
     return nq_lora_forward_add(lora_a, lora_b, h->in, h->out, r_pad, scale, x, x_dtype, reinterpret_cast<float*>(y), M,
                                stream);
 }
@@ -823,6 +827,7 @@ int32_t nq_hessian_create(nq_hessian* out, int32_t n) {
     if (!h) return fail(NQ_ERR_HIP, "nq_hessian_create: out of host memory");
     h->n = n;
     hipError_t e = hipGetDevice(&h->device);
+    if (e == hipSuccess) hinv_dev_setup();
     if (e == hipSuccess) e = hipMalloc((void**)&h->d_h, (size_t)n * n * 8);
     if (e == hipSuccess) e = hipMemset(h->d_h, 0, (size_t)n * n * 8);
     if (e != hipSuccess) {

@@ -227,6 +227,7 @@ int32_t launch_hessian_add(double* H, int n, const void* x, int32_t x_dtype, int
 int32_t launch_hinv_upper_f64(double* h, int n, double* u, int* status_dev, hipStream_t s);
 int32_t run_hinv_upper_f64_dev(const double* h_dev, int n, double* u_dev, int* pivot_dev, hipStream_t s);
 int32_t hinv_dev_max_n();
+void hinv_dev_setup();
 int32_t run_gptq_q4_0(float* w_dev, int64_t n, int k, double* h_dev, double damp_frac, uint8_t* blocks_dev,
                       double* stats_host, hipStream_t s);
 int32_t run_q4_0_objective(const float* w_dev, const float* deq_dev, int64_t n, int k, const double* h_dev,

@@ -334,13 +334,13 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
         for (int j = 0; j < JPW; j++) {
             const int64_t at = (int64_t)tile * p.NJ + min(J0 + j, p.NJ - 1);
             const u32x4* const src = p.tile + at * 64 + lane;
-            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(s.wv[j]) : "v"(src));
+            asm volatile("global_load_dwordx4 %0, %1, off nt ; pf" : "=v"(s.wv[j]) : "v"(src));
             if constexpr (!G128) {
                 const uint2* const ssrc = reinterpret_cast<const uint2*>(p.tscales) + at * 16 + c;
-                asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(s.sc[j]) : "v"(ssrc));
+                asm volatile("global_load_dwordx2 %0, %1, off ; pf" : "=v"(s.sc[j]) : "v"(ssrc));
             } else {
                 const uint32_t* const ssrc = reinterpret_cast<const uint32_t*>(p.tscales) + at * 16 + c;
-                asm volatile("global_load_dword %0, %1, off" : "=v"(s.sc[j].x) : "v"(ssrc));
+                asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(s.sc[j].x) : "v"(ssrc));
                 s.sc[j].y = 0;
             }
         }
@@ -354,15 +354,15 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
             asm volatile("s_waitcnt vmcnt(0)");
         }
         if constexpr (G128) {
-            if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]), "+v"(s.sc[0].x));
-            if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0].x), "+v"(s.sc[1].x));
+            if constexpr (JPW == 1) asm volatile("; pfh %0 %1" : "+v"(s.wv[0]), "+v"(s.sc[0].x));
+            if constexpr (JPW == 2) asm volatile("; pfh %0 %1 %2 %3" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0].x), "+v"(s.sc[1].x));
             if constexpr (JPW == 3)
-                asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0].x), "+v"(s.sc[1].x), "+v"(s.sc[2].x));
+                asm volatile("; pfh %0 %1 %2 %3 %4 %5" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0].x), "+v"(s.sc[1].x), "+v"(s.sc[2].x));
         } else {
-            if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]), "+v"(s.sc[0]));
-            if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0]), "+v"(s.sc[1]));
+            if constexpr (JPW == 1) asm volatile("; pfh %0 %1" : "+v"(s.wv[0]), "+v"(s.sc[0]));
+            if constexpr (JPW == 2) asm volatile("; pfh %0 %1 %2 %3" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0]), "+v"(s.sc[1]));
             if constexpr (JPW == 3)
-                asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0]), "+v"(s.sc[1]), "+v"(s.sc[2]));
+                asm volatile("; pfh %0 %1 %2 %3 %4 %5" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0]), "+v"(s.sc[1]), "+v"(s.sc[2]));
         }
     };
 
@@ -924,17 +924,17 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
             const u32x4* const src = wbase + (min(J0 + j, p.NJ - 1) * 64 + lane);
-            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(s.wv[j]) : "v"(src));
+            asm volatile("global_load_dwordx4 %0, %1, off nt ; pf" : "=v"(s.wv[j]) : "v"(src));
         }
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
             const int64_t at = (R * p.NJ + min(J0 + j, p.NJ - 1)) * 16 + c;
             if constexpr (!G128) {
                 const uint16_t* const src = reinterpret_cast<const uint16_t*>(p.tscales) + (at * 4 + q);  // chunk q's scale
-                asm volatile("global_load_ushort %0, %1, off" : "=v"(s.sc[j]) : "v"(src));
+                asm volatile("global_load_ushort %0, %1, off ; pf" : "=v"(s.sc[j]) : "v"(src));
             } else {
                 const uint32_t* const src = reinterpret_cast<const uint32_t*>(p.tscales) + at;
-                asm volatile("global_load_dword %0, %1, off" : "=v"(s.sc[j]) : "v"(src));
+                asm volatile("global_load_dword %0, %1, off ; pf" : "=v"(s.sc[j]) : "v"(src));
             }
         }
     };
@@ -947,12 +947,12 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
         } else {
             asm volatile("s_waitcnt vmcnt(0)");
         }
-        if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]), "+v"(s.sc[0]));
-        if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0]), "+v"(s.sc[1]));
+        if constexpr (JPW == 1) asm volatile("; pfh %0 %1" : "+v"(s.wv[0]), "+v"(s.sc[0]));
+        if constexpr (JPW == 2) asm volatile("; pfh %0 %1 %2 %3" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.sc[0]), "+v"(s.sc[1]));
         if constexpr (JPW == 3)
-            asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0]), "+v"(s.sc[1]), "+v"(s.sc[2]));
+            asm volatile("; pfh %0 %1 %2 %3 %4 %5" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.sc[0]), "+v"(s.sc[1]), "+v"(s.sc[2]));
         if constexpr (JPW == 4)
-            asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.wv[3]), "+v"(s.sc[0]), "+v"(s.sc[1]),
+            asm volatile("; pfh %0 %1 %2 %3 %4 %5 %6 %7" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.wv[3]), "+v"(s.sc[0]), "+v"(s.sc[1]),
                          "+v"(s.sc[2]), "+v"(s.sc[3]));
     };
     // what finishing needs, for all of this workgroup's tiles: thread (tile i, row r) requests it first of all
@@ -1305,7 +1305,7 @@ __global__ __launch_bounds__(1024) void gemv_tile8_rows_kernel(const TileMrParam
 #pragma unroll
         for (int j = 0; j < JPW; j++) {
             const u32x4* const src = p.tile + (((int64_t)tile * p.NJ + min(J0 + j, p.NJ - 1)) * 64 + lane);
-            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(s.wv[j]) : "v"(src));
+            asm volatile("global_load_dwordx4 %0, %1, off nt ; pf" : "=v"(s.wv[j]) : "v"(src));
         }
     };
     auto arrived = [&](int tile, Slot& s) {  // (the next tile is under way if there is one)
@@ -1318,10 +1318,10 @@ __global__ __launch_bounds__(1024) void gemv_tile8_rows_kernel(const TileMrParam
         } else {
             asm volatile("s_waitcnt vmcnt(0)");
         }
-        if constexpr (JPW == 1) asm volatile("" : "+v"(s.wv[0]));
-        if constexpr (JPW == 2) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]));
-        if constexpr (JPW == 3) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]));
-        if constexpr (JPW == 4) asm volatile("" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.wv[3]));
+        if constexpr (JPW == 1) asm volatile("; pfh %0" : "+v"(s.wv[0]));
+        if constexpr (JPW == 2) asm volatile("; pfh %0 %1" : "+v"(s.wv[0]), "+v"(s.wv[1]));
+        if constexpr (JPW == 3) asm volatile("; pfh %0 %1 %2" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]));
+        if constexpr (JPW == 4) asm volatile("; pfh %0 %1 %2 %3" : "+v"(s.wv[0]), "+v"(s.wv[1]), "+v"(s.wv[2]), "+v"(s.wv[3]));
     };
     // ---- the activations first (the oldest loads: waiting for them leaves the tiles' loads under way), then two tiles
     u32x4 xraw[JPW][2][XF32 ? 2 : 1];

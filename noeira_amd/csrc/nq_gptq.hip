@@ -362,10 +362,22 @@ int32_t run_hinv_upper_f64_dev(const double* h_dev, int n, double* u_dev, int* p
     if (rc) return rc;
     const int64_t nn = (int64_t)n * n;
     hipLaunchKernelGGL(copy_f64_kernel, dim3(blocks_for(nn)), dim3(256), 0, s, h_dev, work, nn, pivot_dev);
+    NQ_HIP(hipGetLastError());
     return launch_hinv_upper_f64(work, n, u_dev, pivot_dev, s);
 }
 
 int32_t hinv_dev_max_n() { return HINV_DEV_MAX_N; }
+
+// Set-up: looks the scratch array's address up for the current device, so that the first call of the entry point
+// above - which may stand inside a stream capture - finds it known.  Called where a layer or a Hessian is created.
+void hinv_dev_setup() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return;  // (the entry point reports it)
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev]) return;
+    double* ptr = nullptr;
+    if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) == hipSuccess) g_scratch_ptr[dev] = ptr;
+}
 
 int32_t launch_hessian_add(double* H, int n, const void* x, int32_t x_dtype, int rows, hipStream_t s) {
     if (rows <= 0) return NQ_OK;

@@ -65,7 +65,7 @@ class LoRAAdapter:
         return y
 
     def forward_with(self, base, x: torch.Tensor, bias: torch.Tensor | None = None,
-                     out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                     out_dtype: torch.dtype = torch.float32, out: torch.Tensor | None = None) -> torch.Tensor:
         """``base.forward(x)`` and this adapter's share in one call (`nq_forward_lora`): one launch where the base
         call runs on the kernel that keeps its rows' activations resident, the two of `forward` + `forward_add`
         elsewhere.  B = 0 returns the bits of ``base.forward(x)``."""
@@ -76,7 +76,8 @@ class LoRAAdapter:
         if base.IN != self.IN or base.OUT != self.OUT:
             raise L.NQError(L.NQ_ERR_INVALID, "LoRAAdapter.forward_with: the adapter and the base layer differ in shape")
         T = x.shape[0]
-        y = torch.empty((T, self.OUT), dtype=out_dtype, device=x.device)
+        y = out if (out is not None and out.dtype == out_dtype and out.numel() >= T * self.OUT and out.is_cuda) else \
+            torch.empty((T, self.OUT), dtype=out_dtype, device=x.device)
         null = C.c_void_p(0)
         L.check(L.lib().nq_forward_lora(base._h, _dev_ptr(x), _TORCH_DT[x.dtype], _dev_ptr(y), _TORCH_DT[out_dtype], T,
                                         _dev_ptr(bias) if bias is not None else null,

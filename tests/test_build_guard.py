@@ -69,3 +69,46 @@ def test_a_prefetched_register_named_before_its_wait_is_reported():
     for src in B.PREFETCH_MARKED:
         text = open(os.path.join(B.CSRC, src)).read()
         assert "; pf\"" in text and "; pfw\"" in text, src
+
+
+LOOP_ASM = """\t.text
+_ZN2nq4loopEv: ; @_ZN2nq4loopEv
+\tglobal_load_dwordx4 v[0:3], v[8:9], off nt ; pf
+\ts_branch .LBB0_2
+.LBB0_1:
+\ts_waitcnt vmcnt(1)
+\t; pfh v[4:7]
+\tv_mfma_f32_16x16x32_bf16 a[0:3], v[4:7], v[10:13], a[0:3]
+\tglobal_load_dwordx4 v[0:3], v[8:9], off nt ; pf
+.LBB0_2:
+\tglobal_load_dwordx4 v[4:7], v[8:9], off nt ; pf
+{extra}
+\ts_waitcnt vmcnt(1)
+\t; pfh v[0:3]
+\tv_mfma_f32_16x16x32_bf16 a[0:3], v[0:3], v[10:13], a[0:3]
+\ts_cbranch_vccnz .LBB0_1
+\ts_waitcnt vmcnt(0)
+\t; pfh v[4:7]
+\ts_endpgm
+.Lfunc_end0:
+"""
+
+
+def test_inflight_check_follows_the_loop_and_catches_copies_and_spills():
+    """Two slots in turn across a back edge: the second slot's load stands later in the text than its hand-over.  A
+    clean loop passes; a move or a spill that takes a register of a slot in flight is named; a move of a slot that was
+    handed over is not."""
+    assert B._inflight_violations(LOOP_ASM.format(extra="\tv_add_u32_e32 v20, v21, v22")) == []
+    bad = B._inflight_violations(LOOP_ASM.format(extra="\tv_mov_b32_e32 v20, v1"))
+    assert [t for _, t in bad] == ["v_mov_b32_e32 v20, v1"]
+    bad = B._inflight_violations(LOOP_ASM.format(extra="\tscratch_store_dwordx2 off, v[6:7], off"))
+    assert [t for _, t in bad] == ["scratch_store_dwordx2 off, v[6:7], off"]
+    # after its hand-over a slot's registers are ordinary values again
+    ok = LOOP_ASM.format(extra="").replace("\ts_endpgm", "\tv_mov_b32_e32 v30, v5\n\ts_endpgm")
+    assert B._inflight_violations(ok) == []
+
+
+def test_inflight_marks_exist_in_the_sources_that_are_checked():
+    for src in B.INFLIGHT_MARKED:
+        text = open(os.path.join(B.CSRC, src)).read()
+        assert text.count("; pf\"") >= 3 and text.count("; pfh ") >= 3, src

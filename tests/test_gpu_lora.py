@@ -165,7 +165,11 @@ def test_qlora_one_call_bf16_out_and_errors():
     narrow = QLinear(IN, 320)
     narrow.set_weight((rng.standard_normal((320, IN)) * 0.05).astype(np.float32))
     adn, _, _ = make(rng, IN, 320, 16)
-    with pytest.raises(L.NQError, match="second launch"):        # not folded here: the adapter adds into fp32 only
-        adn.forward_with(narrow, x, out_dtype=torch.bfloat16)
+    # not folded here: the adapter adds into fp32 only.  The answer comes before anything is launched: y is untouched
+    ybn = torch.full((T, 320), 7.0, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(L.NQError, match="second launch"):
+        adn.forward_with(narrow, x, out=ybn, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    assert bool((ybn == 7.0).all())
     with pytest.raises(L.NQError, match="differ in shape"):
         adn.forward_with(base, x)
