@@ -11,6 +11,7 @@ from noeira_amd import _lib as L  # noqa: E402
 from noeira_amd import formats as F  # noqa: E402
 from noeira_amd.qlinear import FP8Linear, FusedRows, QLinear, W4GroupLinear, W8Linear  # noqa: E402
 from oracle import oracle as O  # noqa: E402
+import refw  # noqa: E402
 
 
 def q4_layer(rng, IN, OUT):
@@ -163,7 +164,9 @@ def test_parts_keep_their_bits_between_the_medium_and_the_many_rows_kernel(M):
 
     def w8(n):
         lin = W8Linear(K, n)
-        lin.set_weight(rng.integers(-127, 128, (n, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, n).astype(np.float32))
+        wq, ws = rng.integers(-127, 128, (n, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+        lin.set_weight(wq, ws)
+        lin.ref_deq = lambda: refw.w8(wq, ws)
         return lin
 
     def q4(n):
@@ -172,6 +175,7 @@ def test_parts_keep_their_bits_between_the_medium_and_the_many_rows_kernel(M):
         sc = rng.uniform(1e-3, 1e-2, (n, K // 32)).astype(np.float16).view(np.uint16)
         blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
         lin.set_blocks(blocks.reshape(-1))
+        lin.ref_deq = lambda: refw.q4_0(blocks, n, K)
         return lin
 
     for make in (w8, q4):
@@ -182,7 +186,7 @@ def test_parts_keep_their_bits_between_the_medium_and_the_many_rows_kernel(M):
             for part, y in zip(parts, outs):
                 own = part.forward(x)
                 assert torch.equal(y, own), (make.__name__, widths, part.OUT)
-                exact = x.double() @ part.dequantized_dev().double().T
+                exact = x.double() @ part.ref_deq().T
                 assert float((own.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
             if make is w8:  # bias and ReLU travel with each part when the call runs part by part
                 bias = torch.from_numpy(rng.standard_normal(sum(widths)).astype(np.float32)).cuda()

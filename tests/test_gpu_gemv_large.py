@@ -1,8 +1,8 @@
 """The single-row GEMV over large 4-bit and int8 weights (megabytes of codes), through the C ABI, on both
 device layouts: the tile-ordered copy large layers keep by default (nq_gemv_tile.hip) and the row-ordered
 codes alone (tile_copy=False: nq_gemv_row4 / row8 / split8),
-against fp64 products of the layer's dequantised weights (pinned bit for bit against the CPU
-oracle in tests/test_gpu_qlinear.py and tests/test_gpu_formats.py) and, at a size the oracle
+against fp64 products with the weights the CPU oracle dequantises from the codes each test drew
+(tests/refw.py; the library is not asked what its weights are) and, at a size the oracle
 finishes in seconds, against the oracle's own forward.
 
 Bars: the reference's fp32 band for Q4_0 with fp32 activations (1e-5 of the largest reference
@@ -16,6 +16,7 @@ import torch
 from noeira_amd import formats as F
 from noeira_amd.qlinear import FusedRows, QLinear, W4GroupLinear
 from oracle import oracle as O
+import refw
 
 pytestmark = pytest.mark.gpu
 
@@ -33,6 +34,8 @@ def q4_layer(rng, K, N, scale_kind="uniform", tile_copy=True):
     blocks[:, :, 0] = bits & 0xFF
     blocks[:, :, 1] = bits >> 8
     lin.set_blocks(blocks.reshape(-1))
+    lin.host_blocks = blocks
+    lin.ref_deq = lambda: refw.q4_0(blocks, N, K)
     return lin
 
 
@@ -44,7 +47,7 @@ def q4_layer(rng, K, N, scale_kind="uniform", tile_copy=True):
 def test_q4_0_large_single_row(K, N, xdt, tile_copy):
     rng = np.random.default_rng(K + N)
     lin = q4_layer(rng, K, N, "signed", tile_copy)
-    deq = lin.dequantized_dev().double()
+    deq = lin.ref_deq()
     x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
     y = lin.forward(x)
     exact = x.double() @ deq.T
@@ -59,9 +62,9 @@ def test_q4_0_large_against_oracle_forward():
     lin = q4_layer(rng, K, N)
     x = rng.standard_normal((1, K)).astype(np.float32)
     y = lin.forward(torch.from_numpy(x).cuda()).cpu().numpy()
-    want = O.qlinear_forward_cpu(lin.blocks(), K, N, x)
+    want = O.qlinear_forward_cpu(lin.host_blocks.reshape(-1), K, N, x)
     assert O.rel_max(y, want) < 1e-5
-    exact = O.dense_forward_f64(O.dequantize_q4_0(lin.blocks().reshape(N, -1), N, K), x)
+    exact = O.dense_forward_f64(O.dequantize_q4_0(lin.host_blocks.reshape(N, -1), N, K), x)
     assert O.rel_max(y, exact.astype(np.float32)) < 1e-5
 
 
@@ -76,8 +79,9 @@ def test_w4_group_large_single_row(K, N, group, xdt, tile_copy):
     z = rng.integers(0, 16, (N, G), dtype=np.uint8)
     codes, zps = F.pack_w4g(q, z)
     lin = W4GroupLinear(K, N, group, tile_copy=tile_copy)
-    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
-    deq = lin.dequantized_dev().double()
+    sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+    lin.set_weight(codes, sg, zps)
+    deq = refw.w4g(codes, sg, zps, N, K, group)
     x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
     bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
     exact = x.double() @ deq.T + bias.double()
@@ -244,6 +248,7 @@ def test_tile_copy_agrees_with_row_kernels(K, N):
     assert np.array_equal(a.blocks(), b.blocks())
     ya, yb = a.forward(x), b.forward(x)
     assert float((ya - yb).abs().max()) <= 2e-6 * float(yb.abs().max())
+    assert torch.equal(a.dequantized_dev().double(), a.ref_deq())  # (fp32 values of the oracle, exactly)
     assert torch.equal(a.dequantized_dev(), b.dequantized_dev())
     w = rng.integers(-127, 128, (N, K), dtype=np.int8)
     s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
@@ -279,7 +284,9 @@ def _w4g_layer(rng, K, N, **kw):
     G = K // 128
     codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
     lin = W4GroupLinear(K, N, 128, **kw)
-    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+    sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+    lin.set_weight(codes, sg, zps)
+    lin.ref_deq = lambda: refw.w4g(codes, sg, zps, N, K, 128)
     return lin
 
 
@@ -289,6 +296,7 @@ def _q4_signed(rng, K, N, **kw):
     bits = (rng.uniform(1e-3, 1e-2, (N, K // 32)) * rng.choice([-1.0, 1.0], (N, K // 32))).astype(np.float16).view(np.uint16)
     blocks[:, :, 0], blocks[:, :, 1] = bits & 0xFF, bits >> 8
     lin.set_blocks(blocks.reshape(-1))
+    lin.ref_deq = lambda: refw.q4_0(blocks, N, K)
     return lin
 
 
@@ -306,7 +314,7 @@ def test_four_bit_single_row_on_the_int8_matrix_cores(K, N, prefer, fmt, xdt):
     reference value) holds for fp32 and bf16 activations alike."""
     rng = np.random.default_rng(K + N + len(fmt))
     lin = (_q4_signed if fmt == "q4_0" else _w4g_layer)(rng, K, N, prefer_tile=prefer)
-    deq = lin.dequantized_dev().double()
+    deq = lin.ref_deq()
     x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).to(xdt).cuda()
     bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
     y = lin.forward(x, bias=bias)
@@ -316,12 +324,12 @@ def test_four_bit_single_row_on_the_int8_matrix_cores(K, N, prefer, fmt, xdt):
     yr = lin.forward(x, bias=bias.to(torch.bfloat16), epilogue="relu", out_dtype=torch.bfloat16)
     want = (x.double() @ deq.T + bias.to(torch.bfloat16).double()).clamp_min(0)
     assert float((yr.double() - want).abs().max()) <= 2.0 ** -8 * float(want.abs().max()) + 1e-5 * float(exact.abs().max())
-    del deq, exact, want
+    del exact, want
     # an outlier sixty times the rest: the terms keep 24 bits under the slice's scale
     xo = x.clone()
     xo[0, K // 3] = 60.0
     yo = lin.forward(xo)
-    eo = xo.double() @ lin.dequantized_dev().double().T
+    eo = xo.double() @ deq.T
     assert float((yo.double() - eo).abs().max()) <= 1e-5 * float(eo.abs().max())
     # a NaN or an infinity in x: every output NaN (the exact result would be NaN or +-inf per row)
     xn = x.clone()

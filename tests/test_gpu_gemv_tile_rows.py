@@ -1,6 +1,6 @@
 """A few activation rows (2 .. 16) over a large 4-bit weight: the persistent tile kernel of nq_gemv_tile.hip
-(bf16 rows as the matrix core's A rows, fp32 rows as three A rows each), through the C ABI, against fp64 products of
-the layer's dequantised weights (pinned bit for bit against the oracle elsewhere) and against the oracle's own
+(bf16 rows as the matrix core's A rows, fp32 rows as three A rows each), through the C ABI, against fp64 products with
+the weights the CPU oracle dequantises from the codes each test drew (tests/refw.py) and against the oracle's own
 forward at a size it finishes in seconds.  Bars: 1e-5 of the largest reference value (the reference's fp32 band,
 tests/nn/quant/qlinear_common.mojo:39-45); repeated calls return the same bits."""
 import numpy as np
@@ -10,6 +10,7 @@ import torch
 from noeira_amd import formats as F
 from noeira_amd.qlinear import FusedRows, QLinear, W4GroupLinear
 from oracle import oracle as O
+import refw
 
 pytestmark = pytest.mark.gpu
 
@@ -20,6 +21,7 @@ def q4_layer(rng, K, N, tile_copy=True):
     sc = (rng.uniform(1e-3, 1e-2, (N, K // 32)) * rng.choice([-1.0, 1.0], (N, K // 32))).astype(np.float16).view(np.uint16)
     blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
     lin.set_blocks(blocks.reshape(-1))
+    lin.ref_deq = lambda: refw.q4_0(blocks, N, K)
     return lin
 
 
@@ -27,7 +29,9 @@ def w4g_layer(rng, K, N, tile_copy=True):
     G = K // 128
     codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
     lin = W4GroupLinear(K, N, 128, tile_copy=tile_copy)
-    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+    sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+    lin.set_weight(codes, sg, zps)
+    lin.ref_deq = lambda: refw.w4g(codes, sg, zps, N, K, 128)
     return lin
 
 
@@ -43,7 +47,7 @@ SHAPES = [(2048, 2051), (2176, 1999), (4096, 1100), (4096, 11008), (5504, 800), 
 def test_few_rows_over_tile_copy(K, N, fmt, xdt, M):
     rng = np.random.default_rng(K + N + M + len(fmt))
     lin = q4_layer(rng, K, N) if fmt == "q4_0" else w4g_layer(rng, K, N)
-    deq = lin.dequantized_dev().double()
+    deq = lin.ref_deq()
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
     bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
     y = lin.forward(x, bias=bias)

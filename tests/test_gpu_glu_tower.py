@@ -12,13 +12,17 @@ from noeira_amd import _lib as L
 from noeira_amd import formats as F
 from noeira_amd.qlinear import FusedGLU, FusedRows, QLinear, W4GroupLinear, W8Linear
 from oracle import oracle as O
+import refw
 
 pytestmark = pytest.mark.gpu
 
 
 def q4(rng, IN, OUT, std=0.05):
     lin = QLinear(IN, OUT)
-    lin.set_weight((rng.standard_normal((OUT, IN)) * std).astype(np.float32))
+    w = (rng.standard_normal((OUT, IN)) * std).astype(np.float32)
+    lin.set_weight(w)
+    # deq(W) by the oracle alone: its round-to-nearest quantiser, then its dequantiser
+    lin.ref_deq = lambda: refw.q4_0(O.rtn_q4_0_blocks(w), OUT, IN)
     return lin
 
 
@@ -58,19 +62,22 @@ def test_glu_against_fp64_over_the_dequantised_weights(kind, IN, H, M, xdt):
             layers.append(q4(rng, IN, H))
         elif kind == "w8":
             lin = W8Linear(IN, H)
-            lin.set_weight(*F.quantize_w8_channel((rng.standard_normal((H, IN)) * 0.05).astype(np.float32)))
+            wq, ws = F.quantize_w8_channel((rng.standard_normal((H, IN)) * 0.05).astype(np.float32))
+            lin.set_weight(wq, ws)
+            lin.ref_deq = lambda wq=wq, ws=ws: refw.w8(wq, ws)
             layers.append(lin)
         else:
             lin = W4GroupLinear(IN, H, 128)
             q, s, z = F.quantize_w4g_asym((rng.standard_normal((H, IN)) * 0.05).astype(np.float32), 128)
             codes, zps = F.pack_w4g(q, z)
             lin.set_weight(codes, s, zps)
+            lin.ref_deq = lambda codes=codes, s=s, zps=zps: refw.w4g(codes, s, zps, H, IN, 128)
             layers.append(lin)
     gate, up = layers
     glu = FusedGLU(gate, up)
     x = torch.from_numpy(rng.standard_normal((M, IN)).astype(np.float32)).to(xdt).cuda()
-    g = x.double() @ gate.dequantized_dev().double().T
-    u = x.double() @ up.dequantized_dev().double().T
+    g = x.double() @ gate.ref_deq().T
+    u = x.double() @ up.ref_deq().T
     want = u * (g * torch.sigmoid(g))
     y = glu.forward(x)
     assert y.shape == (M, H) and y.dtype == torch.float32
@@ -168,7 +175,7 @@ class Tower:
 
         def lin(layer, h):
             if mode == "dense":
-                return h @ layer.dequantized_dev().double().T
+                return h @ layer.ref_deq().T
             if mode == "bf16":
                 return layer.forward(h.to(torch.bfloat16).contiguous(), out_dtype=torch.bfloat16).float()
             return layer.forward(h.contiguous())

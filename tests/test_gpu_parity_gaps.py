@@ -14,6 +14,7 @@ from noeira_amd import formats as F
 from noeira_amd.qlinear import (FP8Linear, QLinear, W4GroupLinear, W8Linear, mlp3_w8a8_forward, quantize_rows_i8)
 from noeira_amd.safetensors_io import SafeTensors, SafeTensorsWriter, load_q4_blocks, q4_blocks_key
 from oracle import oracle as O
+import refw
 
 pytestmark = pytest.mark.gpu
 
@@ -213,7 +214,9 @@ def test_from_linear_is_x_at_w_plus_b(kind):
         tol_q = 6e-2
     elif kind == "fp8":
         lin = FP8Linear.from_linear(w, b)
-        deq = lin.dequantized_dev().double().cpu().numpy()
+        # the loader's rule restated with the oracle's encoder: one scale absmax / 448, codes of w / scale
+        sc8 = float(np.abs(w).max()) / 448.0
+        deq = refw.fp8(O.e4m3_encode(np.ascontiguousarray(w.T) / np.float32(sc8)), sc8).cpu().numpy()
         xc = torch.from_numpy(x).to(torch.float8_e4m3fn)
         want = xc.double().numpy() @ deq.T + b
         y = lin.forward(xc.view(torch.uint8).cuda(), torch.ones(1, device="cuda"), out_dtype=torch.float32).cpu().numpy()
@@ -221,7 +224,9 @@ def test_from_linear_is_x_at_w_plus_b(kind):
         tol_q = 2e-1
     elif kind == "w4g":
         lin = W4GroupLinear.from_linear(w, b, group=128)
-        want = x.astype(np.float64) @ lin.dequantized_dev().double().cpu().numpy().T + b
+        q4g, s4g, z4g = F.quantize_w4g_asym(np.ascontiguousarray(w.T), 128)
+        c4g, zp4g = F.pack_w4g(q4g, z4g)
+        want = x.astype(np.float64) @ refw.w4g(c4g, s4g, zp4g, OUT, IN, 128).cpu().numpy().T + b
         y = lin.forward(xd).cpu().numpy()
         tol_q = 5e-1
     else:
@@ -258,6 +263,46 @@ def test_quantize_w8_channel_is_symmetric_absmax():
     assert np.abs(q).max() == 127
 
 
+# ── nq_dequantize at the full-size layer (4096 -> 11008, 45 M weights), bit for bit against the oracle ──
+@pytest.mark.parametrize("fmt,tile_copy", [("q4_0", True), ("q4_0", False), ("w4g", True), ("w4g", False), ("w8", True),
+                                           ("w8", False), ("fp8", True)])
+def test_dequantize_bitwise_at_full_size(fmt, tile_copy):
+    """Whatever device layout the layer keeps (row-ordered codes, the tile-ordered copy), `nq_dequantize` returns
+    the fp32 values the CPU oracle computes from the codes the test drew, every one of the 45 M bit for bit; the forward
+    tests at this size take their reference weights from the oracle, and this ties the library's own view to them."""
+    rng = np.random.default_rng(sum(map(ord, fmt)) + tile_copy)
+    K, N = 4096, 11008
+    if fmt == "q4_0":
+        blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
+        sc = (rng.uniform(1e-3, 1e-2, (N, K // 32)) * rng.choice([-1.0, 1.0], (N, K // 32))).astype(np.float16).view(np.uint16)
+        blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
+        lin = QLinear(K, N, tile_copy=tile_copy)
+        lin.set_blocks(blocks.reshape(-1))
+        want = O.dequantize_q4_0(blocks.reshape(-1), N, K)
+    elif fmt == "w4g":
+        G = K // 128
+        codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
+        sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+        lin = W4GroupLinear(K, N, 128, tile_copy=tile_copy)
+        lin.set_weight(codes, sg, zps)
+        want = O.w4g_dequantize(codes, sg.view(np.uint16), zps, N, K, 128)
+    elif fmt == "w8":
+        w = rng.integers(-128, 128, (N, K), dtype=np.int8)
+        sw = (rng.uniform(1e-3, 1e-2, N) * rng.choice([-1.0, 1.0], N)).astype(np.float32)
+        lin = W8Linear(K, N, tile_copy=tile_copy)
+        lin.set_weight(w, sw)
+        want = w.astype(np.float32) * sw[:, None]  # one fp32 multiply per weight
+    else:
+        codes = rng.integers(0, 256, (N, K), dtype=np.uint8)
+        codes[(codes & 0x7F) == 0x7F] = 0x38  # (the two NaN codes are compared in test_fp8_dequantize_bitwise)
+        scale = np.float32(0.0625) * np.float32(1.37)
+        lin = FP8Linear(K, N)
+        lin.set_weight(codes, float(scale))
+        want = O.e4m3_decode_table()[codes].astype(np.float32) * scale
+    got = lin.dequantized_dev()
+    assert torch.equal(got.view(torch.int32), torch.from_numpy(want).cuda().view(torch.int32))
+
+
 # ── share_scratch: dequantized_dev() writes the shared buffer (qlinear.mojo:330-340) ──
 def test_share_scratch_receives_the_dequantised_weight():
     rng = np.random.default_rng(9)
@@ -285,15 +330,15 @@ def test_share_scratch_receives_the_dequantised_weight():
 def test_fp8_weights_under_16bit_activations(M, K, N, xdt):
     """e4m3fn weights with fp32 / bf16 activations at every M: one row on the GEMV, from two rows on the bf16
     matrix-core kernels (the codes decode to bf16 exactly, fp32 activations enter as three exact bf16 terms), so
-    the result is the fp64 product over the dequantised weights - which `nq_dequantize` pins to the oracle's
-    decode table bit for bit - to fp32 accumulation accuracy.  With bias, ReLU and bf16 out; a NaN code poisons
+    the result is the fp64 product over the weights the oracle's decode table gives for the codes the test drew,
+    to fp32 accumulation accuracy.  With bias, ReLU and bf16 out; a NaN code poisons
     its own output channel and no other."""
     rng = np.random.default_rng(M + K + N)
     lin = FP8Linear(K, N)
     wt = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).to(torch.float8_e4m3fn)
     codes = wt.view(torch.uint8).numpy().copy()
     lin.set_weight(codes, 1.0 / 16)
-    deq = lin.dequantized_dev().double()
+    deq = refw.fp8(codes, 1.0 / 16)
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
     bias = torch.from_numpy((rng.standard_normal(N) * 0.5).astype(np.float32)).cuda()
     want = x.double() @ deq.T

@@ -3,10 +3,9 @@
 Each case draws a format, M (1 .. 1000, dense around the kernel-selection
 thresholds), IN, OUT (ragged on purpose: OUT = 1 .. 3000, IN any legal
 multiple), activation and output dtypes, bias kind and epilogue, and checks
-the result against an fp64 product of the layer's dequantised weights.  Those
-weights come from the library's own dequantise call, which
-tests/test_gpu_qlinear.py and tests/test_gpu_formats.py pin bit for bit
-against the CPU oracle; the int8 x int8 accumulators are compared exactly.
+the result against an fp64 product with the weights the CPU oracle dequantises
+from the codes the case drew (tests/refw.py; the library is never asked what
+its weights are); the int8 x int8 accumulators are compared exactly.
 Bars as everywhere: 1e-3 * RMS (fp8: 1e-2), plus half a bf16 step when the
 output is bf16.
 """
@@ -16,6 +15,7 @@ import torch
 
 from noeira_amd import formats as F
 from noeira_amd.qlinear import FP8Linear, QLinear, W4GroupLinear, W8Linear, quantize_rows_i8
+import refw
 
 pytestmark = pytest.mark.gpu
 
@@ -72,11 +72,14 @@ def test_random_shapes(seed, prefer):
             blocks[:, :, 0] = sc & 0xFF
             blocks[:, :, 1] = sc >> 8
             lin.set_blocks(blocks.reshape(-1))
+            deq = refw.q4_0(blocks, N, K)
         elif fmt in ("w8", "w8a8"):
             K = _pick_k(rng, 128 if (fmt == "w8a8" and rng.integers(0, 2)) else 16, hi)
             lin = W8Linear(K, N, prefer_tile=prefer)
             w = rng.integers(-127, 128, (N, K), dtype=np.int8)
-            lin.set_weight(w, rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+            sw_host = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+            lin.set_weight(w, sw_host)
+            deq = refw.w8(w, sw_host)
         elif fmt == "w4g":
             group = int(rng.choice([128, 128, 64, 32]))
             K = _pick_k(rng, 32, hi)
@@ -85,14 +88,16 @@ def test_random_shapes(seed, prefer):
             z = rng.integers(0, 16, (N, G), dtype=np.uint8)
             codes, zps = F.pack_w4g(q, z)
             lin = W4GroupLinear(K, N, group, prefer_tile=prefer)
-            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+            sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+            lin.set_weight(codes, sg, zps)
+            deq = refw.w4g(codes, sg, zps, N, K, group)
         else:
             K = _pick_k(rng, 16)
             lin = FP8Linear(K, N)
             wt = torch.from_numpy(rng.standard_normal((N, K)).astype(np.float32)).to(torch.float8_e4m3fn)
             lin.set_weight(wt.view(torch.uint8).numpy(), 1.0 / 16)
+            deq = refw.fp8(wt.view(torch.uint8).numpy(), 1.0 / 16)
         tag = "%s M=%d K=%d N=%d x=%s y=%s bias=%d %s" % (fmt, M, K, N, str(xdt)[6:], str(odt)[6:], use_bias, epi)
-        deq = lin.dequantized_dev().double()
         bias = None
         if use_bias:
             bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
@@ -119,10 +124,7 @@ def test_random_shapes(seed, prefer):
             acc_exact = xq.double() @ wd.T  # exact: |acc| < 2^53
             acc = lin.forward_a8(xq, sx, out_dtype=torch.int32)
             assert bool((acc.double() == acc_exact).all()), tag + ": int32 accumulators differ"
-            # the channel scale, read back through the dequantised weights at a nonzero code
-            nz = wd.abs().argmax(dim=1)
-            rows = torch.arange(N, device="cuda")
-            sw = deq[rows, nz] / wd[rows, nz]
+            sw = torch.from_numpy(sw_host).cuda().double()
             y = lin.forward_a8(xq, sx, bias=bias, epilogue=epi, out_dtype=odt)
             _check(tag, y, fin(acc_exact * sx.double()[:, None] * sw[None, :]), odt == torch.bfloat16)
         del lin
@@ -133,7 +135,7 @@ def test_random_shapes(seed, prefer):
 def test_many_rows(fmt, xdt):
     """Many rows (512 and more, where its workgroups fill the chip): bf16 / fp32 activations take the kernel that stages a [64 or 128] x 128 tile per
     workgroup: ragged M, N and K (K not a multiple of its k-step, N not a multiple of 128, M not a multiple
-    of the tile), bias, ReLU and bf16 output, against the fp64 product of the dequantised weights."""
+    of the tile), bias, ReLU and bf16 output, against the fp64 product with the oracle's dequantised weights."""
     rng = np.random.default_rng(sum(map(ord, fmt + str(xdt))))
     for (M, K, N) in ((2048, 960, 1600), (2100, 992, 1200), (5000, 4096, 650), (4096, 160, 1000), (513, 960, 3000)):
         if fmt.startswith("w4g"):
@@ -143,10 +145,14 @@ def test_many_rows(fmt, xdt):
             z = rng.integers(0, 16, (N, G), dtype=np.uint8)
             codes, zps = F.pack_w4g(q, z)
             lin = W4GroupLinear(K, N, group)
-            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+            sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+            lin.set_weight(codes, sg, zps)
+            deq = refw.w4g(codes, sg, zps, N, K, group)
         elif fmt == "w8":
             lin = W8Linear(K, N)
-            lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+            w, sw_host = rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+            lin.set_weight(w, sw_host)
+            deq = refw.w8(w, sw_host)
         else:
             lin = QLinear(K, N)
             blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
@@ -154,7 +160,7 @@ def test_many_rows(fmt, xdt):
             blocks[:, :, 0] = sc & 0xFF
             blocks[:, :, 1] = sc >> 8
             lin.set_blocks(blocks.reshape(-1))
-        deq = lin.dequantized_dev().double()
+            deq = refw.q4_0(blocks, N, K)
         x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
         tag = "%s M=%d K=%d N=%d %s" % (fmt, M, K, N, str(xdt)[6:])
         bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
@@ -202,7 +208,9 @@ def test_single_row_fp32_x_through_lds(fmt):
             z = rng.integers(0, 16, (N, G), dtype=np.uint8)
             codes, zps = F.pack_w4g(q, z)
             lin = W4GroupLinear(K, N, group)
-            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+            sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+            lin.set_weight(codes, sg, zps)
+            deq = refw.w4g(codes, sg, zps, N, K, group)
         else:
             lin = QLinear(K, N)
             blocks = rng.integers(0, 256, (N, K // 32, 18), dtype=np.uint8)
@@ -210,7 +218,7 @@ def test_single_row_fp32_x_through_lds(fmt):
             blocks[:, :, 0] = sc & 0xFF
             blocks[:, :, 1] = sc >> 8
             lin.set_blocks(blocks.reshape(-1))
-        deq = lin.dequantized_dev().double()
+            deq = refw.q4_0(blocks, N, K)
         x = torch.from_numpy(rng.standard_normal((1, K)).astype(np.float32)).cuda()
         tag = "%s M=1 K=%d N=%d fp32" % (fmt, K, N)
         exact = x.double() @ deq.T
@@ -226,7 +234,7 @@ def test_random_large_layers():
     """Layers of 4 M to 100 M weights with ragged OUT, at row counts from 1 to 512 (every kernel's range of rows and
     the counts either side of each hand-over): the kernels over the
     tile-ordered copy and the row-ordered ones (tile copy and preference drawn per case), bias + ReLU, fp32 or bf16
-    out, against the fp64 product of the dequantised weights; a repeated call returns the same bits."""
+    out, against the fp64 product with the oracle's dequantised weights; a repeated call returns the same bits."""
     rng = np.random.default_rng(2026)
     for case in range(90):
         fmt = ["q4_0", "w4g", "w8"][case % 3]
@@ -243,16 +251,20 @@ def test_random_large_layers():
             blocks[:, :, 0] = sc & 0xFF
             blocks[:, :, 1] = sc >> 8
             lin.set_blocks(blocks.reshape(-1))
+            deq = refw.q4_0(blocks, N, K)
         elif fmt == "w4g":
             G = -(-K // 128)
             codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
             lin = W4GroupLinear(K, N, 128, tile_copy=tc, prefer_tile=prefer)
-            lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+            sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+            lin.set_weight(codes, sg, zps)
+            deq = refw.w4g(codes, sg, zps, N, K, 128)
         else:
             lin = W8Linear(K, N, tile_copy=tc, prefer_tile=prefer)
-            lin.set_weight(rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32))
+            w, sw_host = rng.integers(-127, 128, (N, K), dtype=np.int8), rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+            lin.set_weight(w, sw_host)
+            deq = refw.w8(w, sw_host)
         tag = "%s M=%d K=%d N=%d x=%s y=%s prefer=%d tile_copy=%d" % (fmt, M, K, N, str(xdt)[6:], str(odt)[6:], prefer, tc)
-        deq = lin.dequantized_dev().double()
         bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
         x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda().to(xdt)
         y = lin.forward(x, bias=bias, epilogue="relu", out_dtype=odt)

@@ -3,7 +3,7 @@ the A operands of 16 activation rows in registers and walks the 16-row weight ti
 through the C ABI.  The reference's caller runs exactly this regime: T = 135 tokens over 960 -> 960 / 320 / 2560 and
 2560 -> 960 (noeira/deep_agents/smolvla/fused.mojo:255-384), its gate tests/nn/quant/test_qlinear_gpu.mojo.  Against
 the oracle's forward (1e-5 of the largest reference value, tests/nn/quant/qlinear_common.mojo:39-45), against fp64
-over the dequantised weights for every K split the kernel has, row-fused parts and the SwiGLU epilogue included;
+over the oracle's dequantised weights (tests/refw.py, from the codes each test drew) for every K split the kernel has, row-fused parts and the SwiGLU epilogue included;
 repeated calls return the same bits; a row-fused layer returns the bits of its parts' own forwards."""
 import numpy as np
 import pytest
@@ -12,6 +12,7 @@ import torch
 from noeira_amd import formats as F
 from noeira_amd.qlinear import FusedGLU, FusedRows, QLinear, W4GroupLinear
 from oracle import oracle as O
+import refw
 
 pytestmark = pytest.mark.gpu
 
@@ -23,6 +24,7 @@ def q4_layer(rng, K, N, tile_copy=True):
     sc = (rng.uniform(1e-3, 1e-2, (N, K // 32)) * rng.choice([-1.0, 1.0], (N, K // 32))).astype(np.float16).view(np.uint16)
     blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
     lin.set_blocks(blocks.reshape(-1))
+    lin.ref_deq = lambda: refw.q4_0(blocks, N, K)
     return lin
 
 
@@ -30,7 +32,9 @@ def w4g_layer(rng, K, N, tile_copy=True):
     G = -(-K // 128)
     codes, zps = F.pack_w4g(rng.integers(0, 16, (N, K), dtype=np.uint8), rng.integers(0, 16, (N, G), dtype=np.uint8))
     lin = W4GroupLinear(K, N, 128, tile_copy=tile_copy, prefer_tile=True)
-    lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16), zps)
+    sg = rng.uniform(1e-3, 1e-2, (N, G)).astype(np.float16)
+    lin.set_weight(codes, sg, zps)
+    lin.ref_deq = lambda: refw.w4g(codes, sg, zps, N, K, 128)
     return lin
 
 
@@ -66,7 +70,7 @@ SHAPES = [(512, 777), (640, 100), (960, 1000), (992, 48), (2048, 531), (2176, 30
 def test_m_tiles_over_tile_copy(K, N, fmt, xdt, M):
     rng = np.random.default_rng(K + N + M + len(fmt))
     lin = q4_layer(rng, K, N) if fmt == "q4_0" else w4g_layer(rng, K, N)
-    deq = lin.dequantized_dev().double()
+    deq = lin.ref_deq()
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
     bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
     y = torch.full((M, N), float("nan"), device="cuda")
@@ -97,8 +101,8 @@ def test_row_fused_parts_and_glu(M, xdt):
     for part, y in zip((q, k, v), outs):
         assert torch.equal(y, part.forward(x))
     gate, up = q4_layer(rng, IN, 2560), q4_layer(rng, IN, 2560)
-    g = x.double() @ gate.dequantized_dev().double().T
-    u = x.double() @ up.dequantized_dev().double().T
+    g = x.double() @ gate.ref_deq().T
+    u = x.double() @ up.ref_deq().T
     want = u * (g * torch.sigmoid(g))
     glu = FusedGLU(gate, up)
     y = glu.forward(x)
@@ -138,7 +142,7 @@ def test_default_dispatch_below_a_hundred_rows_over_large_layers():
         blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
         lin.set_blocks(blocks.reshape(-1))
         y = lin.forward(x)
-        exact = x.double() @ lin.dequantized_dev().double().T
+        exact = x.double() @ refw.q4_0(blocks, lin.OUT, K).T
         assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
         assert torch.equal(lin.forward(x), y)
     for part, y in zip((big, small), FusedRows([big, small]).forward(x)):
@@ -161,7 +165,7 @@ def test_default_dispatch_at_a_hundred_rows_follows_each_parts_own_rule(M):
             blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
             lin.set_blocks(blocks.reshape(-1))
             y = lin.forward(x)
-            exact = x.double() @ lin.dequantized_dev().double().T
+            exact = x.double() @ refw.q4_0(blocks, lin.OUT, K).T
             assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
             assert torch.equal(lin.forward(x), y)
         for part, y in zip(parts, FusedRows(parts).forward(x)):
@@ -189,17 +193,20 @@ def test_default_dispatch_by_estimate(fmt, K, N, M, xdt):
             sc = rng.uniform(1e-3, 1e-2, (n, K // 32)).astype(np.float16).view(np.uint16)
             blocks[:, :, 0], blocks[:, :, 1] = sc & 0xFF, sc >> 8
             lin.set_blocks(blocks.reshape(-1))
+            lin.ref_deq = lambda: refw.q4_0(blocks, n, K)
             return lin
         G = -(-K // 128)
         codes, zps = F.pack_w4g(rng.integers(0, 16, (n, K), dtype=np.uint8), rng.integers(0, 16, (n, G), dtype=np.uint8))
         lin = W4GroupLinear(K, n, 128)
-        lin.set_weight(codes, rng.uniform(1e-3, 1e-2, (n, G)).astype(np.float16), zps)
+        sg = rng.uniform(1e-3, 1e-2, (n, G)).astype(np.float16)
+        lin.set_weight(codes, sg, zps)
+        lin.ref_deq = lambda: refw.w4g(codes, sg, zps, n, K, 128)
         return lin
     x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).to(xdt).cuda()
     big, small = layer(N), layer(960)
     for lin in (big, small):
         y = lin.forward(x)
-        exact = x.double() @ lin.dequantized_dev().double().T
+        exact = x.double() @ lin.ref_deq().T
         assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max())
         assert torch.equal(lin.forward(x), y)
     for part, y in zip((big, small), FusedRows([big, small]).forward(x)):
