@@ -248,6 +248,69 @@ def make_q4_0(IN, OUT, M, copies, seed=3, bf16_x=False):
                 keep=(layers, x, y))
 
 
+def make_decoder_layer(M, adapters, copies=1, seed=11):
+    """The seven projections of one text layer of the reference's caller (960 wide, 320 k / v, 2560 MLP; Q4_0; fp32
+    activations; noeira/deep_agents/smolvla/fused.mojo:287-363) in the caller's order, each on its own input buffer:
+    `adapters` = "none": q|k|v fused, o, gate|up + SwiGLU fused, down - four launches;
+    "fused": the same groups with a rank-16 adapter on all seven (layer_weights.mojo:713-739): nq_forward_fused_lora for
+    q|k|v and for gate|up (SwiGLU applied to the sums), nq_forward_lora for o and down;
+    "per_projection": what the caller does today, seven `proj_fwd` = forward + forward_add, then SwiGLU left out."""
+    import numpy as np
+    import torch
+
+    from noeira_amd.lora import LoRAAdapter
+    from noeira_amd.qlinear import FusedGLU, FusedRows, QLinear
+
+    rng = np.random.default_rng(seed)
+    W, KV, FF = 960, 320, 2560
+
+    def q4(IN, OUT):
+        blocks = rng.integers(0, 256, OUT * (IN // 32) * 18, dtype=np.uint8)
+        sc = rng.uniform(1e-3, 2e-3, OUT * (IN // 32)).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        blocks.reshape(-1, 18)[:, 0:2] = sc
+        ql = QLinear.make(IN, OUT, "gpu")
+        ql.set_blocks(blocks)
+        return ql
+
+    def ad(IN, OUT):
+        a = LoRAAdapter(IN, OUT, 16, alpha=32.0)
+        a.set_params(((rng.random((IN, 16)) * 2 - 1) / np.sqrt(IN)).astype(np.float32),
+                     (rng.standard_normal((16, OUT)) * 0.05).astype(np.float32))
+        return a
+
+    shapes = [(W, W), (W, KV), (W, KV), (W, W), (W, FF), (W, FF), (FF, W)]  # q k v o gate up down
+    lin = [q4(i, o) for (i, o) in shapes]
+    ads = [ad(i, o) for (i, o) in shapes]
+    qkv, glu, pair = FusedRows(lin[0:3]), FusedGLU(lin[4], lin[5]), FusedRows(lin[4:6])
+    x = torch.from_numpy(rng.standard_normal((M, W)).astype(np.float32)).cuda()
+    h = torch.from_numpy(rng.standard_normal((M, FF)).astype(np.float32)).cuda()
+    yq = [torch.empty((M, n), device="cuda") for n in (W, KV, KV)]
+    yo, yd = torch.empty((M, W), device="cuda"), torch.empty((M, W), device="cuda")
+    gu = [torch.empty((M, FF), device="cuda") for _ in range(2)]
+    yg = torch.empty((M, FF), device="cuda")
+
+    if adapters == "none":
+        def step(i):
+            qkv.forward(x, outs=yq), lin[3].forward(x, out=yo), glu.forward(x, out=yg), lin[6].forward(h, out=yd)
+        launches = 4
+    elif adapters == "fused":
+        def step(i):
+            qkv.forward_lora(x, ads[0:3], outs=yq), ads[3].forward_with(lin[3], x, out=yo)
+            pair.forward_lora(x, ads[4:6], outs=gu, glu_out=yg), ads[6].forward_with(lin[6], h, out=yd)
+        launches = 8
+    else:
+        outs = [yq[0], yq[1], yq[2], yo, gu[0], gu[1], yd]
+
+        def step(i):
+            for l, a_, y in zip(lin, ads, outs):
+                xin = x if l.IN == W else h
+                l.forward(xin, out=y), a_.forward_add(xin, y)
+        launches = 14
+    wbytes = sum(o * (i // 32) * 18 for (i, o) in shapes)
+    return dict(step=step, bytes=wbytes + 4 * M * (2 * W + FF), ops=2 * M * sum(i * o for (i, o) in shapes), launches=launches,
+                keep=(lin, ads, qkv, glu, pair, x, h, yq, yo, yd, gu, yg))
+
+
 def make_q4_0_fused(IN, OUTS, M, copies, seed=7, bf16_x=False, glu=False, bf16_y=False):
     """The reference caller's q|k|v or gate|up projections as one row-fused launch; with `glu` the SwiGLU between
     gate | up and `down` (fused.mojo:337-353) runs in that launch's epilogue and one [M, H] tensor comes out."""
@@ -667,6 +730,13 @@ def sweep(skip_large=False):
         OUTS=[2560, 2560], M=135, copies=1, calls=20, glu=True)
     run("ref Q4_0 gate|up + SwiGLU 960->2560 one launch M=135 bf16 in / bf16 out (warm)", make_q4_0_fused, "mfma",
         "bf16", IN=960, OUTS=[2560, 2560], M=135, copies=1, calls=20, glu=True, bf16_x=True, bf16_y=True)
+    for M in (135, 1):
+        run(f"ref text layer, 7 Q4_0 projections M={M}: q|k|v, o, gate|up+SwiGLU, down (4 launches, no adapters)",
+            make_decoder_layer, "mfma", "bf16", M=M, adapters="none", calls=20)
+        run(f"ref text layer M={M} + rank-16 adapters on all seven, fused calls (8 launches)", make_decoder_layer, "mfma",
+            "bf16", M=M, adapters="fused", calls=20)
+        run(f"ref text layer M={M} + rank-16 adapters, per projection as the caller does (14 launches, SwiGLU not counted)",
+            make_decoder_layer, "mfma", "bf16", M=M, adapters="per_projection", calls=20)
     run("cfg4 W8A8 actor 64->256->256->8 M=4096 (fused, 1 launch)", make_actor_fused, "mfma", "int8", calls=20)
     run("cfg4 W8A8 actor 64->256->256->8 M=4096 (unfused, 6 launches)", make_actor_w8a8, "mfma", "int8", calls=20)
     for N in (4096, 11008):

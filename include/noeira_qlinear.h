@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define NQ_ABI_VERSION 5
+#define NQ_ABI_VERSION 6
 
 /* status codes */
 #define NQ_OK 0
@@ -273,6 +273,30 @@ int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features,
 int32_t nq_forward_lora(nq_handle h, const void* x, int32_t x_dtype, void* y, int32_t y_dtype, int32_t M,
                         const void* bias, int32_t bias_dtype, const float* lora_a, const float* lora_b, int32_t r_pad,
                         float scale, void* stream);
+
+/* One frozen adapter of a fused call: the device parameters and scale nq_lora_forward_add takes; a = b = NULL: the
+ * part has none (the caller's `Optional` adapter slots, noeira/deep_agents/smolvla/layer_weights.mojo:713-739). */
+typedef struct nq_lora_part {
+    const float* a;   /* [IN, R_PAD] fp32 */
+    const float* b;   /* [R_PAD, OUT_t] fp32 */
+    int32_t r_pad;
+    float scale;
+} nq_lora_part;
+
+/* nq_forward_fused of a layer made by nq_fuse_rows, with one adapter per part: what the reference's caller does per
+ * projection - `proj_fwd` = base linear, then `LoRAAdapter.forward_add` (layer_weights.mojo:455-508; q | k | v and
+ * gate | up read the same activations, fused.mojo:287-363) - as two launches for the whole group:
+ *     ys[t][M, OUT_t] = x @ deq(W_t)^T + bias_t + scale_t * (x @ A_t) @ B_t        (fp32)
+ * the base call of nq_forward_fused, then ONE launch that adds every part's share (R_PAD = 16, IN a multiple of 32,
+ * OUT_t multiples of 4 and 16-byte aligned operands; otherwise one adding launch per part).  B_t = 0, or no adapter,
+ * leaves the bits of nq_forward_fused.  x fp32 or bf16; adapters[n_ys].
+ * glu_out != NULL: the layer's two parts are gate and up of one MLP (equal widths, no bias).  The adding launch then
+ * also writes glu_out[M, OUT] = up * silu(gate) (`SwiGLU.forward`, noeira/nn/primitives/swiglu.mojo:41-60; fp32 or
+ * bf16 by glu_dtype) from the sums it formed, and ys[0], ys[1] keep the base projections: they are scratch the caller
+ * lends (the adapters act before the activation, which is why a layer made by nq_fuse_glu cannot take them). */
+int32_t nq_forward_fused_lora(nq_handle h, const void* x, int32_t x_dtype, float* const* ys, int32_t n_ys, int32_t M,
+                              const void* bias, int32_t bias_dtype, const nq_lora_part* adapters, void* glu_out,
+                              int32_t glu_dtype, void* stream);
 
 /* ---- GPTQ onto the Q4_0 grid (load time; noeira/nn/quant/gptq.mojo) ------------------------ */
 

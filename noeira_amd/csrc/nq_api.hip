@@ -775,6 +775,52 @@ int32_t nq_forward_lora(nq_handle h, const void* x, int32_t x_dtype, void* y, in
                                stream);
 }
 
+int32_t nq_forward_fused_lora(nq_handle h, const void* x, int32_t x_dtype, float* const* ys, int32_t n_ys, int32_t M,
+                              const void* bias, int32_t bias_dtype, const nq_lora_part* adapters, void* glu_out,
+                              int32_t glu_dtype, void* stream) {
+    int32_t rc = check_handle(h, "nq_forward_fused_lora");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    const int parts = nq_fused_parts(h);
+    if (h->glu) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: a layer made by nq_fuse_glu applies SwiGLU before an adapter "
+                                            "could add its share; fuse gate and up with nq_fuse_rows and pass glu_out");
+    if (n_ys != parts)
+        return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: " + std::to_string(n_ys) + " outputs for a layer of " +
+                                        std::to_string(parts) + " fused parts");
+    if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: M must be >= 0");
+    if (M == 0) return NQ_OK;
+    if (!x || !ys || !adapters) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: null pointer");
+    if (x_dtype != NQ_DT_F32 && x_dtype != NQ_DT_BF16)
+        return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: x must be fp32 or bf16");
+    SegTable seg{};
+    seg.nseg = parts;
+    LoraPartArgs lp[4];
+    int r0 = 0;
+    for (int t = 0; t < parts; t++) {
+        seg.end[t] = h->seg_end.empty() ? h->out : h->seg_end[t];
+        seg.y[t] = ys[t];
+        if (!ys[t]) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: null output");
+        const nq_lora_part& ad = adapters[t];
+        if ((ad.a == nullptr) != (ad.b == nullptr) || (ad.a && ad.r_pad <= 0))
+            return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: an adapter is (a, b, r_pad > 0) or all null");
+        const int width = seg.end[t] - r0;
+        if ((int64_t)M * h->in >= ((int64_t)1 << 32) || (int64_t)M * width >= ((int64_t)1 << 32))
+            return fail(NQ_ERR_UNSUPPORTED, "nq_forward_fused_lora: M * IN and M * OUT must stay below 2^32");
+        lp[t] = LoraPartArgs{ad.a, ad.b, ys[t], width, ad.r_pad, ad.scale};
+        r0 = seg.end[t];
+    }
+    if (glu_out) {
+        if (parts != 2 || lp[0].out != lp[1].out)
+            return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: glu_out needs a layer of two parts of equal width (gate, up)");
+        if (glu_dtype != NQ_DT_F32 && glu_dtype != NQ_DT_BF16)
+            return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: glu_out must be fp32 or bf16");
+        if (bias) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: a SwiGLU pair takes no bias");
+    }
+    rc = forward_impl(h, x, x_dtype, nullptr, seg, NQ_DT_F32, M, bias, bias_dtype, NQ_EPI_NONE, stream);
+    if (rc) return rc;
+    return launch_lora_multi(x, x_dtype, M, h->in, parts, lp, glu_out, glu_dtype, (hipStream_t)stream);
+}
+
 int32_t nq_lora_forward_add(const float* a, const float* b, int32_t in_features, int32_t out_features, int32_t r_pad,
                             float scale, const void* x, int32_t x_dtype, float* y, int32_t T, void* stream) {
     if (in_features <= 0 || out_features <= 0 || r_pad <= 0)

@@ -221,6 +221,18 @@ int32_t launch_slice_cast_f32(const uint16_t* src, float* dst, int32_t rows, int
 // nq_lora.hip: y += s (x A) B
 int32_t launch_lora_add(const void* x, int32_t x_dtype, const float* A, const float* B, float* y, int32_t T, int32_t IN,
                         int32_t OUT, int32_t R, float s, hipStream_t stream);
+// the adapters of a row-fused layer's parts, added into the parts' fp32 outputs in one launch (b null: the part has
+// none); glu_out non-null: two parts of equal width, gate and up - their sums go through SwiGLU into glu_out
+struct LoraPartArgs {
+    const float* a;
+    const float* b;
+    float* y;
+    int32_t out;
+    int32_t r;
+    float s;
+};
+int32_t launch_lora_multi(const void* x, int32_t x_dtype, int32_t T, int32_t IN, int32_t n, const LoraPartArgs* parts, void* glu_out,
+                          int32_t glu_dtype, hipStream_t stream);
 
 // nq_gptq.hip: the calibration Hessian, the factor of its inverse, GPTQ's column loop, its objective
 int32_t launch_hessian_add(double* H, int n, const void* x, int32_t x_dtype, int rows, hipStream_t s);

@@ -21,6 +21,12 @@ namespace {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float v) {  // round to nearest even, NaN stays NaN
+    const uint32_t bits = __float_as_uint(v);
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+
 constexpr int LR_ROWS = 16;   // tokens per workgroup
 constexpr int LR_COLS = 256;  // output columns per workgroup
 constexpr int LR_R = 16;      // adapter columns handled per pass
@@ -154,10 +160,12 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 constexpr int L16_NB = 4;  // chunks of 32 k whose loads are in flight together, per wavefront
 
+// The adapter's share of one tile: out[i][e] = sum_r (x A)[m0 + 2 rp + i][r] B[r][ncl + e] for thread (cq, rp) of the
+// workgroup (unscaled; the caller adds s * out into what it loaded of y).  Uses the workgroup's LDS; a caller that runs
+// it twice puts a barrier between the runs.
 template <bool XBF16>
-__global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* __restrict__ xv, const float* __restrict__ A,
-                                                                   const float* __restrict__ B, float* __restrict__ y, int T,
-                                                                   int IN, int OUT, float s) {
+__device__ __forceinline__ void lora16_tile(const void* __restrict__ xv, const float* __restrict__ A, const float* __restrict__ B,
+                                            int T, int IN, int OUT, int m0, int ncl, f32x4 (&out)[2]) {
     constexpr int NT = XBF16 ? 1 : 3;
     __shared__ float part[LR_WAVES][LR_ROWS][LR_R + 1];
     __shared__ __attribute__((aligned(16))) float h[LR_ROWS][LR_R];
@@ -165,18 +173,11 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* _
     __shared__ __attribute__((aligned(16))) float bt[LR_R][LR_COLS];      // the tile of B
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, q = lane >> 4;
-    const int m0 = blockIdx.y * LR_ROWS, n0 = blockIdx.x * LR_COLS;
-    // second phase: thread (column quad cq, row pair rp) owns y[m0 + 2 rp .. + 1][n0 + 4 cq .. + 3]
     const int cq = tid & 63, rp = tid >> 6;
-    const bool cols_in = n0 + 4 * cq < OUT;  // (OUT is a multiple of 4: a quad is inside or outside)
-    const int ncl = min(n0 + 4 * cq, OUT - 4);
-    // requested first, used last: the tile of y and the tile of B (rows 2 rp, 2 rp + 1 of it per thread)
-    f32x4 yv[2], bv[2];
+    // requested first, used last: the tile of B (rows 2 rp, 2 rp + 1 of it per thread)
+    f32x4 bv[2];
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        yv[i] = *reinterpret_cast<const f32x4*>(y + (int64_t)min(m0 + 2 * rp + i, T - 1) * OUT + ncl);
-        bv[i] = *reinterpret_cast<const f32x4*>(B + (int64_t)(2 * rp + i) * OUT + ncl);
-    }
+    for (int i = 0; i < 2; i++) bv[i] = *reinterpret_cast<const f32x4*>(B + (int64_t)(2 * rp + i) * OUT + ncl);
 
     // ---- h = x A: wavefront w takes the chunks w, w + 8, ... of 32 k, L16_NB of them under way at a time
     const int nch = IN >> 5;
@@ -267,8 +268,8 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* _
         h[m][rr] = t;
     }
     __syncthreads();
-    // ---- y[m][n] += s sum_r h[m][r] B[r][n], r ascending
-    f32x4 out[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    // ---- sum_r h[m][r] B[r][n], r ascending
+    out[0] = out[1] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int r4 = 0; r4 < LR_R; r4 += 4) {
         const f32x4 h0 = *reinterpret_cast<const f32x4*>(&h[2 * rp][r4]), h1 = *reinterpret_cast<const f32x4*>(&h[2 * rp + 1][r4]);
@@ -279,6 +280,24 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* _
             for (int e = 0; e < 4; e++) out[0][e] = fmaf(h0[rr], bq[e], out[0][e]), out[1][e] = fmaf(h1[rr], bq[e], out[1][e]);
         }
     }
+}
+
+template <bool XBF16>
+__global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* __restrict__ xv, const float* __restrict__ A,
+                                                                   const float* __restrict__ B, float* __restrict__ y, int T,
+                                                                   int IN, int OUT, float s) {
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * LR_ROWS, n0 = blockIdx.x * LR_COLS;
+    // second phase: thread (column quad cq, row pair rp) owns y[m0 + 2 rp .. + 1][n0 + 4 cq .. + 3]
+    const int cq = tid & 63, rp = tid >> 6;
+    const bool cols_in = n0 + 4 * cq < OUT;  // (OUT is a multiple of 4: a quad is inside or outside)
+    const int ncl = min(n0 + 4 * cq, OUT - 4);
+    // requested first, used last: the tile of y
+    f32x4 yv[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) yv[i] = *reinterpret_cast<const f32x4*>(y + (int64_t)min(m0 + 2 * rp + i, T - 1) * OUT + ncl);
+    f32x4 out[2];
+    lora16_tile<XBF16>(xv, A, B, T, IN, OUT, m0, ncl, out);
     if (cols_in) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
@@ -289,6 +308,115 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* _
             *reinterpret_cast<f32x4*>(y + (int64_t)(m0 + 2 * rp + i) * OUT + ncl) = z;
         }
     }
+}
+
+// ---- the adapters of a row-fused layer's parts in one launch ------------------------------------------------------
+// (the caller's q | k | v and gate | up: `DecoderLayerWeights` keeps one adapter per projection, layer_weights.mojo:713-739.)
+// A workgroup looks its part up by its column-tile index and does what lora_add16_kernel does for that part.  GLU: the
+// layer's two parts are gate and up of one MLP; a workgroup takes the same column tile of both, adds each adapter's
+// share to the base projections it reads from ys[0] and ys[1] (which stay as they are) and writes
+// up * silu(gate) (`SwiGLU.forward`, swiglu.mojo:41-60): the adapters act before the activation, so this is where a
+// trailing launch can still apply it.
+struct LoraPartDev {
+    const float* a;
+    const float* b;   // null: the part has no adapter (its tiles return at once; GLU: its share is zero)
+    float* y;
+    int32_t out;
+    int32_t tile0;    // the part's first column tile in the grid
+    float s;
+};
+struct LoraMultiDev {
+    LoraPartDev p[4];
+    int32_t n;
+};
+
+template <bool XBF16, bool GLU>
+__global__ __launch_bounds__(64 * LR_WAVES) void lora_multi16_kernel(const void* __restrict__ xv, const LoraMultiDev mp, int T, int IN,
+                                                                     void* __restrict__ glu_out, int glu_dtype) {
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * LR_ROWS;
+    const int cq = tid & 63, rp = tid >> 6;
+    if constexpr (!GLU) {
+        // (constant indices: the table stays in scalar registers)
+        LoraPartDev me = mp.p[0];
+        if (mp.n > 1 && (int)blockIdx.x >= mp.p[1].tile0) me = mp.p[1];
+        if (mp.n > 2 && (int)blockIdx.x >= mp.p[2].tile0) me = mp.p[2];
+        if (mp.n > 3 && (int)blockIdx.x >= mp.p[3].tile0) me = mp.p[3];
+        if (!me.b) return;
+        const int n0 = ((int)blockIdx.x - me.tile0) * LR_COLS;
+        const bool cols_in = n0 + 4 * cq < me.out;
+        const int ncl = min(n0 + 4 * cq, me.out - 4);
+        f32x4 yv[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) yv[i] = *reinterpret_cast<const f32x4*>(me.y + (int64_t)min(m0 + 2 * rp + i, T - 1) * me.out + ncl);
+        f32x4 out[2];
+        lora16_tile<XBF16>(xv, me.a, me.b, T, IN, me.out, m0, ncl, out);
+        if (cols_in) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                if (m0 + 2 * rp + i >= T) break;
+                f32x4 z;
+#pragma unroll
+                for (int e = 0; e < 4; e++) z[e] = fmaf(me.s, out[i][e], yv[i][e]);
+                *reinterpret_cast<f32x4*>(me.y + (int64_t)(m0 + 2 * rp + i) * me.out + ncl) = z;
+            }
+        }
+    } else {
+        const int OUT = mp.p[0].out;
+        const int n0 = (int)blockIdx.x * LR_COLS;
+        const bool cols_in = n0 + 4 * cq < OUT;
+        const int ncl = min(n0 + 4 * cq, OUT - 4);
+        f32x4 g[2], u[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int64_t at = (int64_t)min(m0 + 2 * rp + i, T - 1) * OUT + ncl;
+            g[i] = *reinterpret_cast<const f32x4*>(mp.p[0].y + at), u[i] = *reinterpret_cast<const f32x4*>(mp.p[1].y + at);
+        }
+        f32x4 out[2];
+        if (mp.p[0].b) {  // (uniform)
+            lora16_tile<XBF16>(xv, mp.p[0].a, mp.p[0].b, T, IN, OUT, m0, ncl, out);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) g[i][e] = fmaf(mp.p[0].s, out[i][e], g[i][e]);
+            __syncthreads();
+        }
+        if (mp.p[1].b) {
+            lora16_tile<XBF16>(xv, mp.p[1].a, mp.p[1].b, T, IN, OUT, m0, ncl, out);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) u[i][e] = fmaf(mp.p[1].s, out[i][e], u[i][e]);
+        }
+        if (cols_in) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                if (m0 + 2 * rp + i >= T) break;
+                f32x4 z;
+#pragma unroll
+                for (int e = 0; e < 4; e++) z[e] = swiglu_f32(u[i][e], g[i][e]);
+                const int64_t at = (int64_t)(m0 + 2 * rp + i) * OUT + ncl;
+                if (glu_dtype == NQ_DT_F32) {
+                    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(glu_out) + at) = z;
+                } else {
+                    uint2 pk;
+                    pk.x = (uint32_t)f32_to_bf16_bits(z[0]) | ((uint32_t)f32_to_bf16_bits(z[1]) << 16);
+                    pk.y = (uint32_t)f32_to_bf16_bits(z[2]) | ((uint32_t)f32_to_bf16_bits(z[3]) << 16);
+                    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(glu_out) + at) = pk;
+                }
+            }
+        }
+    }
+}
+
+// up * silu(gate) over n values (the path of last resort: adapters the fast kernel does not take, then this)
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ g, const float* __restrict__ u, void* __restrict__ out,
+                                                     int64_t n, int dtype) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float z = swiglu_f32(u[i], g[i]);
+    if (dtype == NQ_DT_F32) reinterpret_cast<float*>(out)[i] = z;
+    else reinterpret_cast<uint16_t*>(out)[i] = f32_to_bf16_bits(z);
 }
 
 }  // namespace
@@ -314,6 +442,46 @@ int32_t launch_lora_add(const void* x, int32_t x_dtype, const float* A, const fl
     }
 #undef NQ_LORA
     NQ_HIP(hipGetLastError());
+    return NQ_OK;
+}
+
+int32_t launch_lora_multi(const void* x, int32_t x_dtype, int32_t T, int32_t IN, int32_t n, const LoraPartArgs* parts, void* glu_out,
+                          int32_t glu_dtype, hipStream_t stream) {
+    const auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    const bool bf = x_dtype == NQ_DT_BF16;
+    bool fast = IN % 32 == 0 && al16(x) && (!glu_out || al16(glu_out));
+    for (int t = 0; t < n; t++)
+        fast = fast && parts[t].out % 4 == 0 && al16(parts[t].y) && (!parts[t].b || (parts[t].r == LR_R && al16(parts[t].a) && al16(parts[t].b)));
+    if (fast) {
+        LoraMultiDev mp{};
+        mp.n = n;
+        int tiles = 0;
+        for (int t = 0; t < n; t++) {
+            mp.p[t] = LoraPartDev{parts[t].a, parts[t].b, parts[t].y, parts[t].out, tiles, parts[t].s};
+            tiles += (parts[t].out + LR_COLS - 1) / LR_COLS;
+        }
+        const dim3 grid(glu_out ? (parts[0].out + LR_COLS - 1) / LR_COLS : tiles, (T + LR_ROWS - 1) / LR_ROWS);
+#define NQ_LM(BF, GLU) \
+    hipLaunchKernelGGL((lora_multi16_kernel<BF, GLU>), grid, dim3(64 * LR_WAVES), 0, stream, x, mp, T, IN, glu_out, glu_dtype)
+        if (glu_out) {
+            if (bf) NQ_LM(true, true); else NQ_LM(false, true);
+        } else {
+            if (bf) NQ_LM(true, false); else NQ_LM(false, false);
+        }
+#undef NQ_LM
+        NQ_HIP(hipGetLastError());
+        return NQ_OK;
+    }
+    for (int t = 0; t < n; t++) {
+        if (!parts[t].b) continue;
+        const int32_t rc = launch_lora_add(x, x_dtype, parts[t].a, parts[t].b, parts[t].y, T, IN, parts[t].out, parts[t].r, parts[t].s, stream);
+        if (rc) return rc;
+    }
+    if (glu_out) {
+        const int64_t cnt = (int64_t)T * parts[0].out;
+        hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((cnt + 255) / 256)), dim3(256), 0, stream, parts[0].y, parts[1].y, glu_out, cnt, glu_dtype);
+        NQ_HIP(hipGetLastError());
+    }
     return NQ_OK;
 }
 

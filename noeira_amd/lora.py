@@ -85,3 +85,17 @@ class LoRAAdapter:
                                         _dev_ptr(self.lora_A), _dev_ptr(self.lora_B), self.R_PAD,
                                         C.c_float(self.scale()), _stream_ptr()))
         return y
+
+
+def proj_fwd(base, x: torch.Tensor, adapter: "LoRAAdapter | None" = None, hessian=None, bias: torch.Tensor | None = None,
+             out: torch.Tensor | None = None) -> torch.Tensor:
+    """One projection of the decoder layer as the reference's caller runs it, `DecoderLayerWeights.proj_fwd`
+    (noeira/deep_agents/smolvla/layer_weights.mojo:455-508): when calibrating, the projection's input is added to
+    its Hessian first (`HessianAccumulator.add`, hessian.mojo:41-77: `hessian` is a `noeira_amd.gptq.HessianAccumulator` or
+    None); then the base linear; then the adapter's share, if the projection carries an unmerged one.  x: fp32 or
+    bf16 [T, IN] on the device; returns fp32 [T, OUT]."""
+    if hessian is not None:
+        hessian.add(x)
+    if adapter is None or adapter.merged:
+        return base.forward(x, bias=bias, out=out) if bias is not None or out is not None else base.forward(x)
+    return adapter.forward_with(base, x, bias=bias, out=out)

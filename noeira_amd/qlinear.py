@@ -439,6 +439,51 @@ class FusedRows:
         return outs
 
 
+    def forward_lora(self, x: torch.Tensor, adapters, outs=None, bias=None, glu_out: Optional[torch.Tensor] = None,
+                     glu_dtype: Optional[torch.dtype] = None):
+        """`forward` with one frozen adapter per part (`nq_forward_fused_lora`): the caller's per-projection
+        `proj_fwd` = base linear + `LoRAAdapter.forward_add` (layer_weights.mojo:455-508) for a whole group in two
+        launches.  `adapters`: one `LoRAAdapter` (or None, or a merged one: no share) per part.  Returns the list of
+        fp32 per-part outputs; with `glu_dtype` (or `glu_out`) the two parts are gate and up of one MLP and the
+        call returns up * silu(gate) instead ([M, OUT]; the per-part outputs are then scratch holding the base
+        projections)."""
+        if x.dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward_lora: x must be fp32 or bf16")
+        M = _check_x(x, self.IN, "FusedRows.forward_lora")
+        adapters = list(adapters)
+        if len(adapters) != len(self.OUTS):
+            raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward_lora: one adapter (or None) per part")
+        if outs is None:
+            outs = [torch.empty((M, n), dtype=torch.float32, device=x.device) for n in self.OUTS]
+        if any(o.dtype != torch.float32 or not o.is_cuda for o in outs):
+            raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward_lora: the per-part outputs are fp32 device tensors")
+        table = (L.LoraPart * len(adapters))()
+        for t, ad in enumerate(adapters):
+            if ad is None or ad.merged:
+                table[t] = L.LoraPart(None, None, 0, 0.0)
+                continue
+            if ad.IN != self.IN or ad.OUT != self.OUTS[t]:
+                raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward_lora: adapter %d does not fit its part" % t)
+            table[t] = L.LoraPart(ad.lora_A.data_ptr(), ad.lora_B.data_ptr(), ad.R_PAD, ad.scale())
+        b_dt = L.DT_F32
+        if bias is not None:
+            if bias.dtype not in _TORCH_DT or bias.numel() != self.OUT or not bias.is_cuda:
+                raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward_lora: bias must be a device fp32/bf16 tensor of "
+                                                  "sum(OUT) values")
+            b_dt = _TORCH_DT[bias.dtype]
+        want_glu = glu_out is not None or glu_dtype is not None
+        if want_glu:
+            if glu_out is None:
+                glu_out = torch.empty((M, self.OUTS[0]), dtype=glu_dtype, device=x.device)
+            if glu_out.dtype not in _TORCH_DT or glu_out.numel() < M * self.OUTS[0]:
+                raise L.NQError(L.NQ_ERR_INVALID, "FusedRows.forward_lora: glu_out must be an fp32/bf16 [M, OUT] tensor")
+        ys = (C.c_void_p * len(outs))(*[_dev_ptr(o) for o in outs])
+        L.check(L.lib().nq_forward_fused_lora(self._h, _dev_ptr(x), _TORCH_DT[x.dtype], ys, len(outs), M, _dev_ptr(bias),
+                                              b_dt, table, _dev_ptr(glu_out) if want_glu else C.c_void_p(0),
+                                              _TORCH_DT[glu_out.dtype] if want_glu else L.DT_F32, _stream_ptr()))
+        return glu_out if want_glu else outs
+
+
 class FusedGLU:
     """gate | up of a decoder MLP with the SwiGLU between them and `down` in ONE launch (nq_fuse_glu): the
     reference's caller runs two projections, a concatenation and `SwiGLU.forward`

@@ -173,3 +173,142 @@ def test_qlora_one_call_bf16_out_and_errors():
     assert bool((ybn == 7.0).all())
     with pytest.raises(L.NQError, match="differ in shape"):
         adn.forward_with(base, x)
+
+
+# ── adapters on row-fused layers: a decoder layer's projections with all seven adapters ─────────────────────────
+def _q4(rng, IN, OUT):
+    w = (rng.standard_normal((OUT, IN)) * 0.05).astype(np.float32)
+    lin = QLinear(IN, OUT)
+    lin.set_weight(w)
+    return lin
+
+
+def _oracle_proj(lin, x_host, ad):
+    """`proj_fwd` on the CPU: the oracle's QLinear forward, then its adapter's share (a, b logical blocks)."""
+    want = O.qlinear_forward_cpu(lin.blocks(), lin.IN, lin.OUT, x_host)
+    if ad is not None:
+        adapter, a, b = ad
+        want = O.lora_forward_add(x_host, a, b, adapter.scale(), want)
+    return want
+
+
+@pytest.mark.parametrize("T", [1, 17, 135])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_fused_rows_with_an_adapter_per_part(T, xdt):
+    """q | k | v of the caller's text layer (960 -> 960 / 320 / 320) with R = 16 adapters on all three: every output
+    is `LoRAAdapter.forward_add` over `QLinear.forward` (oracle, 1e-5 of the largest value); B = 0 on every part, and
+    no adapter at all, leave the bits of the adapter-free fused call; a part without an adapter keeps its base bits
+    while its neighbours get their shares."""
+    from noeira_amd.qlinear import FusedRows
+
+    rng = np.random.default_rng(1000 + T)
+    IN, outs = 960, (960, 320, 320)
+    parts = [_q4(rng, IN, n) for n in outs]
+    fused = FusedRows(parts)
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).to(xdt).cuda()
+    xh = x.float().cpu().numpy()
+    base = [y.clone() for y in fused.forward(x)]
+    ads = [make(rng, IN, n, 16) for n in outs]
+    got = fused.forward_lora(x, [ad[0] for ad in ads])
+    for lin, ad, y in zip(parts, ads, got):
+        want = _oracle_proj(lin, xh, ad)
+        assert O.rel_max(y.cpu().numpy(), want) < BAND
+    zero = [make(rng, IN, n, 16, zero_b=True)[0] for n in outs]
+    for y, yb in zip(fused.forward_lora(x, zero), base):
+        assert torch.equal(y, yb)
+    for y, yb in zip(fused.forward_lora(x, [None, None, None]), base):
+        assert torch.equal(y, yb)
+    mixed = fused.forward_lora(x, [ads[0][0], None, ads[2][0]])
+    assert torch.equal(mixed[1], base[1])
+    assert torch.equal(mixed[0], got[0]) and torch.equal(mixed[2], got[2])
+    # a repeated call returns the same bits
+    for y, y2 in zip(fused.forward_lora(x, [ad[0] for ad in ads]), got):
+        assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("T", [1, 135])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+def test_gate_up_with_adapters_through_swiglu(T, gdt):
+    """gate | up (960 -> 2560 each) with an adapter on both and the SwiGLU applied to the SUMS, as the reference's
+    caller orders it (fused.mojo:337-353: `proj_fwd[LORA_GATE]`, `proj_fwd[LORA_UP]`, then `glu`): against the
+    oracle's projections, adapters and `swiglu`; with B = 0 the result is the adapter-free pair's SwiGLU."""
+    from noeira_amd.qlinear import FusedRows
+
+    rng = np.random.default_rng(2000 + T)
+    IN, H = 960, 2560
+    gate, up = _q4(rng, IN, H), _q4(rng, IN, H)
+    pair = FusedRows([gate, up])
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).cuda()
+    xh = x.cpu().numpy()
+    adg, adu = make(rng, IN, H, 16), make(rng, IN, H, 16)
+    out = pair.forward_lora(x, [adg[0], adu[0]], glu_dtype=gdt)
+    assert out.shape == (T, H) and out.dtype == gdt
+    want = O.swiglu(_oracle_proj(up, xh, adu), _oracle_proj(gate, xh, adg))
+    tol = BAND if gdt == torch.float32 else 2.0 ** -8 + BAND
+    assert O.rel_max(out.float().cpu().numpy(), want) < tol
+    g0, u0 = pair.forward(x)
+    zg, zu = make(rng, IN, H, 16, zero_b=True)[0], make(rng, IN, H, 16, zero_b=True)[0]
+    out0 = pair.forward_lora(x, [zg, zu], glu_dtype=torch.float32)
+    # (the base projections' own bits through SwiGLU; the device's exp and the oracle's differ in the last bit)
+    assert O.rel_max(out0.cpu().numpy(), O.swiglu(u0.cpu().numpy(), g0.cpu().numpy())) < 1e-6
+    assert torch.equal(out0, pair.forward_lora(x, [None, None], glu_dtype=torch.float32))
+    # only one of the two carries an adapter
+    out1 = pair.forward_lora(x, [None, adu[0]], glu_dtype=torch.float32)
+    want1 = O.swiglu(_oracle_proj(up, xh, adu), _oracle_proj(gate, xh, None))
+    assert O.rel_max(out1.cpu().numpy(), want1) < BAND
+
+
+def test_fused_adapters_outside_the_fast_kernel_and_errors():
+    """Ranks and widths the 16-byte kernel does not take (R_PAD = 8, a part 70 wide) go part by part through the
+    general kernel, the SwiGLU through its own launch: the same values.  A GLU-fused layer refuses adapters."""
+    from noeira_amd.qlinear import FusedGLU, FusedRows
+
+    rng = np.random.default_rng(77)
+    IN, T = 96, 9
+    a_, b_ = _q4(rng, IN, 70), _q4(rng, IN, 128)
+    fused = FusedRows([a_, b_])
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).cuda()
+    xh = x.cpu().numpy()
+    ads = [make(rng, IN, 70, 3, pad=8), make(rng, IN, 128, 16)]
+    for lin, ad, y in zip((a_, b_), ads, fused.forward_lora(x, [ad[0] for ad in ads])):
+        assert O.rel_max(y.cpu().numpy(), _oracle_proj(lin, xh, ad)) < BAND
+    g, u = _q4(rng, IN, 64), _q4(rng, IN, 64)
+    pair = FusedRows([g, u])
+    adg, adu = make(rng, IN, 64, 3, pad=8), make(rng, IN, 64, 3, pad=8)
+    out = pair.forward_lora(x, [adg[0], adu[0]], glu_dtype=torch.float32)
+    want = O.swiglu(_oracle_proj(u, xh, adu), _oracle_proj(g, xh, adg))
+    assert O.rel_max(out.cpu().numpy(), want) < BAND
+    with pytest.raises(L.NQError, match="equal width"):
+        fused.forward_lora(x, [None, None], glu_dtype=torch.float32)
+    with pytest.raises(L.NQError, match="per part"):
+        fused.forward_lora(x, [None])
+    glu = FusedGLU(g, u)
+    table = (L.LoraPart * 1)(L.LoraPart(None, None, 0, 0.0))
+    import ctypes as C
+    ys = (C.c_void_p * 1)(out.data_ptr())
+    rc = L.lib().nq_forward_fused_lora(glu._h, x.data_ptr(), L.DT_F32, ys, 1, T, None, L.DT_F32, table, None, L.DT_F32, None)
+    assert rc == L.NQ_ERR_INVALID
+
+
+def test_proj_fwd_taps_the_hessian_then_runs_base_and_adapter():
+    """`DecoderLayerWeights.proj_fwd` (layer_weights.mojo:455-508): with calibration on, the projection's input goes
+    into its Hessian first; then the base linear; then the adapter's share."""
+    from noeira_amd.gptq import HessianAccumulator
+    from noeira_amd.lora import proj_fwd
+
+    rng = np.random.default_rng(31)
+    IN, OUT, T = 192, 96, 11
+    lin = _q4(rng, IN, OUT)
+    ad = make(rng, IN, OUT, 4)
+    x = torch.from_numpy(rng.standard_normal((T, IN)).astype(np.float32)).cuda()
+    xh = x.cpu().numpy()
+    hs = HessianAccumulator(IN)
+    y = proj_fwd(lin, x, adapter=ad[0], hessian=hs)
+    assert O.rel_max(y.cpu().numpy(), _oracle_proj(lin, xh, ad)) < BAND
+    assert hs.rows == T
+    want_h = O.hessian_add(np.zeros((IN, IN), np.float64), xh)
+    assert np.array_equal(hs.h.view(np.uint64), want_h.view(np.uint64))
+    # no adapter, no tap: the bare linear's bits
+    assert torch.equal(proj_fwd(lin, x), lin.forward(x))
+    ad[0].merged = True
+    assert torch.equal(proj_fwd(lin, x, adapter=ad[0]), lin.forward(x))
