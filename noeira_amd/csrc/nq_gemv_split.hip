@@ -139,10 +139,11 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
 #pragma unroll
     for (int w = 0; w < WAVES; w++) mbits = max(mbits, wmax[w]);
     const bool finite = mbits < 0x7F800000u;
-    const float absmax = __uint_as_float(mbits);
-    // (below 1e-30 the reciprocal would overflow: such a row counts as zero, an error below 1e-30 * sum |w|)
-    const float inv_s = (finite && absmax > 1e-30f) ? 127.0f / absmax : 0.0f;
-    const float s_x = inv_s != 0.0f ? absmax * (1.0f / 127.0f) : 0.0f;
+    // (a row below 2^-60 is lifted by 2^64 first, exactly: 127 / absmax then stays finite and the row keeps its terms)
+    const float lift = mbits < 0x21800000u ? 0x1p64f : 1.0f;
+    const float absmax = __uint_as_float(mbits) * lift;
+    const float inv_s = (finite && absmax > 0.0f) ? 127.0f / absmax : 0.0f;
+    const float s_x = inv_s != 0.0f ? (absmax * (1.0f / 127.0f)) / lift : 0.0f;
 
     if (tid < NUNIT) {
         uint32_t* const x0 = reinterpret_cast<uint32_t*>(xs[0]) + tid * (EPT / 4);
@@ -161,7 +162,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void gemv_split8_kernel(const SplitP
                     // Round by adding 1.5 * 2^23 (the sum's low byte is the int8), and take every leftover against
                     // the very integer that was packed: the second and third term round the exact product
                     // (one fma each), so that no leftover exceeds a half and no term leaves the int8 range.
-                    const float t = xf[4 * q + e] * inv_s;
+                    const float t = (xf[4 * q + e] * lift) * inv_s;
                     const float b1 = t + MAGIC;
                     a1[e] = __float_as_uint(b1);
                     const float r1 = t - (b1 - MAGIC);

@@ -1002,15 +1002,18 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile4i_kernel(const TileParams p
             mbits = max(sw[0], sw[1]);
         }
         const bool finite = mbits < 0x7F800000u;
-        const float absmax = __uint_as_float(mbits);
-        const float inv_s = (finite && absmax > 1e-30f) ? 127.0f / absmax : 0.0f;
-        s_x = finite ? (inv_s != 0.0f ? absmax * (1.0f / 127.0f) : 0.0f) : __uint_as_float(0x7FC00000u);
+        // a slice whose largest magnitude is below 2^-60 is lifted by 2^64 first (exact), so that 127 / absmax stays
+        // finite and the slice keeps its three terms (an all-tiny x is still a vector with a direction)
+        const float lift = mbits < 0x21800000u ? 0x1p64f : 1.0f;
+        const float absmax = __uint_as_float(mbits) * lift;
+        const float inv_s = (finite && absmax > 0.0f) ? 127.0f / absmax : 0.0f;
+        s_x = finite ? (absmax * (1.0f / 127.0f)) / lift : __uint_as_float(0x7FC00000u);
         uint32_t a1[8], a2[8], a3[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             // round by adding 1.5 * 2^23 (the sum's low byte is the int8) and take every leftover against the very
             // integer that was packed: no leftover exceeds a half, no term leaves the int8 range
-            const float t = xf[e] * inv_s;
+            const float t = (xf[e] * lift) * inv_s;
             const float b1 = t + MAGIC;
             a1[e] = __float_as_uint(b1);
             const float r1 = t - (b1 - MAGIC);
@@ -1205,11 +1208,12 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p)
             mbits = max(sw[0], sw[1]);
         }
         const bool finite = mbits < 0x7F800000u;
-        const float absmax = __uint_as_float(mbits);
-        // (below 1e-30 the reciprocal would overflow: such a slice counts as zero, an error below 1e-30 * sum |w|)
-        const float inv_s = (finite && absmax > 1e-30f) ? 127.0f / absmax : 0.0f;
+        // (a slice below 2^-60 is lifted by 2^64 first, exactly: 127 / absmax then stays finite)
+        const float lift = mbits < 0x21800000u ? 0x1p64f : 1.0f;
+        const float absmax = __uint_as_float(mbits) * lift;
+        const float inv_s = (finite && absmax > 0.0f) ? 127.0f / absmax : 0.0f;
         // a NaN or an infinity in the slice makes the slice's share, hence every output, NaN
-        const float s_x = finite ? (inv_s != 0.0f ? absmax * (1.0f / 127.0f) : 0.0f) : __uint_as_float(0x7FC00000u);
+        const float s_x = finite ? (absmax * (1.0f / 127.0f)) / lift : __uint_as_float(0x7FC00000u);
         uint32_t pk[3][VPL / 4];
 #pragma unroll
         for (int i = 0; i < VPL; i += 4) {
@@ -1218,7 +1222,7 @@ __global__ __launch_bounds__(64 * KW) void gemv_tile8_kernel(const TileParams p)
             for (int e = 0; e < 4; e++) {
                 // round by adding 1.5 * 2^23 (the sum's low byte is the int8) and take every leftover against the
                 // very integer that was packed: no leftover exceeds a half, no term leaves the int8 range
-                const float t = xf[i + e] * inv_s;
+                const float t = (xf[i + e] * lift) * inv_s;
                 const float b1 = t + MAGIC;
                 a1[e] = __float_as_uint(b1);
                 const float r1 = t - (b1 - MAGIC);

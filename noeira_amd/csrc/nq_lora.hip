@@ -160,18 +160,36 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 constexpr int L16_NB = 4;  // chunks of 32 k whose loads are in flight together, per wavefront
 
-// The adapter's share of one tile: out[i][e] = sum_r (x A)[m0 + 2 rp + i][r] B[r][ncl + e] for thread (cq, rp) of the
-// workgroup (unscaled; the caller adds s * out into what it loaded of y).  Uses the workgroup's LDS; a caller that runs
-// it twice puts a barrier between the runs.
+// The LDS one adapter's tile needs (eight wavefronts): where it lies is the caller's business.
+struct Lora16Lds {
+    float (*part)[LR_ROWS][LR_R + 1];  // [LR_WAVES]: the wavefronts' shares of h
+    float (*h)[LR_R];                  // [LR_ROWS]
+    float (*sta)[2][256];              // [LR_WAVES]: a chunk of A per wavefront, turned
+    float (*bt)[LR_COLS];              // [LR_R]: the tile of B
+};
+constexpr int L16_LDS_FLOATS = LR_WAVES * LR_ROWS * (LR_R + 1) + LR_ROWS * LR_R + LR_WAVES * 2 * 256 + LR_R * LR_COLS;
+__device__ __forceinline__ Lora16Lds lora16_lds_at(float* base) {  // (every piece a multiple of 16 bytes)
+    Lora16Lds L;
+    L.part = reinterpret_cast<float (*)[LR_ROWS][LR_R + 1]>(base);
+    L.h = reinterpret_cast<float (*)[LR_R]>(base + LR_WAVES * LR_ROWS * (LR_R + 1));
+    L.sta = reinterpret_cast<float (*)[2][256]>(base + LR_WAVES * LR_ROWS * (LR_R + 1) + LR_ROWS * LR_R);
+    L.bt = reinterpret_cast<float (*)[LR_COLS]>(base + LR_WAVES * LR_ROWS * (LR_R + 1) + LR_ROWS * LR_R + LR_WAVES * 2 * 256);
+    return L;
+}
+
+// The adapter's share of one tile: out[i][e] = sum_r (x A)[m0 + 2 rp + i][r] B[r][ncl + e] for thread tid = (cq, rp) of
+// the eight wavefronts that share `lds` (unscaled; the caller adds s * out into what it loaded of y).  Its barriers are
+// the workgroup's: every wavefront of the workgroup runs it, on its group's adapter, the same number of times; a caller
+// that runs it twice on the same LDS puts a barrier between the runs.
 template <bool XBF16>
-__device__ __forceinline__ void lora16_tile(const void* __restrict__ xv, const float* __restrict__ A, const float* __restrict__ B,
-                                            int T, int IN, int OUT, int m0, int ncl, f32x4 (&out)[2]) {
+__device__ __forceinline__ void lora16_tile(const Lora16Lds& lds, const int tid, const void* __restrict__ xv, const float* __restrict__ A,
+                                            const float* __restrict__ B, int T, int IN, int OUT, int m0, int ncl, f32x4 (&out)[2]) {
     constexpr int NT = XBF16 ? 1 : 3;
-    __shared__ float part[LR_WAVES][LR_ROWS][LR_R + 1];
-    __shared__ __attribute__((aligned(16))) float h[LR_ROWS][LR_R];
-    __shared__ __attribute__((aligned(16))) float sta[LR_WAVES][2][256];  // a chunk of A per wavefront, turned
-    __shared__ __attribute__((aligned(16))) float bt[LR_R][LR_COLS];      // the tile of B
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float (*const part)[LR_ROWS][LR_R + 1] = lds.part;
+    float (*const h)[LR_R] = lds.h;
+    float (*const sta)[2][256] = lds.sta;
+    float (*const bt)[LR_COLS] = lds.bt;
+    const int lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, q = lane >> 4;
     const int cq = tid & 63, rp = tid >> 6;
     // requested first, used last: the tile of B (rows 2 rp, 2 rp + 1 of it per thread)
@@ -297,7 +315,8 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_add16_kernel(const void* _
 #pragma unroll
     for (int i = 0; i < 2; i++) yv[i] = *reinterpret_cast<const f32x4*>(y + (int64_t)min(m0 + 2 * rp + i, T - 1) * OUT + ncl);
     f32x4 out[2];
-    lora16_tile<XBF16>(xv, A, B, T, IN, OUT, m0, ncl, out);
+    __shared__ __attribute__((aligned(16))) float lds_raw[L16_LDS_FLOATS];
+    lora16_tile<XBF16>(lora16_lds_at(lds_raw), tid, xv, A, B, T, IN, OUT, m0, ncl, out);
     if (cols_in) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
@@ -336,6 +355,8 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_multi16_kernel(const void*
     const int tid = threadIdx.x;
     const int m0 = blockIdx.y * LR_ROWS;
     const int cq = tid & 63, rp = tid >> 6;
+    __shared__ __attribute__((aligned(16))) float lds_raw[L16_LDS_FLOATS];
+    const Lora16Lds lds = lora16_lds_at(lds_raw);
     if constexpr (!GLU) {
         // (constant indices: the table stays in scalar registers)
         LoraPartDev me = mp.p[0];
@@ -350,7 +371,7 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_multi16_kernel(const void*
 #pragma unroll
         for (int i = 0; i < 2; i++) yv[i] = *reinterpret_cast<const f32x4*>(me.y + (int64_t)min(m0 + 2 * rp + i, T - 1) * me.out + ncl);
         f32x4 out[2];
-        lora16_tile<XBF16>(xv, me.a, me.b, T, IN, me.out, m0, ncl, out);
+        lora16_tile<XBF16>(lds, tid, xv, me.a, me.b, T, IN, me.out, m0, ncl, out);
         if (cols_in) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
@@ -374,7 +395,7 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_multi16_kernel(const void*
         }
         f32x4 out[2];
         if (mp.p[0].b) {  // (uniform)
-            lora16_tile<XBF16>(xv, mp.p[0].a, mp.p[0].b, T, IN, OUT, m0, ncl, out);
+            lora16_tile<XBF16>(lds, tid, xv, mp.p[0].a, mp.p[0].b, T, IN, OUT, m0, ncl, out);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -382,7 +403,7 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_multi16_kernel(const void*
             __syncthreads();
         }
         if (mp.p[1].b) {
-            lora16_tile<XBF16>(xv, mp.p[1].a, mp.p[1].b, T, IN, OUT, m0, ncl, out);
+            lora16_tile<XBF16>(lds, tid, xv, mp.p[1].a, mp.p[1].b, T, IN, OUT, m0, ncl, out);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -404,6 +425,57 @@ __global__ __launch_bounds__(64 * LR_WAVES) void lora_multi16_kernel(const void*
                     pk.y = (uint32_t)f32_to_bf16_bits(z[2]) | ((uint32_t)f32_to_bf16_bits(z[3]) << 16);
                     *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(glu_out) + at) = pk;
                 }
+            }
+        }
+    }
+}
+
+// gate and up both with an adapter: sixteen wavefronts, the first eight on gate's adapter, the other eight on up's, at
+// the same time (run one after the other in one workgroup of eight the call took 10.7 us at 960 -> 2560 and 135
+// rows); up's sums then cross over through LDS to the threads that hold gate's.
+constexpr int LGLU_LDS_BYTES = (2 * L16_LDS_FLOATS + LR_ROWS * LR_COLS) * 4;
+template <bool XBF16>
+__global__ __launch_bounds__(128 * LR_WAVES) void lora_glu16_kernel(const void* __restrict__ xv, const LoraMultiDev mp, int T, int IN,
+                                                                    void* __restrict__ glu_out, int glu_dtype) {
+    extern __shared__ __attribute__((aligned(16))) float lglu_raw[];
+    const int ga = __builtin_amdgcn_readfirstlane(threadIdx.x >> 9), tid = threadIdx.x & 511;
+    const Lora16Lds lds = lora16_lds_at(lglu_raw + ga * L16_LDS_FLOATS);
+    float (*const ex)[LR_COLS] = reinterpret_cast<float (*)[LR_COLS]>(lglu_raw + 2 * L16_LDS_FLOATS);
+    const LoraPartDev me = ga ? mp.p[1] : mp.p[0];
+    const int m0 = blockIdx.y * LR_ROWS, n0 = (int)blockIdx.x * LR_COLS, OUT = me.out;
+    const int cq = tid & 63, rp = tid >> 6;
+    const bool cols_in = n0 + 4 * cq < OUT;
+    const int ncl = min(n0 + 4 * cq, OUT - 4);
+    f32x4 z[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) z[i] = *reinterpret_cast<const f32x4*>(me.y + (int64_t)min(m0 + 2 * rp + i, T - 1) * OUT + ncl);
+    f32x4 out[2];
+    lora16_tile<XBF16>(lds, tid, xv, me.a, me.b, T, IN, OUT, m0, ncl, out);
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[i][e] = fmaf(me.s, out[i][e], z[i][e]);
+    if (ga == 1) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) *reinterpret_cast<f32x4*>(&ex[2 * rp + i][4 * cq]) = z[i];
+    }
+    __syncthreads();
+    if (ga == 0 && cols_in) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (m0 + 2 * rp + i >= T) break;
+            const f32x4 u = *reinterpret_cast<const f32x4*>(&ex[2 * rp + i][4 * cq]);
+            f32x4 g;
+#pragma unroll
+            for (int e = 0; e < 4; e++) g[e] = swiglu_f32(u[e], z[i][e]);
+            const int64_t at = (int64_t)(m0 + 2 * rp + i) * OUT + ncl;
+            if (glu_dtype == NQ_DT_F32) {
+                *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(glu_out) + at) = g;
+            } else {
+                uint2 pk;
+                pk.x = (uint32_t)f32_to_bf16_bits(g[0]) | ((uint32_t)f32_to_bf16_bits(g[1]) << 16);
+                pk.y = (uint32_t)f32_to_bf16_bits(g[2]) | ((uint32_t)f32_to_bf16_bits(g[3]) << 16);
+                *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(glu_out) + at) = pk;
             }
         }
     }
@@ -461,6 +533,18 @@ int32_t launch_lora_multi(const void* x, int32_t x_dtype, int32_t T, int32_t IN,
             tiles += (parts[t].out + LR_COLS - 1) / LR_COLS;
         }
         const dim3 grid(glu_out ? (parts[0].out + LR_COLS - 1) / LR_COLS : tiles, (T + LR_ROWS - 1) / LR_ROWS);
+        if (glu_out && parts[0].b && parts[1].b) {  // both halves carry an adapter: side by side
+            static LdsAttrOnce attr[2];
+            if (bf) {
+                NQ_HIP(set_max_lds_once(attr[0], reinterpret_cast<const void*>(lora_glu16_kernel<true>), LGLU_LDS_BYTES));
+                hipLaunchKernelGGL((lora_glu16_kernel<true>), grid, dim3(128 * LR_WAVES), LGLU_LDS_BYTES, stream, x, mp, T, IN, glu_out, glu_dtype);
+            } else {
+                NQ_HIP(set_max_lds_once(attr[1], reinterpret_cast<const void*>(lora_glu16_kernel<false>), LGLU_LDS_BYTES));
+                hipLaunchKernelGGL((lora_glu16_kernel<false>), grid, dim3(128 * LR_WAVES), LGLU_LDS_BYTES, stream, x, mp, T, IN, glu_out, glu_dtype);
+            }
+            NQ_HIP(hipGetLastError());
+            return NQ_OK;
+        }
 #define NQ_LM(BF, GLU) \
     hipLaunchKernelGGL((lora_multi16_kernel<BF, GLU>), grid, dim3(64 * LR_WAVES), 0, stream, x, mp, T, IN, glu_out, glu_dtype)
         if (glu_out) {

@@ -335,3 +335,35 @@ def test_four_bit_single_row_on_the_int8_matrix_cores(K, N, prefer, fmt, xdt):
     xn = x.clone()
     xn[0, 5] = float("inf")
     assert bool(torch.isnan(lin.forward(xn)).all())
+
+
+@pytest.mark.parametrize("fmt", ["q4_0", "w4g", "w8_tile", "w8_rows"])
+@pytest.mark.parametrize("mag", [1e-35, 3e-25, 1e20])
+def test_single_row_of_tiny_or_huge_activations_keeps_its_direction(fmt, mag):
+    """The kernels that split x into int8 terms under the slice's largest magnitude: an x whose every value is
+    around 1e-35 (or 1e20) is still a vector with a direction, and y = deq(W) x scales with it - against the fp64
+    product over the oracle's weights, to the fp32 band of the reference (1e-5 of the largest value).  (A slice below
+    2^-60 is lifted by 2^64 before the split; it used to count as zero, which left the zero-point term of a 4-bit
+    layer standing alone.)"""
+    from noeira_amd.qlinear import W8Linear
+    rng = np.random.default_rng(int(abs(np.log10(mag))) + len(fmt))
+    K, N = 4096, 6403
+    if fmt == "q4_0":
+        lin = _q4_signed(rng, K, N, prefer_tile=True)
+        deq = lin.ref_deq()
+    elif fmt == "w4g":
+        lin = _w4g_layer(rng, K, N, prefer_tile=True)
+        deq = lin.ref_deq()
+    else:
+        w = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        s = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+        lin = W8Linear(K, N, tile_copy=fmt == "w8_tile")
+        lin.set_weight(w, s)
+        deq = refw.w8(w, s)
+    for xdt in (torch.float32, torch.bfloat16):
+        x = torch.from_numpy((rng.standard_normal((1, K)) * mag).astype(np.float32)).to(xdt).cuda()
+        y = lin.forward(x)
+        exact = x.double() @ deq.T
+        assert float((y.double() - exact).abs().max()) <= 1e-5 * float(exact.abs().max()), (fmt, mag, xdt)
+        yr = lin.forward(x, epilogue="relu")
+        assert float((yr.double() - exact.clamp_min(0)).abs().max()) <= 1e-5 * float(exact.abs().max())
