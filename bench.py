@@ -754,7 +754,8 @@ def sweep(skip_large=False):
         c8 = max(1, COLD_BYTES // (4096 * 11008))
         run("W8A8 int8 GEMV K=4096 N=11008 M=1 (cold)", make_w8a8_m1, "hbm", K=4096, N=11008, copies=c8, calls=c8)
         # a few rows to several hundred: the 16-row tile kernel's range
-        for M in (16, 64, 256, 512):
+        # (1024: the 128 x 128 tile GEMM's range; 2048: back on the 256 x 256 tiles)
+        for M in (16, 64, 256, 512, 1024, 2048):
             run(f"W8A8 int8 M={M} K=4096 N=4096 (warm)", make_w8a8_gemm, "mfma", "int8", M=M, N=4096, calls=20)
             run(f"fp8 x fp8 M={M} K=4096 N=4096 (warm)", make_fp8, "mfma", "fp8", M=M, N=4096, copies=1, calls=20)
         # e4m3 weights under bf16 activations: the bf16 matrix-core kernels

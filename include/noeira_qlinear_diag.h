@@ -36,10 +36,20 @@ int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream);
  * with every workgroup of the 256 x 256 tile kernel reporting four readings of the GPU's constant 100 MHz clock -
  * entry, first K stage landed, K loop done, stores acknowledged - into stamps (device uint64 [tiles][4], tiles =
  * ceil(M / 256) * ceil(OUT / 256) <= max_tiles, else NQ_ERR_INVALID).  The arguments are nq_forward's for that case
- * (x: int8 with per-row x_scale, or e4m3 codes with one scale; no bias).  The stamp buffer is an argument of this
+ * (x: int8 with per-row x_scale, or e4m3 codes with one scale; y fp32 or bf16, for int8 also the raw int32
+ * accumulators; no bias).  The stamp buffer is an argument of this
  * one launch: no other call, on this or another thread, writes stamps.  Synchronises the stream before it returns. */
 int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y,
                                int32_t y_dtype, int32_t M, uint64_t* stamps, int64_t max_tiles, void* stream);
+
+/* nq_forward for 8-bit activations (int8 with per-row scales over a W8_CHANNEL layer, e4m3 codes with one scale over
+ * an FP8_E4M3 layer; M >= 64, IN a multiple of 128) on the GEMM kernel of the caller's choice (no counterpart in the
+ * reference): tile = 256, the 256 x 256 tile kernel nq_forward takes from about a round and a half of such tiles on,
+ * or 128, the 128 x 128 tile kernel it takes below that where no 16-row tile kernel is estimated faster.  The two
+ * return the same bits; tests hold each against the oracle on shapes the dispatch would give to the other, and
+ * bench.py times them side by side.  Acts on this one launch only. */
+int32_t nq_diag_forward_gemm8(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y, int32_t y_dtype,
+                              int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue, int32_t tile, void* stream);
 
 /* A forward on the 16-row tile kernel that takes 2 .. 511 rows of fp32 / bf16 activations, under a tile shape of
  * the caller's choice (no counterpart in the reference): mw x nw wavefront tiles of 16 x 16 per workgroup, one of

@@ -35,7 +35,7 @@ EXPORTS = [
     "nq_keep_only_repacked", "nq_device_bytes", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
     "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward", "nq_fuse_rows", "nq_fused_parts",
     "nq_forward_fused", "nq_fuse_glu", "nq_hessian_create", "nq_hessian_destroy", "nq_hessian_add", "nq_hessian_rows",
-    "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_hinv_upper_f64_dev", "nq_set_weight_gptq", "nq_q4_0_objective", "nq_lora_forward_add", "nq_forward_lora", "nq_forward_fused_lora", "nq_diag_mfma_rate", "nq_diag_stream_read", "nq_diag_gemm8_timeline", "nq_diag_forward_a16",
+    "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_hinv_upper_f64_dev", "nq_set_weight_gptq", "nq_q4_0_objective", "nq_lora_forward_add", "nq_forward_lora", "nq_forward_fused_lora", "nq_diag_mfma_rate", "nq_diag_stream_read", "nq_diag_gemm8_timeline", "nq_diag_forward_a16", "nq_diag_forward_gemm8",
 ]
 
 
@@ -162,6 +162,8 @@ def lib() -> C.CDLL:
     L.nq_forward_fused_lora.argtypes = [p, p, i32, C.POINTER(p), i32, i32, p, i32, C.POINTER(LoraPart), p, i32, p]
     L.nq_forward_lora.restype = i32
     L.nq_forward_lora.argtypes = [p, p, i32, p, i32, i32, p, i32, p, p, i32, C.c_float, p]
+    L.nq_diag_forward_gemm8.restype = i32
+    L.nq_diag_forward_gemm8.argtypes = [p, p, i32, p, p, i32, i32, p, i32, i32, i32, p]
     L.nq_diag_gemm8_timeline.restype = i32
     L.nq_diag_gemm8_timeline.argtypes = [p, p, i32, p, p, i32, i32, p, i64, p]
     L.nq_device_bytes.restype = i64

@@ -440,10 +440,12 @@ int32_t dispatch(const ForwardArgs& a) {
     }
     if (a.x_dtype == NQ_DT_I8) {
         if (tile8_i8_applicable(a)) return launch_tile8_i8(a);
+        if (gemm8s_applicable(a)) return launch_gemm8s(a);
         if (gemm8_applicable(a)) return launch_gemm8(a);
         return launch_gemv_i8(a);
     }
     if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
+    if (gemm8s_applicable(a)) return launch_gemm8s(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemv_tile_rows_applicable(a)) return launch_gemv_tile_rows(a);
     if (gemv_tile8_rows_applicable(a)) return launch_gemv_tile8_rows(a);
@@ -1070,8 +1072,8 @@ int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, cons
     const int64_t tiles = (int64_t)((M + 255) / 256) * ((h->out + 255) / 256);
     if (tiles > max_tiles) return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: the stamp buffer is smaller than the tile count");
     if ((rc = need_loaded(h, "forward"))) return rc;
-    if (!x || !y || !x_scale || (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16))
-        return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: x, its scale(s) and an fp32 or bf16 y are needed");
+    if (!x || !y || !x_scale || (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16 && !(y_dtype == NQ_DT_I32 && x_dtype == NQ_DT_I8)))
+        return fail(NQ_ERR_INVALID, "nq_diag_gemm8_timeline: x, its scale(s) and an fp32 or bf16 y (int8: or raw int32) are needed");
     SegTable seg{};
     seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
     ForwardArgs a{h, x, x_dtype, x_scale, y, y_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_NONE, (hipStream_t)stream, seg};
@@ -1082,6 +1084,24 @@ int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, cons
     if (rc) return rc;
     NQ_HIP(hipStreamSynchronize((hipStream_t)stream));
     return NQ_OK;
+}
+
+int32_t nq_diag_forward_gemm8(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y, int32_t y_dtype,
+                              int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue, int32_t tile, void* stream) {
+    int32_t rc = check_handle(h, "nq_diag_forward_gemm8");
+    if (rc) return rc;
+    if ((rc = need_loaded(h, "forward"))) return rc;
+    if (tile != 128 && tile != 256) return fail(NQ_ERR_INVALID, "nq_diag_forward_gemm8: tile is 128 or 256");
+    if (!x || !y || !x_scale || ((uintptr_t)x & 15) || ((uintptr_t)y & 3) || (x_dtype != NQ_DT_I8 && x_dtype != NQ_DT_FP8_E4M3) ||
+        (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16 && !(y_dtype == NQ_DT_I32 && x_dtype == NQ_DT_I8 && !bias && epilogue == NQ_EPI_NONE)) ||
+        (epilogue != NQ_EPI_NONE && epilogue != NQ_EPI_RELU) || (bias && bias_dtype != NQ_DT_F32 && bias_dtype != NQ_DT_BF16))
+        return fail(NQ_ERR_INVALID, "nq_diag_forward_gemm8: nq_forward's arguments for 8-bit activations are needed");
+    SegTable seg{};
+    seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = y;
+    ForwardArgs a{h, x, x_dtype, x_scale, y, y_dtype, M, bias, bias_dtype, epilogue, (hipStream_t)stream, seg};
+    if (h->glu || !h->seg_end.empty() || !gemm8_applicable(a))
+        return fail(NQ_ERR_UNSUPPORTED, "nq_diag_forward_gemm8: the 8-bit GEMM does not take this call (format, M >= 64, IN % 128)");
+    return tile == 128 ? launch_gemm8s(a) : launch_gemm8(a);
 }
 
 int32_t nq_diag_forward_a16(nq_handle h, const void* x, int32_t x_dtype, void* y, int32_t y_dtype, int32_t M,

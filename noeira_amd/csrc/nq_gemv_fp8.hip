@@ -490,9 +490,8 @@ static bool tile8_wins(const ForwardArgs& a) {
     if (L->in % 16 != 0) return false;
     if (a.M < 64 || L->in % 128 != 0) return true;  // (the GEMM needs 64 rows and whole 128-byte steps)
     const double steps = (double)L->in / 128.0;
-    const int64_t tiles = (int64_t)((a.M + 255) / 256) * ((L->out + 255) / 256);
     const bool i8 = a.x_dtype == NQ_DT_I8;
-    const double gemm_us = (double)((tiles + 255) / 256) * (i8 ? 14.0 + 1.25 * steps : 10.0 + 1.1 * steps);
+    const double gemm_us = std::min(gemm8_estimate_us(a.M, L->out, L->in, i8, false), gemm8_estimate_us(a.M, L->out, L->in, i8, true));
     const int nt = tile8_weight_tiles(a.M, L->out, L->in);
     double tile_us;
     if (nt == 1) {

@@ -426,3 +426,52 @@ def test_mlp3_other_shapes_and_errors():
     assert rel_rms(y, h) < TOL_RMS
     with pytest.raises(L.NQError, match="do not chain"):
         mlp3_w8a8_forward(layers[0][0], layers[2][0], layers[1][0], torch.from_numpy(x).cuda())
+
+
+# ── the two tile sizes of the 8-bit GEMM ────────────────────────────────────────────────────────────────────────
+def _gemm8(lin, tile, x, x_dt, x_scale, M, out_dtype, bias=None, epilogue="none"):
+    """The 8-bit GEMM on the 128 x 128 (`tile` = 128) or the 256 x 256 tile kernel, whatever nq_forward would choose."""
+    import ctypes as C
+    from noeira_amd import _lib as L
+    out = torch.full((M, lin.OUT), 7, dtype=out_dtype, device="cuda")
+    y_dt = {torch.float32: L.DT_F32, torch.bfloat16: L.DT_BF16, torch.int32: L.DT_I32}[out_dtype]
+    L.check(L.lib().nq_diag_forward_gemm8(lin._h, C.c_void_p(x.data_ptr()), x_dt, C.c_void_p(x_scale.data_ptr()),
+                                          C.c_void_p(out.data_ptr()), y_dt, M, C.c_void_p(bias.data_ptr()) if bias is not None else None,
+                                          L.DT_F32, L.EPI_RELU if epilogue == "relu" else L.EPI_NONE, tile, None))
+    return out
+
+
+@pytest.mark.parametrize("M,K,N", [(520, 1024, 2296), (1000, 512, 520), (2100, 512, 2300), (300, 4096, 1024), (64, 128, 8)])
+def test_gemm_tile_sizes_against_the_oracle_and_each_other(M, K, N):
+    """Both tile sizes on the same ragged problems (last row and column of tiles cut short, N a multiple of 8 and not,
+    a single tile): int32 accumulators equal the oracle's bit for bit, the fused epilogue its fp32 expression, fp8
+    the float64 oracle; and since both kernels add a row's K in the same order and apply the same epilogue, they
+    return the same bits - int32, fp32 and bf16."""
+    from noeira_amd import _lib as L
+    rng = np.random.default_rng(M + K + N)
+    lin, w, s = w8_layer(rng, K, N)
+    xq_h = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    sx_h = rng.uniform(1e-3, 1e-1, M).astype(np.float32)
+    bias_h = (rng.standard_normal(N) * 0.02).astype(np.float32)
+    xq, sx, bias = torch.from_numpy(xq_h).cuda(), torch.from_numpy(sx_h).cuda(), torch.from_numpy(bias_h).cuda()
+    acc_o = O.w8a8_acc_i32(xq_h, w)
+    want = O.w8a8_epilogue(acc_o, sx_h, s, bias_h, relu=True)
+    for tile in (128, 256):
+        assert np.array_equal(_gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.int32).cpu().numpy(), acc_o), tile
+        assert rel_rms(_gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.float32, bias, "relu").cpu().numpy(), want) < 1e-5, tile
+    for dt in (torch.float32, torch.bfloat16):
+        assert torch.equal(_gemm8(lin, 128, xq, L.DT_I8, sx, M, dt, bias, "relu"), _gemm8(lin, 256, xq, L.DT_I8, sx, M, dt, bias, "relu")), dt
+    a, b = fp8_operands(rng, M, N, K)
+    f8 = FP8Linear(K, N)
+    f8.set_weight(b, 0.25)
+    xs = torch.tensor([0.5], dtype=torch.float32, device="cuda")
+    ad = torch.from_numpy(a).cuda()
+    y64, _ = O.fp8_forward_f64(a, b, np.float32(0.5), np.float32(0.25), want_bf16=False)
+    ref = y64 + bias_h.astype(np.float64)
+    for tile in (128, 256):
+        got = _gemm8(f8, tile, ad, L.DT_FP8_E4M3, xs, M, torch.float32, bias).cpu().numpy()
+        assert np.abs(got - ref).max() <= 3e-4 * np.sqrt((ref ** 2).mean()), tile
+    for dt in (torch.float32, torch.bfloat16):
+        assert torch.equal(_gemm8(f8, 128, ad, L.DT_FP8_E4M3, xs, M, dt, bias), _gemm8(f8, 256, ad, L.DT_FP8_E4M3, xs, M, dt, bias)), dt
+    # what nq_forward itself returns for the call (whichever kernel it takes): the oracle's accumulators
+    assert np.array_equal(lin.forward_a8(xq, sx, out_dtype=torch.int32).cpu().numpy(), acc_o)
