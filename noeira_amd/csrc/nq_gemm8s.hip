@@ -3,22 +3,20 @@
 //
 // Why a second tile size.  A 256 x 256 tile takes its 41 - 46 us (fp8, K = 4096) however few of them a call has:
 // 41.6 us at M = 1024 (64 tiles on 256 CUs), 45.8 at 2048.  With 128 x 128 tiles the same call has four times as
-// many workgroups of a quarter of the arithmetic each.  Such a tile is bound by the CU's LDS, not by its matrix
-// cores: a stage's 32 KiB are written once and each fragment is read by two wavefronts, 96 KiB of LDS traffic for
-// 16 MFMAs per wavefront, and LDS moves about 64 bytes per cycle - measured 0.68 us per stage, of which 0.28 the
-// transfers alone and 0.42 the fragment reads and MFMAs alone (they add up: both go through LDS), against 0.22 for
-// the MFMAs.  So a round of 128 x 128 tiles takes 23 - 27 us at K = 4096 where a round of the large ones takes 42 - 46
-// for four times the work: the small tile wins while its tiles fit one round (M = 1024 over 4096 x 4096: 27.4 us
-// against 41.6, int8 30.8 against 48.6) and loses from two rounds on (M = 2048: 49.1 against 45.8).  No split of K,
-// hence no partial sums, no workspace and no second pass: every output is one accumulator's sum over K in
-// ascending order, the order of the large kernel.
+// many workgroups of a quarter of the arithmetic each.  A stage of such a tile has 16 MFMAs per wavefront (0.22 us)
+// behind a barrier and sixteen fragment reads that nothing overlaps, and takes about 0.6 us; a round of 128 x 128
+// tiles then takes 21 - 25 us at K = 4096 where a round of the large ones takes 42 - 46 for four times the work.  The
+// small tile wins while its tiles fit one round (M = 1024 over 4096 x 4096: 24.8 us against 41.6, int8 31.2 against
+// 48.6; M = 512: 21.1 against the 16-row tile kernel's 25.7) and loses from two rounds on (M = 2048: 49 against 45.8).
+// No split of K, hence no partial sums, no workspace and no second pass: every output is one accumulator's sum over
+// K in ascending order, the order of the large kernel.
 //
 // The kernel is the plain form of the large one: 4 wavefronts (2 x 2), each 64 x 64 as 4 x 4 MFMA tiles of 16 x 16;
 // stages of 128 bytes of K, x tile and w tile 16 KiB each, four stages in LDS (128 KiB: one multiplied, three on
-// their way), filled straight from global memory (global_load_lds_dwordx4, 8 per wavefront and stage) with the large
-// kernel's slot permutation applied on the global side, so that the 128-bit fragment reads are conflict-free.  One
-// barrier per stage: it proves the stage landed and that the buffer of the stage before has been read out, and the
-// transfers of the stage three ahead are issued right behind it.  Scheduling inside a stage is the compiler's.
+// their way), filled straight from global memory (global_load_lds_dwordx4, 8 per wavefront and stage, issued one at a
+// time between the MFMAs) with the large kernel's slot permutation applied on the global side, so that the 128-bit
+// fragment reads are conflict-free.  One barrier per stage: it proves the stage landed and that the buffer of the
+// stage before has been read out.  Scheduling inside a stage is otherwise the compiler's.
 // Epilogue: per-token scale x per-channel scale (int8) or the tensor scales (fp8), bias, ReLU, fp32 / bf16 / raw int32
 // out, staged through LDS per wavefront and stored 16 bytes per lane - the large kernel's formulas, so a value is
 // the same bits whichever of the two kernels produced it.
@@ -34,6 +32,15 @@ typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
 
 constexpr int SM = 128, SN = 128, SK = 128;  // tile of y, bytes of K per stage
 constexpr int S_STAGE = (SM + SN) * SK;      // 32 KiB
@@ -97,17 +104,22 @@ __global__ __launch_bounds__(256) void gemm8s_kernel(const Gemm8sParams p) {
     const uint32_t lds_addr0 = (uint32_t)(uintptr_t)(lptr_t*)lds;
     // (M0 holds the LDS destination of the instruction that follows; the compiler sets M0 itself before each of its
     // own uses, so writing it here needs no clobber; SCC does)
-#define NQ_S_DMA(t, buf, src)                                                                              \
-    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"                       \
-                 :                                                                                         \
-                 : "s"(lds_addr0 + (buf) * S_STAGE + ((t) < 4 ? 0 : SM * SK) + wave * 32 * SK), "v"(doff[(t)]), \
-                   "s"(src), "n"(((t) & 3) * 1024)                                                         \
+#define NQ_S_DMA(t, dst, off, src)                                                          \
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"    \
+                 :                                                                      \
+                 : "s"(dst), "v"(off), "s"(src), "n"(((t) & 3) * 1024)                  \
                  : "memory", "scc")
+    // transfer t (0 .. 7) of stage st into buffer buf
+    auto fill1 = [&](auto tc, int buf, int st) {
+        constexpr int t = decltype(tc)::value;
+        const uint8_t* const src = (t < 4 ? abase : bbase) + (int64_t)st * SK;
+        // (named outside the asm statement so that the lambda captures them)
+        const uint32_t dst = lds_addr0 + buf * S_STAGE + (t < 4 ? 0 : SM * SK) + wave * 32 * SK;
+        const uint32_t off = doff[t];
+        NQ_S_DMA(t, dst, off, src);
+    };
     auto fill = [&](int buf, int st) {
-        const uint8_t* const sa = abase + (int64_t)st * SK;
-        const uint8_t* const sb = bbase + (int64_t)st * SK;
-        NQ_S_DMA(0, buf, sa); NQ_S_DMA(1, buf, sa); NQ_S_DMA(2, buf, sa); NQ_S_DMA(3, buf, sa);
-        NQ_S_DMA(4, buf, sb); NQ_S_DMA(5, buf, sb); NQ_S_DMA(6, buf, sb); NQ_S_DMA(7, buf, sb);
+        static_for<8>([&](auto tc) { fill1(tc, buf, st); });
     };
     const float fp8_scale = FP8 ? p.tscale * p.row_scale[0] : 0.0f;  // requested now, used in the epilogue
 
@@ -127,9 +139,16 @@ __global__ __launch_bounds__(256) void gemm8s_kernel(const Gemm8sParams p) {
 
     const int KT = p.K / SK;
     // Stage st lives in buffer st % 4.  A trip from L2 takes longer than a stage's MFMAs, so three stages are under way
-    // while one is multiplied (with one, the loop ran at the latency of a transfer: 0.67 us per stage, 21 us for the
-    // smallest call).  The transfers are this loop's only vector-memory instructions, 8 per wavefront and stage, and
-    // they land in order: "all but the youngest 16" is stage st.
+    // while one is multiplied, and the transfers of the stage three ahead are issued one at a time between this
+    // stage's MFMAs: a wavefront issues in order and a transfer holds its issue for some seventy cycles, which the
+    // matrix core spends on the MFMA before it.  (Measured at M = 64 .. 1024 over 4096 x 4096, microseconds per stage:
+    // one stage under way and the transfers in a batch behind the barrier 0.68 - of which the transfers alone 0.28,
+    // the fragment reads and MFMAs alone 0.42; three under way, still in a batch, the same 0.68; spread between the
+    // MFMAs 0.6.  The MFMAs take 0.22: what remains is the barrier and the fragment reads at the head of every
+    // stage.  Reading a stage's fragments during the MFMAs of the stage before, into a second register set, made the
+    // compiler rotate the sets through copies - four moves per MFMA - and measured slower, 0.8.)
+    // The transfers are the loop's only vector-memory instructions, 8 per wavefront and stage, landing in order:
+    // "all but the youngest 16" is everything up to stage st.
     fill(0, 0);
     if (KT > 1) fill(1, 1);
     if (KT > 2) fill(2, 2);
@@ -139,7 +158,8 @@ __global__ __launch_bounds__(256) void gemm8s_kernel(const Gemm8sParams p) {
         else if (st + 1 < KT) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();  // stage st has landed everywhere; everyone is done reading the buffer of stage st - 1
-        if (st + 3 < KT) fill((st + 3) & (S_NS - 1), st + 3);
+        const bool more = st + 3 < KT;
+        const int nbuf = (st + 3) & (S_NS - 1);
         const uint8_t* const xb = xrow + buf * S_STAGE;
         const uint8_t* const wb = wrow + buf * S_STAGE;
         i32x4 xf[TI][2], wf[TJ][2];
@@ -153,20 +173,21 @@ __global__ __launch_bounds__(256) void gemm8s_kernel(const Gemm8sParams p) {
             wf[j][0] = *reinterpret_cast<const i32x4*>(wb + j * 16 * SK + so0);
             wf[j][1] = *reinterpret_cast<const i32x4*>(wb + j * 16 * SK + so1);
         }
-#pragma unroll
-        for (int i = 0; i < TI; i++)
-#pragma unroll
-            for (int j = 0; j < TJ; j++) {
-                // (the weight fragment first: a lane then holds one token and four consecutive channels)
-                if constexpr (FP8) {
-                    const i32x8 av = {xf[i][0][0], xf[i][0][1], xf[i][0][2], xf[i][0][3], xf[i][1][0], xf[i][1][1], xf[i][1][2], xf[i][1][3]};
-                    const i32x8 bv = {wf[j][0][0], wf[j][0][1], wf[j][0][2], wf[j][0][3], wf[j][1][0], wf[j][1][1], wf[j][1][2], wf[j][1][3]};
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[i][j], 0, 0, 0, 0, 0, 0);
-                } else {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[j][0], xf[i][0], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[j][1], xf[i][1], acc[i][j], 0, 0, 0);
-                }
+        static_for<TI * TJ>([&](auto ijc) {
+            constexpr int ij = decltype(ijc)::value, i = ij / TJ, j = ij % TJ;
+            // (the weight fragment first: a lane then holds one token and four consecutive channels)
+            if constexpr (FP8) {
+                const i32x8 av = {xf[i][0][0], xf[i][0][1], xf[i][0][2], xf[i][0][3], xf[i][1][0], xf[i][1][1], xf[i][1][2], xf[i][1][3]};
+                const i32x8 bv = {wf[j][0][0], wf[j][0][1], wf[j][0][2], wf[j][0][3], wf[j][1][0], wf[j][1][1], wf[j][1][2], wf[j][1][3]};
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, acc[i][j], 0, 0, 0, 0, 0, 0);
+            } else {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[j][0], xf[i][0], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[j][1], xf[i][1], acc[i][j], 0, 0, 0);
             }
+            if constexpr (ij % 2 == 1) {
+                if (more) fill1(std::integral_constant<int, ij / 2>{}, nbuf, st + 3);
+            }
+        });
     }
 #undef NQ_S_DMA
     __syncthreads();  // every wavefront is done with the stage buffers: the epilogue stages through them
@@ -263,7 +284,7 @@ double gemm8_estimate_us(int M, int N, int K, bool i8, bool small_tile) {
     const double steps = (double)K / 128.0;
     if (small_tile) {
         const int64_t tiles = (int64_t)((M + SM - 1) / SM) * ((N + SN - 1) / SN);
-        return (double)((tiles + 255) / 256) * (i8 ? 3.0 + 0.74 * steps : 2.5 + 0.68 * steps);
+        return (double)((tiles + 255) / 256) * (i8 ? 3.0 + 0.74 * steps : 2.5 + 0.6 * steps);
     }
     const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
     return (double)((tiles + 255) / 256) * (i8 ? 14.0 + 1.25 * steps : 10.0 + 1.1 * steps);
