@@ -790,6 +790,39 @@ def sweep(skip_large=False):
     return out
 
 
+def vendor_gemm():
+    """A yardstick, not a product path: the vendor library's fp8 GEMM (torch._scaled_mm -> hipBLASLt) on config 5's
+    shapes, timed the way the GEMM rows are (50 ms of the same launches first, then medians of 20 launches)."""
+    import torch
+
+    out = []
+    g = torch.Generator().manual_seed(6)
+    for (M, N, K) in ((8192, 4096, 4096), (8192, 11008, 4096), (8192, 8192, 8192)):
+        a = torch.randn((M, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).cuda()
+        w = torch.randn((N, K), generator=g).clamp_(-448, 448).to(torch.float8_e4m3fn).cuda()
+        sa, sb = torch.tensor(1.0 / 16, device="cuda"), torch.tensor(1.0 / 16, device="cuda")
+
+        def f(i):
+            torch._scaled_mm(a, w.t(), scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16)
+
+        try:
+            f(0)
+            torch.cuda.synchronize()
+        except Exception as e:  # (a torch build without the call: say so, measure nothing)
+            out.append({"M": M, "N": N, "K": K, "error": repr(e)[:200]})
+            continue
+        tm = Timer()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < SETTLE_S:
+            tm.run(f, 20)
+        t = statistics.median([tm.run(f, 20) / 20 for _ in range(SAMPLES)])
+        out.append({"M": M, "N": N, "K": K, "us_per_call": round(t * 1e6, 2),
+                    "frac_of_fp8_peak": round(2.0 * M * N * K / t / 1e12 / MFMA_PEAK_TOPS["fp8"], 4)})
+        del a, w
+        torch.cuda.empty_cache()
+    return out
+
+
 def only_loop(which, steps, warmup):
     """One kernel, launched call by call `steps` times after `warmup` untimed calls: the loop a
     rocprofv3 run (kernel trace or one counter pass) is wrapped around."""
@@ -876,10 +909,24 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_t8, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "W8A8 and fp8 x fp8 at 4096 x 4096, M = 16, 64, 128, 256, 512, one call each per step"
+    elif which == "gemm_mid":
+        wls = [make_fp8(M, 4096) for M in (512, 1024)] + [make_w8a8_gemm(M, 4096) for M in (512, 1024)]
+
+        def step_gm(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_gm, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "fp8 x fp8 and W8A8 at 4096 x 4096, M = 512 and 1024 (the 128 x 128 tile GEMM), one call each per step"
+    elif which == "adapters":
+        wl = make_decoder_layer(135, "fused")
+        name = "the reference text layer's seven Q4_0 projections at T = 135 with rank-16 adapters, fused calls"
     elif which == "gemm_timeline":
         return {"only": which, "timelines": [gemm_timeline(4096, 4096), gemm_timeline(4096, 8192), gemm_timeline(11008, 4096)]}
     elif which == "mfma_peak":
         return {"only": which, "mfma_only": mfma_only()}
+    elif which == "vendor_gemm":
+        return {"only": which, "vendor_fp8_gemm": vendor_gemm()}
     elif which == "actor":
         wl = make_actor_fused()
         name = "cfg4 W8A8 actor 64->256->256->8 M=4096, fused"
@@ -1080,7 +1127,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "headline", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline", "a16_shapes", "mid_dispatch"],
+    ap.add_argument("--only", default="", choices=["", "headline", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "gemm_mid", "adapters", "manyrows", "hugegemv", "mfma_peak", "vendor_gemm", "gemm_timeline", "a16_shapes", "mid_dispatch"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): headline = the "
                          "headline line alone (graph replays), act = config 2's pair of linears at M=1, fp8gemv / fp8gemm = "
                          "config 5 at N=11008 (the headline's kernel, launched call by call) / N=4096, mid = the M=100..256 "
@@ -1119,7 +1166,7 @@ def main():
             sys.exit("bench.py: --only mid_dispatch is about the 4-bit formats (--a16-class q4, q4f, w4g or w4gf)")
         print(json.dumps(mid_dispatch(a.a16_class)))
         return
-    if a.only in ("act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "manyrows", "hugegemv", "mfma_peak", "gemm_timeline"):
+    if a.only in ("act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "gemm_mid", "adapters", "manyrows", "hugegemv", "mfma_peak", "vendor_gemm", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 
