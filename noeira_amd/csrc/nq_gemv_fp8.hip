@@ -286,26 +286,37 @@ __global__ __launch_bounds__(64 * KW) void tile8_kernel(const Fp8GemvParams p) {
 }
 
 
-// ---- M = 1: one wavefront per weight row, coalesced loads, trace of the MFMA tile
-template <bool I8, int CPL, int WAVES>
+// ---- M = 1: one wavefront per weight row (or SPLIT wavefronts, each on a 1 / SPLIT share of it), coalesced loads,
+// trace of the MFMA tile.  CPL: 16-byte chunks of the row per lane of ONE wavefront (CPL * SPLIT * 64 chunks cover K).
+template <bool I8, int CPL, int WAVES, int SPLIT>
 __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvParams p) {
-    __shared__ u32x4 xs[CPL * 64];  // the activation row, shared by the workgroup's rows
+    constexpr int ROWS = WAVES / SPLIT;   // rows per workgroup
+    constexpr int XCH = CPL * SPLIT * 64; // chunks of x staged
+    __shared__ u32x4 xs[XCH];  // the activation row, shared by the workgroup's rows
+    __shared__ uint32_t part[ROWS][SPLIT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t row = (int64_t)blockIdx.x * WAVES + wave;
+    const int wrow = wave / SPLIT, share = wave % SPLIT;
+    const int64_t row = (int64_t)blockIdx.x * ROWS + wrow;
     const int64_t rowc = min(row, (int64_t)p.N - 1);
     const int nch = p.K >> 4;  // 16-byte chunks per row
     const u32x4* wr = reinterpret_cast<const u32x4*>(p.w + rowc * p.K);
     const u32x4* xr = reinterpret_cast<const u32x4*>(p.x);
+    const int c0 = share * CPL * 64;  // this wavefront's first chunk of the row
 
     // x goes first so that waiting for it leaves the weight loads in flight; every load is
     // unconditional from a clamped chunk index, and a chunk past K meets x = 0
-    constexpr int XPT = (CPL * 64 + 64 * WAVES - 1) / (64 * WAVES);  // chunks of x per thread
+    constexpr int XPT = (XCH + 64 * WAVES - 1) / (64 * WAVES);  // chunks of x per thread
     u32x4 xg[XPT];
+    u32x4 wv[CPL], xv[CPL];
+#ifdef NQ_LAB_XDIRECT
+#pragma unroll
+    for (int j = 0; j < CPL; j++) xv[j] = xr[min(c0 + j * 64 + lane, nch - 1)];
+#else
 #pragma unroll
     for (int i = 0; i < XPT; i++) xg[i] = xr[min((int)threadIdx.x + i * 64 * WAVES, nch - 1)];
-    u32x4 wv[CPL], xv[CPL];
+#endif
 #pragma unroll
-    for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wr + min(j * 64 + lane, nch - 1));
+    for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wr + min(c0 + j * 64 + lane, nch - 1));
     // the epilogue's operands travel with the codes, raw: nothing is computed from them before the end
     const bool raw_out = I8 && p.y_dtype == NQ_DT_I32;
     float xsraw = 1.0f, csraw = 1.0f;
@@ -315,14 +326,20 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvPara
     if (p.bias)
         braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[rowc]
                                            : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[rowc];
+#ifdef NQ_LAB_XDIRECT
+#pragma unroll
+    for (int j = 0; j < CPL; j++)
+        if (c0 + j * 64 + lane >= nch) xv[j] = (u32x4){0, 0, 0, 0};
+#else
 #pragma unroll
     for (int i = 0; i < XPT; i++) {
         const int c = (int)threadIdx.x + i * 64 * WAVES;
-        if (c < CPL * 64) xs[c] = (c < nch) ? xg[i] : (u32x4){0, 0, 0, 0};
+        if (c < XCH) xs[c] = (c < nch) ? xg[i] : (u32x4){0, 0, 0, 0};
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < CPL; j++) xv[j] = xs[j * 64 + lane];
+    for (int j = 0; j < CPL; j++) xv[j] = xs[c0 + j * 64 + lane];
+#endif
 
     // lane holds D[4 (lane / 16) + r][lane % 16]: its diagonal entry, if any, is r = c % 4 where
     // c = lane % 16 and c / 4 == lane / 16
@@ -369,6 +386,15 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvPara
         const auto sw = __builtin_amdgcn_permlane32_swap(vbits, vbits, false, false);
         vbits = add(sw[0], sw[1]);
     }
+    if constexpr (SPLIT > 1) {
+        // the shares of a row meet in LDS, in their order (fixed: the same bits on every call)
+        if (lane == 0) part[wrow][share] = vbits;
+        __syncthreads();
+        if (share != 0) return;
+        vbits = part[wrow][0];
+#pragma unroll
+        for (int k = 1; k < SPLIT; k++) vbits = add(vbits, part[wrow][k]);
+    }
     if (lane == 0 && row < p.N) {
         if (raw_out) {
             reinterpret_cast<int32_t*>(p.y)[row] = (int32_t)vbits;
@@ -384,9 +410,30 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvPara
     }
 }
 
+// How many wavefronts a workgroup has and how many share a row, by the bytes of the weight (measured on e4m3 and int8
+// weights of K = 4096 and 8192, cold, medians of replays of a graph of 60 calls):
+//   16.8 MB (4096 x 4096):    8 x 1: 4.49 us; 4 x 1: 4.62; 8 wavefronts, two per row: 4.71
+//   45 MB   (4096 -> 11008):  8 x 1: 8.62;    4 x 1: 8.40; 4 wavefronts, two per row: 8.45; 8, two per row: 8.51; 2 x 1: 8.50;
+//                             16 wavefronts, two per row: 9.68; x fetched per lane instead of staged in LDS: 8.44
+//   235 MB  (8192 -> 28672):  8 x 1: 36.05;   4 x 1: 34.58; 4, two per row: 33.06; 8, four per row: 32.90 (89 % of 8 TB/s)
+// On the largest layers smaller workgroups with less of a row per wavefront are worth 8 %.  At 45 MB the differences
+// are within what two timing protocols disagree on: under replays of a graph of 200 steps, on one box in turn, 8 x 1
+// took 8.178 / 8.180 / 8.163 us and 4 x 1 8.202 / 8.239 / 8.157, so it stays as it was.  (A kernel that only reads shows
+// the same taste for small pieces - 1 or 2 KiB per wavefront: 7.7 us for 45 MB, 4 KiB: 8.0, 8 KiB: 8.6 - and gains
+// from fewer resident workgroups, 7.75 with two or three per CU; a kernel with a chain behind its loads loses with
+// fewer: 8.9 / 9.6 us.)
 template <bool I8, int CPL>
 int32_t launch_row(const Fp8GemvParams& p, hipStream_t s) {
-    hipLaunchKernelGGL((gemv8_row_kernel<I8, CPL, 8>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
+    // (CPL counts the row's 16-byte chunks per lane of one wavefront that holds the whole row)
+    const int64_t bytes = (int64_t)p.N * p.K;
+    // fp8: a wavefront's chunks go to the MFMA in pairs
+    constexpr bool HALVES_OK = CPL % 2 == 0 && (I8 || (CPL / 2) % 2 == 0 || CPL / 2 == 1);
+    if (HALVES_OK && bytes >= ((int64_t)100 << 20)) {
+        if constexpr (HALVES_OK)
+            hipLaunchKernelGGL((gemv8_row_kernel<I8, CPL / 2, 4, 2>), dim3((unsigned)((p.N + 1) / 2)), dim3(256), 0, s, p);
+    } else {
+        hipLaunchKernelGGL((gemv8_row_kernel<I8, CPL, 8, 1>), dim3((unsigned)((p.N + 7) / 8)), dim3(512), 0, s, p);
+    }
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
