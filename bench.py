@@ -3,8 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu] [--no-sweep]
 
-Prints ONE JSON line.  Configs are numbered 1 .. 5 as BASELINE.md numbers them (config n is
-BASELINE.json's configs[n - 1]).  The headline workload is the largest single-GPU M = 1 configuration, config 5's
+Prints ONE JSON line.  Configs are numbered 1 .. 5: config n is BASELINE.json's configs[n - 1].  The headline workload is the largest single-GPU M = 1 configuration, config 5's
 GEMV: e4m3 weights [11008, 4096] with a per-tensor scale under one e4m3 activation row, fp32 accumulate, bf16
 out - 45 MB per launch, the size at which a fraction of the HBM roofline means something (config 2's 1.66 MB
 layers are launch-bound by construction and stay a row of `results`).  A step is one launch.  Weights, inputs
