@@ -45,7 +45,8 @@ int32_t nq_diag_gemm8_timeline(nq_handle h, const void* x, int32_t x_dtype, cons
 /* nq_forward for 8-bit activations (int8 with per-row scales over a W8_CHANNEL layer, e4m3 codes with one scale over
  * an FP8_E4M3 layer; M >= 64, IN a multiple of 128) on the GEMM kernel of the caller's choice (no counterpart in the
  * reference): tile = 256, the 256 x 256 tile kernel nq_forward takes from about a round and a half of such tiles on,
- * or 128, the 128 x 128 tile kernel it takes below that where no 16-row tile kernel is estimated faster.  The two
+ * or 128, the 128 x 128 tile kernel it takes below that where no 16-row tile kernel is estimated faster; 2564 / 2568:
+ * the 256 x 256 tile kernel on four / eight wavefronts per workgroup (256 takes eight for int8, four for fp8).  All
  * return the same bits; tests hold each against the oracle on shapes the dispatch would give to the other, and
  * bench.py times them side by side.  Acts on this one launch only. */
 int32_t nq_diag_forward_gemm8(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, void* y, int32_t y_dtype,

@@ -13,7 +13,8 @@
 // same loop built on the 32 x 32 shapes took 107 us (fp8) and 127 us (int8) for
 // 8192 x 4096 x 4096 where this one takes 102 and 114.
 //
-// Tiling.  One workgroup of 4 wavefronts (2 x 2) owns a 256 x 256 tile of y;
+// Tiling.  (The fp8 form; int8 runs the same tile on 8 wavefronts, described below.)  One workgroup of 4 wavefronts
+// (2 x 2) owns a 256 x 256 tile of y;
 // each wavefront owns 128 x 128 of it as 8 x 8 MFMA tiles of 16 x 16, i.e. 256
 // fp32/int32 accumulators per lane (the AGPR half of the unified register
 // file), one workgroup per CU.  A tile this large is what keeps operand traffic
@@ -45,6 +46,16 @@
 // transfers of 1 KiB contiguous from a few KiB per wavefront (L2 hits, one line run
 // instead of eight lines) cost half as much.  Moving 64 KiB per stage and CU from L2 is
 // 14 TB/s over the chip, and at the power limit that traffic is paid in clock.
+//
+// Eight wavefronts.  The same tile, stages, layout and epilogue with 8 wavefronts (4 x 2, each 64 x 128: 128
+// accumulators per lane, two wavefronts per SIMD, 256 registers each, so one set of registers per fragment and each
+// requested again one MFMA after its last reader; ev8_slot below).  Every accumulator still adds its stages in the same
+// order: the two forms return the same bits.  int8: 8192 x 4096 x 4096 105 - 108 us against 110 - 112 on the same
+// boxes, 8192^3 386 against 407 - 413, and a single round of tiles (M = 2048 over 4096 x 4096) 42 - 43 against 49.5: the
+// two short phases per stage of the int8 MFMA leave a lone wavefront waiting more often than the fp8 form's one long
+// phase, and a second wavefront on the SIMD fills those waits.  fp8: the same time either way (95.5 - 99 us; N = 11008
+// and 8192^3 1 - 2 % slower), so fp8 stays on four.  Both forms take ~1.08 us per stage with half the CUs busy and no
+// power limit in play: what is left over the MFMAs' 0.85 is not a lone wavefront's issue order.
 //
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= ((row >> 1) + 6) & 7.  A 128-bit read is served in passes of
@@ -191,16 +202,69 @@ __host__ __device__ constexpr int dma_at(int m) {
     return -1;
 }
 
+// ---- the same for the form with eight wavefronts (4 x 2, each 64 x 128 of the tile: 4 token fragments, 8 channel
+// fragments, 32 MFMAs per phase, two wavefronts per SIMD so that one's waits stand under the other's MFMAs).  With 128
+// accumulators a wavefront has 256 registers in all, so every fragment has ONE set of registers and is requested again
+// one MFMA after its last reader.  Order: m -> token fragment i = (m % 16) / 4, channel fragment j = 4 (m / 16) + m % 4:
+// channel fragments 0 .. 3 are done with after MFMAs 12 .. 15, token fragment i after 19 + 4 i, channel fragments
+// 4 .. 7 after 28 .. 31.  The last two requests of a phase's fragments (w7, x3) fall into the phase itself, slots 0, 1.
+//   event e:   0     1     2    3    4    5    6    7    8    9    10   11
+//   brings:    w7'   x3'   w0   w1   w2   w3   x0   x1   x2   w4   w5   w6     (': this phase's own)
+__host__ __device__ constexpr int ev8_slot(int e) {
+    constexpr int s[12] = {0, 1, 13, 14, 15, 16, 20, 24, 28, 29, 30, 31};
+    return s[e];
+}
+__host__ __device__ constexpr int ev8_at(int m) {
+    for (int e = 0; e < 12; e++)
+        if (ev8_slot(e) == m) return e;
+    return -1;
+}
+// events 0 .. 11: the phase before, 12 .. 23: this phase; barrier_at: the MFMA in front of which the stage's barrier
+// (with its lgkmcnt(0)) stands, or -1
+__host__ __device__ constexpr int lds_wait8(int m_want, int reads_per_fragment, int barrier_at) {
+    int landed = 0;
+    for (int m = 0; m < 32; m++) {
+        const int i = (m % 16) / 4, j = 4 * (m / 16) + m % 4;
+        int issued = 12;
+        for (int e = 0; e < 12; e++)
+            if (ev8_slot(e) < m) issued++;
+        const int nx = i < 3 ? 6 + i : 12 + 1;
+        const int nw = j < 4 ? 2 + j : (j < 7 ? 9 + (j - 4) : 12 + 0);
+        const int need = nx > nw ? nx : nw;
+        int w = -1;
+        if (m == barrier_at) {
+            landed = issued;
+        } else if (need >= landed) {
+            int a = issued - 1 - need;
+            const int cap = 15 / reads_per_fragment;
+            if (a > cap) a = cap;
+            w = a * reads_per_fragment;
+            landed = issued - a;
+        }
+        if (m == m_want) return w;
+    }
+    return -1;
+}
+// (the barrier in front of MFMA 2, 4, 8 or 12, the transfers in consecutive slots or every other one: the same time)
+constexpr int BARRIER8_AT = 8;
+// the eight transfers per wavefront and stage: after the barrier, in slots without a request, every other one
+__host__ __device__ constexpr int dma8_at(int m) {
+    constexpr int s[8] = {8, 10, 12, 17, 19, 21, 23, 25};
+    for (int t = 0; t < 8; t++)
+        if (s[t] == m) return t;
+    return -1;
+}
+
 // BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with BK = 128.
 // KIND: the output type the epilogue is built for (0 fp32, 1 bf16, 2 raw int32 accumulators); one
 // kernel per kind, because with all three in one function the register allocator spills.
-template <bool FP8, int KIND_, int BN, int BK>
+template <bool FP8, int KIND_, int BN, int BK, int WAVES>
 __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int STAGE_BYTES = (BM + BN) * BK;
     constexpr int SLOTS = BK / 16;     // 16-byte slots per LDS row
     constexpr int WN = BN / 2;         // channels per wavefront
-    constexpr int TI = 8, TJ = WN / 16;  // fragments of 16 rows: token rows i, channel columns j
-    static_assert(BM == 256 && BN == 256 && BK == 128 && TJ == 8, "the phase model is written for this tile");
+    constexpr int TI = 32 / WAVES, TJ = WN / 16;  // fragments of 16 rows: token rows i, channel columns j
+    static_assert(BM == 256 && BN == 256 && BK == 128 && TJ == 8 && (WAVES == 4 || WAVES == 8), "the phase models are written for this tile");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const unsigned long long t_entry = wall_clock64();
     const int tid = threadIdx.x;
@@ -232,9 +296,9 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     // lane that lands in physical slot s of its row fetches logical slot s ^ swz(row).
     typedef __attribute__((address_space(3))) void lptr_t;
     constexpr int DROWS = 1024 / BK;           // rows per instruction
-    constexpr int DA = BM / 4 / DROWS;         // instructions per wavefront and stage, x tile
-    constexpr int DB = BN / 4 / DROWS;         // ... w tile
-    static_assert(DA + DB == 16, "dma_at() places 16 transfers per wavefront and stage");
+    constexpr int DA = BM / WAVES / DROWS;         // instructions per wavefront and stage, x tile
+    constexpr int DB = BN / WAVES / DROWS;         // ... w tile
+    static_assert(DA + DB == 64 / WAVES, "dma_at() / dma8_at() place every transfer of a wavefront and stage");
     // addresses as a uniform 64-bit tile base (advanced by k0) plus a 32-bit per-lane offset, and
     // the LDS destination as a scalar: two instructions per transfer (set M0, issue)
     const uint8_t* const abase = p.a + (int64_t)m0 * p.K;
@@ -242,13 +306,13 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     uint32_t doff[DA + DB];
 #pragma unroll
     for (int t = 0; t < DA; t++) {
-        const int row = wave * (BM / 4) + t * DROWS + lane / SLOTS;
+        const int row = wave * (BM / WAVES) + t * DROWS + lane / SLOTS;
         const int slot = (lane % SLOTS) ^ swz(row);
         doff[t] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.K + slot * 16;
     }
 #pragma unroll
     for (int t = 0; t < DB; t++) {
-        const int row = wave * (BN / 4) + t * DROWS + lane / SLOTS;
+        const int row = wave * (BN / WAVES) + t * DROWS + lane / SLOTS;
         const int slot = (lane % SLOTS) ^ swz(row);
         doff[DA + t] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.K + slot * 16;
     }
@@ -260,8 +324,8 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     uint32_t dbase[2][2];  // [buffer][x tile, w tile]: this wavefront's first destination
 #pragma unroll
     for (int buf = 0; buf < 2; buf++) {
-        dbase[buf][0] = lds_addr0 + buf * STAGE_BYTES + wave * (BM / 4) * BK;
-        dbase[buf][1] = lds_addr0 + buf * STAGE_BYTES + BM * BK + wave * (BN / 4) * BK;
+        dbase[buf][0] = lds_addr0 + buf * STAGE_BYTES + wave * (BM / WAVES) * BK;
+        dbase[buf][1] = lds_addr0 + buf * STAGE_BYTES + BM * BK + wave * (BN / WAVES) * BK;
     }
 #define NQ_DMA(t, buf, srca, srcb)                                                                     \
     do {                                                                                               \
@@ -296,10 +360,10 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const uint32_t so = (uint32_t)(((FP8 ? 2 * fc + u : 4 * u + fc) ^ fsw) << 4);
-            aaddr[buf][u] = lds_addr0 + buf * STAGE_BYTES + (wm * 128 + frow) * BK + so;
+            aaddr[buf][u] = lds_addr0 + buf * STAGE_BYTES + (wm * (16 * TI) + frow) * BK + so;
             baddr[buf][u] = lds_addr0 + buf * STAGE_BYTES + BM * BK + (wn * WN + frow) * BK + so;
         }
-    i32x4 xf[TI][R], wf[2][TJ][R];
+    i32x4 xf[TI][R], wf[WAVES == 4 ? 2 : 1][TJ][R];
 #define NQ_LDS_READ(dst, addr, imm) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(imm))
 #define NQ_LDS_WAIT(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n))
     // zc: the accumulator's first MFMA of the tile (C = 0)
@@ -390,16 +454,56 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_sched_barrier(0);
         });
     };
+    // The same for eight wavefronts: 32 MFMAs, one set of registers per fragment (see ev8_slot).
+    auto phase8 = [&](auto bufc, auto phc, auto zeroc, bool have2, const uint8_t* srca, const uint8_t* srcb) {
+        constexpr int BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
+        constexpr bool LAST = PHI == PH - 1;
+        constexpr int NBUF = LAST ? BUF ^ 1 : BUF, NPH = LAST ? 0 : PHI + 1;
+        static_for<32>([&](auto mc) {
+            constexpr int m = decltype(mc)::value, i = (m % 16) / 4, j = 4 * (m / 16) + m % 4;
+            if constexpr (LAST && m == BARRIER8_AT) {
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+            } else {
+                constexpr int al = lds_wait8(m, R, LAST ? BARRIER8_AT : -1);
+                if constexpr (al >= 0) NQ_LDS_WAIT(al);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mma(zeroc, i, j, xf[i], wf[0][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            constexpr int e = ev8_at(m);
+            using z0 = integral_constant<int, 0>;
+            if constexpr (e == 0) {
+                read_w(z0{}, integral_constant<int, 7>{}, bufc, phc);
+            } else if constexpr (e == 1) {
+                read_x(integral_constant<int, 3>{}, bufc, phc);
+            } else if constexpr (e >= 2 && e <= 5) {
+                read_w(z0{}, integral_constant<int, e - 2>{}, integral_constant<int, NBUF>{}, integral_constant<int, NPH>{});
+            } else if constexpr (e >= 6 && e <= 8) {
+                read_x(integral_constant<int, e - 6>{}, integral_constant<int, NBUF>{}, integral_constant<int, NPH>{});
+            } else if constexpr (e >= 9) {
+                read_w(z0{}, integral_constant<int, e - 5>{}, integral_constant<int, NBUF>{}, integral_constant<int, NPH>{});
+            }
+            if constexpr (LAST && dma8_at(m) >= 0) {
+                if (have2) {
+                    constexpr int t = dma8_at(m);
+                    NQ_DMA(t, BUF, srca, srcb);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
     // one stage, read from buffer BUF; its last phase refills BUF with stage st + 2
     auto stage = [&](auto bufc, auto zeroc, int st, int KT) {
         const bool have2 = st + 2 < KT;
         const uint8_t* const srca = abase + (int64_t)(st + 2) * BK;
         const uint8_t* const srcb = bbase + (int64_t)(st + 2) * BK;
-        if constexpr (PH == 1) {
-            phase(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
+        if constexpr (WAVES == 8) {
+            phase8(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
+            if constexpr (PH == 2) phase8(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
         } else {
             phase(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
-            phase(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
+            if constexpr (PH == 2) phase(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
         }
     };
 
@@ -411,10 +515,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 #define NQ_DMA_ALL(buf)                                                                            \
     NQ_DMA(0, buf, srca, srcb); NQ_DMA(1, buf, srca, srcb); NQ_DMA(2, buf, srca, srcb);            \
     NQ_DMA(3, buf, srca, srcb); NQ_DMA(4, buf, srca, srcb); NQ_DMA(5, buf, srca, srcb);            \
-    NQ_DMA(6, buf, srca, srcb); NQ_DMA(7, buf, srca, srcb); NQ_DMA(8, buf, srca, srcb);            \
-    NQ_DMA(9, buf, srca, srcb); NQ_DMA(10, buf, srca, srcb); NQ_DMA(11, buf, srca, srcb);          \
-    NQ_DMA(12, buf, srca, srcb); NQ_DMA(13, buf, srca, srcb); NQ_DMA(14, buf, srca, srcb);         \
-    NQ_DMA(15, buf, srca, srcb);
+    NQ_DMA(6, buf, srca, srcb); NQ_DMA(7, buf, srca, srcb);                                        \
+    if constexpr (WAVES == 4) {                                                                    \
+        NQ_DMA(8, buf, srca, srcb); NQ_DMA(9, buf, srca, srcb); NQ_DMA(10, buf, srca, srcb);       \
+        NQ_DMA(11, buf, srca, srcb); NQ_DMA(12, buf, srca, srcb); NQ_DMA(13, buf, srca, srcb);     \
+        NQ_DMA(14, buf, srca, srcb); NQ_DMA(15, buf, srca, srcb);                                  \
+    }
         NQ_DMA_ALL(0)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -450,7 +556,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     // + 0..3 (MFMA rows, registers 0..3).  Per-token work is lane-local and four outputs of a row of y are adjacent.
     // Each wavefront stages its results through its own LDS region as [token][channel] rows, and writes them out as
     // 128-bit stores, 256 B (bf16) or 512 B (fp32 / int32) contiguous per row of y.
-    const int wm0 = m0 + wm * 128, wn0 = n0 + wn * WN;
+    const int wm0 = m0 + wm * (16 * TI), wn0 = n0 + wn * WN;
     const int lm = lane & 15, lq = lane >> 4;
     // whole 16-byte stores wherever the tile's columns all exist and rows of y stay 16-byte aligned
     // (a tile that only M cuts short just skips the rows past M)
@@ -619,14 +725,21 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 template <bool FP8, int KIND>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm8_kernel(const Gemm8Params p) {
-    gemm8_body<FP8, KIND, 256, 128>(p);
+    gemm8_body<FP8, KIND, 256, 128, 4>(p);
+}
+
+template <bool FP8, int KIND>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm8w_kernel(const Gemm8Params p) {
+    gemm8_body<FP8, KIND, 256, 128, 8>(p);
 }
 
 template <typename K>
-int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int bn, int bk, hipStream_t s) {
-    const size_t lds = (size_t)2 * (BM + bn) * bk;
+int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int waves, hipStream_t s) {
+    // two stage buffers of 64 KiB; the eight-wavefront form's epilogue stages 17 KiB per wavefront
+    const size_t lds = waves == 8 ? (size_t)8 * 17408 : (size_t)2 * (BM + 256) * 128;
     NQ_HIP(set_max_lds_once(*attr, reinterpret_cast<const void*>(kernel), lds));
-    hipLaunchKernelGGL(kernel, dim3(p.tiles_m * p.tiles_n), dim3(256), lds, s, p);
+    hipLaunchKernelGGL(kernel, dim3(p.tiles_m * p.tiles_n), dim3(64 * waves), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
 }
@@ -657,14 +770,26 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     const bool i8 = a.x_dtype == NQ_DT_I8;
     p.chan_vec = L->out % 4 == 0 && L->out >= 4 && (!i8 || a.y_dtype == NQ_DT_I32 || (uintptr_t)p.col_scale % 16 == 0) &&
                  (!a.bias || (uintptr_t)a.bias % (a.bias_dtype == NQ_DT_F32 ? 16 : 8) == 0);
-    static LdsAttrOnce attr_set[5];
+    static LdsAttrOnce attr_set[10];
     const bool f32 = a.y_dtype == NQ_DT_F32;
+    // int8 runs on the eight-wavefront form (8192 x 4096 x 4096: 105 - 108 us against 110 - 112; one round of tiles,
+    // M = 2048: 42 - 43 against 49.5), fp8 on the four-wavefront form (the two measure the same, 95.5 - 99 us on the
+    // same box; N = 11008 and 8192^3 1 - 2 % slower with eight)
+    const int waves = a.diag_gemm8_waves ? a.diag_gemm8_waves : (a.x_dtype == NQ_DT_I8 ? 8 : 4);
+    if (waves == 8) {
+        if (a.x_dtype == NQ_DT_FP8_E4M3)
+            return f32 ? launch_cfg(gemm8w_kernel<true, 0>, &attr_set[5], p, 8, a.stream)
+                       : launch_cfg(gemm8w_kernel<true, 1>, &attr_set[6], p, 8, a.stream);
+        if (a.y_dtype == NQ_DT_I32) return launch_cfg(gemm8w_kernel<false, 2>, &attr_set[9], p, 8, a.stream);
+        return f32 ? launch_cfg(gemm8w_kernel<false, 0>, &attr_set[7], p, 8, a.stream)
+                   : launch_cfg(gemm8w_kernel<false, 1>, &attr_set[8], p, 8, a.stream);
+    }
     if (a.x_dtype == NQ_DT_FP8_E4M3)
-        return f32 ? launch_cfg(gemm8_kernel<true, 0>, &attr_set[0], p, 256, 128, a.stream)
-                   : launch_cfg(gemm8_kernel<true, 1>, &attr_set[1], p, 256, 128, a.stream);
-    if (a.y_dtype == NQ_DT_I32) return launch_cfg(gemm8_kernel<false, 2>, &attr_set[4], p, 256, 128, a.stream);
-    return f32 ? launch_cfg(gemm8_kernel<false, 0>, &attr_set[2], p, 256, 128, a.stream)
-               : launch_cfg(gemm8_kernel<false, 1>, &attr_set[3], p, 256, 128, a.stream);
+        return f32 ? launch_cfg(gemm8_kernel<true, 0>, &attr_set[0], p, 4, a.stream)
+                   : launch_cfg(gemm8_kernel<true, 1>, &attr_set[1], p, 4, a.stream);
+    if (a.y_dtype == NQ_DT_I32) return launch_cfg(gemm8_kernel<false, 2>, &attr_set[4], p, 4, a.stream);
+    return f32 ? launch_cfg(gemm8_kernel<false, 0>, &attr_set[2], p, 4, a.stream)
+               : launch_cfg(gemm8_kernel<false, 1>, &attr_set[3], p, 4, a.stream);
 }
 
 }  // namespace nq

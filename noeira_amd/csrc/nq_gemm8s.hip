@@ -287,15 +287,14 @@ double gemm8_estimate_us(int M, int N, int K, bool i8, bool small_tile) {
         return (double)((tiles + 255) / 256) * (i8 ? 3.0 + 0.74 * steps : 2.5 + 0.6 * steps);
     }
     const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-    return (double)((tiles + 255) / 256) * (i8 ? 14.0 + 1.25 * steps : 10.0 + 1.1 * steps);
+    return (double)((tiles + 255) / 256) * (i8 ? 9.5 + 1.03 * steps : 10.0 + 1.1 * steps);
 }
 
 bool gemm8s_applicable(const ForwardArgs& a) {
     if (!gemm8_applicable(a)) return false;
     const nq_layer* L = a.L;
     const bool i8 = a.x_dtype == NQ_DT_I8;
-    // (a tenth in hand for the large tile: where the two estimates meet it measured the faster, 52.4 against 56.8 us
-    // for int8 at M = 2048 over 4096 x 4096)
+    // (a tenth in hand for the large tile: where the two estimates meet it measured the faster)
     return gemm8_estimate_us(a.M, L->out, L->in, i8, true) < 0.9 * gemm8_estimate_us(a.M, L->out, L->in, i8, false);
 }
 

@@ -430,7 +430,8 @@ def test_mlp3_other_shapes_and_errors():
 
 # ── the two tile sizes of the 8-bit GEMM ────────────────────────────────────────────────────────────────────────
 def _gemm8(lin, tile, x, x_dt, x_scale, M, out_dtype, bias=None, epilogue="none"):
-    """The 8-bit GEMM on the 128 x 128 (`tile` = 128) or the 256 x 256 tile kernel, whatever nq_forward would choose."""
+    """The 8-bit GEMM on the 128 x 128 (`tile` = 128) or the 256 x 256 tile kernel (256; 2564 / 2568: on four / eight
+    wavefronts), whatever nq_forward would choose."""
     import ctypes as C
     from noeira_amd import _lib as L
     out = torch.full((M, lin.OUT), 7, dtype=out_dtype, device="cuda")
@@ -456,11 +457,12 @@ def test_gemm_tile_sizes_against_the_oracle_and_each_other(M, K, N):
     xq, sx, bias = torch.from_numpy(xq_h).cuda(), torch.from_numpy(sx_h).cuda(), torch.from_numpy(bias_h).cuda()
     acc_o = O.w8a8_acc_i32(xq_h, w)
     want = O.w8a8_epilogue(acc_o, sx_h, s, bias_h, relu=True)
-    for tile in (128, 256):
+    for tile in (128, 2564, 2568):  # (256: whichever of the last two nq_forward takes)
         assert np.array_equal(_gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.int32).cpu().numpy(), acc_o), tile
         assert rel_rms(_gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.float32, bias, "relu").cpu().numpy(), want) < 1e-5, tile
     for dt in (torch.float32, torch.bfloat16):
-        assert torch.equal(_gemm8(lin, 128, xq, L.DT_I8, sx, M, dt, bias, "relu"), _gemm8(lin, 256, xq, L.DT_I8, sx, M, dt, bias, "relu")), dt
+        for tile in (2564, 2568):
+            assert torch.equal(_gemm8(lin, 128, xq, L.DT_I8, sx, M, dt, bias, "relu"), _gemm8(lin, tile, xq, L.DT_I8, sx, M, dt, bias, "relu")), (dt, tile)
     a, b = fp8_operands(rng, M, N, K)
     f8 = FP8Linear(K, N)
     f8.set_weight(b, 0.25)
@@ -468,10 +470,11 @@ def test_gemm_tile_sizes_against_the_oracle_and_each_other(M, K, N):
     ad = torch.from_numpy(a).cuda()
     y64, _ = O.fp8_forward_f64(a, b, np.float32(0.5), np.float32(0.25), want_bf16=False)
     ref = y64 + bias_h.astype(np.float64)
-    for tile in (128, 256):
+    for tile in (128, 2564, 2568):
         got = _gemm8(f8, tile, ad, L.DT_FP8_E4M3, xs, M, torch.float32, bias).cpu().numpy()
         assert np.abs(got - ref).max() <= 3e-4 * np.sqrt((ref ** 2).mean()), tile
     for dt in (torch.float32, torch.bfloat16):
-        assert torch.equal(_gemm8(f8, 128, ad, L.DT_FP8_E4M3, xs, M, dt, bias), _gemm8(f8, 256, ad, L.DT_FP8_E4M3, xs, M, dt, bias)), dt
+        for tile in (2564, 2568):
+            assert torch.equal(_gemm8(f8, 128, ad, L.DT_FP8_E4M3, xs, M, dt, bias), _gemm8(f8, tile, ad, L.DT_FP8_E4M3, xs, M, dt, bias)), (dt, tile)
     # what nq_forward itself returns for the call (whichever kernel it takes): the oracle's accumulators
     assert np.array_equal(lin.forward_a8(xq, sx, out_dtype=torch.int32).cpu().numpy(), acc_o)
