@@ -1091,8 +1091,8 @@ int32_t nq_diag_forward_gemm8(nq_handle h, const void* x, int32_t x_dtype, const
     int32_t rc = check_handle(h, "nq_diag_forward_gemm8");
     if (rc) return rc;
     if ((rc = need_loaded(h, "forward"))) return rc;
-    if (tile != 128 && tile != 256 && tile != 2564 && tile != 2568)
-        return fail(NQ_ERR_INVALID, "nq_diag_forward_gemm8: tile is 128, 256, or 2564 / 2568 (256 with four / eight wavefronts)");
+    if (tile != 128 && tile != 256 && tile != 2564 && tile != 2568 && tile != 1282)
+        return fail(NQ_ERR_INVALID, "nq_diag_forward_gemm8: tile is 128, 256, 2564 / 2568 (256 with four / eight wavefronts) or 1282 (128 x 256)");
     if (!x || !y || !x_scale || ((uintptr_t)x & 15) || ((uintptr_t)y & 3) || (x_dtype != NQ_DT_I8 && x_dtype != NQ_DT_FP8_E4M3) ||
         (y_dtype != NQ_DT_F32 && y_dtype != NQ_DT_BF16 && !(y_dtype == NQ_DT_I32 && x_dtype == NQ_DT_I8 && !bias && epilogue == NQ_EPI_NONE)) ||
         (epilogue != NQ_EPI_NONE && epilogue != NQ_EPI_RELU) || (bias && bias_dtype != NQ_DT_F32 && bias_dtype != NQ_DT_BF16))
@@ -1102,7 +1102,7 @@ int32_t nq_diag_forward_gemm8(nq_handle h, const void* x, int32_t x_dtype, const
     ForwardArgs a{h, x, x_dtype, x_scale, y, y_dtype, M, bias, bias_dtype, epilogue, (hipStream_t)stream, seg};
     if (h->glu || !h->seg_end.empty() || !gemm8_applicable(a))
         return fail(NQ_ERR_UNSUPPORTED, "nq_diag_forward_gemm8: the 8-bit GEMM does not take this call (format, M >= 64, IN % 128)");
-    if (tile > 256) a.diag_gemm8_waves = tile % 10;
+    if (tile > 256) a.diag_gemm8_waves = tile == 1282 ? 12 : tile % 10;
     return tile == 128 ? launch_gemm8s(a) : launch_gemm8(a);
 }
 

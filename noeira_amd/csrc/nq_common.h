@@ -135,7 +135,7 @@ struct ForwardArgs {
     float lora_s = 0.0f;
     // nq_diag_gemm8_timeline: where the large-tile GEMM writes its per-tile clock readings (null: none)
     unsigned long long* diag_stamps = nullptr;
-    int diag_gemm8_waves = 0;  // 0: the library's choice; 4 / 8: the 256 x 256 tile GEMM with that many wavefronts
+    int diag_gemm8_waves = 0;  // 0: the library's choice; 4 / 8: the 256 x 256 tile GEMM with that many wavefronts; 12: its 128 x 256 tile form
     // nq_diag_forward_a16: the 16-row tile kernel's shape for this launch, mw << 4 | nw (0: the library's choice)
     int32_t diag_a16_shape = 0;
 };

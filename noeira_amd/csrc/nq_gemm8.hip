@@ -57,6 +57,22 @@
 // and 8192^3 1 - 2 % slower), so fp8 stays on four.  Both forms take ~1.08 us per stage with half the CUs busy and no
 // power limit in play: what is left over the MFMAs' 0.85 is not a lone wavefront's issue order.
 //
+// In cycles.  The K loop's own reading of the shader clock beside the constant one (fp8, 8192 x 4096 x 4096, all 256
+// CUs busy): 2283 cycles per stage at 1.86 - 1.88 GHz, against the 2048 cycles the stage's MFMAs occupy the pipe and
+// against 2.18 GHz under the same MFMAs with operands in registers; with half the CUs busy (M = 2048) 2320 cycles at
+// 2.19 - 2.24 GHz.  So nine tenths of the loop's cycles are MFMA cycles wherever it runs, and what a full chip loses
+// beyond that is clock: the transfers and fragment reads are paid in power, not in stalls.
+//
+// Half tiles.  A launch that fills at most half a round of workgroups (128 tiles of 256 x 256) leaves CUs idle for the
+// whole call, and so do the tiles left over after the last full round.  Both go on a 128 x 256 tile instead (4
+// wavefronts, 2 x 2, each 64 x 128 with the eight-wavefront form's phase), twice as many workgroups: the call as a
+// whole, or the leftover tiles in a second launch when they are whole columns of the last band of row tiles (N = 11008
+// at M = 8192: 96 of 1376, 12 columns of 8).  A stage of that tile has half the MFMAs for three quarters of the
+// transfers and is shorter than the transfers' way from L2, so it has three stage buffers (48 KiB each) and a stage's
+// transfers two stages to land in; even so it is delivery that bounds it once most CUs draw on L2 (fp8, K = 4096: 24.7
+// us with 128 workgroups, 26.9 with 192, 31.3 with 256 - against 41 - 43 us for the same calls on 64 .. 128 tiles of
+// 256 x 256).  Same sums in the same order: same bits.
+//
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= ((row >> 1) + 6) & 7.  A 128-bit read is served in passes of
 // sixteen lanes that are not consecutive lanes (per half of the wavefront the quads of lanes
@@ -104,7 +120,6 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 
-constexpr int BM = 256;  // rows of x per workgroup tile (2 wavefronts x 128)
 
 struct Gemm8Params {
     const uint8_t* a;  // x [M][K]
@@ -116,6 +131,8 @@ struct Gemm8Params {
     float tscale;            // fp8: the weight's per-tensor scale
     int32_t M, N, K;
     int32_t tiles_m, tiles_n;
+    int32_t grid;            // workgroups to launch: the first `grid` tiles of the order (0: all tiles_m x tiles_n)
+    int32_t m_base, n_base;  // the first row and channel of the part of y this launch covers (its tiles count from there)
     int32_t y_dtype, bias_dtype, epilogue;
     unsigned long long* stamps;  // a diagnostic: per workgroup, four readings of the constant 100 MHz clock, or null
     int32_t chan_vec;  // N % 4 == 0 and col_scale / bias aligned for one 16-byte (bf16 bias: 8-byte) load per 4 channels
@@ -248,23 +265,26 @@ __host__ __device__ constexpr int lds_wait8(int m_want, int reads_per_fragment, 
 // (the barrier in front of MFMA 2, 4, 8 or 12, the transfers in consecutive slots or every other one: the same time)
 constexpr int BARRIER8_AT = 8;
 // the eight transfers per wavefront and stage: after the barrier, in slots without a request, every other one
-__host__ __device__ constexpr int dma8_at(int m) {
-    constexpr int s[8] = {8, 10, 12, 17, 19, 21, 23, 25};
-    for (int t = 0; t < 8; t++)
-        if (s[t] == m) return t;
+// (twelve for the 128 x 256 tile on four wavefronts)
+__host__ __device__ constexpr int dma8_at(int m, int n) {
+    constexpr int s8[8] = {8, 10, 12, 17, 19, 21, 23, 25};
+    constexpr int s12[12] = {8, 9, 10, 11, 12, 17, 18, 19, 21, 22, 23, 25};
+    for (int t = 0; t < n; t++)
+        if ((n == 8 ? s8[t] : s12[t]) == m) return t;
     return -1;
 }
 
 // BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with BK = 128.
 // KIND: the output type the epilogue is built for (0 fp32, 1 bf16, 2 raw int32 accumulators); one
 // kernel per kind, because with all three in one function the register allocator spills.
-template <bool FP8, int KIND_, int BN, int BK, int WAVES>
+template <bool FP8, int KIND_, int BM, int BN, int BK, int WAVES>
 __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int STAGE_BYTES = (BM + BN) * BK;
     constexpr int SLOTS = BK / 16;     // 16-byte slots per LDS row
     constexpr int WN = BN / 2;         // channels per wavefront
-    constexpr int TI = 32 / WAVES, TJ = WN / 16;  // fragments of 16 rows: token rows i, channel columns j
-    static_assert(BM == 256 && BN == 256 && BK == 128 && TJ == 8 && (WAVES == 4 || WAVES == 8), "the phase models are written for this tile");
+    constexpr int TI = BM / (8 * WAVES), TJ = WN / 16;  // fragments of 16 rows: token rows i, channel columns j
+    static_assert(BN == 256 && BK == 128 && TJ == 8 && ((BM == 256 && (WAVES == 4 || WAVES == 8)) || (BM == 128 && WAVES == 4)),
+                  "the phase models are written for these tiles");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const unsigned long long t_entry = wall_clock64();
     const int tid = threadIdx.x;
@@ -285,7 +305,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     const int in_band = lid - band * GM * p.tiles_n;
     const int tm = first_m + in_band % band_rows;
     const int tn = in_band / band_rows;
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = p.m_base + tm * BM, n0 = p.n_base + tn * BN;
 
     // the slot permutation of an LDS row (see the header): rows 16 f + r of any fragment f share it
     auto swz = [](int row) { return (((row >> 1) & 7) + 6) & 7; };
@@ -298,7 +318,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int DROWS = 1024 / BK;           // rows per instruction
     constexpr int DA = BM / WAVES / DROWS;         // instructions per wavefront and stage, x tile
     constexpr int DB = BN / WAVES / DROWS;         // ... w tile
-    static_assert(DA + DB == 64 / WAVES, "dma_at() / dma8_at() place every transfer of a wavefront and stage");
+    static_assert(DA + DB == 16 || DA + DB == 8 || DA + DB == 12, "dma_at() / dma8_at() place every transfer of a wavefront and stage");
     // addresses as a uniform 64-bit tile base (advanced by k0) plus a 32-bit per-lane offset, and
     // the LDS destination as a scalar: two instructions per transfer (set M0, issue)
     const uint8_t* const abase = p.a + (int64_t)m0 * p.K;
@@ -321,9 +341,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     // offset.  Three instructions per transfer.  (M0 is a reserved register the compiler sets itself
     // right before each of its own uses, so writing it here needs no clobber; SCC does.)
     const uint32_t lds_addr0 = (uint32_t)(uintptr_t)(lptr_t*)lds;
-    uint32_t dbase[2][2];  // [buffer][x tile, w tile]: this wavefront's first destination
+    // stage buffers: two of 64 KiB; the 128-row tile has three of 48 KiB, so that a stage's transfers have two stages
+    // of MFMAs to land in (one stage of its 32 MFMAs per wavefront is shorter than their way from L2)
+    constexpr int NB = BM == 128 ? 3 : 2;
+    uint32_t dbase[NB][2];  // [buffer][x tile, w tile]: this wavefront's first destination
 #pragma unroll
-    for (int buf = 0; buf < 2; buf++) {
+    for (int buf = 0; buf < NB; buf++) {
         dbase[buf][0] = lds_addr0 + buf * STAGE_BYTES + wave * (BM / WAVES) * BK;
         dbase[buf][1] = lds_addr0 + buf * STAGE_BYTES + BM * BK + wave * (BN / WAVES) * BK;
     }
@@ -354,9 +377,9 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     const int frow = lane & 15, fc = lane >> 4;
     const int fsw = swz(frow);
     // LDS byte addresses of this lane's reads: [buffer][u], u = half of the fragment (fp8) or phase of the stage (int8)
-    uint32_t aaddr[2][2], baddr[2][2];
+    uint32_t aaddr[NB][2], baddr[NB][2];
 #pragma unroll
-    for (int buf = 0; buf < 2; buf++)
+    for (int buf = 0; buf < NB; buf++)
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const uint32_t so = (uint32_t)(((FP8 ? 2 * fc + u : 4 * u + fc) ^ fsw) << 4);
@@ -455,14 +478,18 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
         });
     };
     // The same for eight wavefronts: 32 MFMAs, one set of registers per fragment (see ev8_slot).
-    auto phase8 = [&](auto bufc, auto phc, auto zeroc, bool have2, const uint8_t* srca, const uint8_t* srcb) {
+    // keep1 (three buffers): the stage before issued transfers too, and those may stay in flight across the barrier
+    auto phase8 = [&](auto bufc, auto phc, auto zeroc, bool have2, bool keep1, const uint8_t* srca, const uint8_t* srcb) {
         constexpr int BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
         constexpr bool LAST = PHI == PH - 1;
-        constexpr int NBUF = LAST ? BUF ^ 1 : BUF, NPH = LAST ? 0 : PHI + 1;
+        constexpr int NBUF = LAST ? (BUF + 1) % NB : BUF, NPH = LAST ? 0 : PHI + 1;
         static_for<32>([&](auto mc) {
             constexpr int m = decltype(mc)::value, i = (m % 16) / 4, j = 4 * (m / 16) + m % 4;
             if constexpr (LAST && m == BARRIER8_AT) {
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                if (keep1)
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(DA + DB) : "memory");
+                else
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_s_barrier();
             } else {
                 constexpr int al = lds_wait8(m, R, LAST ? BARRIER8_AT : -1);
@@ -484,23 +511,24 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             } else if constexpr (e >= 9) {
                 read_w(z0{}, integral_constant<int, e - 5>{}, integral_constant<int, NBUF>{}, integral_constant<int, NPH>{});
             }
-            if constexpr (LAST && dma8_at(m) >= 0) {
+            if constexpr (LAST && dma8_at(m, DA + DB) >= 0) {
                 if (have2) {
-                    constexpr int t = dma8_at(m);
+                    constexpr int t = dma8_at(m, DA + DB);
                     NQ_DMA(t, BUF, srca, srcb);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         });
     };
-    // one stage, read from buffer BUF; its last phase refills BUF with stage st + 2
+    // one stage, read from buffer BUF; its last phase refills BUF with stage st + NB
     auto stage = [&](auto bufc, auto zeroc, int st, int KT) {
-        const bool have2 = st + 2 < KT;
-        const uint8_t* const srca = abase + (int64_t)(st + 2) * BK;
-        const uint8_t* const srcb = bbase + (int64_t)(st + 2) * BK;
-        if constexpr (WAVES == 8) {
-            phase8(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
-            if constexpr (PH == 2) phase8(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
+        const bool have2 = st + NB < KT;
+        const bool keep1 = NB == 3 && st + 2 < KT;
+        const uint8_t* const srca = abase + (int64_t)(st + NB) * BK;
+        const uint8_t* const srcb = bbase + (int64_t)(st + NB) * BK;
+        if constexpr (TI == 4) {
+            phase8(bufc, integral_constant<int, 0>{}, zeroc, have2, keep1, srca, srcb);
+            if constexpr (PH == 2) phase8(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, keep1, srca, srcb);
         } else {
             phase(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
             if constexpr (PH == 2) phase(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
@@ -516,17 +544,38 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     NQ_DMA(0, buf, srca, srcb); NQ_DMA(1, buf, srca, srcb); NQ_DMA(2, buf, srca, srcb);            \
     NQ_DMA(3, buf, srca, srcb); NQ_DMA(4, buf, srca, srcb); NQ_DMA(5, buf, srca, srcb);            \
     NQ_DMA(6, buf, srca, srcb); NQ_DMA(7, buf, srca, srcb);                                        \
-    if constexpr (WAVES == 4) {                                                                    \
+    if constexpr (DA + DB >= 12) {                                                                 \
         NQ_DMA(8, buf, srca, srcb); NQ_DMA(9, buf, srca, srcb); NQ_DMA(10, buf, srca, srcb);       \
-        NQ_DMA(11, buf, srca, srcb); NQ_DMA(12, buf, srca, srcb); NQ_DMA(13, buf, srca, srcb);     \
+        NQ_DMA(11, buf, srca, srcb);                                                               \
+    }                                                                                              \
+    if constexpr (DA + DB == 16) {                                                                 \
+        NQ_DMA(12, buf, srca, srcb); NQ_DMA(13, buf, srca, srcb);                                  \
         NQ_DMA(14, buf, srca, srcb); NQ_DMA(15, buf, srca, srcb);                                  \
     }
         NQ_DMA_ALL(0)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (KT > 1) {
-            srca = abase + BK, srcb = bbase + BK;
-            NQ_DMA_ALL(1)
+        if constexpr (NB == 3) {
+            // all three buffers at once; stage 0 has landed when at most the other two stages' transfers are out
+            if (KT > 1) {
+                srca = abase + BK, srcb = bbase + BK;
+                NQ_DMA_ALL(1)
+            }
+            if (KT > 2) {
+                srca = abase + 2 * BK, srcb = bbase + 2 * BK;
+                NQ_DMA_ALL(2)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (DA + DB)) : "memory");
+            } else if (KT > 1) {
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DA + DB) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __syncthreads();
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (KT > 1) {
+                srca = abase + BK, srcb = bbase + BK;
+                NQ_DMA_ALL(1)
+            }
         }
 #undef NQ_DMA_ALL
     }
@@ -536,7 +585,16 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     static_for<TJ>([&](auto jc) { read_w(integral_constant<int, 0>{}, jc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
     NQ_LDS_WAIT(0);
     stage(integral_constant<int, 0>{}, std::true_type{}, 0, KT);
-    {
+    if constexpr (NB == 3) {
+        for (int st = 1; st < KT;) {
+            stage(integral_constant<int, 1>{}, std::false_type{}, st, KT);
+            if (++st >= KT) break;
+            stage(integral_constant<int, 2>{}, std::false_type{}, st, KT);
+            if (++st >= KT) break;
+            stage(integral_constant<int, 0>{}, std::false_type{}, st, KT);
+            ++st;
+        }
+    } else {
         int st = 1;
         for (; st + 1 < KT; st += 2) {
             stage(integral_constant<int, 1>{}, std::false_type{}, st, KT);
@@ -725,23 +783,51 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 template <bool FP8, int KIND>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm8_kernel(const Gemm8Params p) {
-    gemm8_body<FP8, KIND, 256, 128, 4>(p);
+    gemm8_body<FP8, KIND, 256, 256, 128, 4>(p);
 }
 
 template <bool FP8, int KIND>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm8w_kernel(const Gemm8Params p) {
-    gemm8_body<FP8, KIND, 256, 128, 8>(p);
+    gemm8_body<FP8, KIND, 256, 256, 128, 8>(p);
+}
+
+// a 128 x 256 tile on four wavefronts (2 x 2, each 64 x 128 as in the eight-wavefront form): for what fills at most
+// half a round of 256 x 256 tiles
+template <bool FP8, int KIND>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm8h_kernel(const Gemm8Params p) {
+    gemm8_body<FP8, KIND, 128, 256, 128, 4>(p);
 }
 
 template <typename K>
-int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int waves, hipStream_t s) {
-    // two stage buffers of 64 KiB; the eight-wavefront form's epilogue stages 17 KiB per wavefront
-    const size_t lds = waves == 8 ? (size_t)8 * 17408 : (size_t)2 * (BM + 256) * 128;
+int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int form, hipStream_t s) {
+    // two stage buffers of 64 KiB each (three of 48 for the 128-row tile); the eight-wavefront form's epilogue stages 17 KiB
+    // per wavefront
+    const size_t lds = form == 8 ? (size_t)8 * 17408 : form == 12 ? (size_t)3 * (128 + 256) * 128 : (size_t)2 * (256 + 256) * 128;
     NQ_HIP(set_max_lds_once(*attr, reinterpret_cast<const void*>(kernel), lds));
-    hipLaunchKernelGGL(kernel, dim3(p.tiles_m * p.tiles_n), dim3(64 * waves), lds, s, p);
+    hipLaunchKernelGGL(kernel, dim3(p.grid ? p.grid : p.tiles_m * p.tiles_n), dim3(form == 8 ? 512 : 256), lds, s, p);
     NQ_HIP(hipGetLastError());
     return NQ_OK;
+}
+
+// form: 4 / 8 = the 256 x 256 tile on that many wavefronts, 12 = the 128 x 256 tile.  kind: 0 fp32, 1 bf16, 2 raw int32
+int32_t launch_form(int form, bool fp8, int kind, const Gemm8Params& p, hipStream_t s) {
+    static LdsAttrOnce attr[3][5];
+    const int f = form == 4 ? 0 : form == 8 ? 1 : 2;
+    const int k = fp8 ? kind : 2 + kind;
+#define NQ_G8_PICK(KERNEL)                                                                     \
+    switch (k) {                                                                               \
+        case 0: return launch_cfg(KERNEL<true, 0>, &attr[f][0], p, form, s);                   \
+        case 1: return launch_cfg(KERNEL<true, 1>, &attr[f][1], p, form, s);                   \
+        case 2: return launch_cfg(KERNEL<false, 0>, &attr[f][2], p, form, s);                  \
+        case 3: return launch_cfg(KERNEL<false, 1>, &attr[f][3], p, form, s);                  \
+        default: return launch_cfg(KERNEL<false, 2>, &attr[f][4], p, form, s);                 \
+    }
+    if (form == 4) { NQ_G8_PICK(gemm8_kernel) }
+    if (form == 8) { NQ_G8_PICK(gemm8w_kernel) }
+    NQ_G8_PICK(gemm8h_kernel)
+#undef NQ_G8_PICK
 }
 
 }  // namespace
@@ -765,31 +851,49 @@ int32_t launch_gemm8(const ForwardArgs& a) {
     p.tscale = L->scale;
     p.M = a.M, p.N = L->out, p.K = L->in;
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
-    p.tiles_m = (a.M + BM - 1) / BM, p.tiles_n = (L->out + 255) / 256;
     p.stamps = a.diag_stamps;
-    const bool i8 = a.x_dtype == NQ_DT_I8;
+    const bool i8 = a.x_dtype == NQ_DT_I8, fp8 = !i8;
     p.chan_vec = L->out % 4 == 0 && L->out >= 4 && (!i8 || a.y_dtype == NQ_DT_I32 || (uintptr_t)p.col_scale % 16 == 0) &&
                  (!a.bias || (uintptr_t)a.bias % (a.bias_dtype == NQ_DT_F32 ? 16 : 8) == 0);
-    static LdsAttrOnce attr_set[10];
-    const bool f32 = a.y_dtype == NQ_DT_F32;
+    const int kind = a.y_dtype == NQ_DT_F32 ? 0 : a.y_dtype == NQ_DT_BF16 ? 1 : 2;
+    const int tm = (a.M + 255) / 256, tn = (L->out + 255) / 256;
+    const int tiles = tm * tn;
+    p.tiles_m = tm, p.tiles_n = tn;
+    if (a.diag_gemm8_waves == 12) {  // everything on 128-row tiles
+        p.tiles_m = (a.M + 127) / 128;
+        return launch_form(12, fp8, kind, p, a.stream);
+    }
     // int8 runs on the eight-wavefront form (8192 x 4096 x 4096: 105 - 108 us against 110 - 112; one round of tiles,
     // M = 2048: 42 - 43 against 49.5), fp8 on the four-wavefront form (the two measure the same, 95.5 - 99 us on the
     // same box; N = 11008 and 8192^3 1 - 2 % slower with eight)
-    const int waves = a.diag_gemm8_waves ? a.diag_gemm8_waves : (a.x_dtype == NQ_DT_I8 ? 8 : 4);
-    if (waves == 8) {
-        if (a.x_dtype == NQ_DT_FP8_E4M3)
-            return f32 ? launch_cfg(gemm8w_kernel<true, 0>, &attr_set[5], p, 8, a.stream)
-                       : launch_cfg(gemm8w_kernel<true, 1>, &attr_set[6], p, 8, a.stream);
-        if (a.y_dtype == NQ_DT_I32) return launch_cfg(gemm8w_kernel<false, 2>, &attr_set[9], p, 8, a.stream);
-        return f32 ? launch_cfg(gemm8w_kernel<false, 0>, &attr_set[7], p, 8, a.stream)
-                   : launch_cfg(gemm8w_kernel<false, 1>, &attr_set[8], p, 8, a.stream);
+    const int form = a.diag_gemm8_waves ? a.diag_gemm8_waves : (i8 ? 8 : 4);
+    if (a.diag_gemm8_waves || a.diag_stamps) return launch_form(form, fp8, kind, p, a.stream);
+    // What fills at most half a round of workgroups goes on 128 x 256 tiles, twice as many: a call that small as a
+    // whole, or the tiles left over after the last full round when they form a rectangle (the kernel deals tiles in
+    // bands of 8 row tiles, rows first, so the last `rest` tiles are whole columns of the last band when its row
+    // count divides `rest`).  Every accumulator adds the same terms in the same order on either tile: same bits.
+    constexpr int CUS = 256;
+    if (tiles <= CUS / 2) {
+        p.tiles_m = (a.M + 127) / 128;
+        return launch_form(12, fp8, kind, p, a.stream);
     }
-    if (a.x_dtype == NQ_DT_FP8_E4M3)
-        return f32 ? launch_cfg(gemm8_kernel<true, 0>, &attr_set[0], p, 4, a.stream)
-                   : launch_cfg(gemm8_kernel<true, 1>, &attr_set[1], p, 4, a.stream);
-    if (a.y_dtype == NQ_DT_I32) return launch_cfg(gemm8_kernel<false, 2>, &attr_set[4], p, 4, a.stream);
-    return f32 ? launch_cfg(gemm8_kernel<false, 0>, &attr_set[2], p, 4, a.stream)
-               : launch_cfg(gemm8_kernel<false, 1>, &attr_set[3], p, 4, a.stream);
+    const int rest = tiles % CUS;
+    const int last_band_rows = tm - (tm - 1) / 8 * 8;
+    if (tiles > CUS && rest > 0 && rest <= CUS / 2 && rest % last_band_rows == 0 && rest / last_band_rows <= tn) {
+        Gemm8Params q = p;
+        // (the kernel regroups workgroup ids over its own grid size: a grid of tiles - rest covers exactly the first
+        // tiles - rest tiles of the order)
+        q.grid = tiles - rest;
+        const int32_t rc = launch_form(form, fp8, kind, q, a.stream);
+        if (rc != NQ_OK) return rc;
+        Gemm8Params t = p;
+        t.m_base = (tm - last_band_rows) * 256;
+        t.n_base = (tn - rest / last_band_rows) * 256;
+        t.tiles_m = (a.M - t.m_base + 127) / 128;
+        t.tiles_n = rest / last_band_rows;
+        return launch_form(12, fp8, kind, t, a.stream);
+    }
+    return launch_form(form, fp8, kind, p, a.stream);
 }
 
 }  // namespace nq

@@ -287,6 +287,14 @@ double gemm8_estimate_us(int M, int N, int K, bool i8, bool small_tile) {
         return (double)((tiles + 255) / 256) * (i8 ? 3.0 + 0.74 * steps : 2.5 + 0.6 * steps);
     }
     const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    if (tiles <= 128) {
+        // the 128 x 256 tile form (what launch_gemm8 takes for at most half a round of 256 x 256 tiles): a stage
+        // lengthens as more than half the CUs draw on L2 at once (fp8, K = 4096: 24.7 us on 128 workgroups, 26.9 on
+        // 192, 31.3 on 256; int8 28.8 / 30.8 / 35.2)
+        const int64_t wgs = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
+        const double crowd = wgs > 128 ? (double)(wgs - 128) / 128.0 : 0.0;
+        return i8 ? 7.0 + steps * (0.68 + 0.2 * crowd) : 6.5 + steps * (0.58 + 0.21 * crowd);
+    }
     return (double)((tiles + 255) / 256) * (i8 ? 9.5 + 1.03 * steps : 10.0 + 1.1 * steps);
 }
 
@@ -294,8 +302,7 @@ bool gemm8s_applicable(const ForwardArgs& a) {
     if (!gemm8_applicable(a)) return false;
     const nq_layer* L = a.L;
     const bool i8 = a.x_dtype == NQ_DT_I8;
-    // (a tenth in hand for the large tile: where the two estimates meet it measured the faster)
-    return gemm8_estimate_us(a.M, L->out, L->in, i8, true) < 0.9 * gemm8_estimate_us(a.M, L->out, L->in, i8, false);
+    return gemm8_estimate_us(a.M, L->out, L->in, i8, true) < gemm8_estimate_us(a.M, L->out, L->in, i8, false);
 }
 
 int32_t launch_gemm8s(const ForwardArgs& a) {

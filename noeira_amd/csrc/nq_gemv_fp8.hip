@@ -526,8 +526,7 @@ static bool row_kernel_fits(const ForwardArgs& a) {
 }
 
 // The tile kernel against the 256 x 256-tile GEMM (nq_gemm8.hip), both measured over K = 512 .. 8192,
-// N = 1024 .. 11008, M = 64 .. 2048.  A round of GEMM tiles (up to 256) takes about 14 us + 1.25 us per 128 k
-// (fp8: 10 + 1.1).
+// N = 1024 .. 11008, M = 64 .. 2048.  What the GEMM takes on either of its tile sizes: gemm8_estimate_us.
 // The tile kernel with 2 or 4 weight tiles per workgroup takes, per round of 256 workgroups, a fixed 5.5 us
 // (3.75 with four wavefronts) + 0.25 / 0.31 us per 128 k, half as much again when 64 rows at a time stream a
 // weight larger than the caches hold; with one weight tile (small launches, short K) about 4 us + 5.6 us per

@@ -431,7 +431,7 @@ def test_mlp3_other_shapes_and_errors():
 # ── the two tile sizes of the 8-bit GEMM ────────────────────────────────────────────────────────────────────────
 def _gemm8(lin, tile, x, x_dt, x_scale, M, out_dtype, bias=None, epilogue="none"):
     """The 8-bit GEMM on the 128 x 128 (`tile` = 128) or the 256 x 256 tile kernel (256; 2564 / 2568: on four / eight
-    wavefronts), whatever nq_forward would choose."""
+    wavefronts; 1282: its 128 x 256 tile form), whatever nq_forward would choose."""
     import ctypes as C
     from noeira_amd import _lib as L
     out = torch.full((M, lin.OUT), 7, dtype=out_dtype, device="cuda")
@@ -440,6 +440,36 @@ def _gemm8(lin, tile, x, x_dt, x_scale, M, out_dtype, bias=None, epilogue="none"
                                           C.c_void_p(out.data_ptr()), y_dt, M, C.c_void_p(bias.data_ptr()) if bias is not None else None,
                                           L.DT_F32, L.EPI_RELU if epilogue == "relu" else L.EPI_NONE, tile, None))
     return out
+
+
+@pytest.mark.parametrize("M,K,N", [(2048, 128, 8704), (2304, 256, 15360), (2240, 128, 15300), (2100, 128, 8500), (8192, 128, 11008)])
+def test_gemm_leftover_tiles_on_the_half_tile_kernel(M, K, N):
+    """More than a round of 256 x 256 tiles with at most half a round left over: nq_forward gives the full rounds to
+    the 256 x 256 kernel and the leftover - whole columns of the last band of row tiles - to the 128 x 256 form in a
+    second launch ((2048, 8704): 16 tiles = 2 columns of 8; (2304, 15360): the last band is one row of tiles, 28
+    columns of it; (2240, 15300): the same with ragged edges in both directions; (2100, 8500): 50 leftover tiles that
+    are no rectangle of the one-row last band's 34, so one launch; (8192, 11008): the config-5 shape, 96 = 12 columns
+    of 8).  int32 accumulators equal the oracle's bit for bit and every element is written once (a sentinel
+    survives nowhere); fp8 returns the bits of the single-kernel form."""
+    from noeira_amd import _lib as L
+    rng = np.random.default_rng(M + K + N)
+    lin, w, s = w8_layer(rng, K, N)
+    xq_h = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    sx_h = rng.uniform(1e-3, 1e-1, M).astype(np.float32)
+    xq, sx = torch.from_numpy(xq_h).cuda(), torch.from_numpy(sx_h).cuda()
+    out = torch.full((M, N), -2 ** 31, dtype=torch.int32, device="cuda")
+    lin.forward_a8(xq, sx, out=out, out_dtype=torch.int32)
+    assert np.array_equal(out.cpu().numpy(), O.w8a8_acc_i32(xq_h, w))
+    bias = torch.from_numpy((rng.standard_normal(N) * 0.02).astype(np.float32)).cuda()
+    assert torch.equal(lin.forward_a8(xq, sx, bias=bias, epilogue="relu", out_dtype=torch.bfloat16),
+                       _gemm8(lin, 2564, xq, L.DT_I8, sx, M, torch.bfloat16, bias, "relu"))
+    a, b = fp8_operands(rng, M, N, K)
+    f8 = FP8Linear(K, N)
+    f8.set_weight(b, 0.25)
+    xs = torch.tensor([0.5], dtype=torch.float32, device="cuda")
+    ad = torch.from_numpy(a).cuda()
+    for dt in (torch.float32, torch.bfloat16):
+        assert torch.equal(f8.forward(ad, xs, out_dtype=dt), _gemm8(f8, 2564, ad, L.DT_FP8_E4M3, xs, M, dt)), dt
 
 
 @pytest.mark.parametrize("M,K,N", [(520, 1024, 2296), (1000, 512, 520), (2100, 512, 2300), (300, 4096, 1024), (64, 128, 8)])
@@ -457,11 +487,11 @@ def test_gemm_tile_sizes_against_the_oracle_and_each_other(M, K, N):
     xq, sx, bias = torch.from_numpy(xq_h).cuda(), torch.from_numpy(sx_h).cuda(), torch.from_numpy(bias_h).cuda()
     acc_o = O.w8a8_acc_i32(xq_h, w)
     want = O.w8a8_epilogue(acc_o, sx_h, s, bias_h, relu=True)
-    for tile in (128, 2564, 2568):  # (256: whichever of the last two nq_forward takes)
+    for tile in (128, 2564, 2568, 1282):  # (256: whichever of the last three nq_forward takes)
         assert np.array_equal(_gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.int32).cpu().numpy(), acc_o), tile
         assert rel_rms(_gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.float32, bias, "relu").cpu().numpy(), want) < 1e-5, tile
     for dt in (torch.float32, torch.bfloat16):
-        for tile in (2564, 2568):
+        for tile in (2564, 2568, 1282):
             assert torch.equal(_gemm8(lin, 128, xq, L.DT_I8, sx, M, dt, bias, "relu"), _gemm8(lin, tile, xq, L.DT_I8, sx, M, dt, bias, "relu")), (dt, tile)
     a, b = fp8_operands(rng, M, N, K)
     f8 = FP8Linear(K, N)
@@ -470,11 +500,11 @@ def test_gemm_tile_sizes_against_the_oracle_and_each_other(M, K, N):
     ad = torch.from_numpy(a).cuda()
     y64, _ = O.fp8_forward_f64(a, b, np.float32(0.5), np.float32(0.25), want_bf16=False)
     ref = y64 + bias_h.astype(np.float64)
-    for tile in (128, 2564, 2568):
+    for tile in (128, 2564, 2568, 1282):
         got = _gemm8(f8, tile, ad, L.DT_FP8_E4M3, xs, M, torch.float32, bias).cpu().numpy()
         assert np.abs(got - ref).max() <= 3e-4 * np.sqrt((ref ** 2).mean()), tile
     for dt in (torch.float32, torch.bfloat16):
-        for tile in (2564, 2568):
+        for tile in (2564, 2568, 1282):
             assert torch.equal(_gemm8(f8, 128, ad, L.DT_FP8_E4M3, xs, M, dt, bias), _gemm8(f8, tile, ad, L.DT_FP8_E4M3, xs, M, dt, bias)), (dt, tile)
     # what nq_forward itself returns for the call (whichever kernel it takes): the oracle's accumulators
     assert np.array_equal(lin.forward_a8(xq, sx, out_dtype=torch.int32).cpu().numpy(), acc_o)
