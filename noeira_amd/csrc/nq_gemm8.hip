@@ -60,8 +60,9 @@
 // In cycles.  The K loop's own reading of the shader clock beside the constant one (fp8, 8192 x 4096 x 4096, all 256
 // CUs busy): 2283 cycles per stage at 1.86 - 1.88 GHz, against the 2048 cycles the stage's MFMAs occupy the pipe and
 // against 2.18 GHz under the same MFMAs with operands in registers; with half the CUs busy (M = 2048) 2320 cycles at
-// 2.19 - 2.24 GHz.  So nine tenths of the loop's cycles are MFMA cycles wherever it runs, and what a full chip loses
-// beyond that is clock: the transfers and fragment reads are paid in power, not in stalls.
+// 2.19 - 2.24 GHz; int8 on eight wavefronts 2317 cycles at 1.72 - 1.76 GHz (2.05 GHz under its MFMAs alone).  So nine
+// tenths of the loop's cycles are MFMA cycles wherever it runs, and what a full chip loses beyond that is clock: the
+// transfers and fragment reads are paid in power, not in stalls.
 //
 // Half tiles.  A launch that fills at most half a round of workgroups (128 tiles of 256 x 256) leaves CUs idle for the
 // whole call, and so do the tiles left over after the last full round.  Both go on a 128 x 256 tile instead (4
