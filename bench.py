@@ -586,11 +586,12 @@ def mfma_only(iters=4096, reps=5):
     return out
 
 
-def gemm_timeline(N=4096, K=4096, M=8192):
+def gemm_timeline(N=4096, K=4096, M=8192, i8=False):
     """Where a config-5 GEMM call's time goes: every workgroup of the 256 x 256 tile kernel stamps the GPU's
     constant 100 MHz clock at entry, when its first K stage has landed, after its K loop and after its stores
-    are acknowledged (nq_diag_gemm8_timeline).  Reported per round of workgroups (the hardware hands out the
-    next tile as a CU frees up): medians in microseconds."""
+    are acknowledged, and the shader clock's cycle counter at the second and third of them
+    (nq_diag_gemm8_timeline).  Reported per round of workgroups (the hardware hands out the next tile as a CU
+    frees up): medians in microseconds; the K loop also in cycles per stage with the clock that follows."""
     import ctypes as C
 
     import numpy as np
@@ -598,13 +599,18 @@ def gemm_timeline(N=4096, K=4096, M=8192):
 
     from noeira_amd import _lib as L
 
-    wl = make_fp8(M, N, K=K)
-    layers, a, sa, y = wl["keep"]
+    if i8:
+        wl = make_w8a8_gemm(M, N, K=K)
+        lin, a, sa, _, y = wl["keep"]
+        layers = [lin]
+    else:
+        wl = make_fp8(M, N, K=K)
+        layers, a, sa, y = wl["keep"]
     for i in range(5):
         wl["step"](i)
     torch.cuda.synchronize()
     tiles = (M // 256) * ((N + 255) // 256)
-    buf = torch.zeros((tiles, 4), dtype=torch.int64, device="cuda")
+    buf = torch.zeros((tiles, 6), dtype=torch.int64, device="cuda")
     null = C.c_void_p(0)
     t = None
     for _ in range(7):  # single launches differ by a few percent with the clock the chip happens to be at: the fastest
@@ -615,13 +621,14 @@ def gemm_timeline(N=4096, K=4096, M=8192):
             torch.cuda.synchronize()
         for i in range(20):
             wl["step"](i)
-        L.check(L.lib().nq_diag_gemm8_timeline(layers[0]._h, C.c_void_p(a.data_ptr()), L.DT_FP8_E4M3,
+        L.check(L.lib().nq_diag_gemm8_timeline(layers[0]._h, C.c_void_p(a.data_ptr()), L.DT_I8 if i8 else L.DT_FP8_E4M3,
                                                 C.c_void_p(sa.data_ptr()), C.c_void_p(y.data_ptr()), L.DT_BF16, M,
                                                 C.c_void_p(buf.data_ptr()), tiles, null))
-        ti = buf.cpu().numpy().astype(np.float64) * 0.01  # ticks of 10 ns -> us
+        raw = buf.cpu().numpy().astype(np.float64)
+        ti = raw[:, :4] * 0.01  # ticks of 10 ns -> us
         ti -= ti[:, 0].min()
         if t is None or ti[:, 3].max() < t[:, 3].max():
-            t = ti
+            t, cyc = ti, raw[:, 5] - raw[:, 4]
     order = np.argsort(t[:, 0])
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     rounds = []
@@ -634,8 +641,11 @@ def gemm_timeline(N=4096, K=4096, M=8192):
                        "epilogue_us": round(float(np.median(t[idx, 3] - t[idx, 2])), 2),
                        "end_us": [round(float(t[idx, 3].min()), 2), round(float(t[idx, 3].max()), 2)]})
     stages = K // 128
-    return {"workload": f"fp8 GEMM M={M} K={K} N={N}, bf16 out", "tiles": tiles, "kernel_us": round(float(t[:, 3].max()), 2),
+    ghz = cyc / np.maximum(t[:, 2] - t[:, 1], 1e-3) / 1e3
+    return {"workload": f"{'int8' if i8 else 'fp8'} GEMM M={M} K={K} N={N}, bf16 out", "tiles": tiles, "kernel_us": round(float(t[:, 3].max()), 2),
             "stage_us": round(float(np.median(t[:, 2] - t[:, 1])) / stages, 4), "stages_per_tile": stages,
+            "stage_cycles": round(float(np.median(cyc)) / stages, 1), "mfma_cycles_per_stage": 2048,
+            "shader_clock_GHz": [round(float(np.median(ghz)), 3), round(float(ghz.min()), 3), round(float(ghz.max()), 3)],
             "epilogue_bytes_per_round": min(tiles, cus) * 256 * 256 * 2, "rounds": rounds}
 
 
@@ -921,7 +931,8 @@ def only_loop(which, steps, warmup):
         wl = make_decoder_layer(135, "fused")
         name = "the reference text layer's seven Q4_0 projections at T = 135 with rank-16 adapters, fused calls"
     elif which == "gemm_timeline":
-        return {"only": which, "timelines": [gemm_timeline(4096, 4096), gemm_timeline(4096, 8192), gemm_timeline(11008, 4096)]}
+        return {"only": which, "timelines": [gemm_timeline(4096, 4096), gemm_timeline(4096, 8192), gemm_timeline(11008, 4096),
+                                            gemm_timeline(4096, 4096, 2048), gemm_timeline(4096, 4096, i8=True)]}
     elif which == "mfma_peak":
         return {"only": which, "mfma_only": mfma_only()}
     elif which == "vendor_gemm":

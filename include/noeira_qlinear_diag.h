@@ -34,8 +34,10 @@ int32_t nq_diag_stream_read(const void* src, int64_t nbytes, void* stream);
 /* Where the time of a large-tile 8-bit GEMM goes (no counterpart in the reference): the launch nq_forward makes
  * for 8-bit activations and M >= 64 rows over a layer whose IN is a multiple of 128 (NQ_ERR_UNSUPPORTED otherwise),
  * with every workgroup of the 256 x 256 tile kernel reporting four readings of the GPU's constant 100 MHz clock -
- * entry, first K stage landed, K loop done, stores acknowledged - into stamps (device uint64 [tiles][4], tiles =
- * ceil(M / 256) * ceil(OUT / 256) <= max_tiles, else NQ_ERR_INVALID).  The arguments are nq_forward's for that case
+ * entry, first K stage landed, K loop done, stores acknowledged - and the shader clock's cycle counter at the second
+ * and third of them (so that the K loop can be read in cycles and the clock it ran at follows) into stamps (device
+ * uint64 [tiles][6], tiles = ceil(M / 256) * ceil(OUT / 256) <= max_tiles, else NQ_ERR_INVALID).  The kernel is the
+ * form nq_forward takes for the operand type (fp8: four wavefronts, int8: eight), on 256 x 256 tiles throughout.  The arguments are nq_forward's for that case
  * (x: int8 with per-row x_scale, or e4m3 codes with one scale; y fp32 or bf16, for int8 also the raw int32
  * accumulators; no bias).  The stamp buffer is an argument of this
  * one launch: no other call, on this or another thread, writes stamps.  Synchronises the stream before it returns. */

@@ -135,7 +135,7 @@ struct Gemm8Params {
     int32_t grid;            // workgroups to launch: the first `grid` tiles of the order (0: all tiles_m x tiles_n)
     int32_t m_base, n_base;  // the first row and channel of the part of y this launch covers (its tiles count from there)
     int32_t y_dtype, bias_dtype, epilogue;
-    unsigned long long* stamps;  // a diagnostic: per workgroup, four readings of the constant 100 MHz clock, or null
+    unsigned long long* stamps;  // a diagnostic: per workgroup, four readings of the constant 100 MHz clock and two of the shader clock, or null
     int32_t chan_vec;  // N % 4 == 0 and col_scale / bias aligned for one 16-byte (bf16 bias: 8-byte) load per 4 channels
 };
 
@@ -581,6 +581,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
 #undef NQ_DMA_ALL
     }
     const unsigned long long t_first = wall_clock64();  // stage 0 has landed
+    const unsigned long long c_first = p.stamps ? clock64() : 0;  // (the shader clock's own count, for the loop in cycles)
     // what a phase before the first would have requested: all fragments of (buffer 0, phase 0)
     static_for<TI>([&](auto ic) { read_x(ic, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
     static_for<TJ>([&](auto jc) { read_w(integral_constant<int, 0>{}, jc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
@@ -606,6 +607,7 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     NQ_LDS_WAIT(0);  // requests past the last stage still target registers: let them land
     __syncthreads();  // every wavefront is done with the stage buffers: the epilogue stages through them
     const unsigned long long t_loop = wall_clock64();
+    const unsigned long long c_loop = p.stamps ? clock64() : 0;
 #undef NQ_DMA
 #undef NQ_LDS_READ
 #undef NQ_LDS_WAIT
@@ -772,11 +774,12 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
         else if (p.bias_dtype == NQ_DT_F32) emit(kind_t{}, std::integral_constant<int, 2>{});
         else emit(kind_t{}, std::integral_constant<int, 3>{});
     }
-    if (p.stamps) {  // (uniform) entry, first stage landed, loop done, stores acknowledged
+    if (p.stamps) {  // (uniform) entry, first stage landed, loop done, stores acknowledged; the shader clock at the middle two
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (tid == 0) {
-            unsigned long long* o = p.stamps + 4 * (size_t)blockIdx.x;
+            unsigned long long* o = p.stamps + 6 * (size_t)blockIdx.x;
             o[0] = t_entry, o[1] = t_first, o[2] = t_loop, o[3] = wall_clock64();
+            o[4] = c_first, o[5] = c_loop;
         }
     }
 }

@@ -363,7 +363,8 @@ def test_fp8_weights_under_16bit_activations(M, K, N, xdt):
 
 def test_gemm8_timeline_diagnostic_reports_ordered_stamps_and_the_same_output():
     """nq_diag_gemm8_timeline: the call nq_forward would make, with every workgroup of the large-tile kernel
-    reporting its four clock readings: ordered, all written, and y as without them."""
+    reporting its four readings of the constant clock and two of the shader clock: ordered, all written, a
+    plausible clock between them, and y as without them."""
     import ctypes as C
 
     from noeira_amd import _lib as L
@@ -378,15 +379,17 @@ def test_gemm8_timeline_diagnostic_reports_ordered_stamps_and_the_same_output():
     want = lin.forward(xc, sa)
     y = torch.zeros_like(want)
     tiles = 8 * 9
-    stamps = torch.zeros((tiles, 4), dtype=torch.int64, device="cuda")
+    stamps = torch.zeros((tiles, 6), dtype=torch.int64, device="cuda")
     args = (lin._h, C.c_void_p(xc.data_ptr()), L.DT_FP8_E4M3, C.c_void_p(sa.data_ptr()), C.c_void_p(y.data_ptr()),
             L.DT_BF16, M, C.c_void_p(stamps.data_ptr()))
     assert L.lib().nq_diag_gemm8_timeline(*args, tiles - 1, C.c_void_p(0)) == L.NQ_ERR_INVALID
     L.check(L.lib().nq_diag_gemm8_timeline(*args, tiles, C.c_void_p(0)))
     assert torch.equal(y, want)
     t = stamps.cpu().numpy()
-    assert (t > 0).all() and (np.diff(t, axis=1) >= 0).all()
+    assert (t > 0).all() and (np.diff(t[:, :4], axis=1) >= 0).all()
     assert (t[:, 3] - t[:, 0]).max() < 100000   # under a millisecond of 10 ns ticks
+    ghz = (t[:, 5] - t[:, 4]) / np.maximum(t[:, 2] - t[:, 1], 1) / 10.0   # cycles per 10 ns tick -> GHz
+    assert 0.3 < np.median(ghz) < 3.0
     # and the next ordinary call writes no stamps
     stamps.zero_()
     lin.forward(xc, sa)
