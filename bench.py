@@ -927,6 +927,21 @@ def only_loop(which, steps, warmup):
 
         wl = dict(step=step_gm, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
         name = "fp8 x fp8 and W8A8 at 4096 x 4096, M = 512 and 1024 (the 128 x 128 tile GEMM), one call each per step"
+    elif which == "i8gemm":
+        wl = make_w8a8_gemm(8192, 4096)
+        name = "W8A8 int8 GEMM M=8192 K=4096 N=4096, scales + bias, bf16 out (the 256 x 256 tile on eight wavefronts)"
+    elif which == "fp8gemm_n11008":
+        wl = make_fp8(8192, 11008)
+        name = "cfg5 fp8 GEMM M=8192 K=4096 N=11008 (five rounds of 256 x 256 tiles, then the 96 left over as 192 tiles of 128 x 256)"
+    elif which == "gemm_half":
+        wls = [make_fp8(2048, 4096), make_w8a8_gemm(2048, 4096)]
+
+        def step_gh(i):
+            for w in wls:
+                w["step"](i)
+
+        wl = dict(step=step_gh, bytes=sum(w["bytes"] for w in wls), ops=sum(w["ops"] for w in wls), keep=wls)
+        name = "fp8 x fp8 and W8A8 at M=2048 over 4096 x 4096 (128 x 256 tiles), one call each per step"
     elif which == "adapters":
         wl = make_decoder_layer(135, "fused")
         name = "the reference text layer's seven Q4_0 projections at T = 135 with rank-16 adapters, fused calls"
@@ -1137,7 +1152,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", choices=["", "headline", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "gemm_mid", "adapters", "manyrows", "hugegemv", "mfma_peak", "vendor_gemm", "gemm_timeline", "a16_shapes", "mid_dispatch"],
+    ap.add_argument("--only", default="", choices=["", "headline", "act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "gemm_mid", "i8gemm", "fp8gemm_n11008", "gemm_half", "adapters", "manyrows", "hugegemv", "mfma_peak", "vendor_gemm", "gemm_timeline", "a16_shapes", "mid_dispatch"],
                     help="run one loop only and print a short JSON line (for rocprofv3 runs): headline = the "
                          "headline line alone (graph replays), act = config 2's pair of linears at M=1, fp8gemv / fp8gemm = "
                          "config 5 at N=11008 (the headline's kernel, launched call by call) / N=4096, mid = the M=100..256 "
@@ -1146,7 +1161,8 @@ def main():
                          "three 4096->11008 layers with 16-bit or fp32 activations at M=1 / M=16, hugegemv = the two 4-bit layers at 8192->28672, M=1, tile8 = int8 and fp8 "
                          "activations at M = 16 .. 512 over 4096 x 4096, manyrows = bf16 / fp32 activations at M = 1120 "
                          "and 4096, mfma_peak = the matrix cores alone (nq_diag_mfma_rate) on constant and random operands, gemm_timeline = the "
-                         "config-5 GEMM's workgroups stamping entry / first stage / K loop / stores (nq_diag_gemm8_timeline)")
+                         "config-5 GEMM's workgroups stamping entry / first stage / K loop / stores (nq_diag_gemm8_timeline), i8gemm / fp8gemm_n11008 / "
+                         "gemm_half = the int8 GEMM 8192 x 4096 x 4096, config 5's GEMM at N = 11008, the two at M = 2048 over 4096 x 4096")
     ap.add_argument("--eager", action="store_true", help="with --only: launch call by call, no HIP graph")
     ap.add_argument("--rows-layout", action="store_true",
                     help="large layers keep only their row-ordered codes (NQ_FLAG_NO_TILE_COPY): the single-row kernels "
@@ -1176,7 +1192,7 @@ def main():
             sys.exit("bench.py: --only mid_dispatch is about the 4-bit formats (--a16-class q4, q4f, w4g or w4gf)")
         print(json.dumps(mid_dispatch(a.a16_class)))
         return
-    if a.only in ("act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "gemm_mid", "adapters", "manyrows", "hugegemv", "mfma_peak", "vendor_gemm", "gemm_timeline"):
+    if a.only in ("act", "fp8gemv", "fp8gemm", "mid", "actor", "copy", "biggemv", "smallm", "tile8", "gemm_mid", "i8gemm", "fp8gemm_n11008", "gemm_half", "adapters", "manyrows", "hugegemv", "mfma_peak", "vendor_gemm", "gemm_timeline"):
         print(json.dumps(only_loop(a.only, a.steps, a.warmup)))
         return
 
