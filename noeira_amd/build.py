@@ -24,7 +24,7 @@ OBJ = os.path.join(HERE, "csrc", "_obj")
 LIB = os.path.join(HERE, "libnoeira_qlinear.so")
 ROOT = os.path.dirname(HERE)
 
-SOURCES = ["nq_api.hip", "nq_q4_0.hip", "nq_gemv.hip", "nq_quant.hip", "nq_gemm8.hip", "nq_gemm8s.hip", "nq_gemm_a16.hip", "nq_mlp.hip", "nq_gemv_m1.hip", "nq_gemv_fp8.hip", "nq_gptq.hip", "nq_lora.hip", "nq_gemv_row4.hip", "nq_gemv_row8.hip", "nq_gemv_split.hip", "nq_gemv_tile.hip", "nq_diag.hip"]
+SOURCES = ["nq_api.hip", "nq_q4_0.hip", "nq_gemv.hip", "nq_quant.hip", "nq_gemm8.hip", "nq_gemm_a16.hip", "nq_mlp.hip", "nq_gemv_m1.hip", "nq_gemv_fp8.hip", "nq_gptq.hip", "nq_lora.hip", "nq_gemv_row4.hip", "nq_gemv_row8.hip", "nq_gemv_split.hip", "nq_gemv_tile.hip", "nq_diag.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -440,12 +440,10 @@ int32_t dispatch(const ForwardArgs& a) {
     }
     if (a.x_dtype == NQ_DT_I8) {
         if (tile8_i8_applicable(a)) return launch_tile8_i8(a);
-        if (gemm8s_applicable(a)) return launch_gemm8s(a);
         if (gemm8_applicable(a)) return launch_gemm8(a);
         return launch_gemv_i8(a);
     }
     if (gemv_fp8_applicable(a)) return launch_gemv_fp8(a);
-    if (gemm8s_applicable(a)) return launch_gemm8s(a);
     if (gemm8_applicable(a)) return launch_gemm8(a);
     if (gemv_tile_rows_applicable(a)) return launch_gemv_tile_rows(a);
     if (gemv_tile8_rows_applicable(a)) return launch_gemv_tile8_rows(a);
@@ -1103,7 +1101,8 @@ int32_t nq_diag_forward_gemm8(nq_handle h, const void* x, int32_t x_dtype, const
     if (h->glu || !h->seg_end.empty() || !gemm8_applicable(a))
         return fail(NQ_ERR_UNSUPPORTED, "nq_diag_forward_gemm8: the 8-bit GEMM does not take this call (format, M >= 64, IN % 128)");
     if (tile > 256) a.diag_gemm8_waves = tile == 1282 ? 12 : tile % 10;
-    return tile == 128 ? launch_gemm8s(a) : launch_gemm8(a);
+    if (tile == 128) a.diag_gemm8_waves = 16;
+    return launch_gemm8(a);
 }
 
 int32_t nq_diag_forward_a16(nq_handle h, const void* x, int32_t x_dtype, void* y, int32_t y_dtype, int32_t M,

@@ -203,9 +203,7 @@ bool tile8_i8_applicable(const ForwardArgs& a);
 int32_t launch_tile8_i8(const ForwardArgs& a);
 
 // nq_gemm8.hip: LDS-tiled fp8 / int8 MFMA GEMM for large M
-bool gemm8s_applicable(const ForwardArgs& a);
-double gemm8_estimate_us(int M, int N, int K, bool i8, bool small_tile);
-int32_t launch_gemm8s(const ForwardArgs& a);
+double gemm8_estimate_us(int M, int N, int K, bool i8);  // what launch_gemm8 is expected to take, on the tile form it picks
 bool gemm8_applicable(const ForwardArgs& a);
 int32_t launch_gemm8(const ForwardArgs& a);
 

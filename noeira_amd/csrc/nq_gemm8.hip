@@ -74,6 +74,13 @@
 // us with 128 workgroups, 26.9 with 192, 31.3 with 256 - against 41 - 43 us for the same calls on 64 .. 128 tiles of
 // 256 x 256).  Same sums in the same order: same bits.
 //
+// Quarter tiles.  Calls whose 128 x 128 tiles fit about a round of workgroups (M = 512 .. 1152 over 4096 x 4096) run the
+// body on that tile: 4 wavefronts of 64 x 64, a phase of 16 MFMAs (ev16_slot), four stage buffers of 32 KiB.  fp8 /
+// int8 over 4096 x 4096: M = 512 15.8 / 18.0 us, M = 1024 18.1 - 20.2 / 20.2 - 22.3 (a plainer kernel on the same tile, with a
+// stage's fragment reads at the head of the stage: 19.5 / 23.4 and 21.3 / 24.5; 256 x 256 tiles: 39 - 48).  Twice the
+// bytes from L2 per operation: with all CUs on such tiles a stage is 0.39 - 0.45 us for 0.22 - 0.25 of MFMA, 18 - 21 TB/s
+// into LDS over the chip.  launch_gemm8 takes the form of lowest estimated time (estimate_form).
+//
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= ((row >> 1) + 6) & 7.  A 128-bit read is served in passes of
 // sixteen lanes that are not consecutive lanes (per half of the wavefront the quads of lanes
@@ -275,6 +282,52 @@ __host__ __device__ constexpr int dma8_at(int m, int n) {
     return -1;
 }
 
+// ---- and for a 128 x 128 tile on four wavefronts (2 x 2, each 64 x 64: 4 token and 4 channel fragments, 16 MFMAs per
+// phase), again one register set per fragment.  Order: m -> token fragment i = (m % 8) / 2, channel fragment
+// j = 2 (m / 8) + m % 2: channel fragments 0, 1 are done with after MFMAs 6, 7, token fragment i after 9 + 2 i, channel
+// fragments 2, 3 after 14, 15.  Each is requested again one MFMA after its last reader; x3 and w3 fall into the phase
+// that uses them (slots 0, 1).
+//   event e:   0     1     2    3    4    5    6    7
+//   brings:    x3'   w3'   w0   w1   x0   x1   x2   w2     (': this phase's own)
+__host__ __device__ constexpr int ev16_slot(int e) {
+    constexpr int s[8] = {0, 1, 7, 8, 10, 12, 14, 15};
+    return s[e];
+}
+__host__ __device__ constexpr int ev16_at(int m) {
+    for (int e = 0; e < 8; e++)
+        if (ev16_slot(e) == m) return e;
+    return -1;
+}
+__host__ __device__ constexpr int lds_wait16(int m_want, int reads_per_fragment, int barrier_at) {
+    int landed = 0;
+    for (int m = 0; m < 16; m++) {
+        const int i = (m % 8) / 2, j = 2 * (m / 8) + m % 2;
+        int issued = 8;
+        for (int e = 0; e < 8; e++)
+            if (ev16_slot(e) < m) issued++;
+        const int nx = i < 3 ? 4 + i : 8 + 0;
+        const int nw = j < 2 ? 2 + j : (j == 2 ? 7 : 8 + 1);
+        const int need = nx > nw ? nx : nw;
+        int w = -1;
+        if (m == barrier_at) {
+            landed = issued;
+        } else if (need >= landed) {
+            int a = issued - 1 - need;
+            const int cap = 15 / reads_per_fragment;
+            if (a > cap) a = cap;
+            w = a * reads_per_fragment;
+            landed = issued - a;
+        }
+        if (m == m_want) return w;
+    }
+    return -1;
+}
+constexpr int BARRIER16_AT = 4;
+// eight transfers per wavefront and stage behind the barrier: two each after MFMAs 4 and 5, then one per slot that holds
+// no request (barrier in front of MFMA 2 or 6, or all eight transfers right behind it: the same time or slower)
+__host__ __device__ constexpr int dma16_first(int m) { return m == 4 ? 0 : m == 5 ? 2 : m == 6 ? 4 : m == 9 ? 5 : m == 11 ? 6 : m == 13 ? 7 : -1; }
+__host__ __device__ constexpr int dma16_count(int m) { return (m == 4 || m == 5) ? 2 : (m == 6 || m == 9 || m == 11 || m == 13) ? 1 : 0; }
+
 // BN and BK are parameters of the body for the arithmetic's sake; the tile built is 256 x 256 with BK = 128.
 // KIND: the output type the epilogue is built for (0 fp32, 1 bf16, 2 raw int32 accumulators); one
 // kernel per kind, because with all three in one function the register allocator spills.
@@ -284,7 +337,8 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     constexpr int SLOTS = BK / 16;     // 16-byte slots per LDS row
     constexpr int WN = BN / 2;         // channels per wavefront
     constexpr int TI = BM / (8 * WAVES), TJ = WN / 16;  // fragments of 16 rows: token rows i, channel columns j
-    static_assert(BN == 256 && BK == 128 && TJ == 8 && ((BM == 256 && (WAVES == 4 || WAVES == 8)) || (BM == 128 && WAVES == 4)),
+    static_assert(BK == 128 && ((BN == 256 && TJ == 8 && ((BM == 256 && (WAVES == 4 || WAVES == 8)) || (BM == 128 && WAVES == 4))) ||
+                                (BN == 128 && BM == 128 && WAVES == 4 && TI == 4 && TJ == 4)),
                   "the phase models are written for these tiles");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const unsigned long long t_entry = wall_clock64();
@@ -342,9 +396,10 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     // offset.  Three instructions per transfer.  (M0 is a reserved register the compiler sets itself
     // right before each of its own uses, so writing it here needs no clobber; SCC does.)
     const uint32_t lds_addr0 = (uint32_t)(uintptr_t)(lptr_t*)lds;
-    // stage buffers: two of 64 KiB; the 128-row tile has three of 48 KiB, so that a stage's transfers have two stages
-    // of MFMAs to land in (one stage of its 32 MFMAs per wavefront is shorter than their way from L2)
-    constexpr int NB = BM == 128 ? 3 : 2;
+    // stage buffers: two of 64 KiB; the 128-row tiles have three of 48 KiB (128 x 256) or four of 32 KiB (128 x 128), so
+    // that a stage's transfers have two or three stages of MFMAs to land in (one stage of 32 or 16 MFMAs per wavefront
+    // is shorter than their way from L2)
+    constexpr int NB = BM == 128 ? (BN == 128 ? 4 : 3) : 2;
     uint32_t dbase[NB][2];  // [buffer][x tile, w tile]: this wavefront's first destination
 #pragma unroll
     for (int buf = 0; buf < NB; buf++) {
@@ -478,20 +533,26 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_sched_barrier(0);
         });
     };
+    // A stage's barrier with more than two buffers: the transfers of the `keep` stages after the next one may stay in
+    // flight across it (loads return in the order of issue)
+    auto barrier_keep = [&](int keep) {
+        if (keep >= 2)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * (DA + DB)) : "memory");
+        else if (keep == 1)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(DA + DB) : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+    };
     // The same for eight wavefronts: 32 MFMAs, one set of registers per fragment (see ev8_slot).
-    // keep1 (three buffers): the stage before issued transfers too, and those may stay in flight across the barrier
-    auto phase8 = [&](auto bufc, auto phc, auto zeroc, bool have2, bool keep1, const uint8_t* srca, const uint8_t* srcb) {
+    auto phase8 = [&](auto bufc, auto phc, auto zeroc, bool have2, int keep, const uint8_t* srca, const uint8_t* srcb) {
         constexpr int BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
         constexpr bool LAST = PHI == PH - 1;
         constexpr int NBUF = LAST ? (BUF + 1) % NB : BUF, NPH = LAST ? 0 : PHI + 1;
         static_for<32>([&](auto mc) {
             constexpr int m = decltype(mc)::value, i = (m % 16) / 4, j = 4 * (m / 16) + m % 4;
             if constexpr (LAST && m == BARRIER8_AT) {
-                if (keep1)
-                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(DA + DB) : "memory");
-                else
-                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                __builtin_amdgcn_s_barrier();
+                barrier_keep(keep);
             } else {
                 constexpr int al = lds_wait8(m, R, LAST ? BARRIER8_AT : -1);
                 if constexpr (al >= 0) NQ_LDS_WAIT(al);
@@ -521,15 +582,59 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             __builtin_amdgcn_sched_barrier(0);
         });
     };
+    // And for the 128 x 128 tile: 16 MFMAs (see ev16_slot).
+    auto phase16 = [&](auto bufc, auto phc, auto zeroc, bool have2, int keep, const uint8_t* srca, const uint8_t* srcb) {
+        constexpr int BUF = decltype(bufc)::value, PHI = decltype(phc)::value;
+        constexpr bool LAST = PHI == PH - 1;
+        constexpr int NBUF = LAST ? (BUF + 1) % NB : BUF, NPH = LAST ? 0 : PHI + 1;
+        static_for<16>([&](auto mc) {
+            constexpr int m = decltype(mc)::value, i = (m % 8) / 2, j = 2 * (m / 8) + m % 2;
+            if constexpr (LAST && m == BARRIER16_AT) {
+                barrier_keep(keep);
+            } else {
+                constexpr int al = lds_wait16(m, R, LAST ? BARRIER16_AT : -1);
+                if constexpr (al >= 0) NQ_LDS_WAIT(al);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mma(zeroc, i, j, xf[i], wf[0][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            constexpr int e = ev16_at(m);
+            using z0 = integral_constant<int, 0>;
+            using nb = integral_constant<int, NBUF>;
+            using np = integral_constant<int, NPH>;
+            if constexpr (e == 0) {
+                read_x(integral_constant<int, 3>{}, bufc, phc);
+            } else if constexpr (e == 1) {
+                read_w(z0{}, integral_constant<int, 3>{}, bufc, phc);
+            } else if constexpr (e == 2 || e == 3) {
+                read_w(z0{}, integral_constant<int, e - 2>{}, nb{}, np{});
+            } else if constexpr (e >= 4 && e <= 6) {
+                read_x(integral_constant<int, e - 4>{}, nb{}, np{});
+            } else if constexpr (e == 7) {
+                read_w(z0{}, integral_constant<int, 2>{}, nb{}, np{});
+            }
+            if constexpr (LAST && dma16_count(m) > 0) {
+                if (have2) {
+                    constexpr int t = dma16_first(m);
+                    NQ_DMA(t, BUF, srca, srcb);
+                    if constexpr (dma16_count(m) == 2) NQ_DMA(t + 1, BUF, srca, srcb);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
     // one stage, read from buffer BUF; its last phase refills BUF with stage st + NB
     auto stage = [&](auto bufc, auto zeroc, int st, int KT) {
         const bool have2 = st + NB < KT;
-        const bool keep1 = NB == 3 && st + 2 < KT;
+        const int keep = max(0, min(NB - 2, KT - st - 2));
         const uint8_t* const srca = abase + (int64_t)(st + NB) * BK;
         const uint8_t* const srcb = bbase + (int64_t)(st + NB) * BK;
-        if constexpr (TI == 4) {
-            phase8(bufc, integral_constant<int, 0>{}, zeroc, have2, keep1, srca, srcb);
-            if constexpr (PH == 2) phase8(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, keep1, srca, srcb);
+        if constexpr (TJ == 4) {
+            phase16(bufc, integral_constant<int, 0>{}, zeroc, have2, keep, srca, srcb);
+            if constexpr (PH == 2) phase16(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, keep, srca, srcb);
+        } else if constexpr (TI == 4) {
+            phase8(bufc, integral_constant<int, 0>{}, zeroc, have2, keep, srca, srcb);
+            if constexpr (PH == 2) phase8(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, keep, srca, srcb);
         } else {
             phase(bufc, integral_constant<int, 0>{}, zeroc, have2, srca, srcb);
             if constexpr (PH == 2) phase(bufc, integral_constant<int, 1>{}, std::false_type{}, have2, srca, srcb);
@@ -554,8 +659,8 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
         NQ_DMA(14, buf, srca, srcb); NQ_DMA(15, buf, srca, srcb);                                  \
     }
         NQ_DMA_ALL(0)
-        if constexpr (NB == 3) {
-            // all three buffers at once; stage 0 has landed when at most the other two stages' transfers are out
+        if constexpr (NB >= 3) {
+            // all buffers at once; stage 0 has landed when at most the other stages' transfers are out
             if (KT > 1) {
                 srca = abase + BK, srcb = bbase + BK;
                 NQ_DMA_ALL(1)
@@ -563,12 +668,22 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
             if (KT > 2) {
                 srca = abase + 2 * BK, srcb = bbase + 2 * BK;
                 NQ_DMA_ALL(2)
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (DA + DB)) : "memory");
-            } else if (KT > 1) {
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DA + DB) : "memory");
-            } else {
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             }
+            if constexpr (NB == 4) {
+                if (KT > 3) {
+                    srca = abase + 3 * BK, srcb = bbase + 3 * BK;
+                    NQ_DMA_ALL(3)
+                }
+            }
+            const int out = min(KT, NB) - 1;  // stages that may still be on their way
+            if (out >= 3)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (DA + DB)) : "memory");
+            else if (out == 2)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (DA + DB)) : "memory");
+            else if (out == 1)
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DA + DB) : "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
         } else {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -587,7 +702,18 @@ __device__ __forceinline__ void gemm8_body(const Gemm8Params& p) {
     static_for<TJ>([&](auto jc) { read_w(integral_constant<int, 0>{}, jc, integral_constant<int, 0>{}, integral_constant<int, 0>{}); });
     NQ_LDS_WAIT(0);
     stage(integral_constant<int, 0>{}, std::true_type{}, 0, KT);
-    if constexpr (NB == 3) {
+    if constexpr (NB == 4) {
+        for (int st = 1; st < KT;) {
+            stage(integral_constant<int, 1>{}, std::false_type{}, st, KT);
+            if (++st >= KT) break;
+            stage(integral_constant<int, 2>{}, std::false_type{}, st, KT);
+            if (++st >= KT) break;
+            stage(integral_constant<int, 3>{}, std::false_type{}, st, KT);
+            if (++st >= KT) break;
+            stage(integral_constant<int, 0>{}, std::false_type{}, st, KT);
+            ++st;
+        }
+    } else if constexpr (NB == 3) {
         for (int st = 1; st < KT;) {
             stage(integral_constant<int, 1>{}, std::false_type{}, st, KT);
             if (++st >= KT) break;
@@ -804,11 +930,18 @@ void gemm8h_kernel(const Gemm8Params p) {
     gemm8_body<FP8, KIND, 128, 256, 128, 4>(p);
 }
 
+// a 128 x 128 tile on four wavefronts of 64 x 64: for what fills at most a round of such tiles
+template <bool FP8, int KIND>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm8q_kernel(const Gemm8Params p) {
+    gemm8_body<FP8, KIND, 128, 128, 128, 4>(p);
+}
+
 template <typename K>
 int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int form, hipStream_t s) {
     // two stage buffers of 64 KiB each (three of 48 for the 128-row tile); the eight-wavefront form's epilogue stages 17 KiB
     // per wavefront
-    const size_t lds = form == 8 ? (size_t)8 * 17408 : form == 12 ? (size_t)3 * (128 + 256) * 128 : (size_t)2 * (256 + 256) * 128;
+    const size_t lds = form == 8 ? (size_t)8 * 17408 : form == 12 ? (size_t)3 * (128 + 256) * 128 : form == 16 ? (size_t)4 * (128 + 128) * 128 : (size_t)2 * (256 + 256) * 128;
     NQ_HIP(set_max_lds_once(*attr, reinterpret_cast<const void*>(kernel), lds));
     hipLaunchKernelGGL(kernel, dim3(p.grid ? p.grid : p.tiles_m * p.tiles_n), dim3(form == 8 ? 512 : 256), lds, s, p);
     NQ_HIP(hipGetLastError());
@@ -817,8 +950,8 @@ int32_t launch_cfg(K kernel, LdsAttrOnce* attr, const Gemm8Params& p, int form, 
 
 // form: 4 / 8 = the 256 x 256 tile on that many wavefronts, 12 = the 128 x 256 tile.  kind: 0 fp32, 1 bf16, 2 raw int32
 int32_t launch_form(int form, bool fp8, int kind, const Gemm8Params& p, hipStream_t s) {
-    static LdsAttrOnce attr[3][5];
-    const int f = form == 4 ? 0 : form == 8 ? 1 : 2;
+    static LdsAttrOnce attr[4][5];
+    const int f = form == 4 ? 0 : form == 8 ? 1 : form == 12 ? 2 : 3;
     const int k = fp8 ? kind : 2 + kind;
 #define NQ_G8_PICK(KERNEL)                                                                     \
     switch (k) {                                                                               \
@@ -830,11 +963,59 @@ int32_t launch_form(int form, bool fp8, int kind, const Gemm8Params& p, hipStrea
     }
     if (form == 4) { NQ_G8_PICK(gemm8_kernel) }
     if (form == 8) { NQ_G8_PICK(gemm8w_kernel) }
+    if (form == 16) { NQ_G8_PICK(gemm8q_kernel) }
     NQ_G8_PICK(gemm8h_kernel)
 #undef NQ_G8_PICK
 }
 
 }  // namespace
+
+// What a call takes on each tile form, from measurements over K = 1024 .. 8192, M = 256 .. 8192, N = 4096 .. 11008: rounds
+// of 256 workgroups x (a fixed part + a part per stage of 128 bytes of K); the smaller tiles' stages lengthen as more
+// than half the CUs draw on L2 at once (`crowd`: the share of the round's workgroups beyond 128).
+//   128 x 128 (one round, fp8, K = 4096): 15.7 - 15.9 us on 128 workgroups, 18.1 - 20.2 on 256; int8 18.0 / 20.2 - 22.3
+//   128 x 256 (at most 128 tiles of 256 x 256): fp8 24.7 us on 128 workgroups, 26.9 on 192, 29.6 - 31.3 on 256; int8 28.8 / 30.8 / 33.4 - 35.2
+//   256 x 256: 41 - 43 us a round fp8 (four wavefronts), 40 - 42 int8 (eight)
+namespace {
+double estimate_form(int form, int M, int N, int K, bool i8) {
+    const double steps = (double)K / 128.0;
+    if (form == 16) {
+        const int64_t wgs = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+        const int64_t rounds = (wgs + 255) / 256;
+        const int64_t in_round = (wgs + rounds - 1) / rounds;
+        const double crowd = in_round > 128 ? (double)(in_round - 128) / 128.0 : 0.0;
+        return (double)rounds * (5.6 + steps * ((i8 ? 0.385 : 0.32) + 0.08 * crowd));
+    }
+    const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    if (form == 12) {
+        const int64_t wgs = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
+        const double crowd = wgs > 128 ? (double)(wgs - 128) / 128.0 : 0.0;
+        return i8 ? 7.0 + steps * (0.68 + 0.2 * crowd) : 6.5 + steps * (0.58 + 0.21 * crowd);
+    }
+    return (double)((tiles + 255) / 256) * (i8 ? 9.5 + 1.03 * steps : 10.0 + 1.1 * steps);
+}
+// the form a call runs on: 16 = 128 x 128 tiles, 12 = 128 x 256 tiles (calls of at most 128 tiles of 256 x 256), else the
+// 256 x 256 tile on 4 (fp8) or 8 (int8) wavefronts
+int pick_form(int M, int N, int K, bool i8, double* us) {
+    const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    int form = i8 ? 8 : 4;
+    double best = estimate_form(form, M, N, K, i8);
+    if (tiles <= 128) {
+        const double h = estimate_form(12, M, N, K, i8);
+        if (h < best) best = h, form = 12;
+    }
+    const double q = estimate_form(16, M, N, K, i8);
+    if (q < best) best = q, form = 16;
+    if (us) *us = best;
+    return form;
+}
+}  // namespace
+
+double gemm8_estimate_us(int M, int N, int K, bool i8) {
+    double us = 0.0;
+    pick_form(M, N, K, i8, &us);
+    return us;
+}
 
 bool gemm8_applicable(const ForwardArgs& a) {
     const nq_layer* L = a.L;
@@ -867,17 +1048,25 @@ int32_t launch_gemm8(const ForwardArgs& a) {
         p.tiles_m = (a.M + 127) / 128;
         return launch_form(12, fp8, kind, p, a.stream);
     }
+    if (a.diag_gemm8_waves == 16) {  // everything on 128 x 128 tiles
+        p.tiles_m = (a.M + 127) / 128, p.tiles_n = (L->out + 127) / 128;
+        return launch_form(16, fp8, kind, p, a.stream);
+    }
     // int8 runs on the eight-wavefront form (8192 x 4096 x 4096: 105 - 108 us against 110 - 112; one round of tiles,
     // M = 2048: 42 - 43 against 49.5), fp8 on the four-wavefront form (the two measure the same, 95.5 - 99 us on the
     // same box; N = 11008 and 8192^3 1 - 2 % slower with eight)
-    const int form = a.diag_gemm8_waves ? a.diag_gemm8_waves : (i8 ? 8 : 4);
-    if (a.diag_gemm8_waves || a.diag_stamps) return launch_form(form, fp8, kind, p, a.stream);
+    if (a.diag_gemm8_waves || a.diag_stamps) return launch_form(a.diag_gemm8_waves ? a.diag_gemm8_waves : (i8 ? 8 : 4), fp8, kind, p, a.stream);
+    const int form = pick_form(a.M, L->out, L->in, i8, nullptr);
+    if (form == 16) {
+        p.tiles_m = (a.M + 127) / 128, p.tiles_n = (L->out + 127) / 128;
+        return launch_form(16, fp8, kind, p, a.stream);
+    }
     // What fills at most half a round of workgroups goes on 128 x 256 tiles, twice as many: a call that small as a
     // whole, or the tiles left over after the last full round when they form a rectangle (the kernel deals tiles in
     // bands of 8 row tiles, rows first, so the last `rest` tiles are whole columns of the last band when its row
     // count divides `rest`).  Every accumulator adds the same terms in the same order on either tile: same bits.
     constexpr int CUS = 256;
-    if (tiles <= CUS / 2) {
+    if (form == 12) {
         p.tiles_m = (a.M + 127) / 128;
         return launch_form(12, fp8, kind, p, a.stream);
     }

@@ -526,7 +526,7 @@ static bool row_kernel_fits(const ForwardArgs& a) {
 }
 
 // The tile kernel against the 256 x 256-tile GEMM (nq_gemm8.hip), both measured over K = 512 .. 8192,
-// N = 1024 .. 11008, M = 64 .. 2048.  What the GEMM takes on either of its tile sizes: gemm8_estimate_us.
+// N = 1024 .. 11008, M = 64 .. 2048.  What the GEMM takes on the tile form it picks: gemm8_estimate_us.
 // The tile kernel with 2 or 4 weight tiles per workgroup takes, per round of 256 workgroups, a fixed 5.5 us
 // (3.75 with four wavefronts) + 0.25 / 0.31 us per 128 k, half as much again when 64 rows at a time stream a
 // weight larger than the caches hold; with one weight tile (small launches, short K) about 4 us + 5.6 us per
@@ -537,7 +537,7 @@ static bool tile8_wins(const ForwardArgs& a) {
     if (a.M < 64 || L->in % 128 != 0) return true;  // (the GEMM needs 64 rows and whole 128-byte steps)
     const double steps = (double)L->in / 128.0;
     const bool i8 = a.x_dtype == NQ_DT_I8;
-    const double gemm_us = std::min(gemm8_estimate_us(a.M, L->out, L->in, i8, false), gemm8_estimate_us(a.M, L->out, L->in, i8, true));
+    const double gemm_us = gemm8_estimate_us(a.M, L->out, L->in, i8);
     const int nt = tile8_weight_tiles(a.M, L->out, L->in);
     double tile_us;
     if (nt == 1) {
