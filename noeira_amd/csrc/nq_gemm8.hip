@@ -105,7 +105,10 @@
 // registers (no first-stage wait, but the slower store shape: equal); a finished tile held
 // in registers as packed bf16 and stored one piece per stage under the next tile's K loop
 // (the moves that rotate the pieces cost the loop what the epilogue saved); workgroups
-// started 0 .. 5 us apart so that epilogues do not coincide (equal).  At the power
+// started 0 .. 5 us apart so that epilogues do not coincide (equal); one workgroup per CU walking its tiles with the
+// LDS-staged stores kept - the next tile's first stage requested into the first buffer under the epilogue, which stages
+// in the second (in twice the passes), the second stage requested after it: 2 % slower for fp8, 8 % for int8 (whose
+// epilogue's own loads of scales and bias then queue behind the requested stage), on one box in turn.  At the power
 // limit, time that one part stops taking is handed back as clock to the others only
 // when energy is saved with it.
 //
