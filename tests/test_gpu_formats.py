@@ -442,6 +442,26 @@ def _gemm8(lin, tile, x, x_dt, x_scale, M, out_dtype, bias=None, epilogue="none"
     return out
 
 
+def test_gemm_tile_forms_on_random_ragged_shapes():
+    """Every tile form of the 8-bit GEMM (128 x 128, 128 x 256, 256 x 256 on four and on eight wavefronts) on a dozen
+    seeded random shapes - M from 64, any N from 1, K = 128 .. 640 in steps of 128 (one stage up to five: the stage
+    buffers' wrap-around for two, three and four buffers) - against the oracle's int32 accumulators, bit for bit,
+    with a sentinel under every output."""
+    from noeira_amd import _lib as L
+    rng = np.random.default_rng(20240611)
+    shapes = [(int(rng.integers(64, 700)), 128 * int(rng.integers(1, 6)), int(rng.integers(1, 900))) for _ in range(10)]
+    shapes += [(64, 128, 1), (65, 640, 257), (129, 512, 129), (513, 384, 511)]
+    for M, K, N in shapes:
+        lin, w, s = w8_layer(rng, K, N)
+        xq_h = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        xq = torch.from_numpy(xq_h).cuda()
+        sx = torch.from_numpy(rng.uniform(1e-3, 1e-1, M).astype(np.float32)).cuda()
+        want = O.w8a8_acc_i32(xq_h, w)
+        for tile in (128, 1282, 2564, 2568):
+            got = _gemm8(lin, tile, xq, L.DT_I8, sx, M, torch.int32).cpu().numpy()
+            assert np.array_equal(got, want), (M, K, N, tile)
+
+
 @pytest.mark.parametrize("M,K,N", [(2048, 128, 8704), (2304, 256, 15360), (2240, 128, 15300), (2100, 128, 8500), (8192, 128, 11008)])
 def test_gemm_leftover_tiles_on_the_half_tile_kernel(M, K, N):
     """More than a round of 256 x 256 tiles with at most half a round left over: nq_forward gives the full rounds to
