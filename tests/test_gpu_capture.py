@@ -106,9 +106,11 @@ def test_recorded_forward_float_activations(name, maker, K, N, M, xdt, kw):
     replay_equals_eager(call, [x], lambda i: [xs[i]])
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 4096, 1040), (16, 512, 200), (256, 1024, 1040), (1024, 256, 520)])
+@pytest.mark.parametrize("M,K,N", [(1, 4096, 1040), (16, 512, 200), (256, 1024, 1040), (1024, 256, 520), (2048, 128, 8704), (1536, 256, 2304)])
 def test_recorded_forward_int8_and_fp8_activations(M, K, N):
-    """gemv8_row, tile8 and gemm8 under int8 and e4m3 activations, and the row quantiser that feeds the first."""
+    """gemv8_row, tile8 and gemm8 under int8 and e4m3 activations, and the row quantiser that feeds the first.
+    ((2048, 128, 8704): the GEMM as two launches, full rounds of 256 x 256 tiles and the leftover on 128 x 256 tiles;
+    (1536, 256, 2304): all of it on 128 x 256 or 128 x 128 tiles.)"""
     rng = np.random.default_rng(M + K + N)
     lin, lin8 = w8(rng, K, N), fp8(rng, K, N)
     xs = [torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).cuda() for _ in range(4)]
