@@ -38,7 +38,7 @@
 extern "C" {
 #endif
 
-#define NQ_ABI_VERSION 6
+#define NQ_ABI_VERSION 7
 
 /* status codes */
 #define NQ_OK 0
@@ -215,8 +215,18 @@ int32_t nq_forward_fused(nq_handle h, const void* x, int32_t x_dtype, const floa
 /* The device twin of `dequantize_q4_0` (`dequant_q4_0_kernel`,
  * q4_0.mojo:242-266; `QLinear.dequantized`, qlinear.mojo:326-328): deq(W)
  * [OUT, IN] fp32 into out_dev (n_values >= OUT*IN else NQ_ERR_SIZE, the
- * `share_scratch` rule of qlinear.mojo:330-340).  Any format. */
+ * `share_scratch` rule of qlinear.mojo:330-340), or, with out_dev = NULL and
+ * n_values = 0, into the workspace shared by nq_set_workspace.  Any format. */
 int32_t nq_dequantize(nq_handle h, float* out_dev, int64_t n_values, void* stream);
+
+/* `QLinear.share_scratch` (qlinear.mojo:330-340): the caller's buffer takes the place of the layer's own dequantize
+ * scratch; every layer of a model can share one, they run one at a time.  nq_workspace_bytes: the bytes that scratch
+ * holds, 4 * OUT * IN, whatever M (no forward of this library dequantizes to memory, so none reads or writes the
+ * workspace; M is taken for callers written against a forward that does); 0 for a null handle.  nq_set_workspace:
+ * NQ_ERR_SIZE with share_scratch's sentence if nbytes is smaller, NQ_ERR_INVALID for a null or misaligned buffer;
+ * (NULL, 0) takes the workspace away again.  The buffer stays the caller's: the library neither frees nor outlives it. */
+int64_t nq_workspace_bytes(nq_handle h, int32_t M);
+int32_t nq_set_workspace(nq_handle h, void* dev, int64_t nbytes);
 
 /* `QLinear.vjp` (qlinear.mojo:479-518): gx[M, IN] = gy[M, OUT] @ deq(W),
  * fp32 in and out, overwriting gx.  Q4_0 only. */

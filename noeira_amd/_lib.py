@@ -18,7 +18,7 @@ NQ_OK, NQ_ERR_INVALID, NQ_ERR_NOT_LOADED, NQ_ERR_NO_BLOCKS, NQ_ERR_SIZE, NQ_ERR_
 FMT_Q4_0, FMT_W8_CHANNEL, FMT_W4_GROUP, FMT_FP8_E4M3 = range(4)
 DT_F32, DT_BF16, DT_I8, DT_FP8_E4M3, DT_I32 = range(5)
 EPI_NONE, EPI_RELU, EPI_SWIGLU = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 FLAG_NO_TILE_COPY = 1
 FLAG_PREFER_TILE = 2
@@ -32,7 +32,7 @@ class LoraPart(C.Structure):
 EXPORTS = [
     "nq_abi_version", "nq_last_error", "nq_create", "nq_destroy", "nq_set_blocks", "nq_set_weight_f32",
     "nq_set_weight_i8", "nq_set_weight_w4g", "nq_set_weight_fp8", "nq_blocks_bytes", "nq_get_blocks",
-    "nq_keep_only_repacked", "nq_device_bytes", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
+    "nq_keep_only_repacked", "nq_device_bytes", "nq_workspace_bytes", "nq_set_workspace", "nq_forward", "nq_dequantize", "nq_grad_input", "nq_quantize_rows_i8",
     "nq_cast_pad_bf16", "nq_slice_cast_f32", "nq_mlp3_w8a8_forward", "nq_fuse_rows", "nq_fused_parts",
     "nq_forward_fused", "nq_fuse_glu", "nq_hessian_create", "nq_hessian_destroy", "nq_hessian_add", "nq_hessian_rows",
     "nq_hessian_get", "nq_hessian_set", "nq_hinv_upper_f64", "nq_hinv_upper_f64_dev", "nq_set_weight_gptq", "nq_q4_0_objective", "nq_lora_forward_add", "nq_forward_lora", "nq_forward_fused_lora", "nq_diag_mfma_rate", "nq_diag_stream_read", "nq_diag_gemm8_timeline", "nq_diag_forward_a16", "nq_diag_forward_gemm8",
@@ -168,6 +168,10 @@ def lib() -> C.CDLL:
     L.nq_diag_gemm8_timeline.argtypes = [p, p, i32, p, p, i32, i32, p, i64, p]
     L.nq_device_bytes.restype = i64
     L.nq_device_bytes.argtypes = [p]
+    L.nq_workspace_bytes.restype = i64
+    L.nq_workspace_bytes.argtypes = [p, i32]
+    L.nq_set_workspace.restype = i32
+    L.nq_set_workspace.argtypes = [p, p, i64]
     L.nq_diag_forward_a16.restype = i32
     L.nq_diag_forward_a16.argtypes = [p, p, i32, p, i32, i32, i32, i32, p]
     got = L.nq_abi_version()

@@ -732,12 +732,38 @@ int32_t nq_dequantize(nq_handle h, float* out_dev, int64_t n_values, void* strea
     int32_t rc = check_handle(h, "nq_dequantize");
     if (rc) return rc;
     if ((rc = need_loaded(h, "dequantized"))) return rc;
+    if (!out_dev && n_values == 0) {  // into the workspace the caller shared
+        if (!h->workspace) return fail(NQ_ERR_INVALID, "nq_dequantize: no output and no workspace (nq_set_workspace)");
+        return launch_dequantize(h, h->workspace, (hipStream_t)stream);
+    }
     if (n_values < (int64_t)h->in * h->out)  // qlinear.mojo:334-338
         return fail(NQ_ERR_SIZE, "QLinear.share_scratch: " + std::to_string(n_values) + " values for a [" +
                                      std::to_string(h->out) + ", " + std::to_string(h->in) + "] weight");
     if (!out_dev || ((uintptr_t)out_dev & 15))
         return fail(NQ_ERR_INVALID, "nq_dequantize: the output must be a 16-byte aligned device buffer");
     return launch_dequantize(h, out_dev, (hipStream_t)stream);
+}
+
+int64_t nq_workspace_bytes(nq_handle h, int32_t M) {
+    (void)M;  // (no forward of this library dequantizes to memory: the scratch is nq_dequantize's alone)
+    if (!h) return 0;
+    return (int64_t)h->in * h->out * 4;
+}
+
+int32_t nq_set_workspace(nq_handle h, void* dev, int64_t nbytes) {
+    int32_t rc = check_handle(h, "nq_set_workspace");
+    if (rc) return rc;
+    if (!dev && nbytes == 0) {
+        h->workspace = nullptr, h->workspace_bytes = 0;
+        return NQ_OK;
+    }
+    if (nbytes < nq_workspace_bytes(h, 0))  // qlinear.mojo:334-338
+        return fail(NQ_ERR_SIZE, "QLinear.share_scratch: " + std::to_string(nbytes < 0 ? 0 : nbytes / 4) + " values for a [" +
+                                     std::to_string(h->out) + ", " + std::to_string(h->in) + "] weight");
+    if (!dev || ((uintptr_t)dev & 15))
+        return fail(NQ_ERR_INVALID, "nq_set_workspace: the workspace must be a 16-byte aligned device buffer");
+    h->workspace = reinterpret_cast<float*>(dev), h->workspace_bytes = nbytes;
+    return NQ_OK;
 }
 
 int32_t nq_grad_input(nq_handle h, const float* gy, float* gx, int32_t M, void* stream) {

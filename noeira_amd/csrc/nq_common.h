@@ -69,6 +69,8 @@ struct nq_layer {
     // at a time, and (4-bit) of the group records in the same order; tile_nj = steps of K per row tile
     uint8_t* d_tile16 = nullptr;
     void* d_tile16_scales = nullptr;
+    float* workspace = nullptr;     // caller-owned dequantize scratch (nq_set_workspace), never read by a forward
+    int64_t workspace_bytes = 0;
     int32_t tile_nj = 0;
     bool no_tile_copy = false;  // NQ_FLAG_NO_TILE_COPY
     bool prefer_tile = false;   // NQ_FLAG_PREFER_TILE

@@ -127,7 +127,9 @@ class _Layer:
         if out is None:
             shared = getattr(self, "deq", None)
             if shared is not None:
-                out = shared.view(-1)[: self.OUT * self.IN].view(self.OUT, self.IN)
+                # (the library writes the workspace it was handed by nq_set_workspace)
+                L.check(L.lib().nq_dequantize(self._h, None, 0, _stream_ptr()))
+                return shared.view(-1)[: self.OUT * self.IN].view(self.OUT, self.IN)
             else:
                 out = torch.empty((self.OUT, self.IN), dtype=torch.float32, device="cuda")
         L.check(L.lib().nq_dequantize(self._h, _dev_ptr(out), out.numel(), _stream_ptr()))
@@ -207,6 +209,7 @@ class QLinear(_Layer):
                             f"QLinear.share_scratch: {min(n, buf.numel())} values for a [{self.OUT}, {self.IN}] weight")
         if buf.dtype != torch.float32 or not buf.is_cuda or not buf.is_contiguous():
             raise L.NQError(L.NQ_ERR_INVALID, "QLinear.share_scratch: the scratch must be a contiguous fp32 device tensor")
+        L.check(L.lib().nq_set_workspace(self._h, _dev_ptr(buf), 4 * n))
         self.deq = buf
 
     def keep_only_repacked(self):

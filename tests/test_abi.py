@@ -81,6 +81,16 @@ def test_lifecycle_errors_before_load():
     assert "10 values for a [4, 64] weight" in L.last_error()
     # a layer of one format refuses another format's loader
     assert lib.nq_set_weight_fp8(h, buf.ctypes.data_as(C.c_void_p), C.c_float(1.0), None) == L.NQ_ERR_INVALID
+    # the shared dequantize scratch (`share_scratch`, qlinear.mojo:330-340): its size, and the reference's sentence
+    # for a buffer that is too small; no buffer is touched by either call
+    assert lib.nq_workspace_bytes(h, 1) == lib.nq_workspace_bytes(h, 4096) == 4 * 4 * 64
+    assert lib.nq_workspace_bytes(None, 1) == 0
+    assert lib.nq_set_workspace(h, C.c_void_p(4096), 4 * 4 * 64 - 4) == L.NQ_ERR_SIZE
+    assert L.last_error() == "QLinear.share_scratch: 255 values for a [4, 64] weight"
+    assert lib.nq_set_workspace(h, C.c_void_p(4104), 4 * 4 * 64) == L.NQ_ERR_INVALID   # not 16-byte aligned
+    assert lib.nq_set_workspace(h, None, 4 * 4 * 64) == L.NQ_ERR_INVALID
+    assert lib.nq_set_workspace(h, C.c_void_p(4096), 4 * 4 * 64) == 0
+    assert lib.nq_set_workspace(h, None, 0) == 0
     lib.nq_destroy(h)
 
 
