@@ -252,7 +252,8 @@ def make_decoder_layer(M, adapters, copies=1, seed=11):
     activations; noeira/deep_agents/smolvla/fused.mojo:287-363) in the caller's order, each on its own input buffer:
     `adapters` = "none": q|k|v fused, o, gate|up + SwiGLU fused, down - four launches;
     "fused": the same groups with a rank-16 adapter on all seven (layer_weights.mojo:713-739): nq_forward_fused_lora for
-    q|k|v and for gate|up (SwiGLU applied to the sums), nq_forward_lora for o and down;
+    q|k|v and for gate|up (SwiGLU applied to the sums; on the nq_fuse_glu layer in one launch at 17 .. 511 rows),
+    nq_forward_lora for o and down;
     "per_projection": what the caller does today, seven `proj_fwd` = forward + forward_add, then SwiGLU left out."""
     import numpy as np
     import torch
@@ -293,10 +294,18 @@ def make_decoder_layer(M, adapters, copies=1, seed=11):
             qkv.forward(x, outs=yq), lin[3].forward(x, out=yo), glu.forward(x, out=yg), lin[6].forward(h, out=yd)
         launches = 4
     elif adapters == "fused":
+        # gate | up: the nq_fuse_glu layer adds both adapters ahead of SwiGLU in its one launch where its kernel takes
+        # the rows (17 .. 511); elsewhere the row-fused pair, an adding launch and the activation
+        glu_folds = 17 <= M <= 511
+
         def step(i):
             qkv.forward_lora(x, ads[0:3], outs=yq), ads[3].forward_with(lin[3], x, out=yo)
-            pair.forward_lora(x, ads[4:6], outs=gu, glu_out=yg), ads[6].forward_with(lin[6], h, out=yd)
-        launches = 8
+            if glu_folds:
+                glu.forward_lora(x, ads[4], ads[5], out=yg)
+            else:
+                pair.forward_lora(x, ads[4:6], outs=gu, glu_out=yg)
+            ads[6].forward_with(lin[6], h, out=yd)
+        launches = 7 if glu_folds else 8
     else:
         outs = [yq[0], yq[1], yq[2], yo, gu[0], gu[1], yd]
 

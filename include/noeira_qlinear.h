@@ -303,7 +303,14 @@ typedef struct nq_lora_part {
  * glu_out != NULL: the layer's two parts are gate and up of one MLP (equal widths, no bias).  The adding launch then
  * also writes glu_out[M, OUT] = up * silu(gate) (`SwiGLU.forward`, noeira/nn/primitives/swiglu.mojo:41-60; fp32 or
  * bf16 by glu_dtype) from the sums it formed, and ys[0], ys[1] keep the base projections: they are scratch the caller
- * lends (the adapters act before the activation, which is why a layer made by nq_fuse_glu cannot take them). */
+ * lends.
+ * A layer made by nq_fuse_glu (gate and up interleaved, SwiGLU in the kernel's epilogue) takes the call too, as ONE
+ * launch: adapters[0] is the gate projection's, adapters[1] the up projection's, both present with one R_PAD <= 16 (or
+ * both absent), glu_out [M, OUT / 2] is the only output and ys is not read.  Both shares enter the accumulators ahead
+ * of the activation, which only the kernel for 17 .. 511 rows over rows of at most 4096 codes can do: other shapes
+ * return NQ_ERR_UNSUPPORTED before anything is launched (fuse gate and up with nq_fuse_rows then).  B = 0 on both
+ * leaves the bits of nq_forward on that layer wherever nq_forward takes the same kernel (by default from a few tens
+ * of rows on). */
 int32_t nq_forward_fused_lora(nq_handle h, const void* x, int32_t x_dtype, float* const* ys, int32_t n_ys, int32_t M,
                               const void* bias, int32_t bias_dtype, const nq_lora_part* adapters, void* glu_out,
                               int32_t glu_dtype, void* stream);

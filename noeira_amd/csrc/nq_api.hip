@@ -475,6 +475,10 @@ struct LoraArgs {
     const float* b;
     int32_t r;
     float s;
+    // a gate | up layer's second adapter (the up projection's; a / b / s are then the gate's), or null
+    const float* a2 = nullptr;
+    const float* b2 = nullptr;
+    float s2 = 0.0f;
 };
 int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x_scale, const SegTable& seg,
                      int32_t y_dtype, int32_t M, const void* bias, int32_t bias_dtype, int32_t epilogue,
@@ -520,6 +524,18 @@ int32_t forward_impl(nq_handle h, const void* x, int32_t x_dtype, const float* x
         a.lora_a = lora->a, a.lora_b = lora->b, a.lora_r = lora->r, a.lora_s = lora->s;
         *folded = true;
         return launch_gemm_tile_mt(a);
+    }
+    if (lora && lora->a2) {
+        // a gate | up layer: both adapters' shares enter the accumulators ahead of the SwiGLU epilogue, in the M-tile
+        // kernel only (nothing can add them afterwards: the layer's only output is the activation's)
+        if (h->glu && lora->r <= 16 && gemm_tile_mt_takes_shape(a) && gemm_tile_mt_lora_foldable(a)) {
+            a.lora_a = lora->a, a.lora_b = lora->b, a.lora_r = lora->r, a.lora_s = lora->s;
+            a.lora_a2 = lora->a2, a.lora_b2 = lora->b2, a.lora_s2 = lora->s2;
+            *folded = true;
+            return launch_gemm_tile_mt(a);
+        }
+        return fail(NQ_ERR_UNSUPPORTED, "nq_forward_fused_lora: for this layer and M no kernel adds adapters ahead of SwiGLU; "
+                                        "fuse gate and up with nq_fuse_rows and pass glu_out");
     }
     // (decided before anything is launched: a caller whose y cannot take a second, adding launch gets its answer
     // with y untouched)
@@ -808,8 +824,30 @@ int32_t nq_forward_fused_lora(nq_handle h, const void* x, int32_t x_dtype, float
     if (rc) return rc;
     if ((rc = need_loaded(h, "forward"))) return rc;
     const int parts = nq_fused_parts(h);
-    if (h->glu) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: a layer made by nq_fuse_glu applies SwiGLU before an adapter "
-                                            "could add its share; fuse gate and up with nq_fuse_rows and pass glu_out");
+    if (h->glu) {
+        // a gate | up layer (nq_fuse_glu): adapters[0] is the gate projection's, adapters[1] the up projection's; the
+        // only output is glu_out [M, OUT / 2] (ys is not read)
+        if (M < 0) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: M must be >= 0");
+        if (M == 0) return NQ_OK;
+        if (!x || !adapters || !glu_out) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: null pointer");
+        if (bias) return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: a SwiGLU pair takes no bias");
+        if (glu_dtype != NQ_DT_F32 && glu_dtype != NQ_DT_BF16)
+            return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: glu_out must be fp32 or bf16");
+        const nq_lora_part &g = adapters[0], &u = adapters[1];
+        for (const nq_lora_part* ad : {&g, &u})
+            if ((ad->a == nullptr) != (ad->b == nullptr) || (ad->a && ad->r_pad <= 0))
+                return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: an adapter is (a, b, r_pad > 0) or all null");
+        SegTable seg{};
+        seg.nseg = 1, seg.end[0] = h->out, seg.y[0] = glu_out;
+        if (!g.a && !u.a) return forward_impl(h, x, x_dtype, nullptr, seg, glu_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_SWIGLU, stream);
+        if (!g.a || !u.a || g.r_pad != u.r_pad)
+            return fail(NQ_ERR_UNSUPPORTED, "nq_forward_fused_lora: a layer made by nq_fuse_glu takes adapters on both projections, "
+                                            "of one padded rank; otherwise fuse gate and up with nq_fuse_rows and pass glu_out");
+        LoraArgs lora{g.a, g.b, g.r_pad, g.scale};
+        lora.a2 = u.a, lora.b2 = u.b, lora.s2 = u.scale;
+        bool folded = false;
+        return forward_impl(h, x, x_dtype, nullptr, seg, glu_dtype, M, nullptr, NQ_DT_F32, NQ_EPI_SWIGLU, stream, &lora, &folded, true);
+    }
     if (n_ys != parts)
         return fail(NQ_ERR_INVALID, "nq_forward_fused_lora: " + std::to_string(n_ys) + " outputs for a layer of " +
                                         std::to_string(parts) + " fused parts");

@@ -135,6 +135,9 @@ struct ForwardArgs {
     const float* lora_b = nullptr;
     int32_t lora_r = 0;
     float lora_s = 0.0f;
+    const float* lora_a2 = nullptr;  // a gate | up layer's second adapter (the up projection's; lora_a / lora_b: the gate's)
+    const float* lora_b2 = nullptr;
+    float lora_s2 = 0.0f;
     // nq_diag_gemm8_timeline: where the large-tile GEMM writes its per-tile clock readings (null: none)
     unsigned long long* diag_stamps = nullptr;
     int diag_gemm8_waves = 0;  // 0: the library's choice; 4 / 8: the 256 x 256 tile GEMM with that many wavefronts; 12: its 128 x 256 tile form
@@ -193,6 +196,7 @@ int32_t launch_gemv_tile8_rows(const ForwardArgs& a);
 bool gemm_tile_mt_applicable(const ForwardArgs& a);
 bool gemm_tile_mt_splits_parts(const ForwardArgs& a);
 bool gemm_tile_mt_lora_foldable(const ForwardArgs& a);
+bool gemm_tile_mt_takes_shape(const ForwardArgs& a);
 int32_t launch_gemm_tile_mt(const ForwardArgs& a);
 int32_t launch_gemv_tile_rows(const ForwardArgs& a);
 int32_t launch_gemv_tile(const ForwardArgs& a);

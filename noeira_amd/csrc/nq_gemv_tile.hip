@@ -285,6 +285,11 @@ struct TileMrParams {
     const float* lb;  // [lr][OUT] fp32
     int32_t lr;       // rank as stored (padded), <= 16
     float ls;
+    // a second adapter, for a gate | up layer (nq_fuse_glu: gate in the even columns, up in the odd ones): la / lb are
+    // the gate projection's adapter, la2 / lb2 the up projection's, each B [lr][OUT / 2]; null = none
+    const float* la2;
+    const float* lb2;
+    float ls2;
 };
 
 constexpr int TR_MAXT = 64;  // row tiles per workgroup of the rows kernels: its 1024 threads stage one tile column each
@@ -544,8 +549,11 @@ __global__ __launch_bounds__(1024) void gemv_tile4_rows_kernel(const TileMrParam
 // LORA: `y += s (x A) B` of a frozen adapter (noeira/nn/peft/lora.mojo:292-349) in the same launch.  The workgroup
 // holds its rows' x for all of K already, so h = x A [16 x rank] costs it a handful of MFMAs once (A's fp32 values as
 // three exact bf16 terms against the one or three terms of x, products below 2^-24 of the largest left out), summed
-// over the K split through LDS; s * h . B[:, columns] then enters each tile as four fp32 MFMAs into the accumulator of
-// the group's first wavefront.  With B = 0 that adds exact zeros and the base result keeps its bits.
+// over the K split through LDS; s * h . B[:, columns] then enters each tile as four fp32 MFMAs, one each in the
+// accumulators of the group's first four wavefronts (ranks 4 w .. 4 w + 3), whose shares meet in LDS with the K split's.
+// With B = 0 that adds exact zeros and the base result keeps its bits.  A gate | up layer takes two adapters, the gate
+// projection's on its even columns and the up projection's on the odd ones: two such MFMAs per wavefront, each with the
+// other projection's columns of B set to zero.
 // the sum of N wavefronts' shares of one output (256 floats apart), in wave order: all reads issued, then the additions
 template <int N>
 __device__ __forceinline__ float sum_shares(const float* r0) {
@@ -576,9 +584,11 @@ __device__ __forceinline__ float sum_shares_n(const float* r0, int n) {
     }
 }
 
-template <int FMT, bool XF32, int JPW, int TB, bool LORA>
+// LORA: 0 none, 1 one adapter over the layer's columns, 2 a gate | up layer's pair of adapters (both added before SwiGLU)
+template <int FMT, bool XF32, int JPW, int TB, int LORA>
 __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams pm, const int kw) {
     const TileParams& p = pm.t;
+    constexpr int LN = LORA == 2 ? 2 : 1;  // adapters
     constexpr bool G128 = FMT == NQ_FMT_W4_GROUP;
     constexpr int NT = XF32 ? 3 : 1;
     constexpr bool XS_REGS = (G128 || JPW <= 2) && !(LORA && !G128 && JPW >= 2);  // (registers: the adapter's operands need them)
@@ -689,8 +699,11 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
     const bool finisher = active && f < 256;
     const int fr = (f >> 4) & 15, fc = f & 15;
 
-    __shared__ float hfin[LORA ? 4 : 1][16][17];
-    if constexpr (LORA) {
+    __shared__ float hfin[LN][LORA ? 4 : 1][16][17];
+    if constexpr (LORA != 0) {
+#pragma unroll
+      for (int ad = 0; ad < LN; ad++) {
+        const float* const lap = ad ? pm.la2 : pm.la;
         // h = x A over this wavefront's share of K: the MFMA's B operand is A[k][r] for 8 consecutive k of column
         // r = lane % 16 (ranks past lr, and k past K, are zero)
         // (the groups of a workgroup hold the same x: each forms h over every ng-th chunk and all sixteen shares
@@ -710,7 +723,7 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
                 uint32_t av[8];
 #pragma unroll
                 for (int i = 0; i < 8; i++)
-                    av[i] = reinterpret_cast<const uint32_t*>(pm.la)[(int64_t)min(k0 + i, p.K - 1) * pm.lr + rc];
+                    av[i] = reinterpret_cast<const uint32_t*>(lap)[(int64_t)min(k0 + i, p.K - 1) * pm.lr + rc];
                 u32x4 pl[3];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
@@ -737,22 +750,25 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
         if (finisher) {
             const int at = (fc + 16 * (fr >> 2)) * 4 + (fr & 3);  // D[token fr][rank fc]
             const float hv = sum_shares_n(&red[0][0][at], ng * kw);
-            hfin[grp][fr][fc] = hv;
+            hfin[ad][grp][fr][fc] = hv;
         }
         __syncthreads();
+      }
     }
-    // The adapter's share of a tile, s h B[:, columns], is four fp32 MFMAs of 16x16x4 (rank 16 as four k-extents) into
-    // the accumulator of each group's first wavefront before the K split's shares meet: its A operand is s h (token
-    // lane % 16, rank 4 m + lane / 16), kept in registers for the whole call; its B operand B[rank][column lane % 16],
-    // four loads per lane and tile.  (The threads that finish a tile used to do it: sixteen loads of B, sixteen LDS
-    // reads of h and sixteen FMAs per output.)
-    float hA[LORA ? 4 : 1];
-    if constexpr (LORA) {
+    // The adapter's share of a tile, s h B[:, columns], is four fp32 MFMAs of 16x16x4 (rank 16 as four k-extents)
+    // before the K split's shares meet: the A operand is s h (token lane % 16, rank 4 m + lane / 16), kept in registers
+    // for the whole call; the B operand B[rank][column lane % 16], one load per lane, tile and k-extent.  (The threads
+    // that finish a tile used to do it: sixteen loads of B, sixteen LDS reads of h and sixteen FMAs per output; then
+    // the group's first wavefront alone, all four MFMAs: on a tile of twelve bf16 MFMAs per wavefront that made the
+    // group wait for it - 3 us on a 9 us call, 9 us with two adapters.)
+    // (one of the four k-extents per wavefront: the first four wavefronts of a group take ranks 4 kwi .. 4 kwi + 3
+    // each, so that no wavefront's tile is more than one such MFMA per adapter longer than the others')
+    float hA[LN];
+    const int lrank = 4 * kwi + q;
+    if constexpr (LORA != 0) {
 #pragma unroll
-        for (int m = 0; m < 4; m++) {
-            const int r = 4 * m + q;
-            hA[m] = (kwi == 0 && active && r < pm.lr) ? pm.ls * hfin[grp][c][r] : 0.0f;
-        }
+        for (int ad = 0; ad < LN; ad++)
+            hA[ad] = (kwi < 4 && active && lrank < pm.lr) ? (ad ? pm.ls2 : pm.ls) * hfin[ad][grp][c][min(lrank, 15)] : 0.0f;
     }
 
     const int iters = (ntiles + stride - 1) / stride;
@@ -771,12 +787,20 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
         if (p.bias && finisher)
             braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[fn]
                                                : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[fn];
-        float lbf[LORA ? 4 : 1];
-        if constexpr (LORA) {
-            if (kwi == 0 && active) {  // (uniform per wavefront)
+        float lbf[LN];
+        if constexpr (LORA == 1) {
+            if (kwi < 4 && active) {  // (uniform per wavefront)
                 const int64_t nb = min((int64_t)tile * 16 + c, (int64_t)p.N - 1);
-#pragma unroll
-                for (int m = 0; m < 4; m++) lbf[m] = pm.lb[(int64_t)min(4 * m + q, pm.lr - 1) * p.N + nb];
+                lbf[0] = pm.lb[(int64_t)min(lrank, pm.lr - 1) * p.N + nb];
+            }
+        } else if constexpr (LORA == 2) {
+            // the lane's column is a gate column (even) or an up column (odd) of projection row nb / 2: one adapter's B
+            // is loaded, the other's operand is zero there
+            if (kwi < 4 && active) {
+                const int64_t nb = min((int64_t)tile * 16 + c, (int64_t)p.N - 1);
+                const bool up = (nb & 1) != 0;
+                const float v = (up ? pm.lb2 : pm.lb)[(int64_t)min(lrank, pm.lr - 1) * (p.N >> 1) + (nb >> 1)];
+                lbf[0] = up ? 0.0f : v, lbf[1] = up ? v : 0.0f;
             }
         }
         if (have) {
@@ -821,10 +845,10 @@ __global__ __launch_bounds__(1024) void gemm_tile4_mt_kernel(const TileMrParams 
                     for (int t = 0; t < 4; t++) acc[t] = fmaf(d, dd[t], acc[t]);
                 }
             }
-            if constexpr (LORA) {
-                if (kwi == 0) {
+            if constexpr (LORA != 0) {
+                if (kwi < 4) {
 #pragma unroll
-                    for (int m = 0; m < 4; m++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(hA[m], lbf[m], acc, 0, 0, 0);
+                    for (int ad = 0; ad < LN; ad++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(hA[ad], lbf[ad], acc, 0, 0, 0);
                 }
             }
             *reinterpret_cast<f32x4*>(&red[buf][wave][lane * 4]) = acc;
@@ -1627,8 +1651,9 @@ int32_t launch4_mt(const TileMrParams& pm, hipStream_t s) {
     const int gx = std::max(1, std::min((ntiles + ng - 1) / ng, std::max(cus, 1) / mt));
     const dim3 grid((unsigned)gx, (unsigned)mt);
 #define NQ_MT(XF, J)                                                                                             \
-    if (pm.la) hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, true>), grid, dim3(1024), 0, s, pm, kw);      \
-    else hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, false>), grid, dim3(1024), 0, s, pm, kw);
+    if (pm.la2) hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, 2>), grid, dim3(1024), 0, s, pm, kw);        \
+    else if (pm.la) hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, 1>), grid, dim3(1024), 0, s, pm, kw);    \
+    else hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, XF, J, 1, 0>), grid, dim3(1024), 0, s, pm, kw);
     if constexpr (XF32) {
         NQ_MT(true, 1)
     } else {
@@ -1636,7 +1661,7 @@ int32_t launch4_mt(const TileMrParams& pm, hipStream_t s) {
             case 1: NQ_MT(false, 1) break;
             case 2: NQ_MT(false, 2) break;
             default:  // (three steps per wavefront leave no registers for an adapter's operands: lora_foldable says no)
-                hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 3, 1, false>), grid, dim3(1024), 0, s, pm, kw);
+                hipLaunchKernelGGL((gemm_tile4_mt_kernel<FMT, false, 3, 1, 0>), grid, dim3(1024), 0, s, pm, kw);
                 break;
         }
     }
@@ -1840,6 +1865,9 @@ bool gemm_tile_mt_applicable(const ForwardArgs& a) {
     return true;
 }
 
+// whether the kernel can run the call at all (its shapes), whatever the estimates say about other kernels
+bool gemm_tile_mt_takes_shape(const ForwardArgs& a) { return mt_shape_ok(a); }
+
 // an adapter can ride along where a wavefront holds at most two steps of K (IN <= 4096; measured there at
 // 4096 -> 4096, T = 135, bf16 x: 36.3 us folded against 38.2 us as two launches)
 bool gemm_tile_mt_lora_foldable(const ForwardArgs& a) {
@@ -1865,6 +1893,7 @@ int32_t launch_gemm_tile_mt(const ForwardArgs& a) {
     p.y_dtype = a.y_dtype, p.bias_dtype = a.bias_dtype, p.epilogue = a.epilogue;
     pm.M = a.M;
     pm.la = a.lora_a, pm.lb = a.lora_b, pm.lr = a.lora_r, pm.ls = a.lora_s;
+    pm.la2 = a.lora_a2, pm.lb2 = a.lora_b2, pm.ls2 = a.lora_s2;
     const bool xf32 = a.x_dtype == NQ_DT_F32;
     if (L->format == NQ_FMT_Q4_0)
         return xf32 ? launch4_mt<NQ_FMT_Q4_0, true>(pm, a.stream) : launch4_mt<NQ_FMT_Q4_0, false>(pm, a.stream);

@@ -526,6 +526,32 @@ class FusedGLU:
                                    _TORCH_DT[out_dtype], M, C.c_void_p(0), L.DT_F32, L.EPI_SWIGLU, _stream_ptr()))
         return out
 
+    def forward_lora(self, x: torch.Tensor, gate_adapter, up_adapter, out: Optional[torch.Tensor] = None,
+                     out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """`forward` with the gate and the up projection's frozen adapters added ahead of the activation, in the same
+        single launch (`nq_forward_fused_lora` on a layer made by nq_fuse_glu): up'(x) * silu(gate'(x)) with
+        p'(x) = p(x) + scale_p * (x A_p) B_p, i.e. `proj_fwd` on both projections (layer_weights.mojo:455-508) and
+        `SwiGLU.forward`.  Both adapters (one padded rank) or neither; raises NQ_ERR_UNSUPPORTED where no kernel can
+        add them ahead of SwiGLU (then: `FusedRows.forward_lora(..., glu_dtype=...)`)."""
+        if out is not None:
+            out_dtype = out.dtype
+        if x.dtype not in _TORCH_DT or out_dtype not in _TORCH_DT:
+            raise L.NQError(L.NQ_ERR_INVALID, "FusedGLU.forward_lora: x and y must be fp32 or bf16")
+        M = _check_x(x, self.IN, "FusedGLU.forward_lora")
+        if out is None or out.numel() < M * self.OUT:
+            out = torch.empty((M, self.OUT), dtype=out_dtype, device=x.device)
+        table = (L.LoraPart * 2)()
+        for t, ad in enumerate((gate_adapter, up_adapter)):
+            if ad is None or ad.merged:
+                table[t] = L.LoraPart(None, None, 0, 0.0)
+                continue
+            if ad.IN != self.IN or ad.OUT != self.OUT:
+                raise L.NQError(L.NQ_ERR_INVALID, "FusedGLU.forward_lora: adapter %d does not fit its projection" % t)
+            table[t] = L.LoraPart(ad.lora_A.data_ptr(), ad.lora_B.data_ptr(), ad.R_PAD, ad.scale())
+        L.check(L.lib().nq_forward_fused_lora(self._h, _dev_ptr(x), _TORCH_DT[x.dtype], None, 0, M, C.c_void_p(0), L.DT_F32,
+                                              table, _dev_ptr(out), _TORCH_DT[out_dtype], _stream_ptr()))
+        return out
+
 
 def quantize_rows_i8(x: torch.Tensor, q: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None):
     """Per-token absmax int8 quantisation on the device: (q int8 [M, K], s fp32 [M])."""

@@ -258,9 +258,54 @@ def test_gate_up_with_adapters_through_swiglu(T, gdt):
     assert O.rel_max(out1.cpu().numpy(), want1) < BAND
 
 
+@pytest.mark.parametrize("T", [17, 135, 300])
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+def test_glu_layer_with_both_adapters_in_one_launch(T, xdt):
+    """A gate | up layer made by nq_fuse_glu (960 -> 2560 each, SwiGLU in the kernel's epilogue) with an adapter on both
+    projections, in the layer's single launch: against the oracle's projections, adapters and `swiglu`
+    (fused.mojo:337-353 orders them that way); B = 0 on both leaves the bits of the layer's plain forward wherever that
+    runs on the same kernel, no adapters at all always; shapes the kernel does not take, and an adapter on one projection only, are refused before any launch."""
+    from noeira_amd.qlinear import FusedGLU
+
+    rng = np.random.default_rng(3000 + T)
+    IN, H = 960, 2560
+    gate, up = _q4(rng, IN, H), _q4(rng, IN, H)
+    glu = FusedGLU(gate, up)
+    xf = rng.standard_normal((T, IN)).astype(np.float32)
+    x = torch.from_numpy(xf).cuda().to(xdt)
+    xh = x.float().cpu().numpy()
+    adg, adu = make(rng, IN, H, 16), make(rng, IN, H, 16)
+    for odt in (torch.float32, torch.bfloat16):
+        out = glu.forward_lora(x, adg[0], adu[0], out_dtype=odt)
+        assert out.shape == (T, H) and out.dtype == odt
+        want = O.swiglu(_oracle_proj(up, xh, adu), _oracle_proj(gate, xh, adg))
+        tol = BAND if odt == torch.float32 else 2.0 ** -8 + BAND
+        assert O.rel_max(out.float().cpu().numpy(), want) < tol, odt
+    base = glu.forward(x)
+    zg, zu = make(rng, IN, H, 16, zero_b=True)[0], make(rng, IN, H, 16, zero_b=True)[0]
+    zero = glu.forward_lora(x, zg, zu)
+    if T >= 135:  # (where the layer's plain forward runs on the same kernel; at 17 rows it takes another one)
+        assert torch.equal(zero.view(torch.int32), base.view(torch.int32))
+    else:
+        assert O.rel_max(zero.cpu().numpy(), base.cpu().numpy()) < BAND
+    assert torch.equal(glu.forward_lora(x, None, None).view(torch.int32), base.view(torch.int32))
+    # a sentinel under the output: every element is written
+    out = torch.full((T, H), float("nan"), dtype=torch.float32, device="cuda")
+    glu.forward_lora(x, adg[0], adu[0], out=out)
+    assert not torch.isnan(out).any()
+    with pytest.raises(L.NQError, match="both projections"):
+        glu.forward_lora(x, adg[0], None)
+    for bad_T in (1, 600):
+        xb = torch.from_numpy(rng.standard_normal((bad_T, IN)).astype(np.float32)).cuda().to(xdt)
+        keep = torch.full((bad_T, H), 7.0, dtype=torch.float32, device="cuda")
+        with pytest.raises(L.NQError, match="ahead of SwiGLU"):
+            glu.forward_lora(xb, adg[0], adu[0], out=keep)
+        assert bool((keep == 7.0).all())   # refused before anything ran
+
+
 def test_fused_adapters_outside_the_fast_kernel_and_errors():
     """Ranks and widths the 16-byte kernel does not take (R_PAD = 8, a part 70 wide) go part by part through the
-    general kernel, the SwiGLU through its own launch: the same values.  A GLU-fused layer refuses adapters."""
+    general kernel, the SwiGLU through its own launch: the same values.  A GLU-fused layer needs its glu_out."""
     from noeira_amd.qlinear import FusedGLU, FusedRows
 
     rng = np.random.default_rng(77)
