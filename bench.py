@@ -751,7 +751,7 @@ def sweep(skip_large=False):
     for M in (135, 1):
         run(f"ref text layer, 7 Q4_0 projections M={M}: q|k|v, o, gate|up+SwiGLU, down (4 launches, no adapters)",
             make_decoder_layer, "mfma", "bf16", M=M, adapters="none", calls=20)
-        run(f"ref text layer M={M} + rank-16 adapters on all seven, fused calls (8 launches)", make_decoder_layer, "mfma",
+        run(f"ref text layer M={M} + rank-16 adapters on all seven, fused calls ({7 if 17 <= M <= 511 else 8} launches)", make_decoder_layer, "mfma",
             "bf16", M=M, adapters="fused", calls=20)
         run(f"ref text layer M={M} + rank-16 adapters, per projection as the caller does (14 launches, SwiGLU not counted)",
             make_decoder_layer, "mfma", "bf16", M=M, adapters="per_projection", calls=20)
