@@ -308,13 +308,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvPara
     constexpr int XPT = (XCH + 64 * WAVES - 1) / (64 * WAVES);  // chunks of x per thread
     u32x4 xg[XPT];
     u32x4 wv[CPL], xv[CPL];
-#ifdef NQ_LAB_XDIRECT
-#pragma unroll
-    for (int j = 0; j < CPL; j++) xv[j] = xr[min(c0 + j * 64 + lane, nch - 1)];
-#else
 #pragma unroll
     for (int i = 0; i < XPT; i++) xg[i] = xr[min((int)threadIdx.x + i * 64 * WAVES, nch - 1)];
-#endif
 #pragma unroll
     for (int j = 0; j < CPL; j++) wv[j] = __builtin_nontemporal_load(wr + min(c0 + j * 64 + lane, nch - 1));
     // the epilogue's operands travel with the codes, raw: nothing is computed from them before the end
@@ -326,11 +321,6 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvPara
     if (p.bias)
         braw = (p.bias_dtype == NQ_DT_F32) ? reinterpret_cast<const uint32_t*>(p.bias)[rowc]
                                            : (uint32_t)reinterpret_cast<const uint16_t*>(p.bias)[rowc];
-#ifdef NQ_LAB_XDIRECT
-#pragma unroll
-    for (int j = 0; j < CPL; j++)
-        if (c0 + j * 64 + lane >= nch) xv[j] = (u32x4){0, 0, 0, 0};
-#else
 #pragma unroll
     for (int i = 0; i < XPT; i++) {
         const int c = (int)threadIdx.x + i * 64 * WAVES;
@@ -339,7 +329,6 @@ __global__ __launch_bounds__(64 * WAVES) void gemv8_row_kernel(const Fp8GemvPara
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < CPL; j++) xv[j] = xs[c0 + j * 64 + lane];
-#endif
 
     // lane holds D[4 (lane / 16) + r][lane % 16]: its diagonal entry, if any, is r = c % 4 where
     // c = lane % 16 and c / 4 == lane / 16
