@@ -80,6 +80,9 @@
 // stage's fragment reads at the head of the stage: 19.5 / 23.4 and 21.3 / 24.5; 256 x 256 tiles: 39 - 48).  Twice the
 // bytes from L2 per operation: with all CUs on such tiles a stage is 0.39 - 0.45 us for 0.22 - 0.25 of MFMA, 18 - 21 TB/s
 // into LDS over the chip.  launch_gemm8 takes the form of lowest estimated time (estimate_form).
+// (int8 is 2 - 2.5 us behind fp8 on this tile.  Its two phases of 16 short MFMAs per stage request the next phase's
+// fragments only six to nine MFMAs - about a hundred cycles - ahead; a form with two register sets, one per half of a
+// stage, each fragment requested a whole stage ahead, measured the same: 18.3 / 21.3 us at M = 512 / 1024.  Not kept.)
 //
 // LDS layout.  Row-major [256][128 B] with the eight 16-byte slots of a row
 // permuted by slot ^= ((row >> 1) + 6) & 7.  A 128-bit read is served in passes of
