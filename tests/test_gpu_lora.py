@@ -258,23 +258,23 @@ def test_gate_up_with_adapters_through_swiglu(T, gdt):
     assert O.rel_max(out1.cpu().numpy(), want1) < BAND
 
 
+@pytest.mark.parametrize("IN,H,R,pad", [(960, 2560, 16, 16), (2048, 2048, 5, 8)])
 @pytest.mark.parametrize("T", [17, 135, 300])
 @pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
-def test_glu_layer_with_both_adapters_in_one_launch(T, xdt):
-    """A gate | up layer made by nq_fuse_glu (960 -> 2560 each, SwiGLU in the kernel's epilogue) with an adapter on both
+def test_glu_layer_with_both_adapters_in_one_launch(T, xdt, IN, H, R, pad):
+    """A gate | up layer made by nq_fuse_glu (960 -> 2560 each with rank 16, 2048 -> 2048 with rank 5 stored as 8; SwiGLU in the kernel's epilogue) with an adapter on both
     projections, in the layer's single launch: against the oracle's projections, adapters and `swiglu`
     (fused.mojo:337-353 orders them that way); B = 0 on both leaves the bits of the layer's plain forward wherever that
     runs on the same kernel, no adapters at all always; shapes the kernel does not take, and an adapter on one projection only, are refused before any launch."""
     from noeira_amd.qlinear import FusedGLU
 
-    rng = np.random.default_rng(3000 + T)
-    IN, H = 960, 2560
+    rng = np.random.default_rng(3000 + T + IN)
     gate, up = _q4(rng, IN, H), _q4(rng, IN, H)
     glu = FusedGLU(gate, up)
     xf = rng.standard_normal((T, IN)).astype(np.float32)
     x = torch.from_numpy(xf).cuda().to(xdt)
     xh = x.float().cpu().numpy()
-    adg, adu = make(rng, IN, H, 16), make(rng, IN, H, 16)
+    adg, adu = make(rng, IN, H, R, pad=pad), make(rng, IN, H, R, pad=pad)
     for odt in (torch.float32, torch.bfloat16):
         out = glu.forward_lora(x, adg[0], adu[0], out_dtype=odt)
         assert out.shape == (T, H) and out.dtype == odt
@@ -282,7 +282,7 @@ def test_glu_layer_with_both_adapters_in_one_launch(T, xdt):
         tol = BAND if odt == torch.float32 else 2.0 ** -8 + BAND
         assert O.rel_max(out.float().cpu().numpy(), want) < tol, odt
     base = glu.forward(x)
-    zg, zu = make(rng, IN, H, 16, zero_b=True)[0], make(rng, IN, H, 16, zero_b=True)[0]
+    zg, zu = make(rng, IN, H, R, pad=pad, zero_b=True)[0], make(rng, IN, H, R, pad=pad, zero_b=True)[0]
     zero = glu.forward_lora(x, zg, zu)
     if T >= 135:  # (where the layer's plain forward runs on the same kernel; at 17 rows it takes another one)
         assert torch.equal(zero.view(torch.int32), base.view(torch.int32))
